@@ -1,0 +1,108 @@
+"""ctypes binding of ``libareal_hip.so`` (the C ABI declared in ``include/areal_hip.h``).
+
+There is no CPU implementation behind these entry points: if the library is missing or a
+tensor is not on a HIP device the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_double, c_int, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "libareal_hip.so"
+
+_STATUS = {
+    0: "ok",
+    -1: "bad argument",
+    -2: "pointer or leading dimension not suitably aligned",
+    -3: "workspace too small",
+    -4: "kernel launch failed",
+    -5: "unsupported shape",
+}
+
+P = c_void_p
+I64 = c_int64
+F = c_float
+D = c_double
+I = c_int
+SZ = c_size_t
+
+# name -> (restype, argtypes).  Must list every symbol declared in include/areal_hip.h.
+SIGNATURES: dict[str, tuple] = {
+    "areal_gemm_nt_bf16": (I, [P, I64, P, I64, P, I64, I64, I64, I64, I, P]),
+    "areal_lmhead_fwd_workspace_bytes": (SZ, [I64, I64, I64]),
+    "areal_lmhead_fwd": (
+        I,
+        [P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, P, P, P, P, SZ, P],
+    ),
+    "areal_lmhead_bwd_workspace_bytes": (SZ, [I64, I64, I64, I64]),
+    "areal_lmhead_bwd": (
+        I,
+        [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, P, I, I64, P, SZ, P],
+    ),
+    "areal_cast_f32_to_bf16": (I, [P, P, I64, P]),
+}
+
+_lib = None
+
+
+class ArealHipError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the kernel library, raising if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise ArealHipError(
+            f"{LIB_PATH} is missing: build it with `python -m areal_amd.build` "
+            "(areal_amd has no CPU fallback)"
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise ArealHipError(f"{what} failed: {_STATUS.get(status, status)} (code {status})")
+
+
+def ptr(t: torch.Tensor | None) -> c_void_p:
+    """Device pointer of a tensor (None -> NULL)."""
+    if t is None:
+        return c_void_p(0)
+    return c_void_p(t.data_ptr())
+
+
+def stream_ptr(device: torch.device) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def require_gpu(*tensors: torch.Tensor | None) -> torch.device:
+    """All given tensors must live on one HIP device; returns it."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ArealHipError(
+                "areal_amd kernels run on an MI355X only; got a tensor on "
+                f"{t.device} (there is no CPU fallback)"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ArealHipError(f"tensors on different devices: {dev} and {t.device}")
+    if dev is None:
+        raise ArealHipError("no tensor given")
+    return dev

@@ -1,0 +1,732 @@
+// Fused lm_head -> log-softmax -> label log-prob + entropy, forward and backward, for gfx950.
+//
+// One bf16 MFMA contraction D[i][j] = sum_k A[i][k] * B[j][k] (both operands k-contiguous)
+// serves all four matrix products of the path; only the epilogue differs:
+//   forward   : A = W [V,H],        B = hidden [T,H]      -> online softmax statistics
+//   recompute : A = W [V,H],        B = hidden [Tc,H]     -> dlogits (bf16, two layouts)
+//   dHidden   : A = W^T [H,V'],     B = dlogits [Tc,V']   -> bf16 store
+//   dWeight   : A = hidden^T [H,T'],B = dlogits^T [V,T']  -> fp32 accumulate
+// The vocabulary is put on the MFMA "A" side so that, in the accumulator layout of
+// v_mfma_f32_32x32x16_bf16 (lane -> column j, registers -> rows i), each lane owns one token
+// and 16 vocabulary entries per 32x32 block: the softmax reductions over the vocabulary run
+// inside a lane and the [T,V] logits never leave registers.
+//
+// Follows the algorithm of the reference's chunked LM head
+// (areal/models/mcore/vocab_parallel_head.py:564-735 forward, :737-938 backward) and the
+// backward formula of areal/utils/functional/vocab_parallel_kernels.py:99-137.
+#include "common.hpp"
+
+namespace {
+
+constexpr int TILE = 256;        // rows of A and of B per workgroup tile
+constexpr int BK = 64;           // k extent of one LDS stage
+constexpr int LDK = BK + 8;      // LDS row pitch in elements (144 B: conflict-free b128 reads)
+constexpr int OPER = TILE * LDK; // elements of one operand stage
+constexpr int NTHREADS = 256;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+struct GemmArgs {
+  const u16* A; int64_t lda; int M;   // A rows (index i)
+  const u16* B; int64_t ldb; int N;   // B rows (index j)
+  int K;                              // multiple of 8
+};
+
+// Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
+// the 8 XCDs, so the 32 workgroups resident on one XCD are id = xcd + 8*q for 32 consecutive
+// q. They are laid out as an RB x RS block of (B tiles) x (splits) so that they share operand
+// tiles through that XCD's L2.
+struct Sched {
+  int nbj;     // number of B tiles
+  int nai;     // number of A tiles
+  int S;       // splits of the A-tile range
+  int RB, RS;  // RB * RS == 32
+  int n_sb_j;  // super-blocks along j
+  int n_sb;    // total super-blocks
+};
+
+DEVI bool sched_decode(const Sched& sc, int id, int& bj, int& split) {
+  const int xcd = id & 7, q = id >> 3;
+  const int sb = (q >> 5) * 8 + xcd;
+  const int r = q & 31;
+  if (sb >= sc.n_sb) return false;
+  const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
+  bj = sbj * sc.RB + (r % sc.RB);
+  split = sbs * sc.RS + (r / sc.RB);
+  return bj < sc.nbj && split < sc.S;
+}
+
+static Sched make_sched(int nbj, int nai, int S) {
+  Sched sc;
+  sc.nbj = nbj; sc.nai = nai; sc.S = S;
+  sc.RS = S >= 8 ? 8 : (S >= 4 ? 4 : (S >= 2 ? 2 : 1));
+  sc.RB = 32 / sc.RS;
+  sc.n_sb_j = (nbj + sc.RB - 1) / sc.RB;
+  const int n_sb_s = (S + sc.RS - 1) / sc.RS;
+  sc.n_sb = sc.n_sb_j * n_sb_s;
+  return sc;
+}
+static int sched_grid(const Sched& sc) { return ((sc.n_sb + 7) / 8) * 8 * 32; }
+
+// ---------------------------------------------------------------------------------------
+// Main loop pieces
+// ---------------------------------------------------------------------------------------
+
+// Each thread moves 8 chunks of 16 B per operand per stage: chunk c = tid + 256*i covers
+// row c/8 (= 32*i + tid/8), k offset (c%8)*8.
+struct TileLoader {
+  const u32x4* ptr[8];
+  bool kvalid;  // recomputed per stage
+  DEVI void init(const u16* base, int64_t ld, int row0, int nrows, int tid) {
+    const int kc = (tid & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int row = row0 + i * 32 + (tid >> 3);
+      row = row < nrows ? row : nrows - 1;  // clamp: out-of-range rows are discarded later
+      ptr[i] = (const u32x4*)(base + (int64_t)row * ld + kc);
+    }
+  }
+};
+
+DEVI void global_load_stage(const TileLoader& ld, u32x4 (&regs)[8], int k0, int K, int tid) {
+  const bool ok = (k0 + (tid & 7) * 8 + 8) <= K;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (ok) v = ld.ptr[i][k0 >> 3];
+    regs[i] = v;
+  }
+}
+
+DEVI void lds_store_stage(u16* stage, const u32x4 (&regs)[8], int tid) {
+  u16* p = stage + (tid >> 3) * LDK + (tid & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) *(u32x4*)(p + i * 32 * LDK) = regs[i];
+}
+
+DEVI void mma_ksteps(const u16* pa, const u16* pb, f32x16 (&acc)[4][4], int s_begin, int s_end) {
+#pragma unroll
+  for (int s = s_begin; s < s_end; ++s) {
+    bf16x8 af[4], bf[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) af[a] = *(const bf16x8*)(pa + a * 32 * LDK + s * 16);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) bf[b] = *(const bf16x8*)(pb + b * 32 * LDK + s * 16);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b], 0, 0, 0);
+  }
+}
+
+// Workgroup (4 waves as 2x2, each wave a 128x128 block of 4x4 MFMA 32x32 blocks) sweeps the
+// A tiles [ai_begin, ai_end) against one fixed B tile. Epi::tile() consumes each finished
+// accumulator block.
+//
+// Accumulator layout inside a wave: acc[a][b][r] holds
+//   i = a*32 + 8*(r/4) + 4*(lane/32) + (r%4)   (A row inside the wave's 128)
+//   j = b*32 + (lane%32)                        (B row inside the wave's 128)
+template <class Epi>
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
+                                                          typename Epi::Params ep) {
+  __shared__ __attribute__((aligned(16))) u16 lds[2 * 2 * OPER];
+  int bj, split;
+  if (!sched_decode(sc, blockIdx.x, bj, split)) return;
+  const int ai_begin = (int)(((int64_t)split * sc.nai) / sc.S);
+  const int ai_end = (int)(((int64_t)(split + 1) * sc.nai) / sc.S);
+  if (ai_begin >= ai_end) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wa = wave >> 1, wb = wave & 1;
+  const int nk = (g.K + BK - 1) / BK;
+
+  TileLoader lb;
+  lb.init(g.B, g.ldb, bj * TILE, g.N, tid);
+
+  typename Epi::State st;
+  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
+
+  const int frag_off = (lane & 31) * LDK + (lane >> 5) * 8;
+
+  for (int ai = ai_begin; ai < ai_end; ++ai) {
+    TileLoader la;
+    la.init(g.A, g.lda, ai * TILE, g.M, tid);
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+    u32x4 ra[8], rb[8];
+    global_load_stage(la, ra, 0, g.K, tid);
+    global_load_stage(lb, rb, 0, g.K, tid);
+    __syncthreads();  // every wave is done reading LDS of the previous tile
+    lds_store_stage(lds, ra, tid);
+    lds_store_stage(lds + OPER, rb, tid);
+    if (nk > 1) {
+      global_load_stage(la, ra, BK, g.K, tid);
+      global_load_stage(lb, rb, BK, g.K, tid);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+      const int cur = kt & 1;
+      const u16* sA = lds + cur * 2 * OPER;
+      const u16* sB = sA + OPER;
+      const u16* pa = sA + wa * 128 * LDK + frag_off;
+      const u16* pb = sB + wb * 128 * LDK + frag_off;
+      mma_ksteps(pa, pb, acc, 0, 2);
+      if (kt + 1 < nk) {
+        u16* nA = lds + (cur ^ 1) * 2 * OPER;
+        lds_store_stage(nA, ra, tid);
+        lds_store_stage(nA + OPER, rb, tid);
+        if (kt + 2 < nk) {
+          global_load_stage(la, ra, (kt + 2) * BK, g.K, tid);
+          global_load_stage(lb, rb, (kt + 2) * BK, g.K, tid);
+        }
+      }
+      mma_ksteps(pa, pb, acc, 2, 4);
+      __syncthreads();
+    }
+    Epi::tile(st, ep, acc, ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
+  }
+  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// Epilogue 0: plain store (bf16 store, fp32 store, fp32 accumulate). Used for dHidden and
+// dWeight and for the stand-alone GEMM entry point. Output is indexed out[j * ldo + i]
+// (B row major, A row contiguous), so a lane's 4 consecutive i values are contiguous.
+// ---------------------------------------------------------------------------------------
+struct StoreEpi {
+  struct Params {
+    void* out; int64_t ldo; int M; int N;
+    int mode;  // 0: bf16 store, 1: fp32 store, 2: fp32 accumulate
+  };
+  struct State {};
+  static DEVI void begin(State&, const Params&, int, int, int, int) {}
+  static DEVI void end(State&, const Params&, int, int, int, int) {}
+  static DEVI void tile(State&, const Params& p, f32x16 (&acc)[4][4], int i0, int j0, int lane) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int j = j0 + b * 32 + (lane & 31);
+      if (j >= p.N) continue;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int i = i0 + a * 32 + 8 * rq + 4 * (lane >> 5);
+          if (i >= p.M) continue;
+          float x0 = acc[a][b][rq * 4 + 0], x1 = acc[a][b][rq * 4 + 1];
+          float x2 = acc[a][b][rq * 4 + 2], x3 = acc[a][b][rq * 4 + 3];
+          const int64_t off = (int64_t)j * p.ldo + i;
+          if (i + 3 < p.M) {
+            if (p.mode == 0) {
+              u32x2 v;
+              v[0] = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
+              v[1] = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
+              *(u32x2*)((u16*)p.out + off) = v;
+            } else {
+              f32x4* dst = (f32x4*)((float*)p.out + off);
+              f32x4 v = {x0, x1, x2, x3};
+              if (p.mode == 2) v += *dst;
+              *dst = v;
+            }
+          } else {
+            const float xs[4] = {x0, x1, x2, x3};
+            for (int e = 0; e < 4 && i + e < p.M; ++e) {
+              if (p.mode == 0) ((u16*)p.out)[off + e] = f32_to_bf16_bits(xs[e]);
+              else if (p.mode == 1) ((float*)p.out)[off + e] = xs[e];
+              else ((float*)p.out)[off + e] += xs[e];
+            }
+          }
+        }
+      }
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------
+// Epilogue 1: online softmax statistics over the vocabulary (forward).
+// Per token the lane keeps: running max m of the logits x, s = sum exp((x-m)/T),
+// q = sum ((x-m)/T * log2e) * exp((x-m)/T), the label's logit, min, sum x, sum x^2.
+// ---------------------------------------------------------------------------------------
+constexpr int NSTAT = 7;  // m, s, q, xlabel, min, sumx, sumx2
+
+struct FwdEpi {
+  struct Params {
+    const int64_t* labels; int T; int V;
+    float scale;   // logit_scale
+    float c2;      // inv_temperature * log2(e)
+    const float* bias;  // nullable, [V]
+    float* ws;     // [NSTAT][P][T]
+    int P;         // partial slots = 4 * S
+  };
+  struct State {
+    float m[4], s[4], q[4], xl[4], mn[4], sx[4], sx2[4];
+    int lab[4];
+  };
+  static DEVI void begin(State& st, const Params& p, int t0, int, int, int lane) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      st.m[b] = neg_inf(); st.s[b] = 0.f; st.q[b] = 0.f; st.xl[b] = 0.f;
+      st.mn[b] = pos_inf(); st.sx[b] = 0.f; st.sx2[b] = 0.f;
+      const int t = t0 + b * 32 + (lane & 31);
+      int64_t l = t < p.T ? p.labels[t] : -1;
+      st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+    }
+  }
+
+  template <bool EDGE>
+  static DEVI void tile_impl(State& st, const Params& p, f32x16 (&acc)[4][4], int v0, int lane) {
+    const int vl = v0 + 4 * (lane >> 5);
+    const bool affine = (p.scale != 1.0f) || (p.bias != nullptr);
+    if (affine) {
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
+          float bv = 0.f;
+          if (p.bias != nullptr && (!EDGE || v < p.V)) bv = p.bias[v];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) acc[a][b][r] = (acc[a][b][r] + bv) * p.scale;
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float x = acc[a][b][r];
+          if (EDGE) {
+            const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
+            if (v < p.V) {
+              tmax = fmaxf(tmax, x); tmin = fminf(tmin, x); sx += x; sx2 = fmaf(x, x, sx2);
+            }
+          } else {
+            tmax = fmaxf(tmax, x); tmin = fminf(tmin, x); sx += x; sx2 = fmaf(x, x, sx2);
+          }
+        }
+      st.mn[b] = fminf(st.mn[b], tmin);
+      st.sx[b] += sx;
+      st.sx2[b] += sx2;
+      const float m_old = st.m[b];
+      const float m_new = fmaxf(m_old, tmax);
+      if (m_new > neg_inf()) {
+        float s = 0.f, q = 0.f;
+        if (m_old > neg_inf()) {
+          const float dl = (m_old - m_new) * p.c2;
+          const float alpha = fast_exp2(dl);
+          q = alpha * fmaf(dl, st.s[b], st.q[b]);
+          s = alpha * st.s[b];
+        }
+        const float mc = m_new * p.c2;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float x = acc[a][b][r];
+            const float t = fmaf(x, p.c2, -mc);
+            const float e = fast_exp2(t);
+            if (EDGE) {
+              const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
+              if (v < p.V) { s += e; q = fmaf(t, e, q); }
+            } else {
+              s += e; q = fmaf(t, e, q);
+            }
+          }
+        st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
+      }
+      const int lab = st.lab[b];
+      const bool hit = (lab >= v0) && (lab < v0 + 128);
+      if (__builtin_amdgcn_ballot_w64(hit) != 0) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
+            if (v == lab) st.xl[b] = acc[a][b][r];
+          }
+      }
+    }
+  }
+
+  static DEVI void tile(State& st, const Params& p, f32x16 (&acc)[4][4], int i0, int, int lane) {
+    if (i0 + 128 <= p.V) tile_impl<false>(st, p, acc, i0, lane);
+    else tile_impl<true>(st, p, acc, i0, lane);
+  }
+
+  static DEVI void end(State& st, const Params& p, int t0, int split, int wa, int lane) {
+    const int slot = split * 4 + wa * 2 + (lane >> 5);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int t = t0 + b * 32 + (lane & 31);
+      if (t >= p.T) continue;
+      const int64_t PT = (int64_t)p.P * p.T;
+      float* w = p.ws + (int64_t)slot * p.T + t;
+      w[0 * PT] = st.m[b]; w[1 * PT] = st.s[b]; w[2 * PT] = st.q[b]; w[3 * PT] = st.xl[b];
+      w[4 * PT] = st.mn[b]; w[5 * PT] = st.sx[b]; w[6 * PT] = st.sx2[b];
+    }
+  }
+};
+
+// Merge the partial statistics of one token over all slots.
+__global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, int V,
+                                    float inv_temp, float c2, float* __restrict__ logprobs,
+                                    float* __restrict__ entropy, float* __restrict__ vmin,
+                                    float* __restrict__ vmax, float* __restrict__ vmean,
+                                    float* __restrict__ vnorm, float* __restrict__ row_max,
+                                    float* __restrict__ sum_exp) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const int64_t PT = (int64_t)P * T;
+  float M = neg_inf();
+  for (int p = 0; p < P; ++p) M = fmaxf(M, ws[(int64_t)p * T + t]);
+  float S = 0.f, Q = 0.f, xl = 0.f, mn = pos_inf();
+  double sx = 0.0, sx2 = 0.0;
+  for (int p = 0; p < P; ++p) {
+    const float* w = ws + (int64_t)p * T + t;
+    const float m = w[0];
+    if (m > neg_inf()) {
+      const float dl = (m - M) * c2;
+      const float alpha = exp2f(dl);
+      S += alpha * w[1 * PT];
+      Q += alpha * fmaf(dl, w[1 * PT], w[2 * PT]);
+    }
+    xl += w[3 * PT];
+    mn = fminf(mn, w[4 * PT]);
+    sx += (double)w[5 * PT];
+    sx2 += (double)w[6 * PT];
+  }
+  const float logS = logf(S);
+  if (logprobs) logprobs[t] = (xl - M) * inv_temp - logS;
+  if (entropy) entropy[t] = logS - (Q * LN2) / S;
+  if (vmin) vmin[t] = mn;
+  if (vmax) vmax[t] = M;
+  if (vmean) vmean[t] = (float)(sx / (double)V);
+  if (vnorm) vnorm[t] = (float)sqrt(sx2);
+  if (row_max) row_max[t] = M;
+  if (sum_exp) sum_exp[t] = S;
+}
+
+// ---------------------------------------------------------------------------------------
+// Epilogue 2: recompute logits and emit dlogits = (onehot - p) * g * invT * scale in bf16,
+// in two layouts: dl [Tc, ldv] (vocabulary contiguous) and dlT [V, ldt] (token contiguous).
+// ---------------------------------------------------------------------------------------
+struct BwdEpi {
+  struct Params {
+    const int64_t* labels;     // [Tc]
+    const float* row_max;      // [Tc]
+    const float* sum_exp;      // [Tc]
+    const float* grad;         // [Tc] dLoss/dlogprob
+    int T; int V;
+    float scale; float c2; float inv_temp;
+    const float* bias;
+    u16* dl; int64_t ldv;      // ldv >= V rounded to 8; columns [V, ldv) are written as zero
+    u16* dlT; int64_t ldt;     // ldt >= T rounded to 8; columns [T, ldt) are written as zero
+  };
+  struct State {
+    float nb[4], gs[4];
+    int lab[4];
+  };
+  static DEVI void begin(State& st, const Params& p, int t0, int, int, int lane) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int t = t0 + b * 32 + (lane & 31);
+      if (t < p.T) {
+        const int64_t l = p.labels[t];
+        st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+        st.nb[b] = -(p.row_max[t] * p.c2 + fast_log2(p.sum_exp[t]));
+        st.gs[b] = p.grad[t] * p.inv_temp * p.scale;
+      } else {
+        st.lab[b] = -1; st.nb[b] = 0.f; st.gs[b] = 0.f;
+      }
+    }
+  }
+  static DEVI void end(State&, const Params&, int, int, int, int) {}
+
+  static DEVI void tile(State& st, const Params& p, f32x16 (&acc)[4][4], int v0, int t0, int lane) {
+    const int vl = v0 + 4 * (lane >> 5);
+    const bool affine = (p.scale != 1.0f) || (p.bias != nullptr);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int t = t0 + b * 32 + (lane & 31);
+      const float nb = st.nb[b], gs = st.gs[b];
+      const int lab = st.lab[b];
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int vq = vl + a * 32 + 8 * rq;
+          u16 d[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int v = vq + e;
+            float x = acc[a][b][rq * 4 + e];
+            if (affine) {
+              float bv = 0.f;
+              if (p.bias != nullptr && v < p.V) bv = p.bias[v];
+              x = (x + bv) * p.scale;
+            }
+            const float pr = fast_exp2(fmaf(x, p.c2, nb));
+            float dv = -pr * gs;
+            if (v == lab) dv += gs;
+            if (v >= p.V || t >= p.T) dv = 0.f;
+            d[e] = f32_to_bf16_bits(dv);
+          }
+          if (t < p.T && vq < p.ldv) {
+            u32x2 pk;
+            pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
+            pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+            *(u32x2*)(p.dl + (int64_t)t * p.ldv + vq) = pk;
+          }
+          if (t < p.ldt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (vq + e < p.V) p.dlT[(int64_t)(vq + e) * p.ldt + t] = d[e];
+          }
+        }
+    }
+  }
+};
+
+// dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ldd. 64x64 tiles.
+__global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __restrict__ src,
+                                                                 int64_t lds_, int R, int C,
+                                                                 u16* __restrict__ dst,
+                                                                 int64_t ldd) {
+  __shared__ u16 tile[64][66];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? src[(int64_t)r * lds_ + c] : (u16)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < C && r < ldd) dst[(int64_t)c * ldd + r] = tile[tx][i];
+  }
+}
+
+__global__ void cast_f32_to_bf16_kernel(const float* __restrict__ src, u16* __restrict__ dst,
+                                        int64_t n) {
+  int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
+  for (; i + 3 < n; i += stride) {
+    const f32x4 v = *(const f32x4*)(src + i);
+    u32x2 o;
+    o[0] = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+    o[1] = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+    *(u32x2*)(dst + i) = o;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (int64_t j = n & ~(int64_t)3; j < n; ++j) dst[j] = f32_to_bf16_bits(src[j]);
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+int pick_splits(int nbj, int nai, int target_wgs) {
+  int S = 1;
+  while (nbj * S < target_wgs && S * 2 <= nai && S < 64) S *= 2;
+  return S;
+}
+
+template <class Epi>
+int launch_gemm(const GemmArgs& g, int S, const typename Epi::Params& ep, hipStream_t stream) {
+  const int nbj = (g.N + TILE - 1) / TILE, nai = (g.M + TILE - 1) / TILE;
+  if (nbj <= 0 || nai <= 0) return AREAL_OK;
+  if (S > nai) S = nai;
+  if (S < 1) S = 1;
+  const Sched sc = make_sched(nbj, nai, S);
+  hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g, sc,
+                     ep);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+int check_operand(const void* p, int64_t ld) {
+  if (p == nullptr) return AREAL_ERR_BAD_ARG;
+  if (!aligned16(p) || (ld % 8) != 0) return AREAL_ERR_ALIGNMENT;
+  return AREAL_OK;
+}
+
+}  // namespace
+
+// =======================================================================================
+// C ABI
+// =======================================================================================
+extern "C" {
+
+// out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]; A, B bf16; K % 8 == 0.
+int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, void* out,
+                       int64_t ldo, int64_t M, int64_t N, int64_t K, int out_mode,
+                       hipStream_t stream) {
+  if (M < 0 || N < 0 || K < 0 || out == nullptr || out_mode < 0 || out_mode > 2)
+    return AREAL_ERR_BAD_ARG;
+  if (M == 0 || N == 0) return AREAL_OK;
+  if (K % 8 != 0) return AREAL_ERR_ALIGNMENT;
+  int rc;
+  if ((rc = check_operand(A, lda)) != AREAL_OK) return rc;
+  if ((rc = check_operand(B, ldb)) != AREAL_OK) return rc;
+  if (out_mode == 0 ? (ldo % 4 != 0 || ((uintptr_t)out & 7)) : (ldo % 4 != 0 || !aligned16(out)))
+    return AREAL_ERR_ALIGNMENT;
+  GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K};
+  StoreEpi::Params ep{out, ldo, (int)M, (int)N, out_mode};
+  const int nai = (int)ceil_div_i64(M, TILE);
+  return launch_gemm<StoreEpi>(g, nai, ep, stream);
+}
+
+static int fwd_splits(int64_t T, int64_t V) {
+  const int nbj = (int)ceil_div_i64(T, TILE), nai = (int)ceil_div_i64(V, TILE);
+  return pick_splits(nbj, nai, 512);
+}
+
+size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  (void)H;
+  if (T <= 0 || V <= 0) return 0;
+  const int S = fwd_splits(T, V);
+  return (size_t)NSTAT * 4 * S * (size_t)T * sizeof(float);
+}
+
+// Forward. hidden [T,H] bf16, weight [V,H] bf16, labels [T] int64 (out-of-range labels give
+// a label logit of 0, like the reference's masked local target). Outputs are fp32 [T]; any
+// output pointer other than row_max / sum_exp may be null.
+int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
+                     const int64_t* labels, int64_t T, int64_t H, int64_t V,
+                     float inv_temperature, float logit_scale, float* logprobs, float* entropy,
+                     float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
+                     float* row_max, float* sum_exp, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
+  if (T < 0 || H <= 0 || V <= 0 || labels == nullptr) return AREAL_ERR_BAD_ARG;
+  if (!(inv_temperature > 0.f) || !(logit_scale > 0.f)) return AREAL_ERR_BAD_ARG;
+  if (T == 0) return AREAL_OK;
+  if (T > (1 << 30) || V > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  int rc;
+  if ((rc = check_operand(hidden, H)) != AREAL_OK) return rc;
+  if ((rc = check_operand(weight, H)) != AREAL_OK) return rc;
+  const size_t need = areal_lmhead_fwd_workspace_bytes(T, H, V);
+  if (workspace == nullptr || workspace_bytes < need) return AREAL_ERR_WORKSPACE;
+  const int S = fwd_splits(T, V);
+  GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H};
+  FwdEpi::Params ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
+                    (float*)workspace, 4 * S};
+  if ((rc = launch_gemm<FwdEpi>(g, S, ep, stream)) != AREAL_OK) return rc;
+  const int threads = 256;
+  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, threads)), dim3(threads),
+                     0, stream, (const float*)workspace, 4 * S, (int)T, (int)V, inv_temperature,
+                     inv_temperature * LOG2E, logprobs, entropy, vocab_min, vocab_max, vocab_mean,
+                     vocab_norm, row_max, sum_exp);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// Backward workspace: W^T [H, ldv] + per token chunk: hidden^T [H, ldt], dl [Tc, ldv],
+// dlT [V, ldt], all bf16.
+size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk) {
+  if (T <= 0 || H <= 0 || V <= 0 || token_chunk <= 0) return 0;
+  const int64_t Tc = token_chunk < T ? token_chunk : T;
+  const int64_t ldv = round_up_i64(V, 8), ldt = round_up_i64(Tc, 8);
+  int64_t elems = H * ldv + H * ldt + Tc * ldv + V * ldt;
+  return (size_t)elems * 2 + 4 * 256;  // slack for 256-byte sub-buffer alignment
+}
+
+// Backward. grad_logprobs [T] fp32 = dLoss/dlogprobs. Writes dhidden [T,H] bf16 and adds the
+// weight gradient into dweight_f32 [V,H] fp32 (overwrites it when accumulate == 0).
+int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
+                     const int64_t* labels, const float* row_max, const float* sum_exp,
+                     const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
+                     float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
+                     int accumulate, int64_t token_chunk, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
+  if (T < 0 || H <= 0 || V <= 0 || token_chunk <= 0) return AREAL_ERR_BAD_ARG;
+  if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr)
+    return AREAL_ERR_BAD_ARG;
+  if (dhidden == nullptr && dweight_f32 == nullptr) return AREAL_ERR_BAD_ARG;
+  if (T == 0) return AREAL_OK;
+  if (T > (1 << 30) || V > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  int rc;
+  if ((rc = check_operand(hidden, H)) != AREAL_OK) return rc;
+  if ((rc = check_operand(weight, H)) != AREAL_OK) return rc;
+  if (dhidden != nullptr && !aligned16(dhidden)) return AREAL_ERR_ALIGNMENT;
+  if (dweight_f32 != nullptr && !aligned16(dweight_f32)) return AREAL_ERR_ALIGNMENT;
+  if (workspace == nullptr ||
+      workspace_bytes < areal_lmhead_bwd_workspace_bytes(T, H, V, token_chunk))
+    return AREAL_ERR_WORKSPACE;
+
+  const int64_t Tc_max = token_chunk < T ? token_chunk : T;
+  const int64_t ldv = round_up_i64(V, 8), ldt = round_up_i64(Tc_max, 8);
+  auto carve = [](char*& p, int64_t bytes) {
+    char* r = (char*)(((uintptr_t)p + 255) & ~(uintptr_t)255);
+    p = r + bytes;
+    return (u16*)r;
+  };
+  char* wp = (char*)workspace;
+  u16* wT = carve(wp, H * ldv * 2);
+  u16* hT = carve(wp, H * ldt * 2);
+  u16* dl = carve(wp, Tc_max * ldv * 2);
+  u16* dlT = carve(wp, V * ldt * 2);
+
+  const float c2 = inv_temperature * LOG2E;
+  if (dhidden != nullptr) {
+    // W^T [H, ldv]: rows = h, columns = v (zero padded to ldv).
+    hipLaunchKernelGGL(transpose_pad_bf16_kernel,
+                       dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
+                       dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
+    AREAL_CHECK_LAUNCH();
+  }
+  for (int64_t t0 = 0; t0 < T; t0 += Tc_max) {
+    const int64_t Tc = (T - t0) < Tc_max ? (T - t0) : Tc_max;
+    const int64_t ldt_c = round_up_i64(Tc, 8);
+    const u16* hid_c = (const u16*)hidden + t0 * H;
+    // 1. recompute logits of the chunk, emit dlogits in both layouts
+    {
+      GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H};
+      BwdEpi::Params ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
+                        (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
+      const int nbj = (int)ceil_div_i64(Tc, TILE), nai = (int)ceil_div_i64(V, TILE);
+      if ((rc = launch_gemm<BwdEpi>(g, pick_splits(nbj, nai, 512), ep, stream)) != AREAL_OK)
+        return rc;
+    }
+    // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
+    if (dhidden != nullptr) {
+      GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv};
+      StoreEpi::Params ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc, 0};
+      if ((rc = launch_gemm<StoreEpi>(g, (int)ceil_div_i64(H, TILE), ep, stream)) != AREAL_OK)
+        return rc;
+    }
+    // 3. dWeight[v, h] += sum_t dlT[v, t] * hidden^T[h, t]
+    if (dweight_f32 != nullptr) {
+      hipLaunchKernelGGL(transpose_pad_bf16_kernel,
+                         dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldt_c, 64)),
+                         dim3(256), 0, stream, hid_c, H, (int)Tc, (int)H, hT, ldt_c);
+      AREAL_CHECK_LAUNCH();
+      GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c};
+      StoreEpi::Params ep{dweight_f32, H, (int)H, (int)V, (accumulate || t0 > 0) ? 2 : 1};
+      if ((rc = launch_gemm<StoreEpi>(g, (int)ceil_div_i64(H, TILE), ep, stream)) != AREAL_OK)
+        return rc;
+    }
+  }
+  return AREAL_OK;
+}
+
+int areal_cast_f32_to_bf16(const float* src, void* dst, int64_t n, hipStream_t stream) {
+  if (n < 0 || (n > 0 && (src == nullptr || dst == nullptr))) return AREAL_ERR_BAD_ARG;
+  if (n == 0) return AREAL_OK;
+  if (!aligned16(src) || ((uintptr_t)dst & 7)) return AREAL_ERR_ALIGNMENT;
+  int64_t blocks = ceil_div_i64(n, 256 * 4);
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, src,
+                     (u16*)dst, n);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+}  // extern "C"

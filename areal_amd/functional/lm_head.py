@@ -1,0 +1,191 @@
+"""Fused lm_head -> log-softmax -> label log-prob + entropy on MI355X.
+
+Host-side counterpart of the reference's chunked LM head
+(``areal/models/mcore/vocab_parallel_head.py:560-938`` and its wrapper
+``chunked_lm_head_logprobs_entropy`` at ``:941-982``): same outputs
+(``ChunkedLMHeadOutput``), same saved state (row max and sum of exponentials per token, never
+a ``[T, V]`` tensor), same error behaviour.  The arithmetic runs in the HIP kernels of
+``csrc/lmhead.hip`` through the C ABI.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import NamedTuple
+
+import torch
+
+from areal_amd import _lib
+
+# Default budget for the backward workspace (bf16 dlogits of one token chunk in two layouts,
+# plus transposed operands).  An MI355X has 288 GB of HBM, so one chunk normally covers the
+# whole micro-batch.
+DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
+
+
+class ChunkedLMHeadOutput(NamedTuple):
+    """Per-token outputs produced without materialising ``[T, V]`` logits.
+
+    Field names and order follow ``vocab_parallel_head.py:497-506``.
+    """
+
+    logprobs: torch.Tensor
+    entropy: torch.Tensor
+    vocab_min_logits: torch.Tensor
+    vocab_max_logits: torch.Tensor
+    vocab_mean_logits: torch.Tensor
+    vocab_norm_logits: torch.Tensor
+
+
+def default_token_chunk(T: int, H: int, V: int, budget: int = DEFAULT_BWD_WORKSPACE_BYTES) -> int:
+    """Largest token chunk (multiple of 256) whose backward workspace fits ``budget``."""
+    per_token = 2 * (2 * V + H) + 64
+    fixed = 2 * H * (V + 8)
+    chunk = max((budget - fixed) // per_token, 256)
+    chunk = (chunk // 256) * 256
+    return int(min(max(chunk, 256), max(T, 1)))
+
+
+class _FusedLMHead(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, labels, temperature, logit_scale, token_chunk):
+        lib = _lib.load()
+        dev = _lib.require_gpu(hidden, weight, labels, bias)
+        H = hidden.size(-1)
+        V = weight.size(0)
+        hidden_2d = hidden.reshape(-1, H).contiguous()
+        weight_c = weight.contiguous()
+        labels_1d = labels.reshape(-1).to(torch.int64).contiguous()
+        T = hidden_2d.size(0)
+        bias_f = bias.detach().float().contiguous() if bias is not None else None
+
+        outs = [torch.empty(labels.shape, dtype=torch.float32, device=dev) for _ in range(6)]
+        outs += [torch.empty(T, dtype=torch.float32, device=dev) for _ in range(2)]
+        logprobs, entropy, vmin, vmax, vmean, vnorm, row_max, sum_exp = outs
+        if T > 0:
+            nbytes = lib.areal_lmhead_fwd_workspace_bytes(T, H, V)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            rc = lib.areal_lmhead_fwd(
+                _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(bias_f), _lib.ptr(labels_1d),
+                T, H, V, 1.0 / temperature, logit_scale,
+                *[_lib.ptr(o) for o in outs],
+                _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+            )
+            _lib.check(rc, "areal_lmhead_fwd")
+
+        ctx.save_for_backward(hidden_2d, weight_c, labels_1d, row_max, sum_exp)
+        ctx.bias_f = bias_f
+        ctx.temperature = temperature
+        ctx.logit_scale = logit_scale
+        ctx.token_chunk = token_chunk
+        ctx.hidden_shape = hidden.shape
+        ctx.weight_dtype = weight.dtype
+        ctx.set_materialize_grads(False)
+        ctx.mark_non_differentiable(entropy, vmin, vmax, vmean, vnorm)
+        return tuple(outs[:6])
+
+    @staticmethod
+    def backward(ctx, grad_logprobs, *unused):
+        hidden_2d, weight_c, labels_1d, row_max, sum_exp = ctx.saved_tensors
+        need_h, need_w, need_b = ctx.needs_input_grad[:3]
+        if need_b:
+            raise NotImplementedError("gradient of the lm_head bias is not implemented")
+        if grad_logprobs is None or not (need_h or need_w):
+            return (None,) * 7
+        lib = _lib.load()
+        dev = hidden_2d.device
+        T, H = hidden_2d.shape
+        V = weight_c.size(0)
+        g = grad_logprobs.reshape(-1).to(torch.float32).contiguous()
+        dh = torch.empty_like(hidden_2d) if need_h else None
+        dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if need_w else None
+        if T == 0:
+            if dw32 is not None:
+                dw32.zero_()
+        else:
+            chunk = ctx.token_chunk or default_token_chunk(T, H, V)
+            nbytes = lib.areal_lmhead_bwd_workspace_bytes(T, H, V, chunk)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            rc = lib.areal_lmhead_bwd(
+                _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(ctx.bias_f),
+                _lib.ptr(labels_1d), _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(g),
+                T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
+                _lib.ptr(dh), _lib.ptr(dw32), 0, chunk,
+                _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+            )
+            _lib.check(rc, "areal_lmhead_bwd")
+        dw = None
+        if dw32 is not None:
+            if ctx.weight_dtype == torch.float32:
+                dw = dw32
+            else:
+                dw = torch.empty((V, H), dtype=ctx.weight_dtype, device=dev)
+                rc = lib.areal_cast_f32_to_bf16(
+                    _lib.ptr(dw32), _lib.ptr(dw), dw32.numel(), _lib.stream_ptr(dev)
+                )
+                _lib.check(rc, "areal_cast_f32_to_bf16")
+        if dh is not None:
+            dh = dh.view(ctx.hidden_shape)
+        return dh, dw, None, None, None, None, None
+
+
+def fused_lm_head_logprobs_entropy(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    temperature: float = 1.0,
+    vocab_chunk: int | None = None,
+    logit_scale: float = 1.0,
+    bias: torch.Tensor | None = None,
+    token_chunk: int | None = None,
+) -> ChunkedLMHeadOutput:
+    """Label log-probabilities, entropy and vocabulary statistics of ``hidden @ weight.T``.
+
+    Args:
+        hidden: ``[..., H]`` bf16 final hidden states (packed tokens).
+        weight: ``[V, H]`` bf16 lm_head weight (row = vocabulary id).
+        labels: ``[...]`` integer labels, leading dimensions matching ``hidden``.
+        temperature: softmax temperature (> 0).
+        vocab_chunk: accepted for signature compatibility; the kernel sweeps the vocabulary
+            in 256-row tiles whatever its value.
+        logit_scale: multiplier applied to the logits before the softmax (> 0).
+        bias: optional ``[V]`` bias added to the logits.
+        token_chunk: tokens per backward chunk (bounds the bf16 dlogits workspace);
+            ``None`` picks the largest chunk within ``DEFAULT_BWD_WORKSPACE_BYTES``.
+
+    Gradient flows through ``logprobs`` only (to ``hidden`` and ``weight``), as in the
+    reference (``vocab_parallel_head.py:732-734``).
+    """
+    del vocab_chunk
+    if not math.isfinite(temperature) or temperature <= 0:
+        raise ValueError(f"temperature must be positive, got {temperature}")
+    if not math.isfinite(logit_scale) or logit_scale <= 0:
+        raise ValueError(f"logit_scale must be positive, got {logit_scale}")
+    if token_chunk is not None and token_chunk <= 0:
+        raise ValueError(f"chunk_size must be positive, got {token_chunk}")
+    if hidden.dtype != weight.dtype:
+        raise ValueError(
+            "chunked LM Head requires matching hidden and weight dtypes, got "
+            f"{hidden.dtype} and {weight.dtype}"
+        )
+    if weight.ndim != 2 or hidden.size(-1) != weight.size(1):
+        raise ValueError(
+            f"weight must be [V, H] with H == hidden.size(-1); got {tuple(weight.shape)} "
+            f"and {tuple(hidden.shape)}"
+        )
+    if hidden.numel() // max(hidden.size(-1), 1) != labels.numel():
+        raise ValueError(
+            "LM Head hidden leading dimensions must match labels: "
+            f"got {tuple(hidden.shape)} and {tuple(labels.shape)}"
+        )
+    if hidden.dtype != torch.bfloat16:
+        raise ValueError(f"the fused LM head computes in bf16; got {hidden.dtype}")
+    if hidden.size(-1) % 8 != 0:
+        raise ValueError(f"hidden size must be a multiple of 8, got {hidden.size(-1)}")
+    if bias is not None and bias.shape != (weight.size(0),):
+        raise ValueError(f"bias must have shape ({weight.size(0)},), got {tuple(bias.shape)}")
+    values = _FusedLMHead.apply(
+        hidden, weight, bias, labels, float(temperature), float(logit_scale), token_chunk
+    )
+    return ChunkedLMHeadOutput(*values)
