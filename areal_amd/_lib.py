@@ -44,7 +44,51 @@ SIGNATURES: dict[str, tuple] = {
         [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, P, I, I64, P, SZ, P],
     ),
     "areal_cast_f32_to_bf16": (I, [P, P, I64, P]),
+    "areal_logits_logprobs_entropy_fwd": (I, [P, I, I64, P, I64, I64, F, P, P, P, P]),
+    "areal_logits_logprobs_entropy_bwd": (
+        I,
+        [P, I, I64, P, I64, I64, F, P, P, P, P, P, I64, P],
+    ),
+    "areal_actor_loss_workspace_bytes": (SZ, [I64, I64]),
+    "areal_actor_loss": (
+        I,
+        [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
+    ),
+    "areal_actor_loss_grad": (I, [P, P, P, P, I64, P]),
+    "areal_gae_workspace_bytes": (SZ, [I64]),
+    "areal_gae_packed": (
+        I,
+        [P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, SZ, P],
+    ),
+    "areal_group_norm_workspace_bytes": (SZ, [I64, I64]),
+    "areal_group_norm": (
+        I,
+        [P, P, I64, P, P, I64, I64, I, I, I, I, I, D, P, P, SZ, P],
+    ),
+    "areal_masked_norm_workspace_bytes": (SZ, [I64]),
+    "areal_masked_norm": (I, [P, P, I64, I, D, P, P, SZ, P]),
 }
+
+
+class LossConfig(ctypes.Structure):
+    """Mirror of ``areal_loss_config`` in include/areal_hip.h (a host-side struct)."""
+
+    _fields_ = [
+        ("loss_kind", c_int),
+        ("clip_lo", c_float),
+        ("clip_hi", c_float),
+        ("has_c_clip", c_int),
+        ("c_clip", c_float),
+        ("seq_is", c_int),
+        ("rs_enabled", c_int),
+        ("rs_seq_level", c_int),
+        ("rs_clamp", c_int),
+        ("rs_metric", c_int),
+        ("rs_agg", c_int),
+        ("rs_upper", c_float),
+        ("rs_has_lower", c_int),
+        ("rs_lower", c_float),
+    ]
 
 _lib = None
 
@@ -75,6 +119,11 @@ def load() -> ctypes.CDLL:
 def check(status: int, what: str) -> None:
     if status != 0:
         raise ArealHipError(f"{what} failed: {_STATUS.get(status, status)} (code {status})")
+
+
+def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """Scratch buffer owned by the caller (PyTorch's caching allocator)."""
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
 
 
 def ptr(t: torch.Tensor | None) -> c_void_p:

@@ -1,0 +1,577 @@
+// Packed-sequence GAE (segmented reverse scan) and masked group/batch normalisation.
+//
+// GAE follows areal/trainer/ppo/gae.py:10-36 (token-level recurrence on padded [bs, L]
+// tensors); here it runs on the packed layout (or on the padded layout seen as bs sequences of
+// length L). Normalisation follows areal/utils/data.py:1382-1637 (class Normalization) and
+// areal/utils/functional/functional.py:16-53 (masked_normalization).
+//
+// GAE as a scan.  Going right to left, the carried state is (A, nv) = (last advantage, next
+// value) and token t applies the affine map
+//     A'  = A*((1-m) + c*m) + nv*(gamma*m) + (r - v)*m        c = gamma*lambda_seq
+//     nv' = nv*(1-m) + v*m
+// while the last token of a sequence applies the constant map (A', nv') = (0, no_eos ? v : 0).
+// Affine maps compose associatively and constant maps absorb whatever lies to their right, so
+// one unsegmented suffix scan over the whole packed array gives every sequence its own
+// recurrence. Maps are held in fp64 (five coefficients); outputs are rounded to fp32.
+#include "common.hpp"
+
+namespace {
+
+constexpr int GAE_THREADS = 256;
+constexpr int GAE_ITEMS = 4;
+constexpr int GAE_TILE = GAE_THREADS * GAE_ITEMS;
+
+struct Map {
+  double a11, a12, a22, b1, b2;
+};
+DEVI Map map_identity() { return Map{1.0, 0.0, 1.0, 0.0, 0.0}; }
+// (f o g): apply g first, then f.
+DEVI Map compose(const Map& f, const Map& g) {
+  Map r;
+  r.a11 = f.a11 * g.a11;
+  r.a12 = f.a11 * g.a12 + f.a12 * g.a22;
+  r.a22 = f.a22 * g.a22;
+  r.b1 = f.a11 * g.b1 + f.a12 * g.b2 + f.b1;
+  r.b2 = f.a22 * g.b2 + f.b2;
+  return r;
+}
+DEVI Map shfl_down_map(const Map& m, int d) {
+  Map r;
+  r.a11 = __shfl_down(m.a11, d, 64); r.a12 = __shfl_down(m.a12, d, 64);
+  r.a22 = __shfl_down(m.a22, d, 64); r.b1 = __shfl_down(m.b1, d, 64);
+  r.b2 = __shfl_down(m.b2, d, 64);
+  return r;
+}
+
+struct GaeArgs {
+  const float* rewards;
+  const float* values;
+  const float* mask;         // float 0/1
+  const int32_t* cu;         // [n_seqs+1] or null when uniform_len > 0
+  const uint8_t* no_eos;     // [n_seqs] or null (all false)
+  const float* lam_seq;      // [n_seqs] per-sequence lambda or null
+  int64_t n;
+  int n_seqs;
+  int64_t uniform_len;
+  float discount;
+  float lam;
+  float* adv;
+  float* ret;
+};
+
+DEVI int gae_seq_of(const GaeArgs& g, int64_t t) {
+  if (g.uniform_len > 0) return (int)(t / g.uniform_len);
+  int lo = 0, hi = g.n_seqs;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)g.cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+DEVI int64_t gae_seq_end(const GaeArgs& g, int s) {
+  return g.uniform_len > 0 ? (int64_t)(s + 1) * g.uniform_len : (int64_t)g.cu[s + 1];
+}
+
+// Maps of the thread's GAE_ITEMS consecutive tokens starting at t0 (identity beyond n).
+DEVI void load_maps(const GaeArgs& g, int64_t t0, Map (&mp)[GAE_ITEMS], float (&v)[GAE_ITEMS]) {
+  if (t0 >= g.n) {
+#pragma unroll
+    for (int i = 0; i < GAE_ITEMS; ++i) { mp[i] = map_identity(); v[i] = 0.f; }
+    return;
+  }
+  int s = gae_seq_of(g, t0);
+  int64_t e = gae_seq_end(g, s);
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) {
+    const int64_t t = t0 + i;
+    if (t >= g.n) { mp[i] = map_identity(); v[i] = 0.f; continue; }
+    while (t >= e && s + 1 < g.n_seqs) { ++s; e = gae_seq_end(g, s); }
+    const float val = g.values[t];
+    v[i] = val;
+    if (t == e - 1) {
+      const bool ne = g.no_eos != nullptr && g.no_eos[s] != 0;
+      mp[i] = Map{0.0, 0.0, 0.0, 0.0, ne ? (double)val : 0.0};
+    } else {
+      const double m = (double)g.mask[t];
+      const double lam = g.lam_seq != nullptr ? (double)g.lam_seq[s] : (double)g.lam;
+      const double c = (double)g.discount * lam;
+      Map f;
+      f.a11 = (1.0 - m) + c * m;
+      f.a12 = (double)g.discount * m;
+      f.a22 = 1.0 - m;
+      f.b1 = ((double)g.rewards[t] - (double)val) * m;
+      f.b2 = (double)val * m;
+      mp[i] = f;
+    }
+  }
+}
+
+// Composition of the thread's maps: leftmost applied last.
+DEVI Map thread_total(const Map (&mp)[GAE_ITEMS]) {
+  Map r = mp[GAE_ITEMS - 1];
+#pragma unroll
+  for (int i = GAE_ITEMS - 2; i >= 0; --i) r = compose(mp[i], r);
+  return r;
+}
+
+// Inclusive suffix scan over the block: returns for each thread the composition of the maps
+// of threads tid..blockDim-1 (thread tid applied last). smem: [4] wave totals.
+DEVI Map block_suffix_scan(Map mine, Map* smem, Map& block_total) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  Map acc = mine;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const Map other = shfl_down_map(acc, d);
+    if (lane + d < 64) acc = compose(acc, other);
+  }
+  __syncthreads();
+  if (lane == 0) smem[w] = acc;  // wave total (lanes 0..63)
+  __syncthreads();
+  const int nw = blockDim.x >> 6;
+  Map right = map_identity();
+  for (int i = nw - 1; i > w; --i) right = compose(smem[i], right);
+  Map tot = right;
+  for (int i = w; i >= 0; --i) tot = compose(smem[i], tot);
+  block_total = tot;
+  return compose(acc, right);
+}
+
+__global__ __launch_bounds__(GAE_THREADS) void gae_block_total_kernel(GaeArgs g, Map* totals) {
+  __shared__ Map smem[4];
+  const int64_t t0 = (int64_t)blockIdx.x * GAE_TILE + (int64_t)threadIdx.x * GAE_ITEMS;
+  Map mp[GAE_ITEMS];
+  float v[GAE_ITEMS];
+  load_maps(g, t0, mp, v);
+  Map total;
+  block_suffix_scan(thread_total(mp), smem, total);
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+// carry[b] = state (A, nv) entering block b from its right = (F_{b+1} o F_{b+2} o ...)(0, 0).
+__global__ __launch_bounds__(GAE_THREADS) void gae_carry_kernel(const Map* totals, int nblocks,
+                                                                double* carry) {
+  __shared__ Map smem[4];
+  const int per = (nblocks + GAE_THREADS - 1) / GAE_THREADS;
+  const int b0 = threadIdx.x * per;
+  // composition of this thread's blocks b0 .. b0+per-1
+  Map mine = map_identity();
+  for (int i = per - 1; i >= 0; --i) {
+    const int b = b0 + i;
+    if (b < nblocks) mine = compose(totals[b], mine);
+  }
+  Map total;
+  const Map incl = block_suffix_scan(mine, smem, total);
+  // exclusive: composition of everything right of this thread's range
+  Map excl;
+  {
+    // incl = mine o right  =>  right is what enters after this thread's range; recompute it
+    // from the neighbour: thread tid+1's inclusive scan equals our exclusive one.
+    __shared__ Map all[GAE_THREADS];
+    all[threadIdx.x] = incl;
+    __syncthreads();
+    excl = threadIdx.x + 1 < blockDim.x ? all[threadIdx.x + 1] : map_identity();
+  }
+  // walk this thread's blocks right to left
+  double A = excl.b1, nv = excl.b2;  // map applied to the zero state
+  for (int i = per - 1; i >= 0; --i) {
+    const int b = b0 + i;
+    if (b >= nblocks) continue;
+    carry[2 * b] = A;
+    carry[2 * b + 1] = nv;
+    const Map f = totals[b];
+    const double A2 = f.a11 * A + f.a12 * nv + f.b1;
+    const double nv2 = f.a22 * nv + f.b2;
+    A = A2; nv = nv2;
+  }
+}
+
+__global__ __launch_bounds__(GAE_THREADS) void gae_apply_kernel(GaeArgs g, const double* carry) {
+  __shared__ Map smem[4];
+  __shared__ Map all[GAE_THREADS];
+  const int64_t t0 = (int64_t)blockIdx.x * GAE_TILE + (int64_t)threadIdx.x * GAE_ITEMS;
+  Map mp[GAE_ITEMS];
+  float v[GAE_ITEMS];
+  load_maps(g, t0, mp, v);
+  Map total;
+  const Map incl = block_suffix_scan(thread_total(mp), smem, total);
+  all[threadIdx.x] = incl;
+  __syncthreads();
+  const Map excl = threadIdx.x + 1 < blockDim.x ? all[threadIdx.x + 1] : map_identity();
+  const double A0 = carry[2 * blockIdx.x], nv0 = carry[2 * blockIdx.x + 1];
+  double A = excl.a11 * A0 + excl.a12 * nv0 + excl.b1;
+  double nv = excl.a22 * nv0 + excl.b2;
+#pragma unroll
+  for (int i = GAE_ITEMS - 1; i >= 0; --i) {
+    const int64_t t = t0 + i;
+    if (t >= g.n) continue;
+    const Map& f = mp[i];
+    const double A2 = f.a11 * A + f.a12 * nv + f.b1;
+    const double nv2 = f.a22 * nv + f.b2;
+    A = A2; nv = nv2;
+    const float a = (float)A;
+    g.adv[t] = a;
+    g.ret[t] = a + v[i];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Normalisation
+// ---------------------------------------------------------------------------------------
+constexpr int NORM_THREADS = 256;
+enum { LEVEL_NONE = 0, LEVEL_BATCH = 1, LEVEL_GROUP = 2 };
+
+struct NormArgs {
+  const float* x;
+  const float* mask;       // nullable
+  int64_t n;
+  const int64_t* goff;     // [G+1] element offsets of the groups (cover [0, n))
+  const int64_t* grows;    // [G] rows in each group (for the singleton rules)
+  int G;
+  int tail_group;          // index of the group holding ungrouped tail rows, or -1
+  int nsplit;              // blocks per group
+  int mean_level, std_level;
+  int leave1out, unbiased;
+  double eps;
+  double* part;            // [3][G][nsplit]: count, sum, sum of squares
+  float* out;
+};
+
+DEVI double block_sum_d(double v, double* smem) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[w] = v;
+  __syncthreads();
+  double r = 0.0;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i];
+  return r;
+}
+
+DEVI void split_range(const NormArgs& a, int g, int sp, int64_t& lo, int64_t& hi) {
+  const int64_t g0 = a.goff[g], g1 = a.goff[g + 1];
+  const int64_t len = g1 - g0;
+  const int64_t per = (len + a.nsplit - 1) / a.nsplit;
+  lo = g0 + (int64_t)sp * per;
+  hi = lo + per;
+  if (hi > g1) hi = g1;
+  if (lo > g1) lo = g1;
+}
+
+// Sum of one partial array over all splits of group g (fixed order).
+DEVI double group_partial(const NormArgs& a, int which, int g) {
+  double r = 0.0;
+  const double* p = a.part + ((int64_t)which * a.G + g) * a.nsplit;
+  for (int i = 0; i < a.nsplit; ++i) r += p[i];
+  return r;
+}
+// Sum over every group and split, computed cooperatively by the block.
+DEVI double batch_partial(const NormArgs& a, int which, double* smem) {
+  double r = 0.0;
+  const double* p = a.part + (int64_t)which * a.G * a.nsplit;
+  const int64_t tot = (int64_t)a.G * a.nsplit;
+  for (int64_t i = threadIdx.x; i < tot; i += blockDim.x) r += p[i];
+  return block_sum_d(r, smem);
+}
+
+struct MeanCtx {
+  int level;      // LEVEL_*
+  bool identity;  // singleton group with leave-one-out: mean = x
+  bool zero;      // tail group, or leave-one-out with count <= 1, or empty: mean = 0
+  bool loo;
+  double cnt, sum;
+};
+
+DEVI MeanCtx make_mean_ctx(const NormArgs& a, int g, double* smem) {
+  MeanCtx c;
+  c.level = a.mean_level; c.identity = false; c.zero = false; c.loo = a.leave1out != 0;
+  c.cnt = 0.0; c.sum = 0.0;
+  if (a.mean_level == LEVEL_BATCH) {
+    c.cnt = batch_partial(a, 0, smem);
+    c.sum = batch_partial(a, 1, smem);
+  } else if (a.mean_level == LEVEL_GROUP) {
+    if (g == a.tail_group) { c.zero = true; return c; }
+    if (a.grows[g] == 1 && c.loo) { c.identity = true; return c; }
+    c.cnt = group_partial(a, 0, g);
+    c.sum = group_partial(a, 1, g);
+  } else {
+    c.zero = true;
+    return c;
+  }
+  if (c.loo) { if (c.cnt <= 1.0) c.zero = true; }
+  else if (c.cnt == 0.0) c.zero = true;
+  return c;
+}
+
+// Mean seen by one element, as the reference stores it: group-level means are rounded to
+// fp32 (they are written into a zeros_like(x) tensor), batch-level means stay fp64.
+DEVI double elem_mean(const MeanCtx& c, float x, float m, bool has_mask) {
+  double mean;
+  if (c.zero) mean = 0.0;
+  else if (c.identity) mean = (double)x;
+  else if (!c.loo) mean = c.sum / c.cnt;
+  else if (!has_mask) mean = (c.sum - (double)x) / (c.cnt - 1.0);
+  else {
+    const double md = (double)m;
+    if (md > 0.0) {
+      double den = c.cnt - md;
+      if (den < 1.0) den = 1.0;
+      mean = (c.sum - (double)x * md) / den;
+    } else {
+      mean = c.sum / c.cnt;
+    }
+  }
+  if (c.level != LEVEL_BATCH) mean = (double)(float)mean;
+  return mean;
+}
+
+// pass 1: count and sum per (group, split)
+__global__ __launch_bounds__(NORM_THREADS) void norm_stats1_kernel(NormArgs a) {
+  __shared__ double smem[4];
+  const int g = blockIdx.x, sp = blockIdx.y;
+  int64_t lo, hi;
+  split_range(a, g, sp, lo, hi);
+  double cnt = 0.0, sum = 0.0;
+  for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const double m = a.mask ? (double)a.mask[i] : 1.0;
+    cnt += m;
+    sum += (double)a.x[i] * m;
+  }
+  cnt = block_sum_d(cnt, smem);
+  sum = block_sum_d(sum, smem);
+  if (threadIdx.x == 0) {
+    a.part[((int64_t)0 * a.G + g) * a.nsplit + sp] = cnt;
+    a.part[((int64_t)1 * a.G + g) * a.nsplit + sp] = sum;
+  }
+}
+
+// pass 2: sum of squared masked deviations per (group, split)
+__global__ __launch_bounds__(NORM_THREADS) void norm_stats2_kernel(NormArgs a) {
+  __shared__ double smem[4];
+  const int g = blockIdx.x, sp = blockIdx.y;
+  const MeanCtx mc = make_mean_ctx(a, g, smem);
+  int64_t lo, hi;
+  split_range(a, g, sp, lo, hi);
+  double ss = 0.0;
+  const bool has_mask = a.mask != nullptr;
+  for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const float x = a.x[i];
+    const float m = has_mask ? a.mask[i] : 1.0f;
+    const double mean = elem_mean(mc, x, m, has_mask);
+    const double d = has_mask ? ((double)x * (double)m - mean * (double)m) : ((double)x - mean);
+    ss += d * d;
+  }
+  ss = block_sum_d(ss, smem);
+  if (threadIdx.x == 0) a.part[((int64_t)2 * a.G + g) * a.nsplit + sp] = ss;
+}
+
+// pass 3: normalise
+__global__ __launch_bounds__(NORM_THREADS) void norm_apply_kernel(NormArgs a) {
+  __shared__ double smem[4];
+  const int g = blockIdx.x, sp = blockIdx.y;
+  const bool has_mask = a.mask != nullptr;
+  int64_t lo, hi;
+  split_range(a, g, sp, lo, hi);
+  if (has_mask) {
+    const double total = batch_partial(a, 0, smem);
+    if (total == 0.0) {  // nothing active: the input is returned unchanged
+      for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) a.out[i] = a.x[i];
+      return;
+    }
+  }
+  const MeanCtx mc = make_mean_ctx(a, g, smem);
+  // standard deviation
+  double std_d = 1.0;
+  double eps = a.eps;
+  if (a.std_level == LEVEL_BATCH) {
+    const double cnt = batch_partial(a, 0, smem);
+    const double ss = batch_partial(a, 2, smem);
+    if (a.unbiased) std_d = cnt <= 1.0 ? 1.0 : sqrt(ss / (cnt - 1.0));
+    else std_d = cnt == 0.0 ? 1.0 : sqrt(ss / cnt);
+  } else if (a.std_level == LEVEL_GROUP) {
+    if (g == a.tail_group) std_d = 0.0;
+    else if (a.grows[g] == 1 && a.unbiased) std_d = 1.0;
+    else {
+      const double cnt = group_partial(a, 0, g);
+      const double ss = group_partial(a, 2, g);
+      if (a.unbiased) std_d = cnt <= 1.0 ? 1.0 : sqrt(ss / (cnt - 1.0));
+      else std_d = cnt == 0.0 ? 1.0 : sqrt(ss / cnt);
+    }
+    std_d = (double)(float)std_d;
+  } else {
+    eps = 0.0;
+  }
+  const bool mean64 = a.mean_level == LEVEL_BATCH, std64 = a.std_level == LEVEL_BATCH;
+  for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const float x = a.x[i];
+    const float m = has_mask ? a.mask[i] : 1.0f;
+    const double mean = elem_mean(mc, x, m, has_mask);
+    float r;
+    if (mean64 || std64) {
+      double c = mean64 ? ((double)x - mean) : (double)(x - (float)mean);
+      if (has_mask) c = mean64 ? c * (double)m : (double)((float)c * m);
+      const double den = std64 ? (std_d + eps) : (double)((float)std_d + (float)eps);
+      r = (float)(c / den);
+    } else {
+      float c = x - (float)mean;
+      if (has_mask) c = c * m;
+      r = c / ((float)std_d + (float)eps);
+    }
+    a.out[i] = r;
+  }
+}
+
+// masked_normalization (functional.py:16-53): one group, var = E[x^2] - E[x]^2 in fp64,
+// (x*mask - mean) / (sqrt(var) + eps); the centred value is not re-masked.
+__global__ __launch_bounds__(NORM_THREADS) void masked_norm_stats_kernel(const float* x,
+                                                                          const float* mask,
+                                                                          int64_t n, double* part) {
+  __shared__ double smem[4];
+  double cnt = 0.0, s = 0.0, s2 = 0.0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const double m = mask ? (double)mask[i] : 1.0;
+    const double v = (double)x[i] * m;
+    cnt += m; s += v; s2 += v * v;
+  }
+  cnt = block_sum_d(cnt, smem); s = block_sum_d(s, smem); s2 = block_sum_d(s2, smem);
+  if (threadIdx.x == 0) {
+    part[blockIdx.x] = cnt; part[gridDim.x + blockIdx.x] = s; part[2 * gridDim.x + blockIdx.x] = s2;
+  }
+}
+__global__ __launch_bounds__(NORM_THREADS) void masked_norm_apply_kernel(
+    const float* x, const float* mask, int64_t n, const double* part, int nparts, int unbiased,
+    double eps, float* out) {
+  __shared__ double smem[4];
+  double cnt = 0.0, s = 0.0, s2 = 0.0;
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    cnt += part[i]; s += part[nparts + i]; s2 += part[2 * nparts + i];
+  }
+  cnt = block_sum_d(cnt, smem); s = block_sum_d(s, smem); s2 = block_sum_d(s2, smem);
+  const double mean = s / cnt;
+  double var = s2 / cnt - mean * mean;
+  if (unbiased) var *= cnt / (cnt - 1.0);
+  const double den = sqrt(var) + eps;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const double v = (double)x[i] * (mask ? (double)mask[i] : 1.0);
+    out[i] = (float)((v - mean) / den);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t areal_gae_workspace_bytes(int64_t n_tokens) {
+  if (n_tokens <= 0) return 0;
+  const int64_t nb = ceil_div_i64(n_tokens, GAE_TILE);
+  return (size_t)nb * (sizeof(Map) + 2 * sizeof(double)) + 256;
+}
+
+// Generalised advantage estimation over packed sequences.
+//   sequences: cu_seqlens [n_seqs+1] (int32), or uniform_len > 0 for a padded [n_seqs, L] array
+//   no_eos [n_seqs] (uint8, nullable): bootstrap from the last value of the sequence
+//   lambda_seq [n_seqs] (nullable): per-sequence lambda, else the scalar gae_lambda
+int areal_gae_packed(const float* rewards, const float* values, const float* loss_mask,
+                     const int32_t* cu_seqlens, const uint8_t* no_eos, const float* lambda_seq,
+                     int64_t n_tokens, int64_t n_seqs, int64_t uniform_len, float discount,
+                     float gae_lambda, float* advantages, float* returns, void* workspace,
+                     size_t workspace_bytes, hipStream_t stream) {
+  if (n_tokens < 0 || n_seqs < 0) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!rewards || !values || !loss_mask || !advantages || !returns) return AREAL_ERR_BAD_ARG;
+  if (n_seqs == 0 || (uniform_len <= 0 && cu_seqlens == nullptr)) return AREAL_ERR_BAD_ARG;
+  if (uniform_len > 0 && uniform_len * n_seqs != n_tokens) return AREAL_ERR_BAD_ARG;
+  if (n_seqs > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  if (workspace == nullptr || workspace_bytes < areal_gae_workspace_bytes(n_tokens))
+    return AREAL_ERR_WORKSPACE;
+  const int64_t nb = ceil_div_i64(n_tokens, GAE_TILE);
+  if (nb > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  Map* totals = (Map*)wp;
+  double* carry = (double*)(wp + (size_t)nb * sizeof(Map));
+  GaeArgs g{rewards, values, loss_mask, cu_seqlens, no_eos, lambda_seq, n_tokens, (int)n_seqs,
+            uniform_len, discount, gae_lambda, advantages, returns};
+  hipLaunchKernelGGL(gae_block_total_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g,
+                     totals);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(gae_carry_kernel, dim3(1), dim3(GAE_THREADS), 0, stream, totals, (int)nb,
+                     carry);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(gae_apply_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g, carry);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+static int norm_nsplit(int64_t max_group_len) {
+  int64_t s = ceil_div_i64(max_group_len, 16384);
+  if (s < 1) s = 1;
+  if (s > 512) s = 512;
+  return (int)s;
+}
+
+size_t areal_group_norm_workspace_bytes(int64_t n_groups, int64_t max_group_len) {
+  if (n_groups <= 0) return 0;
+  return (size_t)3 * n_groups * norm_nsplit(max_group_len) * sizeof(double) + 256;
+}
+
+// Normalization(x, mask, groups): levels 0 = none, 1 = batch, 2 = group.
+//   group_offsets [G+1] int64 element offsets (device) partitioning [0, n);
+//   group_rows [G] int64 (device): number of rows (samples) of each group;
+//   tail_group: index of a group made of rows that belong to no group (mean 0, std 0 at group
+//   level, still part of batch statistics), or -1.
+int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t* group_offsets,
+                     const int64_t* group_rows, int64_t n_groups, int64_t max_group_len,
+                     int tail_group, int mean_level, int std_level, int leave_one_out,
+                     int unbiased, double eps, float* out, void* workspace,
+                     size_t workspace_bytes, hipStream_t stream) {
+  if (n < 0 || n_groups < 0) return AREAL_ERR_BAD_ARG;
+  if (n == 0) return AREAL_OK;
+  if (!x || !out || !group_offsets || !group_rows || n_groups == 0) return AREAL_ERR_BAD_ARG;
+  if (mean_level < 0 || mean_level > 2 || std_level < 0 || std_level > 2) return AREAL_ERR_BAD_ARG;
+  if (n_groups > 65535 * 16) return AREAL_ERR_UNSUPPORTED;
+  if (workspace == nullptr ||
+      workspace_bytes < areal_group_norm_workspace_bytes(n_groups, max_group_len))
+    return AREAL_ERR_WORKSPACE;
+  NormArgs a;
+  a.x = x; a.mask = mask; a.n = n; a.goff = group_offsets; a.grows = group_rows;
+  a.G = (int)n_groups; a.tail_group = tail_group; a.nsplit = norm_nsplit(max_group_len);
+  a.mean_level = mean_level; a.std_level = std_level; a.leave1out = leave_one_out;
+  a.unbiased = unbiased; a.eps = eps;
+  a.part = (double*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  a.out = out;
+  const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
+  hipLaunchKernelGGL(norm_stats1_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(norm_stats2_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(norm_apply_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+size_t areal_masked_norm_workspace_bytes(int64_t n) {
+  (void)n;
+  return (size_t)3 * 256 * sizeof(double) + 256;
+}
+
+int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased, double eps,
+                      float* out, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (n < 0) return AREAL_ERR_BAD_ARG;
+  if (n == 0) return AREAL_OK;
+  if (!x || !out) return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_masked_norm_workspace_bytes(n))
+    return AREAL_ERR_WORKSPACE;
+  double* part = (double*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  int64_t nb = ceil_div_i64(n, NORM_THREADS * 8);
+  if (nb > 256) nb = 256;
+  hipLaunchKernelGGL(masked_norm_stats_kernel, dim3((unsigned)nb), dim3(NORM_THREADS), 0, stream, x,
+                     mask, n, part);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(masked_norm_apply_kernel, dim3((unsigned)nb), dim3(NORM_THREADS), 0, stream, x,
+                     mask, n, (const double*)part, (int)nb, unbiased, eps, out);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,528 @@
+// PPO / GRPO / CISPO actor loss with rejection sampling (IcePop ratio bounds, KPop binary KL,
+// k1/k2/k3 estimators), token and sequence level, forward and closed-form backward.
+//
+// Follows areal/utils/functional/functional.py: apply_rejection_sampling (:185-437),
+// compute_binary_kl_divergence (:440-449), ppo_actor_loss_fn (:452-596), cispo_loss_fn
+// (:678-793), _compute_sequence_level_ratio_and_advantages (:56-149) and
+// KLEstimator._compute_approx_kl (areal/utils/data.py:1662-1698).
+//
+// All per-token arithmetic is fp32 and is written operation by operation in the order of the
+// reference's tensor expressions (this file is compiled with -ffp-contract=off), so that the
+// boolean outputs agree with a CPU evaluation except where exp/log differ in their last bit.
+// Sums use fp64 block partials reduced in a fixed order: results are run-to-run identical.
+#include "common.hpp"
+
+namespace {
+
+constexpr int LOSS_THREADS = 256;
+constexpr int MAX_LOSS_BLOCKS = 1024;
+
+enum { METRIC_RATIO = 0, METRIC_K1 = 1, METRIC_K2 = 2, METRIC_K3 = 3, METRIC_BINARY_KL = 4 };
+enum { AGG_SUM = 0, AGG_MEAN = 1, AGG_MAX = 2 };
+enum { LOSS_NONE = -1, LOSS_PPO = 0, LOSS_CISPO = 1 };
+
+struct LossCfg {
+  int loss_kind;       // LOSS_*
+  float clip_lo;       // 1 - eps_clip (rounded from double on the host)
+  float clip_hi;       // 1 + eps_clip_higher
+  int has_c_clip;
+  float c_clip;
+  int seq_is;          // importance_sampling_level == "sequence"
+  int rs_enabled;
+  int rs_seq_level;    // rejection_sampling.level == "sequence"
+  int rs_clamp;        // action == "clamp"
+  int rs_metric;       // METRIC_*
+  int rs_agg;          // AGG_*
+  float rs_upper;
+  int rs_has_lower;
+  float rs_lower;
+};
+
+struct LossIO {
+  const float* lp;      // current policy log-probs (null when loss_kind == LOSS_NONE)
+  const float* prox;
+  const float* old;     // may be null when !rs_enabled
+  const float* adv;
+  const uint8_t* mask;  // bool loss mask (pre rejection)
+  const int32_t* cu;    // [n_seqs + 1] or null
+  int64_t n;
+  int n_seqs;
+  int64_t uniform_len;  // > 0: sequence s covers [s*uniform_len, (s+1)*uniform_len)
+  // per-sequence inputs produced by the segmented kernels
+  const float* seq_rs;    // [n_seqs][2]: {in_bounds (0/1), uniform weight}
+  const float* seq_is;    // [n_seqs][4]: {ratio_s, adv_mean_s, sum_w_s, 1/count_s}
+  // outputs (any may be null)
+  float* dlp;             // d(loss_sum)/dlp, not yet divided by the token count
+  float* stat_loss;
+  float* stat_ratio;
+  float* stat_kl;
+  uint8_t* clip_mask;
+  uint8_t* dual_mask;
+  uint8_t* new_mask;
+  float* behave_w;
+  float* behave_kl;
+  uint8_t* behave_mask;
+};
+
+struct Partial {
+  double loss_sum;
+  long long n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave;
+};
+
+DEVI int seq_of(const LossIO& io, int64_t t) {
+  if (io.uniform_len > 0) return (int)(t / io.uniform_len);
+  int lo = 0, hi = io.n_seqs;  // find last s with cu[s] <= t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)io.cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// torch.clamp keeps NaN (fminf/fmaxf would drop it).
+DEVI float torch_clamp(float x, float lo, float hi) {
+  if (x != x) return x;
+  return x < lo ? lo : (x > hi ? hi : x);
+}
+DEVI float torch_max(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a > b ? a : b); }
+DEVI float torch_min(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a < b ? a : b); }
+
+// Bernoulli KL(P||Q) with p = clamp(exp(log_p), 1e-8, 1 - 1e-8): in fp32 the upper bound
+// rounds to 1.0f, which is what the reference's fp32 tensors see.
+DEVI float binary_kl(float log_p, float log_q) {
+  const float lo = 1e-8f, hi = (float)(1.0 - 1e-8);
+  const float p = torch_clamp(expf(log_p), lo, hi);
+  const float q = torch_clamp(expf(log_q), lo, hi);
+  const float a = p * logf(p / q);
+  const float b = (1.0f - p) * logf((1.0f - p) / (1.0f - q));
+  return a + b;
+}
+
+DEVI bool in_bounds(float metric, const LossCfg& c) {
+  bool ok = metric <= c.rs_upper;
+  if (c.rs_has_lower) ok = ok && (metric >= c.rs_lower);
+  return ok;
+}
+
+// Per-token divergence metric between proximal and behaviour policy.
+DEVI float rs_metric(float prox, float old, float lr_sane, int metric) {
+  switch (metric) {
+    case METRIC_RATIO: return expf(lr_sane);
+    case METRIC_K1: return prox - old;
+    case METRIC_K2: { const float d = prox - old; return (d * d) / 2.0f; }
+    case METRIC_K3: { const float d = -(prox - old); return (expf(d) - 1.0f) - d; }
+    default: return torch_max(binary_kl(prox, old), binary_kl(old, prox));
+  }
+}
+
+DEVI float sane_log_ratio(float prox, float old) {
+  const float lr = prox - old;
+  return __builtin_isfinite(lr) ? lr : 0.0f;
+}
+
+template <typename T>
+DEVI T block_sum(T v, T* smem) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[w] = v;
+  __syncthreads();
+  T r = 0;
+  const int nw = (blockDim.x + 63) >> 6;
+  for (int i = 0; i < nw; ++i) r += smem[i];
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------
+// Segmented pass 1: per-sequence aggregate of the rejection metric (one block per sequence).
+// Writes seq_rs[s] = {in_bounds, uniform weight exp(mean log ratio)}.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(LOSS_THREADS) void seq_rs_kernel(LossIO io, LossCfg c, float* seq_rs) {
+  __shared__ double sm_d[8];
+  __shared__ float sm_f[8];
+  const int s = blockIdx.x;
+  int64_t t0, t1;
+  if (io.uniform_len > 0) { t0 = (int64_t)s * io.uniform_len; t1 = t0 + io.uniform_len; }
+  else { t0 = io.cu[s]; t1 = io.cu[s + 1]; }
+  if (t1 > io.n) t1 = io.n;
+  double sum_lr = 0.0, sum_m = 0.0;
+  float mx = neg_inf();
+  long long cnt = 0;
+  const bool log_agg = (c.rs_metric == METRIC_RATIO);
+  for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
+    if (!io.mask[t]) continue;
+    const float prox = io.prox[t], old = io.old[t];
+    const float lr = sane_log_ratio(prox, old);
+    const float v = log_agg ? lr : rs_metric(prox, old, lr, c.rs_metric);
+    cnt += 1;
+    sum_lr += (double)lr;
+    sum_m += (double)v;
+    mx = (v != v || mx != mx) ? __builtin_nanf("") : fmaxf(mx, v);
+  }
+  sum_lr = block_sum(sum_lr, sm_d);
+  sum_m = block_sum(sum_m, sm_d);
+  // max with NaN propagation: reduce a NaN flag and the max separately
+  float nanflag = (mx != mx) ? 1.f : 0.f;
+  float mxc = (mx != mx) ? neg_inf() : mx;
+  mxc = wave_max(mxc);
+  nanflag = wave_max(nanflag);
+  {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) { sm_f[w] = mxc; sm_f[4 + w] = nanflag; }
+    __syncthreads();
+    mxc = fmaxf(fmaxf(sm_f[0], sm_f[1]), fmaxf(sm_f[2], sm_f[3]));
+    nanflag = fmaxf(fmaxf(sm_f[4], sm_f[5]), fmaxf(sm_f[6], sm_f[7]));
+  }
+  __shared__ long long sm_l[8];
+  const long long total = block_sum(cnt, sm_l);
+  if (threadIdx.x == 0) {
+    const float denom = (float)(total > 0 ? total : 1);
+    float agg;
+    if (c.rs_agg == AGG_SUM) agg = (float)sum_m;
+    else if (c.rs_agg == AGG_MEAN) agg = (float)sum_m / denom;
+    else agg = total == 0 ? 0.0f : (nanflag > 0.f ? __builtin_nanf("") : mxc);
+    const float seq_metric = log_agg ? expf(agg) : agg;
+    seq_rs[2 * s + 0] = in_bounds(seq_metric, c) ? 1.0f : 0.0f;
+    seq_rs[2 * s + 1] = log_agg ? expf((float)sum_lr / denom) : 0.0f;
+  }
+}
+
+// Rejection sampling for one token. Returns the narrowed mask; sets w (not yet zeroed outside
+// the mask) and whether the token counts as filtered / clamped.
+DEVI bool rs_token(const LossIO& io, const LossCfg& c, int64_t t, bool m, float& w, bool& counted) {
+  const float prox = io.prox[t], old = io.old[t];
+  const float lr = sane_log_ratio(prox, old);
+  w = expf(lr);
+  bool keep = true;
+  counted = false;
+  if (c.rs_seq_level) {
+    const int s = seq_of(io, t);
+    const bool seq_ok = io.seq_rs[2 * s] != 0.0f;
+    if (c.rs_metric == METRIC_RATIO) w = io.seq_rs[2 * s + 1];
+    if (c.rs_clamp) {
+      const float orig = w;
+      if (!seq_ok) w = torch_clamp(w, c.rs_has_lower ? c.rs_lower : 0.0f, c.rs_upper);
+      counted = m && (orig != w);
+    } else {
+      keep = seq_ok;
+      counted = m && !keep;
+    }
+  } else if (c.rs_clamp) {
+    const float orig = w;
+    w = torch_clamp(w, c.rs_has_lower ? c.rs_lower : 0.0f, c.rs_upper);
+    counted = m && (orig != w);
+  } else {
+    keep = in_bounds(rs_metric(prox, old, lr, c.rs_metric), c);
+    counted = m && !keep;
+  }
+  return c.rs_clamp ? m : (m && keep);
+}
+
+// ---------------------------------------------------------------------------------------
+// Segmented pass 2 (GSPO): per-sequence geometric-mean ratio and mean advantage over the
+// narrowed mask. Writes seq_is[s] = {ratio_s, adv_mean_s, sum of behave weights, 1/count}.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(LOSS_THREADS) void seq_is_kernel(LossIO io, LossCfg c, float* seq_is) {
+  __shared__ double sm_d[8];
+  const int s = blockIdx.x;
+  int64_t t0, t1;
+  if (io.uniform_len > 0) { t0 = (int64_t)s * io.uniform_len; t1 = t0 + io.uniform_len; }
+  else { t0 = io.cu[s]; t1 = io.cu[s + 1]; }
+  if (t1 > io.n) t1 = io.n;
+  double sum_lr = 0.0, sum_adv = 0.0, sum_w = 0.0, cnt = 0.0;
+  for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
+    const bool m2 = c.rs_enabled ? (io.new_mask[t] != 0) : (io.mask[t] != 0);
+    if (!m2) continue;
+    cnt += 1.0;
+    sum_lr += (double)(io.lp[t] - io.prox[t]);
+    sum_adv += (double)io.adv[t];
+    sum_w += c.rs_enabled ? (double)io.behave_w[t] : 1.0;
+  }
+  sum_lr = block_sum(sum_lr, sm_d);
+  sum_adv = block_sum(sum_adv, sm_d);
+  sum_w = block_sum(sum_w, sm_d);
+  cnt = block_sum(cnt, sm_d);
+  if (threadIdx.x == 0) {
+    const float denom = (float)(cnt > 0.0 ? cnt : 1.0);
+    seq_is[4 * s + 0] = expf((float)sum_lr / denom);
+    seq_is[4 * s + 1] = (float)sum_adv / denom;
+    seq_is[4 * s + 2] = (float)sum_w;
+    seq_is[4 * s + 3] = 1.0f / denom;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Token kernel
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, LossCfg c,
+                                                                   Partial* partials) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double loss_sum = 0.0;
+  long long n_valid = 0, n_kept = 0, n_filtered = 0, n_clip = 0, n_dual = 0, n_behave = 0;
+
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < io.n;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const bool m = io.mask[t] != 0;
+    bool m2 = m;
+    float w = 1.0f;
+    if (c.rs_enabled) {
+      bool counted;
+      m2 = rs_token(io, c, t, m, w, counted);
+      w = m2 ? w : 0.0f;
+      n_filtered += counted;
+      if (io.new_mask) io.new_mask[t] = m2;
+      if (io.behave_w) io.behave_w[t] = w;
+    }
+    n_valid += m;
+    n_kept += m2;
+    if (c.loss_kind == LOSS_NONE) continue;
+
+    const float lp = io.lp[t], prox = io.prox[t], adv = io.adv[t];
+    const float kl = lp - prox;
+    float pg, dsel, ratio_out;
+    bool clip = false, dual = false;
+    if (c.loss_kind == LOSS_CISPO) {
+      const float ratio = expf(kl);
+      const float rc = torch_clamp(ratio, c.clip_lo, c.clip_hi);
+      const float coef = (-rc) * adv;
+      pg = coef * lp;
+      dsel = coef;  // d pg / d lp
+      clip = (rc != ratio) && m2;
+      ratio_out = ratio;
+    } else {
+      float ratio, a = adv, dratio;  // dratio = d ratio / d lp[t] factor handled below
+      if (c.seq_is) {
+        const int s = seq_of(io, t);
+        ratio = m2 ? io.seq_is[4 * s + 0] : 0.0f;
+        a = m2 ? io.seq_is[4 * s + 1] : 0.0f;
+        dratio = 0.f;  // gradient assembled per sequence below
+      } else {
+        ratio = m ? expf(kl) : 0.0f;
+        dratio = ratio;
+      }
+      const float clipped = torch_clamp(ratio, c.clip_lo, c.clip_hi);
+      const float pg1 = (-a) * ratio;
+      const float pg2 = (-a) * clipped;
+      clip = pg1 < pg2;
+      pg = torch_max(pg1, pg2);
+      // d pg / d ratio following torch.max (ties split evenly) and clamp (closed interval)
+      const float in_band = (ratio >= c.clip_lo && ratio <= c.clip_hi) ? 1.0f : 0.0f;
+      float g1 = pg1 > pg2 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
+      float g2 = pg2 > pg1 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
+      float dpg = (-a) * (g1 + g2 * in_band);
+      if (c.has_c_clip) {
+        const float sgn = a > 0.f ? 1.0f : (a < 0.f ? -1.0f : 0.0f);
+        const float pg3 = (sgn * c.c_clip) * a;
+        dual = pg3 < pg;
+        const float keep = pg < pg3 ? 1.0f : (pg == pg3 ? 0.5f : 0.0f);
+        pg = torch_min(pg, pg3);
+        dpg *= keep;
+      }
+      if (c.seq_is) {
+        // every kept token of the sequence receives ratio_s/count_s * sum_w_s * dpg_s
+        const int s = seq_of(io, t);
+        dsel = m2 ? dpg * ratio * io.seq_is[4 * s + 2] * io.seq_is[4 * s + 3] : 0.0f;
+      } else {
+        dsel = dpg * dratio;
+      }
+      clip = clip && m;
+      dual = dual && m;
+      ratio_out = ratio;
+    }
+    if (c.rs_enabled) {
+      pg = pg * w;
+      if (!(c.loss_kind == LOSS_PPO && c.seq_is)) dsel = dsel * w;
+      const bool bm = (w > 0.0f) && m2;
+      n_behave += bm;
+      if (io.behave_mask) io.behave_mask[t] = bm;
+      if (io.behave_kl) io.behave_kl[t] = bm ? (prox - io.old[t]) : 0.0f;
+    }
+    if (m2) loss_sum += (double)pg;
+    n_clip += clip;
+    n_dual += dual;
+    if (io.dlp) io.dlp[t] = m2 ? dsel : 0.0f;
+    if (io.stat_loss) io.stat_loss[t] = pg;
+    if (io.stat_ratio) io.stat_ratio[t] = ratio_out;
+    if (io.stat_kl) io.stat_kl[t] = kl;
+    if (io.clip_mask) io.clip_mask[t] = clip;
+    if (io.dual_mask) io.dual_mask[t] = dual;
+  }
+  loss_sum = block_sum(loss_sum, sm_d);
+  n_valid = block_sum(n_valid, sm_l);
+  n_kept = block_sum(n_kept, sm_l);
+  n_filtered = block_sum(n_filtered, sm_l);
+  n_clip = block_sum(n_clip, sm_l);
+  n_dual = block_sum(n_dual, sm_l);
+  n_behave = block_sum(n_behave, sm_l);
+  if (threadIdx.x == 0) {
+    Partial p{loss_sum, n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave};
+    partials[blockIdx.x] = p;
+  }
+}
+
+// counters: [0] loss_sum [1] n_valid [2] n_kept [3] n_filtered [4] n_clip [5] n_dual
+//           [6] n_behave [7] loss = loss_sum / max(n_valid, 1)
+__global__ void loss_finalize_kernel(const Partial* partials, int nparts, float* loss_out,
+                                     double* counters) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double ls = 0.0;
+  long long a[6] = {0, 0, 0, 0, 0, 0};
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    const Partial p = partials[i];
+    ls += p.loss_sum;
+    a[0] += p.n_valid; a[1] += p.n_kept; a[2] += p.n_filtered;
+    a[3] += p.n_clip; a[4] += p.n_dual; a[5] += p.n_behave;
+  }
+  // fixed-order reduction: thread partials -> wave shuffles -> 4 wave slots
+  ls = block_sum(ls, sm_d);
+  for (int k = 0; k < 6; ++k) a[k] = block_sum(a[k], sm_l);
+  if (threadIdx.x == 0) {
+    counters[0] = ls;
+    for (int k = 0; k < 6; ++k) counters[1 + k] = (double)a[k];
+    const double denom = a[0] > 0 ? (double)a[0] : 1.0;
+    const float loss = (float)ls / (float)denom;
+    counters[7] = (double)loss;
+    if (loss_out) *loss_out = loss;
+  }
+}
+
+// out[t] = dlp[t] * upstream[0] / max(n_valid, 1)
+__global__ void loss_grad_scale_kernel(const float* __restrict__ dlp,
+                                       const float* __restrict__ upstream,
+                                       const double* __restrict__ counters,
+                                       float* __restrict__ out, int64_t n) {
+  const float nv = (float)(counters[1] > 0.0 ? counters[1] : 1.0);
+  const float g = upstream[0];
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
+       t += (int64_t)gridDim.x * blockDim.x)
+    out[t] = (dlp[t] * g) / nv;
+}
+
+int loss_grid(int64_t n) {
+  int64_t b = ceil_div_i64(n, LOSS_THREADS);
+  if (b > MAX_LOSS_BLOCKS) b = MAX_LOSS_BLOCKS;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Plain-C mirror of LossCfg (see include/areal_hip.h).
+struct areal_loss_config {
+  int loss_kind;
+  float clip_lo, clip_hi;
+  int has_c_clip;
+  float c_clip;
+  int seq_is;
+  int rs_enabled, rs_seq_level, rs_clamp, rs_metric, rs_agg;
+  float rs_upper;
+  int rs_has_lower;
+  float rs_lower;
+};
+
+size_t areal_actor_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
+  (void)n_tokens;
+  if (n_seqs < 0) n_seqs = 0;
+  return (size_t)MAX_LOSS_BLOCKS * sizeof(Partial) + (size_t)n_seqs * 6 * sizeof(float) + 256;
+}
+
+// Actor loss forward + backward in one pass over the tokens.
+//   loss_kind -1: rejection sampling only (lp / adv / loss outputs ignored)
+//              0: PPO clip (optionally dual clip, optionally sequence-level ratio)
+//              1: CISPO
+// Sequences are given by cu_seqlens [n_seqs+1] (packed) or by uniform_len (> 0, padded
+// [n_seqs, uniform_len] layout); both are needed only for sequence-level options.
+// counters is a device array of 8 doubles (layout above loss_finalize_kernel).
+int areal_actor_loss(const float* logprobs, const float* proximal, const float* old_logprobs,
+                     const float* advantages, const uint8_t* loss_mask,
+                     const int32_t* cu_seqlens, int64_t n_tokens, int64_t n_seqs,
+                     int64_t uniform_len, const areal_loss_config* cfg, float* loss,
+                     float* dlogprobs, float* stat_loss, float* stat_ratio, float* stat_approx_kl,
+                     uint8_t* clip_mask, uint8_t* dual_clip_mask, uint8_t* new_mask,
+                     float* behave_imp_weight, float* behave_approx_kl, uint8_t* behave_mask,
+                     double* counters, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
+  if (cfg == nullptr || n_tokens < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
+  if (cfg->loss_kind < LOSS_NONE || cfg->loss_kind > LOSS_CISPO) return AREAL_ERR_BAD_ARG;
+  if (n_tokens > 0 && (proximal == nullptr || loss_mask == nullptr)) return AREAL_ERR_BAD_ARG;
+  if (cfg->loss_kind != LOSS_NONE && n_tokens > 0 && (logprobs == nullptr || advantages == nullptr))
+    return AREAL_ERR_BAD_ARG;
+  if (cfg->rs_enabled && n_tokens > 0 && old_logprobs == nullptr) return AREAL_ERR_BAD_ARG;
+  const bool need_seq = (cfg->rs_enabled && cfg->rs_seq_level) || (cfg->loss_kind == LOSS_PPO && cfg->seq_is);
+  if (need_seq && n_tokens > 0) {
+    if (n_seqs <= 0) return AREAL_ERR_BAD_ARG;
+    if (uniform_len <= 0 && cu_seqlens == nullptr) return AREAL_ERR_BAD_ARG;
+    if (cfg->rs_enabled && (new_mask == nullptr || behave_imp_weight == nullptr) && cfg->seq_is)
+      return AREAL_ERR_BAD_ARG;
+  }
+  if (workspace == nullptr || workspace_bytes < areal_actor_loss_workspace_bytes(n_tokens, n_seqs))
+    return AREAL_ERR_WORKSPACE;
+
+  LossCfg c;
+  c.loss_kind = cfg->loss_kind; c.clip_lo = cfg->clip_lo; c.clip_hi = cfg->clip_hi;
+  c.has_c_clip = cfg->has_c_clip; c.c_clip = cfg->c_clip;
+  c.seq_is = (cfg->loss_kind == LOSS_PPO) ? cfg->seq_is : 0;
+  c.rs_enabled = cfg->rs_enabled; c.rs_seq_level = cfg->rs_seq_level; c.rs_clamp = cfg->rs_clamp;
+  c.rs_metric = cfg->rs_metric; c.rs_agg = cfg->rs_agg; c.rs_upper = cfg->rs_upper;
+  c.rs_has_lower = cfg->rs_has_lower; c.rs_lower = cfg->rs_lower;
+
+  char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  Partial* partials = (Partial*)wp;
+  float* seq_rs = (float*)(wp + (size_t)MAX_LOSS_BLOCKS * sizeof(Partial));
+  float* seq_is = seq_rs + 2 * (n_seqs > 0 ? n_seqs : 0);
+
+  LossIO io;
+  io.lp = logprobs; io.prox = proximal; io.old = old_logprobs; io.adv = advantages;
+  io.mask = loss_mask; io.cu = cu_seqlens; io.n = n_tokens; io.n_seqs = (int)n_seqs;
+  io.uniform_len = uniform_len; io.seq_rs = seq_rs; io.seq_is = seq_is;
+  io.dlp = dlogprobs; io.stat_loss = stat_loss; io.stat_ratio = stat_ratio;
+  io.stat_kl = stat_approx_kl; io.clip_mask = clip_mask; io.dual_mask = dual_clip_mask;
+  io.new_mask = new_mask; io.behave_w = behave_imp_weight; io.behave_kl = behave_approx_kl;
+  io.behave_mask = behave_mask;
+
+  const int grid = loss_grid(n_tokens);
+  if (n_tokens > 0 && c.rs_enabled && c.rs_seq_level) {
+    hipLaunchKernelGGL(seq_rs_kernel, dim3((unsigned)n_seqs), dim3(LOSS_THREADS), 0, stream, io, c,
+                       seq_rs);
+    AREAL_CHECK_LAUNCH();
+  }
+  if (n_tokens > 0 && c.seq_is) {
+    if (c.rs_enabled) {
+      // first materialise the narrowed mask and the behaviour weight, then aggregate on them
+      LossCfg c0 = c;
+      c0.loss_kind = LOSS_NONE;
+      LossIO io0 = io;
+      hipLaunchKernelGGL(loss_token_kernel, dim3(grid), dim3(LOSS_THREADS), 0, stream, io0, c0,
+                         partials);
+      AREAL_CHECK_LAUNCH();
+    }
+    hipLaunchKernelGGL(seq_is_kernel, dim3((unsigned)n_seqs), dim3(LOSS_THREADS), 0, stream, io, c,
+                       seq_is);
+    AREAL_CHECK_LAUNCH();
+  }
+  hipLaunchKernelGGL(loss_token_kernel, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c, partials);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(LOSS_THREADS), 0, stream, partials, grid,
+                     loss, counters);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// grad_logprobs[t] = dlogprobs[t] * upstream[0] / max(counters[1], 1)
+int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const double* counters,
+                          float* grad_logprobs, int64_t n_tokens, hipStream_t stream) {
+  if (n_tokens < 0) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!dlogprobs || !upstream || !counters || !grad_logprobs) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(loss_grad_scale_kernel, dim3(loss_grid(n_tokens)), dim3(LOSS_THREADS), 0,
+                     stream, dlogprobs, upstream, counters, grad_logprobs, n_tokens);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+}  // extern "C"

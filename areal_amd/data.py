@@ -1,0 +1,143 @@
+"""``Normalization`` and ``KLEstimator`` with the reference's interfaces
+(``areal/utils/data.py:1382-1637`` and ``:1640-1698``).
+
+``Normalization.__call__`` runs the three-pass kernel of ``csrc/gae_norm.hip``: fp64 sums,
+group-level statistics rounded to fp32 exactly where the reference stores them in fp32
+tensors.  Multi-rank reduction of batch statistics is outside the one-GPU scope.
+"""
+
+from __future__ import annotations
+
+import functools
+
+import torch
+import torch.distributed as dist
+
+from areal_amd import _lib
+from areal_amd.config import NormConfig
+
+_LEVEL_ID = {None: 0, "none": 0, "batch": 1, "group": 2}
+
+
+@functools.lru_cache(maxsize=64)
+def _group_tables(groups: tuple, tail_rows: int, row_len: int, device_str: str):
+    offsets, rows = [0], []
+    for g in groups:
+        offsets.append(offsets[-1] + g * row_len)
+        rows.append(g)
+    tail_group = -1
+    if tail_rows > 0:
+        tail_group = len(rows)
+        offsets.append(offsets[-1] + tail_rows * row_len)
+        rows.append(tail_rows)
+    dev = torch.device(device_str)
+    max_len = max(b - a for a, b in zip(offsets[:-1], offsets[1:]))
+    return (
+        torch.tensor(offsets, dtype=torch.int64, device=dev),
+        torch.tensor(rows, dtype=torch.int64, device=dev),
+        tail_group,
+        max_len,
+    )
+
+
+class Normalization:
+    """Adaptive normalisation with independent levels for mean and std:
+    ``"batch"``, ``"group"`` (fixed ``group_size`` or explicit ``group_sizes``) or ``None``."""
+
+    def __init__(self, config: NormConfig):
+        self.mean_level = config.mean_level
+        self.mean_leave1out = config.mean_leave1out
+        self.std_level = config.std_level
+        self.std_unbiased = config.std_unbiased
+        self.group_size = config.group_size
+        self.eps = config.eps
+
+    def _group_rows(self, bs: int, group_sizes: list[int] | None) -> tuple[tuple, int]:
+        """Row counts of the groups and the number of trailing rows in no group."""
+        if group_sizes is not None:
+            if any(sz <= 0 for sz in group_sizes):
+                raise ValueError(f"group_sizes must be all positive, got {group_sizes}")
+            if sum(group_sizes) != bs:
+                raise ValueError(
+                    f"group_sizes sum ({sum(group_sizes)}) must equal "
+                    f"batch size ({bs}), got {group_sizes}"
+                )
+            return tuple(int(s) for s in group_sizes), 0
+        n_groups = bs // self.group_size
+        return (self.group_size,) * n_groups, bs - n_groups * self.group_size
+
+    @torch.no_grad()
+    def __call__(
+        self,
+        x: torch.Tensor,
+        loss_mask: torch.Tensor | None = None,
+        high_precision: bool = True,
+        reduce_group=None,
+        group_sizes: list[int] | None = None,
+    ) -> torch.Tensor:
+        del high_precision  # sums are always fp64
+        if dist.is_initialized() and dist.get_world_size(reduce_group) > 1 and "batch" in (
+            self.mean_level, self.std_level,
+        ):
+            raise NotImplementedError("batch-level normalisation over several ranks is not built")
+        lib = _lib.load()
+        dev = _lib.require_gpu(x, loss_mask)
+        bs = x.size(0)
+        xf = x.to(torch.float32).contiguous()
+        n = xf.numel()
+        out = torch.empty_like(xf)
+        if n == 0:
+            return out
+        if loss_mask is not None and loss_mask.shape != x.shape:
+            loss_mask = loss_mask.expand_as(x)
+        mf = loss_mask.to(torch.float32).contiguous() if loss_mask is not None else None
+        row_len = n // bs
+        if self.mean_level == "group" or self.std_level == "group":
+            groups, tail = self._group_rows(bs, group_sizes)
+        else:
+            groups, tail = (bs,), 0
+        if not groups and tail == 0:
+            return xf
+        offsets, rows, tail_group, max_len = _group_tables(groups, tail, row_len, str(dev))
+        n_groups = rows.numel()
+        nbytes = lib.areal_group_norm_workspace_bytes(n_groups, max_len)
+        ws = _lib.workspace(nbytes, dev)
+        rc = lib.areal_group_norm(
+            _lib.ptr(xf), _lib.ptr(mf), n, _lib.ptr(offsets), _lib.ptr(rows), n_groups, max_len,
+            tail_group, _LEVEL_ID[self.mean_level], _LEVEL_ID[self.std_level],
+            int(bool(self.mean_leave1out)), int(bool(self.std_unbiased)), float(self.eps),
+            _lib.ptr(out), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_group_norm")
+        return out
+
+
+class KLEstimator:
+    """k1 / k2 / k3 estimators of KL(new || base) from log-probabilities
+    (``data.py:1640-1698``).  Elementwise tensor arithmetic on whatever device holds the
+    inputs; the rejection-sampling kernel has its own fused copy of these formulas."""
+
+    def __init__(self, kl_estimator: str = "k1", apply_clamp: bool = True):
+        if kl_estimator not in ["k1", "k2", "k3"]:
+            raise ValueError(f"Invalid KL estimator: {kl_estimator}. Valid choices: k1, k2, k3")
+        self.kl_estimator = kl_estimator
+        self.apply_clamp = apply_clamp
+
+    def __call__(self, log_probs: torch.Tensor, log_probs_base: torch.Tensor) -> torch.Tensor:
+        return self._compute_approx_kl(log_probs, log_probs_base, self.kl_estimator, self.apply_clamp)
+
+    @staticmethod
+    def _compute_approx_kl(log_probs, log_probs_base, kl_estimator: str = "k1", apply_clamp: bool = True):
+        diff = log_probs.float() - log_probs_base.float()
+        if kl_estimator == "k1":
+            est = diff
+        elif kl_estimator == "k2":
+            est = diff**2 / 2.0
+        elif kl_estimator == "k3":
+            neg = -diff
+            est = neg.exp() - 1 - neg
+        else:
+            raise ValueError(f"Invalid KL estimator: {kl_estimator}. Valid choices: k1, k2, k3")
+        if apply_clamp:
+            est = est.clamp(min=-10, max=10)
+        return est

@@ -1,0 +1,81 @@
+"""Engine-side glue: what ``FSDPEngine`` does between the model's last hidden states and the
+scaled scalar loss (``areal/engine/fsdp_engine.py:2076-2217``), with the logits replaced by the
+fused lm_head kernel.
+
+The reference computes ``logits = model(...).logits`` and then reads them three times
+(log-softmax, entropy, min/max). Here the caller passes the final hidden states and the
+``lm_head`` weight; label roll, padding trim and loss scaling follow the reference.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+import torch
+
+from areal_amd.functional.lm_head import fused_lm_head_logprobs_entropy
+
+
+def _labels(inputs: dict[str, Any]) -> torch.Tensor:
+    labels = inputs.get("rolled_input_ids")
+    if labels is None:
+        labels = torch.roll(inputs["input_ids"], shifts=-1, dims=-1)
+    if labels.ndim == 2 and labels.shape[0] == 1:
+        labels = labels.squeeze(0)
+    return labels
+
+
+def compute_logprobs(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    inputs: dict[str, Any],
+    temperature: float = 1.0,
+    pad_length: int = 0,
+) -> torch.Tensor:
+    """Forward-only label log-probabilities of a packed micro-batch
+    (``fsdp_engine.py:2107-2134`` with the lm_head folded in)."""
+    if hidden.ndim == 3 and hidden.shape[0] == 1:
+        hidden = hidden.squeeze(0)
+    with torch.no_grad():
+        out = fused_lm_head_logprobs_entropy(
+            hidden, lm_head_weight, _labels(inputs), temperature=temperature
+        )
+    logprobs = out.logprobs
+    return logprobs[:-pad_length] if pad_length > 0 else logprobs
+
+
+def compute_logprobs_and_loss(
+    hidden: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    model_inputs: dict[str, Any],
+    mb_input: dict[str, Any],
+    loss_fn: Callable[..., torch.Tensor],
+    loss_weight_fn: Callable[[dict[str, Any]], torch.Tensor],
+    total_loss_weight: torch.Tensor | float,
+    temperature: float = 1.0,
+    pad_length: int = 0,
+    loss_multiplier: float = 1.0,
+) -> torch.Tensor:
+    """Scaled loss of one micro-batch (``fsdp_engine.py:2147-2217``).
+
+    ``loss_fn(logprobs, entropy, mb_input, vocab_min_logits=..., vocab_max_logits=...)`` is
+    the actor loss (normally a ``functools.partial`` of ``grpo_loss_fn``).  The per-token
+    vocabulary min/max come out of the same kernel sweep instead of a second pass over logits.
+    """
+    local_weight = loss_weight_fn(mb_input)
+    if local_weight == 0:
+        return hidden.float().mean() * 0.0
+    if hidden.ndim == 3 and hidden.shape[0] == 1:
+        hidden = hidden.squeeze(0)
+    out = fused_lm_head_logprobs_entropy(
+        hidden, lm_head_weight, _labels(model_inputs), temperature=temperature
+    )
+    logprobs, entropy = out.logprobs, out.entropy
+    vmin, vmax = out.vocab_min_logits, out.vocab_max_logits
+    if pad_length > 0:
+        logprobs, entropy = logprobs[:-pad_length], entropy[:-pad_length]
+        vmin, vmax = vmin[:-pad_length], vmax[:-pad_length]
+    loss = loss_fn(logprobs, entropy, mb_input, vocab_min_logits=vmin, vocab_max_logits=vmax)
+    loss_scale = local_weight / total_loss_weight * loss_multiplier
+    return loss * loss_scale

@@ -1,11 +1,29 @@
 """Drop-in counterparts of ``areal.utils.functional`` (``__init__.py:3-35`` of the reference)."""
 
+from areal_amd.functional.functional import (
+    RejectionSamplingResult,
+    apply_rejection_sampling,
+    cispo_loss_fn,
+    masked_normalization,
+    ppo_actor_loss_fn,
+)
 from areal_amd.functional.lm_head import (
     ChunkedLMHeadOutput,
     fused_lm_head_logprobs_entropy,
 )
+from areal_amd.functional.vocab_parallel import (
+    gather_logprobs,
+    gather_logprobs_entropy,
+)
 
 __all__ = [
+    "RejectionSamplingResult",
+    "apply_rejection_sampling",
+    "cispo_loss_fn",
+    "masked_normalization",
+    "ppo_actor_loss_fn",
+    "gather_logprobs",
+    "gather_logprobs_entropy",
     "ChunkedLMHeadOutput",
     "fused_lm_head_logprobs_entropy",
 ]

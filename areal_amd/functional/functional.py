@@ -1,0 +1,376 @@
+"""Actor-loss stage of the hot path: same Python signatures as the reference's
+``areal/utils/functional/functional.py`` (``masked_normalization`` :16-53,
+``apply_rejection_sampling`` :185-437, ``ppo_actor_loss_fn`` :452-596, ``cispo_loss_fn``
+:678-793), computed by the HIP kernels of ``csrc/ppo_loss.hip`` and ``csrc/gae_norm.hip``.
+
+Argument checking (types of exception and their messages) happens here, before any device
+work, and follows the reference.  Every call performs exactly one device-to-host copy (the
+eight counters of the loss kernel), where the reference performs one to three ``.item()``
+synchronisations.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from areal_amd import _lib
+from areal_amd.config import RejectionSamplingConfig
+
+_METRIC_ID = {"ratio": 0, "kl_k1": 1, "kl_k2": 2, "kl_k3": 3, "binary_kl": 4}
+_AGG_ID = {"sum": 0, "mean": 1, "max": 2}
+LOSS_NONE, LOSS_PPO, LOSS_CISPO = -1, 0, 1
+
+
+@dataclass
+class RejectionSamplingResult:
+    """Result of rejection sampling (fields as in ``functional.py:152-164``)."""
+
+    loss_mask: torch.Tensor
+    behave_imp_weight: torch.Tensor
+    filtered_fraction: float
+
+
+def _f32(t: torch.Tensor) -> torch.Tensor:
+    return t.detach().to(torch.float32).contiguous().view(-1)
+
+
+def _fill_rs(cfg: _lib.LossConfig, rs: RejectionSamplingConfig | None) -> None:
+    if rs is None:
+        cfg.rs_enabled = 0
+        return
+    if rs.metric not in _METRIC_ID:
+        raise ValueError(f"Unknown metric: {rs.metric}")
+    if rs.agg not in _AGG_ID:
+        raise ValueError(f"Unknown agg method: {rs.agg}")
+    cfg.rs_enabled = 1
+    cfg.rs_seq_level = int(rs.level == "sequence")
+    cfg.rs_clamp = int(rs.action != "mask")
+    cfg.rs_metric = _METRIC_ID[rs.metric]
+    cfg.rs_agg = _AGG_ID[rs.agg]
+    cfg.rs_upper = rs.upper
+    cfg.rs_has_lower = int(rs.lower is not None)
+    cfg.rs_lower = rs.lower if rs.lower is not None else 0.0
+
+
+def _sequence_layout(shape, cu_seqlens, device):
+    """(cu_seqlens int32 tensor or None, n_seqs, uniform_len) for a 1-D or 2-D batch."""
+    if len(shape) == 2:
+        return None, int(shape[0]), int(shape[1])
+    cu = cu_seqlens.to(device=device, dtype=torch.int32).contiguous()
+    return cu, int(cu.numel() - 1), 0
+
+
+def _run_loss_kernel(
+    cfg: _lib.LossConfig,
+    shape,
+    logprobs,
+    proximal,
+    old,
+    advantages,
+    mask_bool,
+    cu_seqlens,
+    want_grad: bool,
+):
+    """Launch ``areal_actor_loss`` and return its outputs and the eight host counters."""
+    lib = _lib.load()
+    dev = _lib.require_gpu(proximal, mask_bool, logprobs, old, advantages)
+    n = int(mask_bool.numel())
+    need_seq = (cfg.rs_enabled and cfg.rs_seq_level) or (cfg.loss_kind == LOSS_PPO and cfg.seq_is)
+    cu, n_seqs, uniform_len = (None, 0, 0)
+    if need_seq:
+        cu, n_seqs, uniform_len = _sequence_layout(shape, cu_seqlens, dev)
+    has_loss = cfg.loss_kind != LOSS_NONE
+    f32 = dict(dtype=torch.float32, device=dev)
+    u8 = dict(dtype=torch.bool, device=dev)
+    out = {
+        "loss": torch.empty((), **f32) if has_loss else None,
+        "dlp": torch.empty(n, **f32) if (has_loss and want_grad) else None,
+        "stat_loss": torch.empty(n, **f32) if has_loss else None,
+        "ratio": torch.empty(n, **f32) if has_loss else None,
+        "approx_kl": torch.empty(n, **f32) if has_loss else None,
+        "clip_mask": torch.empty(n, **u8) if has_loss else None,
+        "dual_clip_mask": torch.empty(n, **u8) if (has_loss and cfg.loss_kind == LOSS_PPO) else None,
+        "new_mask": torch.empty(n, **u8) if cfg.rs_enabled else None,
+        "behave_imp_weight": torch.empty(n, **f32) if cfg.rs_enabled else None,
+        "behave_approx_kl": torch.empty(n, **f32) if (cfg.rs_enabled and has_loss) else None,
+        "behave_mask": torch.empty(n, **u8) if (cfg.rs_enabled and has_loss) else None,
+    }
+    counters = torch.empty(8, dtype=torch.float64, device=dev)
+    nbytes = lib.areal_actor_loss_workspace_bytes(n, n_seqs)
+    ws = _lib.workspace(nbytes, dev)
+    rc = lib.areal_actor_loss(
+        _lib.ptr(logprobs), _lib.ptr(proximal), _lib.ptr(old), _lib.ptr(advantages),
+        _lib.ptr(mask_bool), _lib.ptr(cu), n, n_seqs, uniform_len, ctypes.byref(cfg),
+        _lib.ptr(out["loss"]), _lib.ptr(out["dlp"]), _lib.ptr(out["stat_loss"]),
+        _lib.ptr(out["ratio"]), _lib.ptr(out["approx_kl"]), _lib.ptr(out["clip_mask"]),
+        _lib.ptr(out["dual_clip_mask"]), _lib.ptr(out["new_mask"]),
+        _lib.ptr(out["behave_imp_weight"]), _lib.ptr(out["behave_approx_kl"]),
+        _lib.ptr(out["behave_mask"]), _lib.ptr(counters), _lib.ptr(ws), nbytes,
+        _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_actor_loss")
+    out["counters_dev"] = counters
+    return out
+
+
+class _ActorLoss(torch.autograd.Function):
+    """loss = sum(where(mask', pg, 0)) / N0 with the closed-form gradient w.r.t. logprobs."""
+
+    @staticmethod
+    def forward(ctx, logprobs, cfg, shape, proximal, old, advantages, mask_bool, cu_seqlens, sink):
+        want_grad = logprobs.requires_grad
+        lp = _f32(logprobs)
+        out = _run_loss_kernel(cfg, shape, lp, proximal, old, advantages, mask_bool, cu_seqlens,
+                               want_grad)
+        sink.update(out)
+        if want_grad:
+            ctx.save_for_backward(out["dlp"], out["counters_dev"])
+        ctx.shape = logprobs.shape
+        ctx.in_dtype = logprobs.dtype
+        return out["loss"]
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        dlp, counters = ctx.saved_tensors
+        lib = _lib.load()
+        dev = dlp.device
+        g = grad_loss.detach().to(torch.float32).reshape(1).contiguous()
+        grad = torch.empty_like(dlp)
+        rc = lib.areal_actor_loss_grad(
+            _lib.ptr(dlp), _lib.ptr(g), _lib.ptr(counters), _lib.ptr(grad), dlp.numel(),
+            _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_actor_loss_grad")
+        grad = grad.view(ctx.shape)
+        if ctx.in_dtype != torch.float32:
+            grad = grad.to(ctx.in_dtype)
+        return (grad,) + (None,) * 8
+
+
+def _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask):
+    if proximal_logprobs.shape != old_logprobs.shape:
+        raise ValueError(
+            f"proximal_logprobs shape {proximal_logprobs.shape} != "
+            f"old_logprobs shape {old_logprobs.shape}"
+        )
+    if proximal_logprobs.shape != loss_mask.shape:
+        raise ValueError(
+            f"proximal_logprobs shape {proximal_logprobs.shape} != "
+            f"loss_mask shape {loss_mask.shape}"
+        )
+    if proximal_logprobs.ndim not in (1, 2):
+        raise ValueError(
+            f"Expected 1D (packed) or 2D (padded) tensors, got ndim={proximal_logprobs.ndim}"
+        )
+
+
+def _check_rs_sequences(config, loss_mask, cu_seqlens):
+    if config.level == "sequence" and loss_mask.ndim == 1 and cu_seqlens is None:
+        raise ValueError(
+            "cu_seqlens is required for 1D packed tensors in sequence-level filtering."
+        )
+
+
+def apply_rejection_sampling(
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    loss_mask: torch.Tensor,
+    cu_seqlens: torch.Tensor | None,
+    config: RejectionSamplingConfig,
+) -> RejectionSamplingResult:
+    """Filter (``action='mask'``) or truncate (``action='clamp'``) tokens / sequences whose
+    divergence between proximal and behaviour policy leaves the configured bounds.
+
+    Same contract as ``functional.py:185-437``: the returned mask has the dtype of the input
+    mask; ``filtered_fraction`` is a Python float.
+    """
+    _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask)
+    cfg = _lib.LossConfig()
+    cfg.loss_kind = LOSS_NONE
+    _fill_rs(cfg, config)
+    _check_rs_sequences(config, loss_mask, cu_seqlens)
+    shape = loss_mask.shape
+    mask_bool = loss_mask.detach().bool().contiguous().view(-1)
+    out = _run_loss_kernel(
+        cfg, shape, None, _f32(proximal_logprobs), _f32(old_logprobs), None, mask_bool,
+        cu_seqlens, False,
+    )
+    c = out["counters_dev"].cpu()
+    n_valid, n_filtered = float(c[1]), float(c[3])
+    if config.action == "mask":
+        new_mask = out["new_mask"].view(shape).to(loss_mask.dtype)
+    else:
+        new_mask = loss_mask
+    return RejectionSamplingResult(
+        loss_mask=new_mask,
+        behave_imp_weight=out["behave_imp_weight"].view(shape),
+        filtered_fraction=n_filtered / max(n_valid, 1.0),
+    )
+
+
+def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
+                 rejection_sampling, cu_seqlens):
+    shape = logprobs.shape
+    if rejection_sampling is not None:
+        _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask)
+        _check_rs_sequences(rejection_sampling, loss_mask, cu_seqlens)
+    _fill_rs(cfg, rejection_sampling)
+    mask_bool = loss_mask.detach().bool().contiguous().view(-1)
+    sink: dict = {}
+    loss = _ActorLoss.apply(
+        logprobs, cfg, shape, _f32(proximal_logprobs),
+        _f32(old_logprobs) if (rejection_sampling is not None) else None,
+        _f32(advantages), mask_bool, cu_seqlens, sink,
+    )
+    c = sink["counters_dev"].cpu()  # the one host synchronisation of the call
+    return loss, sink, c, shape
+
+
+def _rs_stats(stat, sink, c, shape, rejection_sampling):
+    if rejection_sampling is None:
+        return
+    stat.update(
+        behave_approx_kl=sink["behave_approx_kl"].view(shape),
+        behave_imp_weight=sink["behave_imp_weight"].view(shape),
+        behave_mask=sink["behave_mask"].view(shape),
+        filtered_fraction=float(c[3]) / max(float(c[1]), 1.0),
+    )
+
+
+def ppo_actor_loss_fn(
+    logprobs: torch.Tensor,
+    proximal_logprobs: torch.Tensor,
+    old_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip: float,
+    loss_mask: torch.Tensor,
+    eps_clip_higher: float | None = None,
+    c_clip: float | None = None,
+    rejection_sampling: RejectionSamplingConfig | None = None,
+    importance_sampling_level: str = "token",
+    cu_seqlens: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """PPO/GRPO clipped surrogate with optional dual clip, GSPO sequence-level ratio and
+    rejection sampling.  Signature, return structure and ``stat`` keys as in
+    ``functional.py:452-596``."""
+    if importance_sampling_level == "sequence":
+        if logprobs.ndim == 1 and cu_seqlens is None:
+            raise ValueError(
+                "cu_seqlens is required for 1D tensors (packed format). "
+                "In AReaL, 1D tensors are produced by pack_tensor_dict() and always have "
+                "cu_seqlens. For a single sequence, use "
+                "cu_seqlens=torch.tensor([0, seq_len], dtype=torch.int32)."
+            )
+    elif importance_sampling_level != "token":
+        raise ValueError(
+            f"Invalid importance_sampling_level: {importance_sampling_level}. "
+            "Must be 'token' or 'sequence'."
+        )
+    if c_clip is not None:
+        assert c_clip > 1.0, c_clip
+    cfg = _lib.LossConfig()
+    cfg.loss_kind = LOSS_PPO
+    cfg.clip_lo = 1.0 - eps_clip
+    cfg.clip_hi = 1.0 + (eps_clip if eps_clip_higher is None else eps_clip_higher)
+    cfg.has_c_clip = int(c_clip is not None)
+    cfg.c_clip = c_clip if c_clip is not None else 0.0
+    cfg.seq_is = int(importance_sampling_level == "sequence")
+    loss, sink, c, shape = _loss_common(
+        cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
+        rejection_sampling, cu_seqlens,
+    )
+    n_total = float(loss_mask.numel())
+    n_valid = float(c[1])
+    stat = dict(
+        loss=sink["stat_loss"].view(shape),
+        importance_weight=sink["ratio"].view(shape),
+        approx_kl=sink["approx_kl"].view(shape),
+        clip_mask=sink["clip_mask"].view(shape),
+        dual_clip_mask=sink["dual_clip_mask"].view(shape),
+        n_total_tokens=n_total,
+        n_valid_tokens=n_valid,
+        n_masked_tokens=n_total - n_valid,
+        masked_token_ratio=1.0 - n_valid / max(n_total, 1.0),
+    )
+    _rs_stats(stat, sink, c, shape, rejection_sampling)
+    return loss, stat
+
+
+def cispo_loss_fn(
+    logprobs: torch.Tensor,
+    proximal_logprobs: torch.Tensor,
+    advantages: torch.Tensor,
+    eps_clip: float,
+    loss_mask: torch.Tensor,
+    eps_clip_higher: float | None = None,
+    old_logprobs: torch.Tensor | None = None,
+    rejection_sampling: RejectionSamplingConfig | None = None,
+    cu_seqlens: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, dict]:
+    """CISPO: clipped importance weight under stop-gradient times ``log pi`` (MiniMax-M1).
+    Signature, errors and ``stat`` keys as in ``functional.py:678-793``."""
+    if eps_clip_higher is None or eps_clip_higher <= 0:
+        raise ValueError(
+            "CISPO requires a positive eps_clip_higher; the asymmetric upper "
+            f"clip is the defining knob (MiniMax-M1 Eq. 4-5). Got {eps_clip_higher!r}."
+        )
+    cfg = _lib.LossConfig()
+    cfg.loss_kind = LOSS_CISPO
+    cfg.clip_lo = 1.0 - eps_clip
+    cfg.clip_hi = 1.0 + eps_clip_higher
+    loss, sink, c, shape = _loss_common(
+        cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
+        rejection_sampling, cu_seqlens,
+    )
+    stat = dict(
+        loss=sink["stat_loss"].view(shape),
+        importance_weight=sink["ratio"].view(shape),
+        approx_kl=sink["approx_kl"].view(shape),
+        clip_mask=sink["clip_mask"].view(shape),
+        dual_clip_mask=torch.zeros(shape, dtype=torch.bool, device=logprobs.device),
+    )
+    _rs_stats(stat, sink, c, shape, rejection_sampling)
+    return loss, stat
+
+
+@torch.no_grad()
+def masked_normalization(
+    x: torch.Tensor,
+    mask: torch.Tensor | None = None,
+    dim=None,
+    unbiased=False,
+    eps=1e-5,
+    high_precision=True,
+    all_reduce=True,
+    reduce_group=None,
+):
+    """Whiten ``x`` over its masked elements (``functional.py:16-53``): fp64 sums,
+    ``var = E[x^2] - E[x]^2``, ``(x * mask - mean) / (sqrt(var) + eps)``.
+
+    Only the reduction over all dimensions is implemented (the only use on this path), in fp64
+    whatever ``high_precision`` says; a multi-rank ``all_reduce`` is outside the one-GPU scope.
+    """
+    if dim is not None and tuple(sorted(d % x.ndim for d in dim)) != tuple(range(x.ndim)):
+        raise NotImplementedError("masked_normalization reduces over all dimensions only")
+    import torch.distributed as dist
+
+    if all_reduce and dist.is_initialized() and dist.get_world_size(reduce_group) > 1:
+        raise NotImplementedError("masked_normalization runs on one GPU; no all_reduce")
+    del high_precision
+    lib = _lib.load()
+    dev = _lib.require_gpu(x, mask)
+    xf = x.to(torch.float32).contiguous()
+    mf = mask.to(torch.float32).contiguous() if mask is not None else None
+    out = torch.empty_like(xf)
+    n = xf.numel()
+    nbytes = lib.areal_masked_norm_workspace_bytes(n)
+    ws = _lib.workspace(nbytes, dev)
+    rc = lib.areal_masked_norm(
+        _lib.ptr(xf), _lib.ptr(mf), n, int(bool(unbiased)), float(eps), _lib.ptr(out),
+        _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_masked_norm")
+    return out

@@ -1,0 +1,96 @@
+"""Generalised advantage estimation on MI355X.
+
+``_compute_token_level_gae`` keeps the reference's padded signature
+(``areal/trainer/ppo/gae.py:10-36``); ``compute_gae_packed`` is the same recurrence on the
+packed layout (``cu_seqlens``), which the reference does not have.  Both run the segmented
+reverse scan of ``csrc/gae_norm.hip``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from areal_amd import _lib
+
+
+def _launch(rewards, values, mask, cu, no_eos, lam_seq, n_seqs, uniform_len, discount, lam):
+    lib = _lib.load()
+    dev = _lib.require_gpu(rewards, values, mask, cu, no_eos, lam_seq)
+    n = rewards.numel()
+    adv = torch.empty(rewards.shape, dtype=torch.float32, device=dev)
+    ret = torch.empty(rewards.shape, dtype=torch.float32, device=dev)
+    if n == 0:
+        return adv, ret
+    nbytes = lib.areal_gae_workspace_bytes(n)
+    ws = _lib.workspace(nbytes, dev)
+    rc = lib.areal_gae_packed(
+        _lib.ptr(rewards), _lib.ptr(values), _lib.ptr(mask), _lib.ptr(cu), _lib.ptr(no_eos),
+        _lib.ptr(lam_seq), n, n_seqs, uniform_len, float(discount), float(lam),
+        _lib.ptr(adv), _lib.ptr(ret), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_gae_packed")
+    return adv, ret
+
+
+def _split_lambda(gae_lambda, n_seqs, device):
+    if isinstance(gae_lambda, torch.Tensor):
+        lam_seq = gae_lambda.to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+        if lam_seq.numel() == 1:
+            lam_seq = lam_seq.expand(n_seqs).contiguous()
+        if lam_seq.numel() != n_seqs:
+            raise ValueError(
+                f"gae_lambda must be a float or hold one value per sequence ({n_seqs}), "
+                f"got {tuple(gae_lambda.shape)}"
+            )
+        return lam_seq, 0.0
+    return None, float(gae_lambda)
+
+
+def _compute_token_level_gae(
+    rewards: torch.Tensor,
+    values: torch.Tensor,
+    loss_mask: torch.Tensor,
+    seq_no_eos_mask: torch.Tensor,
+    discount: float,
+    gae_lambda: float | torch.Tensor,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """GAE with each generated token as one timestep, on padded ``[bs, max_seqlen]`` tensors.
+    Returns ``(advantages, returns)``; ``returns = advantages + values``."""
+    bs, max_seqlen = rewards.shape
+    dev = rewards.device
+    lam_seq, lam = _split_lambda(gae_lambda, bs, dev)
+    return _launch(
+        rewards.to(torch.float32).contiguous(),
+        values.to(torch.float32).contiguous(),
+        loss_mask.to(torch.float32).contiguous(),
+        None,
+        seq_no_eos_mask.to(torch.bool).contiguous(),
+        lam_seq, bs, max_seqlen, discount, lam,
+    )
+
+
+def compute_gae_packed(
+    rewards: torch.Tensor,
+    values: torch.Tensor,
+    loss_mask: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    seq_no_eos_mask: torch.Tensor | None,
+    discount: float,
+    gae_lambda: float | torch.Tensor,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """The same recurrence over 1-D packed tensors: sequence ``i`` is
+    ``[cu_seqlens[i], cu_seqlens[i+1])``; its last position gets advantage 0 and, when
+    ``seq_no_eos_mask[i]``, bootstraps the next value from ``values`` there."""
+    if rewards.ndim != 1:
+        raise ValueError(f"packed GAE expects 1D tensors, got ndim={rewards.ndim}")
+    dev = rewards.device
+    cu = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+    n_seqs = cu.numel() - 1
+    lam_seq, lam = _split_lambda(gae_lambda, n_seqs, dev)
+    no_eos = seq_no_eos_mask.to(device=dev, dtype=torch.bool).contiguous() if seq_no_eos_mask is not None else None
+    return _launch(
+        rewards.to(torch.float32).contiguous(),
+        values.to(torch.float32).contiguous(),
+        loss_mask.to(torch.float32).contiguous(),
+        cu, no_eos, lam_seq, n_seqs, 0, discount, lam,
+    )

@@ -1,0 +1,182 @@
+/* C ABI of libareal_hip.so: MI355X (gfx950) kernels for AReaL's per-token RL training hot path.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless stated otherwise; the library never allocates,
+ *     never synchronises and only touches the stream it is given;
+ *   - scratch memory is passed in by the caller (`workspace`, sized by the matching
+ *     *_workspace_bytes function);
+ *   - return value 0 = success, negative = error (see areal_status);
+ *   - bf16 tensors are passed as `const void*` (raw bfloat16 bit patterns), masks as uint8_t
+ *     (0/1, the memory layout of torch.bool).
+ *
+ * The reference (areal-project/AReaL) is pure Python and has no FFI for this path; each entry
+ * point cites the Python function it replaces (paths relative to the reference root).
+ */
+#ifndef AREAL_HIP_H
+#define AREAL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* areal_stream_t; /* a hipStream_t */
+
+enum areal_status {
+  AREAL_OK = 0,
+  AREAL_ERR_BAD_ARG = -1,
+  AREAL_ERR_ALIGNMENT = -2,
+  AREAL_ERR_WORKSPACE = -3,
+  AREAL_ERR_LAUNCH = -4,
+  AREAL_ERR_UNSUPPORTED = -5
+};
+
+/* ---------------------------------------------------------------------------------------
+ * Fused lm_head -> log-softmax -> label log-prob + entropy
+ * replaces _ChunkedVocabParallelLMHead.forward / .backward
+ * (areal/models/mcore/vocab_parallel_head.py:564-735, :737-938) and the
+ * torch.mm(..., out_dtype=float32) contraction of _linear_chunk_fp32 (:538-557).
+ * ------------------------------------------------------------------------------------- */
+
+size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
+/* hidden [T,H] bf16, weight [V,H] bf16 (H % 8 == 0, 16-byte aligned), bias [V] fp32 or NULL,
+ * labels [T] int64. Outputs fp32 [T]; row_max and sum_exp are the state saved for backward
+ * (vocab_parallel_head.py:704-713). logits = (hidden . weight^T + bias) * logit_scale. */
+int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
+                     const int64_t* labels, int64_t T, int64_t H, int64_t V,
+                     float inv_temperature, float logit_scale, float* logprobs, float* entropy,
+                     float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
+                     float* row_max, float* sum_exp, void* workspace, size_t workspace_bytes,
+                     areal_stream_t stream);
+
+size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
+
+/* grad_logprobs [T] fp32. Writes dhidden [T,H] bf16 (NULL to skip) and dweight_f32 [V,H] fp32
+ * (NULL to skip; added to when accumulate != 0). dlogits are rounded to bf16 before the two
+ * gradient contractions, as in vocab_parallel_head.py:830-839. */
+int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
+                     const int64_t* labels, const float* row_max, const float* sum_exp,
+                     const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
+                     float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
+                     int accumulate, int64_t token_chunk, void* workspace, size_t workspace_bytes,
+                     areal_stream_t stream);
+
+/* out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]  (bf16 in, fp32 accumulate).
+ * out_mode 0: bf16 store, 1: fp32 store, 2: fp32 accumulate. The contraction used by the
+ * entry points above, exported for tests (torch.mm in vocab_parallel_head.py:549-552). */
+int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, void* out,
+                       int64_t ldo, int64_t M, int64_t N, int64_t K, int out_mode,
+                       areal_stream_t stream);
+
+/* dst (bf16) = src (fp32), n elements: the final cast of the weight gradient
+ * (vocab_parallel_head.py:917-918). */
+int areal_cast_f32_to_bf16(const float* src, void* dst, int64_t n, areal_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Logits-in label log-prob + entropy
+ * replaces _gather_logprobs / _gather_logprobs_entropy and their chunked wrappers
+ * (areal/utils/functional/vocab_parallel.py:16-30, :42-82, :564-651).
+ * dtype: 0 = fp32 logits, 1 = bf16 logits; ld = row pitch in elements.
+ * lse2 = log-sum-exp of logits/T in base-2 units (saved for backward).
+ * ------------------------------------------------------------------------------------- */
+int areal_logits_logprobs_entropy_fwd(const void* logits, int dtype, int64_t ld,
+                                      const int64_t* labels, int64_t T, int64_t V,
+                                      float inv_temperature, float* logprobs, float* entropy,
+                                      float* lse2, areal_stream_t stream);
+
+int areal_logits_logprobs_entropy_bwd(const void* logits, int dtype, int64_t ld,
+                                      const int64_t* labels, int64_t T, int64_t V,
+                                      float inv_temperature, const float* lse2,
+                                      const float* entropy, const float* grad_logprobs,
+                                      const float* grad_entropy, void* dlogits, int64_t ldd,
+                                      areal_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Actor loss: PPO / GRPO clip (optionally dual clip, optionally GSPO sequence-level ratio) or
+ * CISPO, with rejection sampling (IcePop ratio bounds, KPop binary KL, k1/k2/k3)
+ * replaces ppo_actor_loss_fn (areal/utils/functional/functional.py:452-596), cispo_loss_fn
+ * (:678-793), apply_rejection_sampling (:185-437), compute_binary_kl_divergence (:440-449) and
+ * _compute_sequence_level_ratio_and_advantages (:56-149).
+ * ------------------------------------------------------------------------------------- */
+typedef struct areal_loss_config {
+  int loss_kind;      /* -1: rejection sampling only, 0: PPO clip, 1: CISPO */
+  float clip_lo;      /* (float)(1.0 - eps_clip) */
+  float clip_hi;      /* (float)(1.0 + eps_clip_higher) */
+  int has_c_clip;
+  float c_clip;
+  int seq_is;         /* importance_sampling_level == "sequence" */
+  int rs_enabled;
+  int rs_seq_level;   /* rejection_sampling.level == "sequence" */
+  int rs_clamp;       /* rejection_sampling.action == "clamp" */
+  int rs_metric;      /* 0 ratio, 1 kl_k1, 2 kl_k2, 3 kl_k3, 4 binary_kl */
+  int rs_agg;         /* 0 sum, 1 mean, 2 max */
+  float rs_upper;
+  int rs_has_lower;
+  float rs_lower;
+} areal_loss_config;
+
+size_t areal_actor_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs);
+
+/* All per-token arrays have n_tokens elements (a packed 1-D batch or a flattened padded one).
+ * Sequences: cu_seqlens [n_seqs+1] int32, or uniform_len > 0 for a padded [n_seqs, uniform_len]
+ * batch; needed only for sequence-level options. cfg is a HOST pointer.
+ * Outputs (each may be NULL): loss [1]; dlogprobs = d(sum of masked token losses)/dlogprobs
+ * (divide by counters[1] for the loss gradient, see areal_actor_loss_grad); the per-token
+ * statistics of the reference's stat dict; new_mask / behave_* of RejectionSamplingResult.
+ * counters [8] double: loss_sum, n_valid (pre-rejection mask count), n_kept, n_filtered
+ * (mask: rejected valid tokens; clamp: valid tokens whose weight changed), n_clip, n_dual_clip,
+ * n_behave, loss. */
+int areal_actor_loss(const float* logprobs, const float* proximal_logprobs,
+                     const float* old_logprobs, const float* advantages,
+                     const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
+                     int64_t n_seqs, int64_t uniform_len, const areal_loss_config* cfg,
+                     float* loss, float* dlogprobs, float* stat_loss, float* stat_ratio,
+                     float* stat_approx_kl, uint8_t* clip_mask, uint8_t* dual_clip_mask,
+                     uint8_t* new_mask, float* behave_imp_weight, float* behave_approx_kl,
+                     uint8_t* behave_mask, double* counters, void* workspace,
+                     size_t workspace_bytes, areal_stream_t stream);
+
+/* grad_logprobs[t] = dlogprobs[t] * upstream[0] / max(counters[1], 1): the backward of
+ * `loss = sum(where(mask, pg, 0)) / loss_mask_count` (functional.py:571). */
+int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const double* counters,
+                          float* grad_logprobs, int64_t n_tokens, areal_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * GAE over packed sequences
+ * replaces _compute_token_level_gae (areal/trainer/ppo/gae.py:10-36); per-sequence lambda as
+ * produced by areal/trainer/ppo/lambda_fn.py:50-112.
+ * ------------------------------------------------------------------------------------- */
+size_t areal_gae_workspace_bytes(int64_t n_tokens);
+
+int areal_gae_packed(const float* rewards, const float* values, const float* loss_mask,
+                     const int32_t* cu_seqlens, const uint8_t* no_eos, const float* lambda_seq,
+                     int64_t n_tokens, int64_t n_seqs, int64_t uniform_len, float discount,
+                     float gae_lambda, float* advantages, float* returns, void* workspace,
+                     size_t workspace_bytes, areal_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Normalisation
+ * replaces Normalization.__call__ / _compute_mean / _compute_std
+ * (areal/utils/data.py:1432-1637) and masked_normalization
+ * (areal/utils/functional/functional.py:16-53). Levels: 0 none, 1 batch, 2 group.
+ * ------------------------------------------------------------------------------------- */
+size_t areal_group_norm_workspace_bytes(int64_t n_groups, int64_t max_group_len);
+
+int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t* group_offsets,
+                     const int64_t* group_rows, int64_t n_groups, int64_t max_group_len,
+                     int tail_group, int mean_level, int std_level, int leave_one_out,
+                     int unbiased, double eps, float* out, void* workspace,
+                     size_t workspace_bytes, areal_stream_t stream);
+
+size_t areal_masked_norm_workspace_bytes(int64_t n);
+
+int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased, double eps,
+                      float* out, void* workspace, size_t workspace_bytes, areal_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AREAL_HIP_H */

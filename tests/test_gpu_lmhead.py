@@ -1,0 +1,136 @@
+"""Fused lm_head -> logprob/entropy kernels against the CPU oracle.
+
+Tolerances: bf16-input logprobs within 2e-3 absolute of the fp32 oracle (measured ~1e-5);
+gradients within 1e-2 relative (relative L2, as the reference compares dW in
+tests/test_megatron_lm_head.py:190-199; measured ~2.5e-3, the bf16 rounding of dlogits)."""
+
+import pytest
+import torch
+
+from areal_amd import _lib
+from areal_amd.functional import fused_lm_head_logprobs_entropy
+from oracle import logprob as L
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
+
+
+@pytest.mark.parametrize("M,N,K", [(32, 32, 16), (256, 256, 64), (300, 200, 72), (1000, 520, 8), (96, 13, 32),
+                                   (260, 513, 200)])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_gemm_nt(dev, M, N, K, mode):
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(M + N + K)
+    A = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    B = torch.randn(N, K, generator=g).bfloat16().to(dev)
+    ref = (B.float() @ A.float().T)
+    if mode == 0:
+        out = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
+    else:
+        out = torch.ones((N, M), dtype=torch.float32, device=dev)
+    rc = lib.areal_gemm_nt_bf16(_lib.ptr(A), K, _lib.ptr(B), K, _lib.ptr(out), M, M, N, K, mode,
+                                _lib.stream_ptr(dev))
+    assert rc == 0
+    if mode == 0:
+        assert torch.equal(out, ref.bfloat16()) or _rel(out.float(), ref) < 4e-3
+    else:
+        torch.testing.assert_close(out, ref + (1.0 if mode == 2 else 0.0), rtol=1e-5, atol=1e-4)
+
+
+SHAPES = [
+    # T, H, V, temperature, logit_scale, bias, token_chunk
+    (13, 32, 96, 0.7, 0.5, True, 5),       # the reference's test shape, chunk 5, scale 0.5, bias
+    (13, 32, 96, 1.0, 1.0, False, None),
+    (2, 8, 3, 1.0, 1.0, False, None),
+    (300, 64, 1000, 1.5, 1.0, False, 128),
+    (700, 128, 5000, 1.0, 2.0, True, None),
+    (515, 896, 151936, 1.0, 1.0, False, 256),
+]
+
+
+@pytest.mark.parametrize("T,H,V,temp,scale,use_bias,chunk", SHAPES)
+def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, chunk):
+    g = torch.Generator().manual_seed(T * 7 + V)
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * (0.5 if V < 10000 else 0.02)).bfloat16()
+    bias = (torch.randn(V, generator=g) * 0.1).bfloat16() if use_bias else None
+    labels = torch.randint(0, V, (T,), generator=g)
+    grad = torch.randn(T, generator=g)
+    grad[::3] = 0
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels.to(dev), temperature=temp, logit_scale=scale,
+                                         bias=bias.to(dev) if use_bias else None, token_chunk=chunk)
+    want = L.lm_head_logprobs_entropy(hidden, weight, labels, temp, scale, bias)
+    names = ["logprobs", "entropy", "vocab_min", "vocab_max", "vocab_mean", "vocab_norm"]
+    for name, a, b in zip(names, out, want):
+        assert a.dtype == torch.float32 and a.shape == (T,)
+        tol = 2e-3 if name in ("logprobs", "entropy") else 2e-3 * max(1.0, b.abs().max().item())
+        err = (a.cpu() - b).abs().max().item()
+        assert err < tol, f"{name}: max abs err {err}"
+    assert out.logprobs.requires_grad and not out.entropy.requires_grad
+    (out.logprobs * grad.to(dev)).sum().backward()
+    dh_want, dw_want = L.lm_head_backward(hidden, weight, labels, grad, temp, scale, bias)
+    assert h.grad.dtype == torch.bfloat16 and w.grad.dtype == torch.bfloat16
+    assert _rel(h.grad.cpu().float(), dh_want) < 1e-2
+    assert _rel(w.grad.cpu().float(), dw_want) < 1e-2
+    assert (h.grad[::3] == 0).all()  # rows with zero upstream gradient get exactly zero
+    cos = torch.nn.functional.cosine_similarity(w.grad.cpu().float().view(-1), dw_want.view(-1), dim=0)
+    assert cos > 0.9999
+
+
+def test_no_vocab_sized_tensor_is_saved(dev):
+    # as the reference checks in tests/test_megatron_lm_head.py:738-741
+    T, H, V = 48, 64, 4096
+    h = torch.randn(T, H, device=dev).bfloat16().requires_grad_(True)
+    w = torch.randn(V, H, device=dev).bfloat16().requires_grad_(True)
+    y = torch.randint(0, V, (T,), device=dev)
+    out = fused_lm_head_logprobs_entropy(h, w, y)
+    for t in out.logprobs.grad_fn.saved_tensors:
+        assert t.numel() < T * V and tuple(t.shape) != (T, V)
+
+
+def test_chunking_and_repeat_runs_are_bit_identical(dev):
+    T, H, V = 600, 128, 3000
+    g = torch.Generator().manual_seed(0)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * 0.3).bfloat16().to(dev)
+    y = torch.randint(0, V, (T,), generator=g).to(dev)
+    grad = torch.randn(T, generator=g).to(dev)
+    res = []
+    for chunk in (None, None, 256):
+        h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+        out = fused_lm_head_logprobs_entropy(h, w, y, token_chunk=chunk)
+        (out.logprobs * grad).sum().backward()
+        res.append((out.logprobs.detach(), out.entropy, h.grad, w.grad))
+    for a, b in zip(res[0], res[1]):
+        assert torch.equal(a, b)
+    assert torch.equal(res[0][0], res[2][0]) and torch.equal(res[0][2], res[2][2])
+    assert _rel(res[2][3].float(), res[0][3].float()) < 1e-2  # dW: different accumulation split
+
+
+def test_large_logits_are_stable(dev):
+    T, H, V = 64, 64, 2048
+    h = (torch.randn(T, H, device=dev) * 30).bfloat16()
+    w = (torch.randn(V, H, device=dev) * 3).bfloat16()
+    y = torch.randint(0, V, (T,), device=dev)
+    out = fused_lm_head_logprobs_entropy(h, w, y)
+    want = L.lm_head_logprobs_entropy(h.cpu(), w.cpu(), y.cpu())
+    assert torch.isfinite(out.logprobs).all() and torch.isfinite(out.entropy).all()
+    torch.testing.assert_close(out.logprobs.cpu(), want[0], rtol=1e-4, atol=2e-3)
+
+
+def test_empty_and_3d_inputs(dev):
+    w = torch.randn(100, 16, device=dev).bfloat16()
+    out = fused_lm_head_logprobs_entropy(torch.empty(0, 16, device=dev).bfloat16(), w,
+                                         torch.empty(0, dtype=torch.long, device=dev))
+    assert out.logprobs.shape == (0,)
+    h = torch.randn(2, 5, 16, device=dev).bfloat16()
+    y = torch.randint(0, 100, (2, 5), device=dev)
+    out = fused_lm_head_logprobs_entropy(h, w, y)
+    want = L.lm_head_logprobs_entropy(h.cpu().view(10, 16), w.cpu(), y.cpu().view(-1))
+    assert out.logprobs.shape == (2, 5)
+    torch.testing.assert_close(out.logprobs.cpu().view(-1), want[0], rtol=1e-4, atol=2e-3)

@@ -1,0 +1,186 @@
+"""Pins the GAE and normalisation oracles with the reference tests' literals and closed forms."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import gae as G
+from oracle import norm as N
+
+
+def _t(x, dtype=torch.float32):
+    return torch.tensor(x, dtype=dtype)
+
+
+def test_gae_per_sample_lambda_literals():
+    # reference tests/test_ppo_gae.py:196-221, atol = 0
+    rewards = _t([[0.0, 0.0, 1.0, 0.0]] * 2)
+    mask = _t([[1.0, 1.0, 1.0, 0.0]] * 2)
+    adv, _ = G.gae_padded(rewards, torch.zeros_like(rewards), mask, torch.tensor([False, False]), 1.0,
+                          _t([0.5, 0.0]))
+    assert torch.equal(adv, _t([[0.25, 0.5, 1.0, 0.0], [0.0, 0.0, 1.0, 0.0]]))
+
+
+def test_gae_closed_form_unmasked():
+    """A_t = sum_k (gamma*lambda)^k delta_{t+k}, delta_t = r_t + gamma V_{t+1} - V_t."""
+    torch.manual_seed(0)
+    L, gamma, lam = 12, 0.9, 0.8
+    r = torch.randn(1, L, dtype=torch.float64)
+    v = torch.randn(1, L, dtype=torch.float64)
+    adv, ret = G.gae_padded(r.float(), v.float(), torch.ones(1, L), torch.tensor([True]), gamma, lam)
+    want = torch.zeros(L, dtype=torch.float64)
+    for t in range(L - 1):
+        acc = 0.0
+        for k in range(L - 1 - t):
+            nv = v[0, t + k + 1]
+            acc += (gamma * lam) ** k * (r[0, t + k] + gamma * nv - v[0, t + k])
+        want[t] = acc
+    torch.testing.assert_close(adv[0].double(), want, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(ret, adv + v.float())
+
+
+def test_gae_no_bootstrap_when_sequence_ended():
+    r = _t([[0.0, 0.0, 1.0, 0.0]])
+    v = _t([[0.5, 0.5, 0.5, 9.0]])
+    a_eos, _ = G.gae_padded(r, v, torch.ones(1, 4), torch.tensor([False]), 1.0, 1.0)
+    a_trunc, _ = G.gae_padded(r, v, torch.ones(1, 4), torch.tensor([True]), 1.0, 1.0)
+    # with gamma = lambda = 1: A_t = sum r + V_boot - V_t
+    assert torch.equal(a_eos, _t([[0.5, 0.5, 0.5, 0.0]]))
+    assert torch.equal(a_trunc, _t([[9.5, 9.5, 9.5, 0.0]]))
+
+
+def test_gae_masked_positions_carry_state():
+    r = _t([[0.0, 5.0, 0.0, 2.0, 0.0]])
+    v = _t([[0.1, 0.2, 0.3, 0.4, 0.0]])
+    m = _t([[1.0, 0.0, 0.0, 1.0, 0.0]])
+    adv, _ = G.gae_padded(r, v, m, torch.tensor([False]), 0.9, 0.8)
+    assert adv[0, 1] == adv[0, 2] == adv[0, 3]  # masked tokens repeat the advantage to their right
+    assert adv[0, 3].item() == pytest.approx(2.0 - 0.4)
+    # the masked reward 5.0 never enters
+    assert adv[0, 0].item() == pytest.approx((0.0 + 0.9 * 0.4 - 0.1) + 0.72 * 1.6, rel=1e-6)
+
+
+def test_gae_packed_equals_padded():
+    """The packed recurrence equals the reference's padded one on the same data, given what the
+    reference's data guarantees: mask 0 on padding and on each sequence's last token (the loss
+    mask is rolled by -1, actor.py:214-215)."""
+    torch.manual_seed(1)
+    lens = [5, 1, 9, 3]
+    L = max(lens)
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+    T = sum(lens)
+    r, v = torch.randn(T), torch.randn(T)
+    m = (torch.rand(T) > 0.3).float()
+    m[cu[1:].long() - 1] = 0.0
+    no_eos = torch.tensor([False, False, True, False])  # only the full-width row may bootstrap
+    lam = _t([0.95, 0.5, 0.9, 1.0])
+    adv_p, ret_p = G.gae_packed(r, v, m, cu, no_eos, 0.99, lam)
+    rp, vp, mp = torch.zeros(4, L), torch.zeros(4, L), torch.zeros(4, L)
+    for i, n in enumerate(lens):
+        s = int(cu[i])
+        rp[i, :n], vp[i, :n], mp[i, :n] = r[s:s + n], v[s:s + n], m[s:s + n]
+    adv_d, ret_d = G.gae_padded(rp, vp, mp, no_eos, 0.99, lam)
+    for i, n in enumerate(lens):
+        s = int(cu[i])
+        assert torch.equal(adv_p[s:s + n], adv_d[i, :n])
+        assert torch.equal(ret_p[s:s + n], ret_d[i, :n])
+
+
+def test_norm_leave_one_out_literals():
+    # reference tests/test_adv_norm_config.py:730-749
+    x = _t([[1.0], [2.0], [3.0], [4.0]])
+    out = N.normalization(x, torch.ones_like(x), mean_level="batch", std_level=None, mean_leave1out=True)
+    torch.testing.assert_close(out, _t([[-2.0], [-2.0 / 3], [2.0 / 3], [2.0]]), atol=1e-6, rtol=0)
+    # :800-810
+    x = _t([[0.0, 0.0], [1.0, 0.0], [0.0, 0.0]])
+    out = N.normalization(x, torch.ones_like(x), mean_level="batch", std_level=None, mean_leave1out=True)
+    torch.testing.assert_close(out, _t([[-0.2, -0.2], [1.0, -0.2], [-0.2, -0.2]]), atol=1e-4, rtol=0)
+
+
+def test_norm_masked_batch_literals():
+    # reference tests/test_adv_norm_config.py:1102-1152: mean 5.0, biased-sample std property
+    x = _t([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0], [7.0, 8.0, 9.0]])
+    m = _t([[1.0, 1.0, 0.0], [1.0, 0.0, 1.0], [0.0, 1.0, 1.0]])
+    out = N.normalization(x, m, mean_level="batch", std_level="batch", group_size=1)
+    assert out[0, 2] == 0 and out[1, 1] == 0 and out[2, 0] == 0
+    vals = out[m.bool()]
+    assert abs(vals.mean().item()) < 1e-5
+    assert abs(vals.std().item() - 1.0) < 1e-5
+    std = math.sqrt(52 / 5)  # unbiased (default) over the six active values
+    torch.testing.assert_close(out[0, 0], _t((1 - 5) / (std + 1e-5)), rtol=1e-5, atol=1e-6)
+
+
+def test_norm_masked_leave_one_out_literals():
+    # reference tests/test_adv_norm_config.py:1209-1224
+    x = _t([[1.0, 2.0], [3.0, 4.0], [5.0, 6.0]])
+    m = _t([[1.0, 1.0], [1.0, 0.0], [0.0, 1.0]])
+    out = N.normalization(x, m, mean_level="batch", std_level="batch", mean_leave1out=True, std_unbiased=True)
+    for got, want in [(out[0, 0], -0.9258), (out[0, 1], -0.4629), (out[1, 0], 0.0), (out[2, 1], 1.3887)]:
+        assert got.item() == pytest.approx(want, abs=1e-3)
+    assert out[1, 1] == 0 and out[2, 0] == 0
+
+
+def test_norm_unbiased_ratio():
+    # reference tests/test_adv_norm_config.py:752-780
+    x = _t([[1.0], [2.0], [3.0]])
+    m = torch.ones_like(x)
+    b = N.normalization(x, m, mean_level="batch", std_level="batch", std_unbiased=False)
+    u = N.normalization(x, m, mean_level="batch", std_level="batch", std_unbiased=True)
+    assert (b.std() / u.std()).item() == pytest.approx(math.sqrt(1.5), abs=1e-4)
+
+
+def test_norm_variable_groups():
+    # reference tests/test_reward_norm_variable_group.py:28-64
+    x = _t([0.0, 3.0, 6.0, 10.0, 20.0, 1.0, 2.0, 3.0])
+    sizes = [3, 2, 3]
+    out = N.normalization(x, None, mean_level="group", std_level="group", group_size=2,
+                          std_unbiased=False, eps=0.0, group_sizes=sizes)
+    off = 0
+    for s in sizes:
+        c = x[off:off + s].double()
+        want = (c - c.mean()) / c.std(unbiased=False)
+        torch.testing.assert_close(out[off:off + s].double(), want, rtol=1e-5, atol=1e-5)
+        off += s
+    a = N.normalization(_t([0.0, 2.0, 10.0, 14.0]), None, mean_level="group", std_level="group", group_size=2,
+                        std_unbiased=False, eps=0.0)
+    b = N.normalization(_t([0.0, 2.0, 10.0, 14.0]), None, mean_level="group", std_level="group", group_size=2,
+                        std_unbiased=False, eps=0.0, group_sizes=[2, 2])
+    torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-6)
+
+
+def test_norm_zero_variance_and_singleton():
+    # reference tests/test_reward_norm_variable_group.py:78-127
+    out = N.normalization(_t([0.0, 3.0, 6.0, 5.0, 5.0]), None, mean_level="group", std_level="group",
+                          group_size=2, std_unbiased=False, eps=1e-5, group_sizes=[3, 2])
+    assert torch.isfinite(out).all() and (out[3:] == 0).all()
+    out = N.normalization(_t([7.0, 1.0, 5.0]), None, mean_level="group", std_level="group", group_size=1,
+                          mean_leave1out=True, std_unbiased=True, eps=1e-5, group_sizes=[1, 2])
+    assert torch.isfinite(out).all() and out[0].item() == 0.0
+
+
+def test_norm_errors_and_all_masked():
+    x = _t([0.0, 1.0, 2.0, 3.0])
+    with pytest.raises(ValueError, match="must equal"):
+        N.normalization(x, None, mean_level="group", std_level="group", group_size=2, group_sizes=[3, 2])
+    with pytest.raises(ValueError, match="positive"):
+        N.normalization(x, None, mean_level="group", std_level="group", group_size=2, group_sizes=[4, 0])
+    out = N.normalization(x, torch.zeros(4))
+    assert torch.equal(out, x)
+
+
+def test_norm_tail_rows_divide_by_eps():
+    # fixed group_size leaves bs % group_size rows with mean 0 / std 0 (data.py:1405-1410)
+    x = _t([1.0, 3.0, 5.0])
+    out = N.normalization(x, None, mean_level="group", std_level="group", group_size=2, eps=1e-5)
+    assert out[2].item() == pytest.approx(5.0 / 1e-5, rel=1e-5)
+
+
+def test_masked_normalization_closed_form():
+    torch.manual_seed(0)
+    x = torch.randn(50) * 3 + 2
+    m = (torch.rand(50) > 0.4).float()
+    out = N.masked_normalization(x, m, unbiased=False, eps=1e-5)
+    act = x[m.bool()].double()
+    want = ((x.double() * m.double()) - act.mean()) / (act.std(unbiased=False) + 1e-5)
+    torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-6)
