@@ -1,0 +1,231 @@
+"""Benchmark of the per-token RL training hot path on one MI355X.
+
+One "step" = fused lm_head -> logprob/entropy forward, GRPO/PPO actor loss with IcePop
+(ratio-bound) rejection sampling, and the backward pass to dHidden and dWeight, on one packed
+micro-batch that is already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py --gpus 1 --steps 10 --warmup 3 [--workload qwen3-8b]
+"""
+
+from __future__ import annotations
+
+import argparse
+import functools
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+V_QWEN = 151936
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak used for the roofline fraction
+
+WORKLOADS = {
+    # name: (T, H, n_seqs, min_len, max_len, seed, description)
+    "qwen3-8b": dict(T=32768, H=4096, n_seqs=32, lo=256, hi=2048, seed=3,
+                     desc="BASELINE config 4: Qwen3-8B shape fwd+bwd, IcePop ratio bounds [0.5, 2.0]"),
+    "qwen2.5-1.5b": dict(T=16384, H=1536, n_seqs=64, lo=32, hi=2048, seed=1,
+                         desc="BASELINE config 2: Qwen2.5-1.5B shape fwd+bwd, decoupled PPO"),
+    "qwen2.5-0.5b": dict(T=4096, H=896, n_seqs=16, lo=64, hi=512, seed=0,
+                         desc="BASELINE config 1 shape (run fwd+bwd here)"),
+}
+
+
+def make_batch(name: str, device):
+    """Synthetic packed micro-batch of the named shape (seeded, random-init weights)."""
+    import torch
+
+    w = WORKLOADS[name]
+    T, H = w["T"], w["H"]
+    g = torch.Generator().manual_seed(w["seed"])
+    lens = torch.randint(w["lo"], w["hi"] + 1, (w["n_seqs"],), generator=g)
+    if int(lens.sum()) > T:  # rescale proportionally so the sequences fit
+        lens = torch.clamp((lens.double() * T / lens.sum()).floor().long(), min=w["lo"])
+        while int(lens.sum()) > T:
+            lens[lens.argmax()] -= 1
+    pad = T - int(lens.sum())
+    seg = lens.tolist() + ([pad] if pad > 0 else [])
+    cu = torch.tensor([0] + torch.tensor(seg).cumsum(0).tolist(), dtype=torch.int32)
+    loss_mask = torch.ones(T, dtype=torch.bool)
+    loss_mask[cu[1 : w["n_seqs"] + 1].long() - 1] = False  # last token of a sequence has no label
+    if pad > 0:
+        loss_mask[T - pad :] = False
+    hidden = torch.randn(T, H, generator=g, dtype=torch.float32).bfloat16()
+    labels = torch.randint(0, V_QWEN, (T,), generator=g)
+    weight = torch.empty(V_QWEN, H, dtype=torch.bfloat16)
+    for i in range(0, V_QWEN, 16384):  # chunked to bound host memory
+        n = min(16384, V_QWEN - i)
+        weight[i : i + n] = (torch.randn(n, H, generator=g) * 0.02).bfloat16()
+    adv_seq = torch.randn(len(seg), generator=g)
+    advantages = adv_seq.repeat_interleave(torch.tensor(seg))
+    return dict(
+        hidden=hidden.to(device), weight=weight.to(device), labels=labels.to(device),
+        cu_seqlens=cu.to(device), loss_mask=loss_mask.to(device), advantages=advantages.to(device),
+        T=T, H=H, V=V_QWEN, seed=w["seed"],
+    )
+
+
+def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int):
+    """The CPU oracle (plain PyTorch port of the reference's op sequence) on a token slice at
+    full vocabulary: fp32 logits from bf16 operands, log-softmax + entropy, PPO loss with
+    rejection sampling, autograd backward to hidden and weight."""
+    import torch
+
+    from oracle import logprob as olp
+    from oracle import loss as oloss
+
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(seed)
+    n = sample_tokens
+    hidden = torch.randn(n, H, generator=g).bfloat16()
+    weight = (torch.randn(V_QWEN, H, generator=g) * 0.02).bfloat16()
+    labels = torch.randint(0, V_QWEN, (n,), generator=g)
+    adv = torch.randn(n, generator=g)
+    mask = torch.ones(n, dtype=torch.bool)
+    t0 = time.perf_counter()
+    h32 = hidden.float().requires_grad_(True)
+    w32 = weight.float().requires_grad_(True)
+    logits = h32 @ w32.T
+    lp, ent = olp.gather_logprobs_entropy(logits, labels, 1.0)
+    old = lp.detach() + 0.05
+    loss, _ = oloss.ppo_actor_loss(lp, lp.detach(), old, adv, 0.2, mask,
+                                   rejection_sampling_cfg=dict(level="token", action="mask", metric="ratio",
+                                                               upper=2.0, lower=0.5))
+    loss.backward()
+    dt = time.perf_counter() - t0
+    return n / dt, dt
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="qwen3-8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-sample-tokens", type=int, default=512)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+
+    from areal_amd import _lib
+    from areal_amd.config import RejectionSamplingConfig
+    from areal_amd.functional import fused_lm_head_logprobs_entropy
+    from areal_amd.ppo.actor import grpo_loss_fn
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X: the hot path has no CPU implementation")
+    _lib.load()
+    dev = torch.device("cuda:0")
+    b = make_batch(args.workload, dev)
+    T, H, V = b["T"], b["H"], b["V"]
+    hidden = b["hidden"].requires_grad_(True)
+    weight = b["weight"].requires_grad_(True)
+
+    # rollout log-probs = train log-probs + Laplace(0, 0.1); proximal = train log-probs
+    with torch.no_grad():
+        logp0 = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0).logprobs
+    torch.manual_seed(b["seed"])
+    old = logp0 + torch.distributions.Laplace(0.0, 0.1).sample((T,)).to(dev)
+    input_data = dict(logprobs=old, advantages=b["advantages"], loss_mask=b["loss_mask"],
+                      prox_logp=logp0, cu_seqlens=b["cu_seqlens"])
+    loss_fn = functools.partial(
+        grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None,
+        rejection_sampling=RejectionSamplingConfig(level="token", action="mask", metric="ratio",
+                                                   lower=0.5, upper=2.0),
+    )
+
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    t_fwd = t_loss = t_bwd = 0.0
+
+    def step(timed: bool):
+        nonlocal t_fwd, t_loss, t_bwd
+        hidden.grad = None
+        weight.grad = None
+        ev[0].record()
+        out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0)
+        ev[1].record()
+        loss = loss_fn(out.logprobs, out.entropy, input_data,
+                       vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
+        ev[2].record()
+        loss.backward()
+        ev[3].record()
+        if timed:
+            torch.cuda.synchronize()
+            t_fwd += ev[0].elapsed_time(ev[1])
+            t_loss += ev[1].elapsed_time(ev[2])
+            t_bwd += ev[2].elapsed_time(ev[3])
+        return loss
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step(True)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    tokens_per_s = T * args.steps / wall
+
+    # Roofline of the MFMA contraction kernel (gemm_nt_sweep): one step launches it four times
+    # (forward, recompute, dHidden, dWeight) for 3 algorithmic GEMMs = 6*T*H*V flops; the
+    # recompute launch carries no algorithmic flops.  Durations are the HIP-event times of the
+    # forward and backward library calls (they also contain the merge, transpose and cast
+    # kernels, which makes the figure slightly pessimistic).
+    gemm_ms = (t_fwd + t_bwd) / args.steps
+    algo_flops = 6.0 * T * H * V
+    achieved = algo_flops / (gemm_ms * 1e-3) / 1e12
+    fwd_tflops = 2.0 * T * H * V / (t_fwd / args.steps * 1e-3) / 1e12
+
+    result = {
+        "metric": "packed tokens/sec, logprob+entropy+PPO loss fwd+bwd; % bf16 MFMA peak",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: {WORKLOADS[args.workload]['desc']}",
+            "tokens": T, "hidden": H, "vocab": V,
+            "loss": "PPO clip eps=0.2, rejection sampling ratio in [0.5, 2.0] (token, mask)",
+            "final_loss": float(loss.detach().item()),
+        },
+        "pct_bf16_mfma_peak": 100.0 * (algo_flops / (ms_per_step * 1e-3) / 1e12) / PEAK_BF16_TFLOPS,
+        "roofline": {
+            "kernel": "gemm_nt_sweep (4 launches/step: forward, recompute, dHidden, dWeight)",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "forward_only_tflops": fwd_tflops,
+            "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
+                   "loss_bwd+lmhead_bwd": t_bwd / args.steps},
+        },
+    }
+    if not args.no_cpu_baseline:
+        threads = min(16, os.cpu_count() or 1)
+        tps, dt = cpu_baseline(args.cpu_sample_tokens, H, b["seed"], threads)
+        result["cpu_baseline"] = {
+            "value": tps, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{args.cpu_sample_tokens}-token slice at full vocabulary, fwd+bwd with the "
+                      f"PyTorch oracle, {dt:.1f} s (rate is per token, so it scales linearly in T)",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

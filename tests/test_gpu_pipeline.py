@@ -1,0 +1,213 @@
+"""End-to-end and full-size checks of the hot path on the GPU: the engine/actor glue against a
+composition of oracle pieces, and the BASELINE-size workloads through size-independent
+properties plus oracle comparison on slices."""
+
+import functools
+import math
+
+import pytest
+import torch
+
+from areal_amd.config import NormConfig, RejectionSamplingConfig
+from areal_amd.data import KLEstimator, Normalization
+from areal_amd.engine import compute_logprobs, compute_logprobs_and_loss
+from areal_amd.functional import fused_lm_head_logprobs_entropy, ppo_actor_loss_fn
+from areal_amd.ppo.actor import compute_advantages, grpo_loss_fn
+from areal_amd.ppo.gae import compute_gae_packed
+from oracle import gae as G
+from oracle import logprob as L
+from oracle import loss as O
+from oracle import norm as N
+
+pytestmark = pytest.mark.gpu
+
+
+def test_compute_advantages_matches_oracle_composition(dev):
+    g = torch.Generator().manual_seed(0)
+    bs, Lw = 8, 96
+    lens = torch.randint(20, Lw + 1, (bs,), generator=g)
+    lens[0] = Lw
+    attn = (torch.arange(Lw)[None] < lens[:, None]).long()
+    prompt = lens // 4
+    loss_mask = ((torch.arange(Lw)[None] >= prompt[:, None]) & attn.bool()).long()
+    data = dict(
+        input_ids=torch.randint(0, 1000, (bs, Lw), generator=g),
+        attention_mask=attn,
+        loss_mask=loss_mask,
+        logprobs=-torch.rand(bs, Lw, generator=g),
+        ref_logp=-torch.rand(bs, Lw, generator=g),
+        rewards=(torch.rand(bs, generator=g) > 0.5).float() * 5,
+        values=torch.randn(bs, Lw, generator=g) * 0.1,
+    )
+    kw = dict(kl_ctl=0.1, reward_bias=-0.5, reward_scaling=2.0, reward_clip=4.0, discount=0.99, gae_lambda=0.9)
+
+    # oracle composition of actor.py:178-323 on CPU
+    rs = torch.clip((data["rewards"] + kw["reward_bias"]) * kw["reward_scaling"], -4.0, 4.0)
+    rs = N.normalization(rs, None, mean_level="group", std_level="group", group_size=4)
+    m = torch.roll(loss_mask.float(), -1, -1)
+    old = torch.roll(data["logprobs"], -1, -1) * m
+    ref = data["ref_logp"] * m
+    rew = -kw["kl_ctl"] * (old - ref).clamp(-10, 10)
+    idx = torch.arange(bs)
+    rew[idx, lens - 1] = 0
+    rew[idx, (lens - 2).clamp(min=0)] += rs
+    adv, ret = G.gae_padded(rew, data["values"], m, lens == Lw, 0.99, 0.9)
+    adv = N.normalization(adv, m, mean_level="batch", std_level="batch")
+
+    gd = {k: v.to(dev) for k, v in data.items()}
+    out = compute_advantages(
+        gd, kl_estimator=KLEstimator("k1"),
+        reward_norm=Normalization(NormConfig(mean_level="group", std_level="group", group_size=4)),
+        adv_norm=Normalization(NormConfig(mean_level="batch", std_level="batch")), **kw)
+    torch.testing.assert_close(out["advantages"].cpu(), adv, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(out["returns"].cpu(), ret, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(out["tot_rewards"].cpu(), rew, rtol=1e-5, atol=1e-6)
+    assert torch.equal(out["loss_mask"].cpu(), m)
+    assert torch.equal(out["logprobs"].cpu(), old)
+
+
+def test_engine_loss_step_matches_oracle(dev):
+    """Label roll, pad trim, loss scaling and the fused kernels together (config-1-like shape)."""
+    g = torch.Generator().manual_seed(1)
+    T, H, V, pad = 512, 64, 3000, 37
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.2).bfloat16()
+    ids = torch.randint(0, V, (1, T), generator=g)
+    n = T - pad
+    cu = torch.tensor([0, 100, 260, n, T], dtype=torch.int32)
+    mask = torch.rand(n, generator=g) > 0.3
+    adv = torch.randn(n, generator=g)
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    with torch.no_grad():
+        prox = compute_logprobs(h, w, dict(input_ids=ids.to(dev)), pad_length=pad)
+    labels = torch.roll(ids, -1, -1)[0]
+    want_lp = L.lm_head_logprobs_entropy(hidden, weight, labels)[0][:n]
+    assert (prox.cpu() - want_lp).abs().max() < 2e-3
+    old = prox.cpu() + torch.randn(n, generator=g) * 0.1
+    mb = dict(logprobs=old.to(dev), advantages=adv.to(dev), loss_mask=mask.to(dev), prox_logp=prox,
+              cu_seqlens=cu[:4].to(dev))
+    stats = {}
+    rs = dict(level="token", action="mask", metric="ratio", upper=2.0, lower=0.5)
+    loss_fn = functools.partial(grpo_loss_fn, eps_clip=0.2, eps_clip_higher=0.28, c_clip=3.0,
+                                rejection_sampling=RejectionSamplingConfig(**rs), stats=stats)
+    loss = compute_logprobs_and_loss(
+        h, w, dict(input_ids=ids.to(dev)), mb, loss_fn, lambda d: d["loss_mask"].count_nonzero(),
+        total_loss_weight=torch.tensor(2.0 * int(mask.sum()), device=dev), pad_length=pad, loss_multiplier=4.0)
+    loss.backward()
+    # oracle: same proximal/old log-probs, loss on the oracle's own log-probs
+    lp_o = want_lp.clone().requires_grad_(True)
+    lo, so = O.ppo_actor_loss(lp_o, prox.cpu(), old, adv, 0.2, mask, eps_clip_higher=0.28, c_clip=3.0,
+                              rejection_sampling_cfg=rs)
+    (lo * 2.0).backward()
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach() * 2.0, rtol=2e-3, atol=1e-5)
+    assert torch.equal(stats["unclipped_behave_tokens"].cpu(), so["behave_mask"])
+    assert stats["vocab_max_logits"].shape == (n,) and stats["entropy"].dtype == torch.float32
+    g_full = torch.zeros(T)
+    g_full[:n] = lp_o.grad
+    dh, dw = L.lm_head_backward(hidden, weight, labels, g_full)
+    assert ((h.grad.cpu().float() - dh).norm() / dh.norm()) < 1e-2
+    assert ((w.grad.cpu().float() - dw).norm() / dw.norm()) < 1e-2
+    # zero-weight micro-batch
+    zero = compute_logprobs_and_loss(h, w, dict(input_ids=ids.to(dev)), mb, loss_fn, lambda d: 0,
+                                     total_loss_weight=1.0)
+    assert zero.item() == 0.0
+
+
+def _lognormal_lengths(n, mu, sigma, lo, hi, g):
+    return torch.clamp((torch.randn(n, generator=g) * sigma + mu).exp().long(), lo, hi)
+
+
+def test_config3_gae_and_group_norm_full_size(dev):
+    """1024 sequences, lognormal(7, 1) lengths in [16, 8192] (~1.6 M tokens), gamma 1, lambda 0.95,
+    then group-of-16 normalisation: oracle on the first 48 sequences, properties on all."""
+    g = torch.Generator().manual_seed(2)
+    lens = _lognormal_lengths(1024, 7.0, 1.0, 16, 8192, g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    T = int(cu[-1])
+    values = torch.randn(T, generator=g)
+    rewards = torch.zeros(T)
+    rewards[cu[1:].long() - 2] = (torch.rand(1024, generator=g) > 0.5).float()
+    pos = torch.arange(T) - cu[:-1].long().repeat_interleave(lens)
+    seq_len = lens.repeat_interleave(lens)
+    mask = ((pos >= seq_len // 4) & (pos < seq_len - 1)).float()
+    adv, ret = compute_gae_packed(rewards.to(dev), values.to(dev), mask.to(dev), cu.to(dev), None, 1.0, 0.95)
+    k = int(cu[48])
+    want_a, want_r = G.gae_packed(rewards[:k], values[:k], mask[:k], cu[:49], None, 1.0, 0.95)
+    scale = want_a.abs().max().item()
+    torch.testing.assert_close(adv[:k].cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
+    torch.testing.assert_close(ret[:k].cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
+    a = adv.cpu()
+    assert torch.isfinite(a).all() and (a[cu[1:].long() - 1] == 0).all()
+    torch.testing.assert_close(ret.cpu(), a + values, rtol=0, atol=0)
+    # prompt tokens repeat the advantage of the first response token (masked carry)
+    s = int(cu[5])
+    p = int(lens[5]) // 4
+    assert (a[s:s + p] == a[s + p]).all()
+
+    # group normalisation on the packed layout = padded [1024, L] semantics per group of 16 rows
+    norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
+    L_pad = int(lens.max())
+    padded_adv = torch.zeros(1024, L_pad)
+    padded_mask = torch.zeros(1024, L_pad)
+    idx = (torch.arange(1024).repeat_interleave(lens), pos)
+    padded_adv[idx] = a
+    padded_mask[idx] = mask
+    out = norm(padded_adv.to(dev), padded_mask.to(dev)).cpu()
+    want = N.normalization(padded_adv[:32], padded_mask[:32], mean_level="group", std_level="group", group_size=16)
+    torch.testing.assert_close(out[:32], want, rtol=1e-4, atol=1e-5)
+    for gi in (0, 17, 63):
+        vals = out[gi * 16:(gi + 1) * 16][padded_mask[gi * 16:(gi + 1) * 16].bool()].double()
+        assert abs(vals.mean().item()) < 1e-4 and abs(vals.std().item() - 1.0) < 1e-3
+    assert (out[padded_mask == 0] == 0).all()
+
+
+def test_config4_full_size_masks_bit_exact(dev):
+    """Qwen3-8B shape forward at T=32768, then IcePop (ratio [0.5, 2]) and KPop (binary KL 0.05)
+    masking: masks and counts bit-exact against the oracle fed the same log-probs; the fused
+    forward against the oracle on a 192-token slice at full vocabulary."""
+    g = torch.Generator().manual_seed(3)
+    T, H, V = 32768, 4096, 151936
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = torch.empty(V, H, dtype=torch.bfloat16, device=dev)
+    for i in range(0, V, 32768):
+        n = min(32768, V - i)
+        weight[i:i + n] = (torch.randn(n, H, generator=g) * 0.02).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    with torch.no_grad():
+        out = fused_lm_head_logprobs_entropy(hidden, weight, labels)
+    lp = out.logprobs.cpu()
+    assert torch.isfinite(lp).all() and (lp <= 0).all()
+    ent = out.entropy.cpu()
+    assert (ent >= 0).all() and (ent <= math.log(V) + 1e-3).all()
+    assert (out.vocab_max_logits >= out.vocab_min_logits).all()
+    rows = torch.arange(0, T, T // 192)[:192]
+    want = L.lm_head_logprobs_entropy(hidden[rows.to(dev)].cpu(), weight.cpu(), labels[rows.to(dev)].cpu())
+    assert (lp[rows] - want[0]).abs().max() < 2e-3
+    assert (ent[rows] - want[1]).abs().max() < 2e-3
+    assert (out.vocab_max_logits.cpu()[rows] - want[3]).abs().max() < 2e-3
+
+    torch.manual_seed(3)
+    old = lp + torch.distributions.Laplace(0.0, 0.1).sample((T,))
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) > 0.1
+    for rs, bounds in ((dict(level="token", action="mask", metric="ratio", lower=0.5, upper=2.0), (0.5, 2.0)),
+                       (dict(level="token", action="mask", metric="binary_kl", upper=0.05), (0.05,))):
+        lo, so = O.ppo_actor_loss(lp.clone(), lp, old, adv, 0.2, mask, rejection_sampling_cfg=rs)
+        lg, sg = ppo_actor_loss_fn(lp.to(dev), lp.to(dev), old.to(dev), adv.to(dev), 0.2, mask.to(dev),
+                                   rejection_sampling=RejectionSamplingConfig(**rs))
+        # guard band: tokens whose metric lies within 2 ulp of a bound (exp/log may differ there)
+        if rs["metric"] == "ratio":
+            metric = torch.exp(lp - old)
+        else:
+            metric = torch.maximum(O.binary_kl(lp, old), O.binary_kl(old, lp))
+        guard = 0
+        for b in bounds:
+            bt = torch.tensor(b)
+            guard += int(((metric - bt).abs() <= 2 * (torch.nextafter(bt, bt + 1) - bt)).sum())
+        assert guard == 0, f"{guard} tokens inside the 2-ulp guard band; pick another seed"
+        assert torch.equal(sg["behave_mask"].cpu(), so["behave_mask"])
+        assert torch.equal(sg["clip_mask"].cpu(), so["clip_mask"])
+        assert sg["n_valid_tokens"] == so["n_valid_tokens"]
+        assert sg["filtered_fraction"] == so["filtered_fraction"]
+        torch.testing.assert_close(lg.cpu(), lo, rtol=1e-4, atol=1e-8)

@@ -1,0 +1,172 @@
+"""Host-side behaviour that needs no GPU: the library loads and exports every symbol declared
+in include/areal_hip.h, argument validation raises the reference's exception types before any
+device work, and the product path refuses CPU tensors instead of falling back."""
+
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from areal_amd import _lib
+from areal_amd.config import NormConfig, RejectionSamplingConfig
+from areal_amd.data import KLEstimator, Normalization
+from areal_amd.functional import (
+    apply_rejection_sampling,
+    cispo_loss_fn,
+    fused_lm_head_logprobs_entropy,
+    gather_logprobs,
+    gather_logprobs_entropy,
+    ppo_actor_loss_fn,
+)
+from areal_amd.functional.lm_head import default_token_chunk
+from areal_amd.ppo.actor import grpo_loss_fn
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "areal_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(areal_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 17
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in areal_hip.h but not exported"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_workspace_size_queries_run_without_gpu():
+    lib = _lib.load()
+    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096, 151936) == 7 * 16 * 32768 * 4
+    assert lib.areal_lmhead_bwd_workspace_bytes(1024, 64, 1000, 256) > 2 * (256 * 1000 + 1000 * 256)
+    assert lib.areal_gae_workspace_bytes(0) == 0
+    assert lib.areal_actor_loss_workspace_bytes(10, 3) > 0
+
+
+def test_no_cpu_fallback():
+    h = torch.randn(4, 8).bfloat16()
+    w = torch.randn(16, 8).bfloat16()
+    y = torch.randint(0, 16, (4,))
+    with pytest.raises(_lib.ArealHipError, match="no CPU fallback"):
+        fused_lm_head_logprobs_entropy(h, w, y)
+    with pytest.raises(_lib.ArealHipError, match="no CPU fallback"):
+        gather_logprobs(torch.randn(4, 16), y)
+    z = torch.zeros(4)
+    with pytest.raises(_lib.ArealHipError, match="no CPU fallback"):
+        ppo_actor_loss_fn(z, z, z, z, 0.2, torch.ones(4, dtype=torch.bool))
+    with pytest.raises(_lib.ArealHipError, match="no CPU fallback"):
+        Normalization(NormConfig())(z)
+
+
+def test_lm_head_argument_errors():
+    h = torch.randn(4, 8).bfloat16()
+    w = torch.randn(16, 8).bfloat16()
+    y = torch.randint(0, 16, (4,))
+    with pytest.raises(ValueError, match="temperature must be positive"):
+        fused_lm_head_logprobs_entropy(h, w, y, temperature=0.0)
+    with pytest.raises(ValueError, match="temperature must be positive"):
+        fused_lm_head_logprobs_entropy(h, w, y, temperature=float("nan"))
+    with pytest.raises(ValueError, match="logit_scale must be positive"):
+        fused_lm_head_logprobs_entropy(h, w, y, logit_scale=-1.0)
+    with pytest.raises(ValueError, match="chunk_size must be positive"):
+        fused_lm_head_logprobs_entropy(h, w, y, token_chunk=0)
+    with pytest.raises(ValueError, match="matching hidden and weight dtypes"):
+        fused_lm_head_logprobs_entropy(h.float(), w, y)
+    with pytest.raises(ValueError, match="leading dimensions must match labels"):
+        fused_lm_head_logprobs_entropy(h, w, y[:3])
+    assert default_token_chunk(32768, 4096, 151936) == 32768
+    assert default_token_chunk(131072, 5120, 151936) % 256 == 0
+
+
+def test_logits_argument_errors():
+    with pytest.raises(ValueError, match="temperature must be positive"):
+        gather_logprobs_entropy(torch.randn(4, 16), torch.zeros(4, dtype=torch.long), temperature=-1.0)
+    with pytest.raises(ValueError, match="leading dimensions must match labels"):
+        gather_logprobs(torch.randn(4, 16), torch.zeros(3, dtype=torch.long))
+
+
+def test_loss_argument_errors():
+    z = torch.zeros(4)
+    m = torch.ones(4, dtype=torch.bool)
+    # messages matched by the reference's tests (tests/test_functional.py:665,762)
+    with pytest.raises(ValueError, match="cu_seqlens is required"):
+        ppo_actor_loss_fn(z, z, z, z, 0.2, m, importance_sampling_level="sequence")
+    with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
+        ppo_actor_loss_fn(z, z, z, z, 0.2, m, importance_sampling_level="invalid")
+    with pytest.raises(AssertionError):
+        ppo_actor_loss_fn(z, z, z, z, 0.2, m, c_clip=1.0)
+    for bad in (None, 0.0, -1.0):  # tests/test_cispo_loss.py:96-108
+        with pytest.raises(ValueError, match="eps_clip_higher"):
+            cispo_loss_fn(z, z, z, 1.0, m, eps_clip_higher=bad)
+    cfg = RejectionSamplingConfig(level="token", metric="ratio", upper=5.0)
+    with pytest.raises(ValueError, match="shape"):  # tests/test_rejection_sampling.py:796-810
+        apply_rejection_sampling(torch.zeros(1, 2), torch.zeros(1, 3), torch.ones(1, 2), None, cfg)
+    seq = RejectionSamplingConfig(level="sequence", metric="ratio", upper=5.0)
+    with pytest.raises(ValueError, match="cu_seqlens is required"):
+        apply_rejection_sampling(z, z, torch.ones(4), None, seq)
+    with pytest.raises(ValueError, match="ndim"):
+        apply_rejection_sampling(torch.zeros(1, 1, 2), torch.zeros(1, 1, 2), torch.ones(1, 1, 2), None, cfg)
+
+
+def test_rejection_sampling_config_validation():
+    # tests/test_rejection_sampling.py:813-839 and :24-42
+    with pytest.raises(ValueError, match="lower.*cannot be greater than upper"):
+        RejectionSamplingConfig(metric="ratio", lower=3.0, upper=2.0)
+    for field in ("level", "action", "metric", "agg"):
+        with pytest.raises(ValueError, match=f"{field} must be one of"):
+            RejectionSamplingConfig(**{field: "invalid"})
+    with pytest.raises(ValueError, match="upper must be > 1.0"):
+        RejectionSamplingConfig(metric="ratio", upper=1.0)
+    with pytest.raises(ValueError, match="lower must be positive"):
+        RejectionSamplingConfig(metric="ratio", lower=0.0, upper=2.0)
+    with pytest.raises(ValueError, match="only supports metric='ratio'"):
+        RejectionSamplingConfig(action="clamp", metric="kl_k2", upper=1.0)
+    assert RejectionSamplingConfig(action="clamp", metric="ratio", upper=5.0).lower == 0.0
+    with pytest.warns(UserWarning, match="ignored when level='token'"):
+        RejectionSamplingConfig(level="token", agg="max")
+    assert RejectionSamplingConfig(metric="binary_kl", upper=0.05).metric == "binary_kl"
+
+
+def test_norm_config_and_group_errors():
+    with pytest.raises(ValueError, match="mean_level"):
+        NormConfig(mean_level="token")
+    with pytest.raises(ValueError, match="group_size must be a positive integer"):
+        NormConfig(mean_level="group", group_size=0)
+    norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=2))
+    with pytest.raises(ValueError, match="must equal"):
+        norm._group_rows(4, [3, 2])
+    with pytest.raises(ValueError, match="positive"):
+        norm._group_rows(4, [4, 0])
+    assert norm._group_rows(5, None) == ((2, 2), 1)
+    assert norm._group_rows(8, [3, 2, 3]) == ((3, 2, 3), 0)
+
+
+def test_kl_estimator_values():
+    a, b = torch.tensor([0.5, -0.5, 20.0]), torch.zeros(3)
+    assert torch.equal(KLEstimator("k1")(a, b), torch.tensor([0.5, -0.5, 10.0]))
+    torch.testing.assert_close(KLEstimator("k2", apply_clamp=False)(a, b), a * a / 2)
+    torch.testing.assert_close(KLEstimator("k3", apply_clamp=False)(a, b), torch.exp(-a) - 1 + a)
+    with pytest.raises(ValueError, match="Invalid KL estimator"):
+        KLEstimator("k4")
+
+
+def test_grpo_loss_fn_rejects_out_of_scope_options():
+    z = torch.zeros(4)
+    data = dict(logprobs=z, advantages=z, loss_mask=torch.ones(4), prox_logp=z)
+    with pytest.raises(NotImplementedError, match="M2PO"):
+        grpo_loss_fn(z, z, data, 0.2, None, None, m2_threshold=0.1)
+    with pytest.raises(ValueError, match="mutually exclusive"):
+        grpo_loss_fn(z, z, data, 0.2, 4.0, None, use_cispo_loss=True, use_sapo_loss=True)
+    with pytest.raises(ValueError, match="CISPO only supports"):
+        grpo_loss_fn(z, z, data, 0.2, 4.0, None, use_cispo_loss=True, importance_sampling_level="sequence")
+    data["prox_logp"] = None
+    with pytest.raises(ValueError, match="prox_logp is None"):
+        grpo_loss_fn(z, z, data, 0.2, None, None)
+    data["prox_logp"] = torch.tensor([0.0, float("nan"), 0.0, 0.0])
+    with pytest.raises(RuntimeError, match="NaN or Inf"):
+        grpo_loss_fn(z, z, data, 0.2, None, None)
