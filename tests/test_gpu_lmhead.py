@@ -90,7 +90,7 @@ def test_no_vocab_sized_tensor_is_saved(dev):
     y = torch.randint(0, V, (T,), device=dev)
     out = fused_lm_head_logprobs_entropy(h, w, y)
     for t in out.logprobs.grad_fn.saved_tensors:
-        assert t.numel() < T * V and tuple(t.shape) != (T, V)
+        assert tuple(t.shape) != (T, V) and t.numel() <= max(T * H, V * H)
 
 
 def test_chunking_and_repeat_runs_are_bit_identical(dev):
