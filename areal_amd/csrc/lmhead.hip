@@ -127,9 +127,12 @@ DEVI void mma_ksteps(const u16* pa, const u16* pb, f32x16 (&acc)[4][4], int s_be
 // Accumulator layout inside a wave: acc[a][b][r] holds
 //   i = a*32 + 8*(r/4) + 4*(lane/32) + (r%4)   (A row inside the wave's 128)
 //   j = b*32 + (lane%32)                        (B row inside the wave's 128)
+//
+// gemm_nt_generic: any K that is a multiple of 8 (k tail zero-filled); operands staged through
+// registers into a padded LDS layout. Used for small or odd shapes.
 template <class Epi>
-__global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
-                                                          typename Epi::Params ep) {
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_generic(GemmArgs g, Sched sc,
+                                                            typename Epi::Params ep) {
   __shared__ __attribute__((aligned(16))) u16 lds[2 * 2 * OPER];
   int bj, split;
   if (!sched_decode(sc, blockIdx.x, bj, split)) return;
@@ -194,6 +197,168 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
     }
     Epi::tile(st, ep, acc, ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
   }
+  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// gemm_nt_sweep: the production main loop, for K % 64 == 0.
+//
+//  * Operand tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR staging). A wave
+//    instruction fills 8 rows x 128 B; which 16-byte chunk of its row a lane fetches is XOR
+//    swizzled so that the MFMA fragment reads (ds_read_b128, 32 rows x one chunk) hit every
+//    LDS bank exactly once (measured: 0 bank conflicts).
+//  * Two 64 KB stages form a ring over the flattened (A tile, k tile) sequence of the whole
+//    sweep: the loads of the next A tile are in flight while the epilogue of the current one
+//    runs. A stage is refilled right after the barrier that retires it (A half during the last
+//    k-step of the current k-tile, B half during the first k-step of the next).
+//  * The loop body is written as 8 slots per k-step, each {2 MFMA, 1 fragment read, 1 direct
+//    load}, fenced with sched_barrier so the compiler keeps the interleave.
+// ---------------------------------------------------------------------------------------
+constexpr int RING_OPER = TILE * BK;       // elements of one operand stage (32 KB)
+constexpr int RING_STAGE = 2 * RING_OPER;  // A then B
+DEVI int swz64(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+#define LDS_AS(p) ((void __attribute__((address_space(3)))*)(p))
+#define GLB_AS(p) ((const void __attribute__((address_space(1)))*)(p))
+
+template <class Epi>
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
+                                                          typename Epi::Params ep) {
+  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
+  int bj, split;
+  if (!sched_decode(sc, blockIdx.x, bj, split)) return;
+  const int ai_begin = (int)(((int64_t)split * sc.nai) / sc.S);
+  const int ai_end = (int)(((int64_t)(split + 1) * sc.nai) / sc.S);
+  if (ai_begin >= ai_end) return;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave >> 1, wb = wave & 1;
+  const int nk = g.K / BK;
+
+  // ---- loader: lane -> (row of the wave's 64-row slice, swizzled chunk)
+  const u16* ga[8];
+  const u16* gb[8];
+  int l_ai = ai_begin, l_kt = 0;
+  auto set_a_rows = [&](int ai) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = wave * 64 + i * 8 + (lane >> 3);
+      int row = ai * TILE + r;
+      row = row < g.M ? row : g.M - 1;  // clamped rows are discarded by the epilogue
+      ga[i] = g.A + (int64_t)row * g.lda + (((lane & 7) ^ swz64(r)) * 8);
+    }
+  };
+  set_a_rows(ai_begin);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = wave * 64 + i * 8 + (lane >> 3);
+    int row = bj * TILE + r;
+    row = row < g.N ? row : g.N - 1;
+    gb[i] = g.B + (int64_t)row * g.ldb + (((lane & 7) ^ swz64(r)) * 8);
+  }
+  int l_stage = 0;  // stage the loader fills next
+  auto load_a = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + wave * 64 * BK + i * 8 * BK;
+    __builtin_amdgcn_global_load_lds(GLB_AS(ga[i] + l_kt * BK), LDS_AS(dst), 16, 0, 0);
+  };
+  auto load_b = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + wave * 64 * BK + i * 8 * BK;
+    __builtin_amdgcn_global_load_lds(GLB_AS(gb[i] + l_kt * BK), LDS_AS(dst), 16, 0, 0);
+  };
+  auto loader_advance = [&]() {  // after both halves of a stage were issued
+    l_stage ^= 1;
+    if (l_kt + 1 < nk) {
+      ++l_kt;
+    } else if (l_ai + 1 < ai_end) {
+      ++l_ai;
+      l_kt = 0;
+      set_a_rows(l_ai);
+    }  // else: keep re-loading the last k-tile into the idle stage (never consumed)
+  };
+
+  // ---- fragments
+  const int rl = lane & 31, ch = lane >> 5;
+  const int sw = swz64(rl);
+  bf16x8 af[2][4], bf[2][4];
+  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
+  auto dsr = [&](int st, int s, int buf, int f) {
+    const int slot = ((s * 2 + ch) ^ sw) * 8;
+    const u16* sA = lds + st * RING_STAGE + wa * 128 * BK + rl * BK + slot;
+    const u16* sB = lds + st * RING_STAGE + RING_OPER + wb * 128 * BK + rl * BK + slot;
+    if (f == 0) af[buf][0] = *(const bf16x8*)(sA);
+    else if (f <= 4) bf[buf][f - 1] = *(const bf16x8*)(sB + (f - 1) * 32 * BK);
+    else af[buf][f - 4] = *(const bf16x8*)(sA + (f - 4) * 32 * BK);
+  };
+  f32x16 acc[4][4];
+  auto mfma2 = [&](int buf, int p) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int idx = 2 * p + q, a = idx >> 2, b = idx & 3;
+      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
+    }
+  };
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  };
+
+  typename Epi::State st;
+  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
+
+  // ---- prologue: stage 0 completely, A half of stage 1
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_b(i);
+  loader_advance();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+  zero_acc();
+  __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): everything but the last 8 loads has landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
+
+  // Outer loop over A tiles, inner (hot) loop over k-tiles; the loader state and the stage
+  // parity run on across tile boundaries.
+  int cs = 0;
+  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
+    for (int c_kt = 0; c_kt < nk; ++c_kt) {
+      // k-steps 0..2: fragments of the next k-step are fetched while this one multiplies;
+      // step 0 also issues the B half of the stage the loader is filling.
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+          mfma2(s & 1, p);
+          dsr(cs, s + 1, (s + 1) & 1, p);
+          if (s == 0) load_b(p);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (s == 0) loader_advance();
+      }
+      // every wave: own fragment reads done, own direct loads landed; then all waves agree
+      __builtin_amdgcn_s_waitcnt(0x0070);
+      __builtin_amdgcn_s_barrier();
+      // k-step 3, with the first fragments of the next k-tile and the A half of the stage
+      // that the barrier has just retired
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        mfma2(1, p);
+        dsr(cs ^ 1, 0, 0, p);
+        load_a(p);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      cs ^= 1;
+    }
+    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
+    zero_acc();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
   Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
 }
 
@@ -429,8 +594,8 @@ struct BwdEpi {
     int T; int V;
     float scale; float c2; float inv_temp;
     const float* bias;
-    u16* dl; int64_t ldv;      // ldv >= V rounded to 8; columns [V, ldv) are written as zero
-    u16* dlT; int64_t ldt;     // ldt >= T rounded to 8; columns [T, ldt) are written as zero
+    u16* dl; int64_t ldv;      // ldv = V rounded up to 64; columns [V, ldv) are written as zero
+    u16* dlT; int64_t ldt;     // ldt = T rounded up to 64; columns [T, ldt) are written as zero
   };
   struct State {
     float nb[4], gs[4];
@@ -546,8 +711,12 @@ int launch_gemm(const GemmArgs& g, int S, const typename Epi::Params& ep, hipStr
   if (S > nai) S = nai;
   if (S < 1) S = 1;
   const Sched sc = make_sched(nbj, nai, S);
-  hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g, sc,
-                     ep);
+  if (g.K % BK == 0 && g.K > 0)
+    hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
+                       sc, ep);
+  else
+    hipLaunchKernelGGL((gemm_nt_generic<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
+                       sc, ep);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -633,7 +802,7 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk) {
   if (T <= 0 || H <= 0 || V <= 0 || token_chunk <= 0) return 0;
   const int64_t Tc = token_chunk < T ? token_chunk : T;
-  const int64_t ldv = round_up_i64(V, 8), ldt = round_up_i64(Tc, 8);
+  const int64_t ldv = round_up_i64(V, BK), ldt = round_up_i64(Tc, BK);
   int64_t elems = H * ldv + H * ldt + Tc * ldv + V * ldt;
   return (size_t)elems * 2 + 4 * 256;  // slack for 256-byte sub-buffer alignment
 }
@@ -662,7 +831,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     return AREAL_ERR_WORKSPACE;
 
   const int64_t Tc_max = token_chunk < T ? token_chunk : T;
-  const int64_t ldv = round_up_i64(V, 8), ldt = round_up_i64(Tc_max, 8);
+  const int64_t ldv = round_up_i64(V, BK), ldt = round_up_i64(Tc_max, BK);
   auto carve = [](char*& p, int64_t bytes) {
     char* r = (char*)(((uintptr_t)p + 255) & ~(uintptr_t)255);
     p = r + bytes;
@@ -684,7 +853,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   }
   for (int64_t t0 = 0; t0 < T; t0 += Tc_max) {
     const int64_t Tc = (T - t0) < Tc_max ? (T - t0) : Tc_max;
-    const int64_t ldt_c = round_up_i64(Tc, 8);
+    const int64_t ldt_c = round_up_i64(Tc, BK);
     const u16* hid_c = (const u16*)hidden + t0 * H;
     // 1. recompute logits of the chunk, emit dlogits in both layouts
     {
