@@ -37,28 +37,32 @@ struct GemmArgs {
 // q. They are laid out as an RB x RS block of (B tiles) x (splits) so that they share operand
 // tiles through that XCD's L2.
 struct Sched {
-  int nbj;     // number of B tiles
-  int nai;     // number of A tiles
-  int S;       // splits of the A-tile range
-  int RB, RS;  // RB * RS == 32
-  int n_sb_j;  // super-blocks along j
-  int n_sb;    // total super-blocks
+  int bj0, nbj;  // B tiles [bj0, bj0 + nbj)
+  int ai0, nai;  // A tiles [ai0, ai0 + nai)
+  int S;         // splits of the A-tile range
+  int RB, RS;    // RB * RS == 32
+  int n_sb_j;    // super-blocks along j
+  int n_sb;      // total super-blocks
 };
 
-DEVI bool sched_decode(const Sched& sc, int id, int& bj, int& split) {
+DEVI bool sched_decode(const Sched& sc, int id, int& bj, int& split, int& ai_begin, int& ai_end) {
   const int xcd = id & 7, q = id >> 3;
   const int sb = (q >> 5) * 8 + xcd;
   const int r = q & 31;
   if (sb >= sc.n_sb) return false;
   const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
-  bj = sbj * sc.RB + (r % sc.RB);
+  const int bl = sbj * sc.RB + (r % sc.RB);
   split = sbs * sc.RS + (r / sc.RB);
-  return bj < sc.nbj && split < sc.S;
+  if (bl >= sc.nbj || split >= sc.S) return false;
+  bj = sc.bj0 + bl;
+  ai_begin = sc.ai0 + (int)(((int64_t)split * sc.nai) / sc.S);
+  ai_end = sc.ai0 + (int)(((int64_t)(split + 1) * sc.nai) / sc.S);
+  return ai_begin < ai_end;
 }
 
-static Sched make_sched(int nbj, int nai, int S) {
+static Sched make_sched(int bj0, int nbj, int ai0, int nai, int S) {
   Sched sc;
-  sc.nbj = nbj; sc.nai = nai; sc.S = S;
+  sc.bj0 = bj0; sc.nbj = nbj; sc.ai0 = ai0; sc.nai = nai; sc.S = S;
   sc.RS = S >= 8 ? 8 : (S >= 4 ? 4 : (S >= 2 ? 2 : 1));
   sc.RB = 32 / sc.RS;
   sc.n_sb_j = (nbj + sc.RB - 1) / sc.RB;
@@ -134,11 +138,8 @@ template <class Epi>
 __global__ __launch_bounds__(NTHREADS) void gemm_nt_generic(GemmArgs g, Sched sc,
                                                             typename Epi::Params ep) {
   __shared__ __attribute__((aligned(16))) u16 lds[2 * 2 * OPER];
-  int bj, split;
-  if (!sched_decode(sc, blockIdx.x, bj, split)) return;
-  const int ai_begin = (int)(((int64_t)split * sc.nai) / sc.S);
-  const int ai_end = (int)(((int64_t)(split + 1) * sc.nai) / sc.S);
-  if (ai_begin >= ai_end) return;
+  int bj, split, ai_begin, ai_end;
+  if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wa = wave >> 1, wb = wave & 1;
@@ -224,11 +225,8 @@ template <class Epi>
 __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
                                                           typename Epi::Params ep) {
   __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
-  int bj, split;
-  if (!sched_decode(sc, blockIdx.x, bj, split)) return;
-  const int ai_begin = (int)(((int64_t)split * sc.nai) / sc.S);
-  const int ai_end = (int)(((int64_t)(split + 1) * sc.nai) / sc.S);
-  if (ai_begin >= ai_end) return;
+  int bj, split, ai_begin, ai_end;
+  if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -363,15 +361,23 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
 }
 
 // ---------------------------------------------------------------------------------------
+// Epilogues. Each is a template on EDGE: the interior of the tile grid (every tile fully inside
+// M x N) runs the EDGE = false instance, which carries no bounds predicates; ragged last tiles
+// are launched separately with EDGE = true. Keeping one variant per kernel keeps the
+// accumulators in registers (several variants behind run-time branches made the compiler spill
+// them, which showed up as tens of GB of scratch traffic per launch).
+//
 // Epilogue 0: plain store (bf16 store, fp32 store, fp32 accumulate). Used for dHidden and
 // dWeight and for the stand-alone GEMM entry point. Output is indexed out[j * ldo + i]
 // (B row major, A row contiguous), so a lane's 4 consecutive i values are contiguous.
 // ---------------------------------------------------------------------------------------
+struct StoreParams {
+  void* out; int64_t ldo; int M; int N;  // M % 4 == 0
+};
+
+template <bool EDGE, int MODE>  // MODE 0: bf16 store, 1: fp32 store, 2: fp32 accumulate
 struct StoreEpi {
-  struct Params {
-    void* out; int64_t ldo; int M; int N;
-    int mode;  // 0: bf16 store, 1: fp32 store, 2: fp32 accumulate
-  };
+  typedef StoreParams Params;
   struct State {};
   static DEVI void begin(State&, const Params&, int, int, int, int) {}
   static DEVI void end(State&, const Params&, int, int, int, int) {}
@@ -379,18 +385,16 @@ struct StoreEpi {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int j = j0 + b * 32 + (lane & 31);
-      if (j >= p.N) continue;
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int i = i0 + a * 32 + 8 * rq + 4 * (lane >> 5);
-          if (i >= p.M) continue;
-          float x0 = acc[a][b][rq * 4 + 0], x1 = acc[a][b][rq * 4 + 1];
-          float x2 = acc[a][b][rq * 4 + 2], x3 = acc[a][b][rq * 4 + 3];
-          const int64_t off = (int64_t)j * p.ldo + i;
-          if (i + 3 < p.M) {
-            if (p.mode == 0) {
+          if (!EDGE || (j < p.N && i < p.M)) {
+            const float x0 = acc[a][b][rq * 4 + 0], x1 = acc[a][b][rq * 4 + 1];
+            const float x2 = acc[a][b][rq * 4 + 2], x3 = acc[a][b][rq * 4 + 3];
+            const int64_t off = (int64_t)j * p.ldo + i;
+            if (MODE == 0) {
               u32x2 v;
               v[0] = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
               v[1] = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
@@ -398,39 +402,42 @@ struct StoreEpi {
             } else {
               f32x4* dst = (f32x4*)((float*)p.out + off);
               f32x4 v = {x0, x1, x2, x3};
-              if (p.mode == 2) v += *dst;
+              if (MODE == 2) v += *dst;
               *dst = v;
-            }
-          } else {
-            const float xs[4] = {x0, x1, x2, x3};
-            for (int e = 0; e < 4 && i + e < p.M; ++e) {
-              if (p.mode == 0) ((u16*)p.out)[off + e] = f32_to_bf16_bits(xs[e]);
-              else if (p.mode == 1) ((float*)p.out)[off + e] = xs[e];
-              else ((float*)p.out)[off + e] += xs[e];
             }
           }
         }
+        __builtin_amdgcn_sched_barrier(0);  // keep the accumulator reads of one block together
       }
     }
   }
 };
+template <bool E> using StoreBf16 = StoreEpi<E, 0>;
+template <bool E> using StoreF32 = StoreEpi<E, 1>;
+template <bool E> using AccumF32 = StoreEpi<E, 2>;
 
 // ---------------------------------------------------------------------------------------
 // Epilogue 1: online softmax statistics over the vocabulary (forward).
 // Per token the lane keeps: running max m of the logits x, s = sum exp((x-m)/T),
-// q = sum ((x-m)/T * log2e) * exp((x-m)/T), the label's logit, min, sum x, sum x^2.
+// q = sum ((x-m)/T * log2e) * exp((x-m)/T), the label's logit, min and (MOMENTS) sum x,
+// sum x^2. One token (its 64 logits in this lane) at a time: the logits are read from the
+// accumulators twice (statistics pass, exponential pass) and never written back.
 // ---------------------------------------------------------------------------------------
 constexpr int NSTAT = 7;  // m, s, q, xlabel, min, sumx, sumx2
 
+struct FwdParams {
+  const int64_t* labels; int T; int V;
+  float scale;        // logit_scale
+  float c2;           // inv_temperature * log2(e)
+  const float* bias;  // nullable, [V]
+  float* ws;          // [NSTAT][P][T]
+  int P;              // total partial slots
+  int slot_base;      // first slot written by this launch
+};
+
+template <bool EDGE, bool AFFINE, bool MOMENTS>
 struct FwdEpi {
-  struct Params {
-    const int64_t* labels; int T; int V;
-    float scale;   // logit_scale
-    float c2;      // inv_temperature * log2(e)
-    const float* bias;  // nullable, [V]
-    float* ws;     // [NSTAT][P][T]
-    int P;         // partial slots = 4 * S
-  };
+  typedef FwdParams Params;
   struct State {
     float m[4], s[4], q[4], xl[4], mn[4], sx[4], sx2[4];
     int lab[4];
@@ -441,27 +448,23 @@ struct FwdEpi {
       st.m[b] = neg_inf(); st.s[b] = 0.f; st.q[b] = 0.f; st.xl[b] = 0.f;
       st.mn[b] = pos_inf(); st.sx[b] = 0.f; st.sx2[b] = 0.f;
       const int t = t0 + b * 32 + (lane & 31);
-      int64_t l = t < p.T ? p.labels[t] : -1;
+      int64_t l = (!EDGE || t < p.T) ? p.labels[t] : -1;
       st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
     }
   }
 
-  template <bool EDGE>
-  static DEVI void tile_impl(State& st, const Params& p, f32x16 (&acc)[4][4], int v0, int lane) {
+  static DEVI void tile(State& st, const Params& p, const f32x16 (&acc)[4][4], int v0, int, int lane) {
     const int vl = v0 + 4 * (lane >> 5);
-    const bool affine = (p.scale != 1.0f) || (p.bias != nullptr);
-    if (affine) {
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
-          float bv = 0.f;
-          if (p.bias != nullptr && (!EDGE || v < p.V)) bv = p.bias[v];
-#pragma unroll
-          for (int b = 0; b < 4; ++b) acc[a][b][r] = (acc[a][b][r] + bv) * p.scale;
-        }
-    }
+    auto vidx = [&](int a, int r) { return vl + a * 32 + 8 * (r >> 2) + (r & 3); };
+    auto logit = [&](int a, int b, int r) -> float {
+      float x = acc[a][b][r];
+      if (AFFINE) {
+        float bv = 0.f;
+        if (p.bias != nullptr && (!EDGE || vidx(a, r) < p.V)) bv = p.bias[vidx(a, r)];
+        x = (x + bv) * p.scale;
+      }
+      return x;
+    };
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
@@ -469,78 +472,65 @@ struct FwdEpi {
       for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float x = acc[a][b][r];
-          if (EDGE) {
-            const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
-            if (v < p.V) {
-              tmax = fmaxf(tmax, x); tmin = fminf(tmin, x); sx += x; sx2 = fmaf(x, x, sx2);
-            }
-          } else {
-            tmax = fmaxf(tmax, x); tmin = fminf(tmin, x); sx += x; sx2 = fmaf(x, x, sx2);
+          const float x = logit(a, b, r);
+          if (!EDGE || vidx(a, r) < p.V) {
+            tmax = fmaxf(tmax, x);
+            tmin = fminf(tmin, x);
+            if (MOMENTS) { sx += x; sx2 = fmaf(x, x, sx2); }
           }
         }
       st.mn[b] = fminf(st.mn[b], tmin);
-      st.sx[b] += sx;
-      st.sx2[b] += sx2;
+      if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
       const float m_old = st.m[b];
       const float m_new = fmaxf(m_old, tmax);
-      if (m_new > neg_inf()) {
-        float s = 0.f, q = 0.f;
-        if (m_old > neg_inf()) {
-          const float dl = (m_old - m_new) * p.c2;
-          const float alpha = fast_exp2(dl);
-          q = alpha * fmaf(dl, st.s[b], st.q[b]);
-          s = alpha * st.s[b];
+      // rescale the running sums to the new maximum; on the first tile m_old = -inf and
+      // s = q = 0, so the factor is taken as 2^0 instead of evaluating -inf - x
+      float s = st.s[b], q = st.q[b];
+      const float dl = (m_old > neg_inf()) ? (m_old - m_new) * p.c2 : 0.f;
+      const float alpha = fast_exp2(dl);
+      q = alpha * fmaf(dl, s, q);
+      s = alpha * s;
+      const float mc = (!EDGE || m_new > neg_inf()) ? m_new * p.c2 : 0.f;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float t = fmaf(logit(a, b, r), p.c2, -mc);
+          const float e = fast_exp2(t);
+          if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
         }
-        const float mc = m_new * p.c2;
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float x = acc[a][b][r];
-            const float t = fmaf(x, p.c2, -mc);
-            const float e = fast_exp2(t);
-            if (EDGE) {
-              const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
-              if (v < p.V) { s += e; q = fmaf(t, e, q); }
-            } else {
-              s += e; q = fmaf(t, e, q);
-            }
-          }
-        st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
-      }
+      st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
       const int lab = st.lab[b];
       const bool hit = (lab >= v0) && (lab < v0 + 128);
       if (__builtin_amdgcn_ballot_w64(hit) != 0) {
 #pragma unroll
         for (int a = 0; a < 4; ++a)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int v = vl + a * 32 + 8 * (r >> 2) + (r & 3);
-            if (v == lab) st.xl[b] = acc[a][b][r];
-          }
+          for (int r = 0; r < 16; ++r)
+            if (vidx(a, r) == lab) st.xl[b] = logit(a, b, r);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-  }
-
-  static DEVI void tile(State& st, const Params& p, f32x16 (&acc)[4][4], int i0, int, int lane) {
-    if (i0 + 128 <= p.V) tile_impl<false>(st, p, acc, i0, lane);
-    else tile_impl<true>(st, p, acc, i0, lane);
   }
 
   static DEVI void end(State& st, const Params& p, int t0, int split, int wa, int lane) {
-    const int slot = split * 4 + wa * 2 + (lane >> 5);
+    const int slot = p.slot_base + split * 4 + wa * 2 + (lane >> 5);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int t = t0 + b * 32 + (lane & 31);
-      if (t >= p.T) continue;
+      if (EDGE && t >= p.T) continue;
       const int64_t PT = (int64_t)p.P * p.T;
       float* w = p.ws + (int64_t)slot * p.T + t;
       w[0 * PT] = st.m[b]; w[1 * PT] = st.s[b]; w[2 * PT] = st.q[b]; w[3 * PT] = st.xl[b];
-      w[4 * PT] = st.mn[b]; w[5 * PT] = st.sx[b]; w[6 * PT] = st.sx2[b];
+      w[4 * PT] = st.mn[b];
+      if (MOMENTS) { w[5 * PT] = st.sx[b]; w[6 * PT] = st.sx2[b]; }
     }
   }
 };
+template <bool E> using FwdPlain = FwdEpi<E, false, false>;
+template <bool E> using FwdPlainMom = FwdEpi<E, false, true>;
+template <bool E> using FwdAffine = FwdEpi<E, true, false>;
+template <bool E> using FwdAffineMom = FwdEpi<E, true, true>;
 
 // Merge the partial statistics of one token over all slots.
 __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, int V,
@@ -552,6 +542,7 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const int64_t PT = (int64_t)P * T;
+  const bool moments = vmean != nullptr || vnorm != nullptr;
   float M = neg_inf();
   for (int p = 0; p < P; ++p) M = fmaxf(M, ws[(int64_t)p * T + t]);
   float S = 0.f, Q = 0.f, xl = 0.f, mn = pos_inf();
@@ -567,8 +558,7 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
     }
     xl += w[3 * PT];
     mn = fminf(mn, w[4 * PT]);
-    sx += (double)w[5 * PT];
-    sx2 += (double)w[6 * PT];
+    if (moments) { sx += (double)w[5 * PT]; sx2 += (double)w[6 * PT]; }
   }
   const float logS = logf(S);
   if (logprobs) logprobs[t] = (xl - M) * inv_temp - logS;
@@ -585,18 +575,21 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
 // Epilogue 2: recompute logits and emit dlogits = (onehot - p) * g * invT * scale in bf16,
 // in two layouts: dl [Tc, ldv] (vocabulary contiguous) and dlT [V, ldt] (token contiguous).
 // ---------------------------------------------------------------------------------------
+struct BwdParams {
+  const int64_t* labels;     // [Tc]
+  const float* row_max;      // [Tc]
+  const float* sum_exp;      // [Tc]
+  const float* grad;         // [Tc] dLoss/dlogprob
+  int T; int V;
+  float scale; float c2; float inv_temp;
+  const float* bias;
+  u16* dl; int64_t ldv;      // ldv = V rounded up to 64; columns [V, ldv) are written as zero
+  u16* dlT; int64_t ldt;     // ldt = T rounded up to 64; columns [T, ldt) are written as zero
+};
+
+template <bool EDGE, bool AFFINE>
 struct BwdEpi {
-  struct Params {
-    const int64_t* labels;     // [Tc]
-    const float* row_max;      // [Tc]
-    const float* sum_exp;      // [Tc]
-    const float* grad;         // [Tc] dLoss/dlogprob
-    int T; int V;
-    float scale; float c2; float inv_temp;
-    const float* bias;
-    u16* dl; int64_t ldv;      // ldv = V rounded up to 64; columns [V, ldv) are written as zero
-    u16* dlT; int64_t ldt;     // ldt = T rounded up to 64; columns [T, ldt) are written as zero
-  };
+  typedef BwdParams Params;
   struct State {
     float nb[4], gs[4];
     int lab[4];
@@ -605,7 +598,7 @@ struct BwdEpi {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int t = t0 + b * 32 + (lane & 31);
-      if (t < p.T) {
+      if (!EDGE || t < p.T) {
         const int64_t l = p.labels[t];
         st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
         st.nb[b] = -(p.row_max[t] * p.c2 + fast_log2(p.sum_exp[t]));
@@ -617,16 +610,17 @@ struct BwdEpi {
   }
   static DEVI void end(State&, const Params&, int, int, int, int) {}
 
-  static DEVI void tile(State& st, const Params& p, f32x16 (&acc)[4][4], int v0, int t0, int lane) {
+  static DEVI void tile(State& st, const Params& p, const f32x16 (&acc)[4][4], int v0, int t0, int lane) {
     const int vl = v0 + 4 * (lane >> 5);
-    const bool affine = (p.scale != 1.0f) || (p.bias != nullptr);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int t = t0 + b * 32 + (lane & 31);
       const float nb = st.nb[b], gs = st.gs[b];
       const int lab = st.lab[b];
+      u16* row = p.dl + (int64_t)t * p.ldv;
+      u16* col = p.dlT + t;
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+      for (int a = 0; a < 4; ++a) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int vq = vl + a * 32 + 8 * rq;
@@ -635,32 +629,36 @@ struct BwdEpi {
           for (int e = 0; e < 4; ++e) {
             const int v = vq + e;
             float x = acc[a][b][rq * 4 + e];
-            if (affine) {
+            if (AFFINE) {
               float bv = 0.f;
-              if (p.bias != nullptr && v < p.V) bv = p.bias[v];
+              if (p.bias != nullptr && (!EDGE || v < p.V)) bv = p.bias[v];
               x = (x + bv) * p.scale;
             }
             const float pr = fast_exp2(fmaf(x, p.c2, nb));
             float dv = -pr * gs;
             if (v == lab) dv += gs;
-            if (v >= p.V || t >= p.T) dv = 0.f;
+            if (EDGE && (v >= p.V || t >= p.T)) dv = 0.f;
             d[e] = f32_to_bf16_bits(dv);
           }
-          if (t < p.T && vq < p.ldv) {
+          if (!EDGE || (t < p.T && vq < p.ldv)) {
             u32x2 pk;
             pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
             pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
-            *(u32x2*)(p.dl + (int64_t)t * p.ldv + vq) = pk;
+            *(u32x2*)(row + vq) = pk;
           }
-          if (t < p.ldt) {
+          if (!EDGE || t < p.ldt) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              if (vq + e < p.V) p.dlT[(int64_t)(vq + e) * p.ldt + t] = d[e];
+              if (!EDGE || vq + e < p.V) col[(int64_t)(vq + e) * p.ldt] = d[e];
           }
         }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 };
+template <bool E> using BwdPlain = BwdEpi<E, false>;
+template <bool E> using BwdAffine = BwdEpi<E, true>;
 
 // dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ldd. 64x64 tiles.
 __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __restrict__ src,
@@ -704,14 +702,14 @@ int pick_splits(int nbj, int nai, int target_wgs) {
   return S;
 }
 
-template <class Epi>
-int launch_gemm(const GemmArgs& g, int S, const typename Epi::Params& ep, hipStream_t stream) {
-  const int nbj = (g.N + TILE - 1) / TILE, nai = (g.M + TILE - 1) / TILE;
+template <class Epi, bool FAST>
+int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
+                  const typename Epi::Params& ep, hipStream_t stream) {
   if (nbj <= 0 || nai <= 0) return AREAL_OK;
   if (S > nai) S = nai;
   if (S < 1) S = 1;
-  const Sched sc = make_sched(nbj, nai, S);
-  if (g.K % BK == 0 && g.K > 0)
+  const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
+  if (FAST)
     hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
   else
@@ -721,11 +719,59 @@ int launch_gemm(const GemmArgs& g, int S, const typename Epi::Params& ep, hipStr
   return AREAL_OK;
 }
 
+// How a GEMM is cut into launches. K % 64 == 0 takes the fast kernel: interior tiles with the
+// predicate-free epilogue, then the ragged last B tile and the ragged last A tile with the
+// EDGE epilogue. Any other K takes the generic kernel over all tiles in one launch.
+struct Regions {
+  bool fast;
+  int nai_full, nbj_full;  // tiles entirely inside M and N
+  bool ragged_a, ragged_b;
+  int S;                   // splits used for the interior and the ragged-B launch
+};
+Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixed) {
+  Regions r;
+  r.fast = (K > 0 && K % BK == 0);
+  if (r.fast) {
+    r.nai_full = (int)(M / TILE); r.nbj_full = (int)(N / TILE);
+    r.ragged_a = (M % TILE) != 0; r.ragged_b = (N % TILE) != 0;
+  } else {
+    r.nai_full = (int)ceil_div_i64(M, TILE); r.nbj_full = (int)ceil_div_i64(N, TILE);
+    r.ragged_a = false; r.ragged_b = false;
+  }
+  const int nbj_all = r.nbj_full + (r.ragged_b ? 1 : 0);
+  r.S = r.nai_full > 0 ? (S_fixed > 0 ? S_fixed : pick_splits(nbj_all, r.nai_full, target_wgs)) : 0;
+  if (r.S > r.nai_full) r.S = r.nai_full;
+  return r;
+}
+
+// EpiT<EDGE>; ep_edge_a is the parameter block of the ragged-A launch (it may differ from ep in
+// where it writes its partial results).
+template <template <bool> class EpiT, class P>
+int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_edge_a,
+                hipStream_t stream) {
+  int rc;
+  if (!r.fast)
+    return launch_region<EpiT<true>, false>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
+  if ((rc = launch_region<EpiT<false>, true>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+    return rc;
+  if (r.ragged_b &&
+      (rc = launch_region<EpiT<true>, true>(g, r.nbj_full, 1, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+    return rc;
+  if (r.ragged_a &&
+      (rc = launch_region<EpiT<true>, true>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
+                                            ep_edge_a, stream)) != AREAL_OK)
+    return rc;
+  return AREAL_OK;
+}
+
 int check_operand(const void* p, int64_t ld) {
   if (p == nullptr) return AREAL_ERR_BAD_ARG;
   if (!aligned16(p) || (ld % 8) != 0) return AREAL_ERR_ALIGNMENT;
   return AREAL_OK;
 }
+
+// Slots of partial softmax statistics per token written by the forward launches.
+int fwd_slots(const Regions& r) { return 4 * r.S + (r.ragged_a ? 4 : 0); }
 
 }  // namespace
 
@@ -734,40 +780,39 @@ int check_operand(const void* p, int64_t ld) {
 // =======================================================================================
 extern "C" {
 
-// out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]; A, B bf16; K % 8 == 0.
+// out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]; A, B bf16; K % 8 == 0, M % 4 == 0.
 int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, void* out,
                        int64_t ldo, int64_t M, int64_t N, int64_t K, int out_mode,
                        hipStream_t stream) {
   if (M < 0 || N < 0 || K < 0 || out == nullptr || out_mode < 0 || out_mode > 2)
     return AREAL_ERR_BAD_ARG;
   if (M == 0 || N == 0) return AREAL_OK;
-  if (K % 8 != 0) return AREAL_ERR_ALIGNMENT;
+  if (K % 8 != 0 || M % 4 != 0) return AREAL_ERR_ALIGNMENT;
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
   int rc;
   if ((rc = check_operand(A, lda)) != AREAL_OK) return rc;
   if ((rc = check_operand(B, ldb)) != AREAL_OK) return rc;
   if (out_mode == 0 ? (ldo % 4 != 0 || ((uintptr_t)out & 7)) : (ldo % 4 != 0 || !aligned16(out)))
     return AREAL_ERR_ALIGNMENT;
   GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K};
-  StoreEpi::Params ep{out, ldo, (int)M, (int)N, out_mode};
-  const int nai = (int)ceil_div_i64(M, TILE);
-  return launch_gemm<StoreEpi>(g, nai, ep, stream);
+  const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
+  const StoreParams ep{out, ldo, (int)M, (int)N};
+  if (out_mode == 0) return launch_gemm<StoreBf16>(g, r, ep, ep, stream);
+  if (out_mode == 1) return launch_gemm<StoreF32>(g, r, ep, ep, stream);
+  return launch_gemm<AccumF32>(g, r, ep, ep, stream);
 }
 
-static int fwd_splits(int64_t T, int64_t V) {
-  const int nbj = (int)ceil_div_i64(T, TILE), nai = (int)ceil_div_i64(V, TILE);
-  return pick_splits(nbj, nai, 512);
-}
+static Regions fwd_regions(int64_t T, int64_t H, int64_t V) { return plan_regions(V, T, H, 512, 0); }
 
 size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
-  (void)H;
-  if (T <= 0 || V <= 0) return 0;
-  const int S = fwd_splits(T, V);
-  return (size_t)NSTAT * 4 * S * (size_t)T * sizeof(float);
+  if (T <= 0 || V <= 0 || H <= 0) return 0;
+  return (size_t)NSTAT * fwd_slots(fwd_regions(T, H, V)) * (size_t)T * sizeof(float);
 }
 
-// Forward. hidden [T,H] bf16, weight [V,H] bf16, labels [T] int64 (out-of-range labels give
-// a label logit of 0, like the reference's masked local target). Outputs are fp32 [T]; any
-// output pointer other than row_max / sum_exp may be null.
+// Forward. hidden [T,H] bf16, weight [V,H] bf16, labels [T] int64 (labels outside [0, V) give
+// a label logit of 0). Outputs are fp32 [T]; any output pointer other than row_max / sum_exp
+// may be null; vocab_mean and vocab_norm cost two extra operations per logit and are computed
+// only when one of them is requested.
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
@@ -783,14 +828,23 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   if ((rc = check_operand(weight, H)) != AREAL_OK) return rc;
   const size_t need = areal_lmhead_fwd_workspace_bytes(T, H, V);
   if (workspace == nullptr || workspace_bytes < need) return AREAL_ERR_WORKSPACE;
-  const int S = fwd_splits(T, V);
+  const Regions r = fwd_regions(T, H, V);
+  const int P = fwd_slots(r);
   GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H};
-  FwdEpi::Params ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
-                    (float*)workspace, 4 * S};
-  if ((rc = launch_gemm<FwdEpi>(g, S, ep, stream)) != AREAL_OK) return rc;
+  FwdParams ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
+               (float*)workspace, P, 0};
+  FwdParams ep_a = ep;
+  ep_a.slot_base = 4 * r.S;
+  const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
+  const bool moments = (vocab_mean != nullptr) || (vocab_norm != nullptr);
+  if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
+  else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
+  else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
+  else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
+  if (rc != AREAL_OK) return rc;
   const int threads = 256;
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, threads)), dim3(threads),
-                     0, stream, (const float*)workspace, 4 * S, (int)T, (int)V, inv_temperature,
+                     0, stream, (const float*)workspace, P, (int)T, (int)V, inv_temperature,
                      inv_temperature * LOG2E, logprobs, entropy, vocab_min, vocab_max, vocab_mean,
                      vocab_norm, row_max, sum_exp);
   AREAL_CHECK_LAUNCH();
@@ -844,6 +898,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   u16* dlT = carve(wp, V * ldt * 2);
 
   const float c2 = inv_temperature * LOG2E;
+  const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
   if (dhidden != nullptr) {
     // W^T [H, ldv]: rows = h, columns = v (zero padded to ldv).
     hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -858,18 +913,19 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     // 1. recompute logits of the chunk, emit dlogits in both layouts
     {
       GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H};
-      BwdEpi::Params ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
-                        (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
-      const int nbj = (int)ceil_div_i64(Tc, TILE), nai = (int)ceil_div_i64(V, TILE);
-      if ((rc = launch_gemm<BwdEpi>(g, pick_splits(nbj, nai, 512), ep, stream)) != AREAL_OK)
-        return rc;
+      BwdParams ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
+                   (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
+      const Regions r = plan_regions(V, Tc, H, 512, 0);
+      rc = affine ? launch_gemm<BwdAffine>(g, r, ep, ep, stream)
+                  : launch_gemm<BwdPlain>(g, r, ep, ep, stream);
+      if (rc != AREAL_OK) return rc;
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
       GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv};
-      StoreEpi::Params ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc, 0};
-      if ((rc = launch_gemm<StoreEpi>(g, (int)ceil_div_i64(H, TILE), ep, stream)) != AREAL_OK)
-        return rc;
+      const StoreParams ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc};
+      const Regions r = plan_regions(H, Tc, ldv, 0, 1 << 20);
+      if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
     }
     // 3. dWeight[v, h] += sum_t dlT[v, t] * hidden^T[h, t]
     if (dweight_f32 != nullptr) {
@@ -878,9 +934,11 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                          dim3(256), 0, stream, hid_c, H, (int)Tc, (int)H, hT, ldt_c);
       AREAL_CHECK_LAUNCH();
       GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c};
-      StoreEpi::Params ep{dweight_f32, H, (int)H, (int)V, (accumulate || t0 > 0) ? 2 : 1};
-      if ((rc = launch_gemm<StoreEpi>(g, (int)ceil_div_i64(H, TILE), ep, stream)) != AREAL_OK)
-        return rc;
+      const StoreParams ep{dweight_f32, H, (int)H, (int)V};
+      const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
+      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32>(g, r, ep, ep, stream)
+                                  : launch_gemm<StoreF32>(g, r, ep, ep, stream);
+      if (rc != AREAL_OK) return rc;
     }
   }
   return AREAL_OK;

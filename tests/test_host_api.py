@@ -42,7 +42,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_workspace_size_queries_run_without_gpu():
     lib = _lib.load()
-    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096, 151936) == 7 * 16 * 32768 * 4
+    # 4 vocabulary splits x 4 slots for the 593 full tiles + 4 slots for the ragged last tile
+    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096, 151936) == 7 * 20 * 32768 * 4
     assert lib.areal_lmhead_bwd_workspace_bytes(1024, 64, 1000, 256) > 2 * (256 * 1000 + 1000 * 256)
     assert lib.areal_gae_workspace_bytes(0) == 0
     assert lib.areal_actor_loss_workspace_bytes(10, 3) > 0
