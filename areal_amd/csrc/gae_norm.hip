@@ -18,7 +18,7 @@
 namespace {
 
 constexpr int GAE_THREADS = 256;
-constexpr int GAE_ITEMS = 4;
+constexpr int GAE_ITEMS = 8;
 constexpr int GAE_TILE = GAE_THREADS * GAE_ITEMS;
 
 struct Map {
@@ -79,6 +79,25 @@ DEVI void load_maps(const GaeArgs& g, int64_t t0, Map (&mp)[GAE_ITEMS], float (&
     for (int i = 0; i < GAE_ITEMS; ++i) { mp[i] = map_identity(); v[i] = 0.f; }
     return;
   }
+  float rw[GAE_ITEMS], ms[GAE_ITEMS];
+  if (t0 + GAE_ITEMS <= g.n) {  // t0 is a multiple of GAE_ITEMS: 16-byte aligned vector loads
+#pragma unroll
+    for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+      const f32x4 a = *(const f32x4*)(g.rewards + t0 + 4 * q);
+      const f32x4 b = *(const f32x4*)(g.values + t0 + 4 * q);
+      const f32x4 c = *(const f32x4*)(g.mask + t0 + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { rw[4 * q + e] = a[e]; v[4 * q + e] = b[e]; ms[4 * q + e] = c[e]; }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < GAE_ITEMS; ++i) {
+      const bool in = t0 + i < g.n;
+      rw[i] = in ? g.rewards[t0 + i] : 0.f;
+      v[i] = in ? g.values[t0 + i] : 0.f;
+      ms[i] = in ? g.mask[t0 + i] : 0.f;
+    }
+  }
   int s = gae_seq_of(g, t0);
   int64_t e = gae_seq_end(g, s);
 #pragma unroll
@@ -86,20 +105,19 @@ DEVI void load_maps(const GaeArgs& g, int64_t t0, Map (&mp)[GAE_ITEMS], float (&
     const int64_t t = t0 + i;
     if (t >= g.n) { mp[i] = map_identity(); v[i] = 0.f; continue; }
     while (t >= e && s + 1 < g.n_seqs) { ++s; e = gae_seq_end(g, s); }
-    const float val = g.values[t];
-    v[i] = val;
+    const float val = v[i];
     if (t == e - 1) {
       const bool ne = g.no_eos != nullptr && g.no_eos[s] != 0;
       mp[i] = Map{0.0, 0.0, 0.0, 0.0, ne ? (double)val : 0.0};
     } else {
-      const double m = (double)g.mask[t];
+      const double m = (double)ms[i];
       const double lam = g.lam_seq != nullptr ? (double)g.lam_seq[s] : (double)g.lam;
       const double c = (double)g.discount * lam;
       Map f;
       f.a11 = (1.0 - m) + c * m;
       f.a12 = (double)g.discount * m;
       f.a22 = 1.0 - m;
-      f.b1 = ((double)g.rewards[t] - (double)val) * m;
+      f.b1 = ((double)rw[i] - (double)val) * m;
       f.b2 = (double)val * m;
       mp[i] = f;
     }

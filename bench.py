@@ -99,14 +99,85 @@ def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int):
     return n / dt, dt
 
 
+def hbm_rooflines(dev):
+    """HBM-bound kernels of the path on their own workloads: algorithmic bytes / HIP-event time.
+    GAE + group normalisation on BASELINE config 3 (1024 packed sequences, lognormal lengths),
+    the actor-loss token kernel on 4 Mi tokens (forward + closed-form backward, full stat dict),
+    and the logits-in row kernel on config 1's [4096, 151936] bf16 logits."""
+    import torch
+
+    from areal_amd.config import NormConfig, RejectionSamplingConfig
+    from areal_amd.data import Normalization
+    from areal_amd.functional import gather_logprobs_entropy, ppo_actor_loss_fn
+    from areal_amd.ppo.gae import compute_gae_packed
+
+    peak = 8000.0
+
+    def timed(fn, iters=20, warm=3):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    out = []
+
+    def add(name, workload, nbytes, ms):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out.append({"kernel": name, "workload": workload, "bound": "hbm", "algorithmic_bytes": nbytes,
+                    "ms": ms, "achieved": gbs, "peak": peak, "unit": "GB/s", "frac": gbs / peak})
+
+    g = torch.Generator().manual_seed(2)
+    lens = torch.clamp((torch.randn(1024, generator=g) + 7.0).exp().long(), 16, 8192)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32).to(dev)
+    T = int(cu[-1])
+    r = torch.zeros(T, device=dev)
+    r[cu[1:].long() - 2] = 1.0
+    v = torch.randn(T, device=dev)
+    m = (torch.rand(T, device=dev) > 0.25).float()
+    add("gae_block_total+gae_carry+gae_apply", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
+        20 * T, timed(lambda: compute_gae_packed(r, v, m, cu, None, 1.0, 0.95)))
+    x = torch.randn(1024, 1600, device=dev)
+    mk = (torch.rand(1024, 1600, device=dev) > 0.25).float()
+    norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
+    add("norm_stats1+norm_stats2+norm_apply", "config 3: [1024, 1600] advantages, groups of 16 rows, 20 B/token",
+        20 * x.numel(), timed(lambda: norm(x, mk)))
+    Tl = 4 << 20
+    lp = (torch.randn(Tl, device=dev) * 0.5 - 1).requires_grad_(True)
+    prox = lp.detach() + torch.randn(Tl, device=dev) * 0.1
+    old = prox + torch.randn(Tl, device=dev) * 0.1
+    adv = torch.randn(Tl, device=dev)
+    mask = torch.rand(Tl, device=dev) > 0.2
+    rs = RejectionSamplingConfig(level="token", metric="ratio", upper=2.0, lower=0.5)
+
+    def loss_step():
+        lp.grad = None
+        loss, _ = ppo_actor_loss_fn(lp, prox, old, adv, 0.2, mask, rejection_sampling=rs)
+        loss.backward()
+
+    add("loss_token+loss_finalize+loss_grad_scale", "PPO + IcePop, 4 Mi tokens, fwd+bwd, 47 B/token + 8 B/token grad scale",
+        55 * Tl, timed(loss_step))
+    lg = torch.randn(4096, V_QWEN, device=dev).bfloat16()
+    lab = torch.randint(0, V_QWEN, (4096,), device=dev)
+    add("rows_fwd_kernel", "config 1: [4096, 151936] bf16 logits, logprob + entropy forward",
+        lg.numel() * 2 + 16 * 4096, timed(lambda: gather_logprobs_entropy(lg, lab), iters=10))
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="qwen3-8b", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-sample-tokens", type=int, default=512)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-hbm-kernels", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -216,9 +287,13 @@ def main() -> None:
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},
         },
     }
+    if not args.no_hbm_kernels:
+        del hidden, weight, b, input_data, old, logp0
+        torch.cuda.empty_cache()
+        result["hbm_rooflines"] = hbm_rooflines(dev)
     if not args.no_cpu_baseline:
         threads = min(16, os.cpu_count() or 1)
-        tps, dt = cpu_baseline(args.cpu_sample_tokens, H, b["seed"], threads)
+        tps, dt = cpu_baseline(args.cpu_sample_tokens, H, WORKLOADS[args.workload]["seed"], threads)
         result["cpu_baseline"] = {
             "value": tps, "unit": "tokens/s", "cores": threads, "kind": "port",
             "sample": f"{args.cpu_sample_tokens}-token slice at full vocabulary, fwd+bwd with the "
