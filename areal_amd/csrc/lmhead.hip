@@ -30,6 +30,8 @@ struct GemmArgs {
   const u16* A; int64_t lda; int M;   // A rows (index i)
   const u16* B; int64_t ldb; int N;   // B rows (index j)
   int K;                              // multiple of 8
+  int acols, bcols;                   // k-major (TN) form only: readable columns of A and B
+  int akrows;                         // k-major form only: rows of A that may be read (<= K)
 };
 
 // Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
@@ -361,6 +363,185 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
 }
 
 // ---------------------------------------------------------------------------------------
+// gemm_tn_sweep: D[i][j] = sum_k A[k][i] * B[k][j], both operands stored k-major (row = k,
+// the i / j index contiguous), K % 64 == 0. Used for dWeight[v][h] = sum_t dl[t][v] hidden[t][h]
+// straight from the row-major dlogits and hidden states, so no transposed copies are needed.
+//
+// A stage holds 64 k-rows x 256 columns per operand (512 B per row). Fragments are fetched with
+// ds_read_b64_tr_b16: inside a group of 16 lanes, lanes 4r..4r+3 point at 16 consecutive columns
+// of row k0+r (r = 0..3) and lane q receives column q for those four k. Two such reads give
+// the 8 k values one MFMA operand needs. The 64-byte chunks of a row are XOR swizzled with
+// (k & 3) so that the four rows a group reads fall into different LDS bank groups.
+// ---------------------------------------------------------------------------------------
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from global memory straight into LDS (lane L lands at lds_addr + 16 L).
+// Issued as inline assembly in the k-major kernel: when the compiler sees the load-to-LDS
+// builtin next to ds_read_b64_tr_b16 it cannot prove they do not alias and puts a full
+// vmcnt(0) wait in front of every transposed read, which serialises the prefetch with the
+// math. The kernel orders the two itself with its explicit vmcnt waits and barriers.
+DEVI void lds_dma16(const u16* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :: "s"(lds_addr), "v"(gptr) : "memory", "m0");
+}
+DEVI uint32_t lds_addr_of(const u16* p) { return (uint32_t)(uintptr_t)LDS_AS(p); }
+
+template <class Epi>
+__global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
+                                                          typename Epi::Params ep) {
+  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
+  int bj, split, ai_begin, ai_end;
+  if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave >> 1, wb = wave & 1;
+  const int nk = g.K / BK;
+
+  // ---- loader. Instruction i of a wave fills rows k = wave*16 + 2*i + (lane >> 5) of the
+  // stage; lane -> 16-byte piece (lane & 31) of the LDS row, i.e. chunk position cp = piece/4.
+  // It fetches the chunk ci = cp ^ (k & 3); k & 3 = ((i & 1) * 2 + (lane >> 5)) & 3.
+  const int hl = lane >> 5, piece = lane & 31;
+  const u16* ga = g.A;
+  int a_row[2], a_col[2];  // i even / odd: row inside a 4-row group, first column of the piece
+  const u16* gb[2];
+  int l_ai = ai_begin, l_kt = 0;
+  // global 16-byte piece of instruction parity par for column tile `tile`
+  auto piece_col = [&](int tile, int ncols, int par) -> int {
+    const int k3 = (par * 2 + hl) & 3;
+    int gp = tile * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + (piece & 3);
+    const int last = ncols / 8 - 1;
+    gp = gp < last ? gp : last;  // columns past the end are discarded by the epilogue
+    return gp * 8;
+  };
+  auto set_a_cols = [&](int ai) {
+    a_col[0] = piece_col(ai, g.acols, 0);
+    a_col[1] = piece_col(ai, g.acols, 1);
+  };
+  a_row[0] = wave * 16 + hl;
+  a_row[1] = wave * 16 + 2 + hl;
+  set_a_cols(ai_begin);
+  gb[0] = g.B + (int64_t)(wave * 16 + hl) * g.ldb + piece_col(bj, g.bcols, 0);
+  gb[1] = g.B + (int64_t)(wave * 16 + 2 + hl) * g.ldb + piece_col(bj, g.bcols, 1);
+  int l_stage = 0;
+  auto load_a = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
+    // rows past the last valid one re-read it; the matching rows of B must then be zero
+    const int kb = l_kt * BK + (i >> 1) * 4;
+    const int lim = g.akrows - 1 - kb;
+    const int rl = a_row[i & 1] < lim ? a_row[i & 1] : lim;
+    const u16* src = ga + (int64_t)(kb + rl) * g.lda + a_col[i & 1];
+    lds_dma16(src, __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+  };
+  auto load_b = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + (wave * 16 + i * 2) * TILE;
+    const u16* src = gb[i & 1] + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.ldb;
+    lds_dma16(src, __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+  };
+  auto loader_advance = [&]() {
+    l_stage ^= 1;
+    if (l_kt + 1 < nk) {
+      ++l_kt;
+    } else if (l_ai + 1 < ai_end) {
+      ++l_ai;
+      l_kt = 0;
+      set_a_cols(l_ai);
+    }
+  };
+
+  // ---- fragments: group G = lane/16 -> column half (G & 1) and k half (G >> 1);
+  // q = lane%16 -> row r = q/4 of the four, column quad q%4.
+  const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
+  // byte offset inside a stage operand, without the block (x) and step (s, half) terms
+  const int frag_row = (G >> 1) * 8 + r4;                         // k within the k-step
+  const int frag_byte = (G & 1) * 32 + (q & 3) * 8;              // inside the 64-byte chunk
+  bf16x8 af[2][4], bf[2][4];
+  auto tr_read = [&](const u16* oper, int wsel, int x, int s) -> bf16x8 {
+    const int ci = wsel * 4 + x;
+    const char* base = (const char*)oper + ((ci ^ r4) << 6) + frag_byte;
+    const int k0 = s * 16 + frag_row;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)(base + (k0 << 9)));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)(base + ((k0 + 4) << 9)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
+  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
+  auto dsr = [&](int st, int s, int buf, int f) {
+    const u16* sA = lds + st * RING_STAGE;
+    const u16* sB = sA + RING_OPER;
+    if (f == 0) af[buf][0] = tr_read(sA, wa, 0, s);
+    else if (f <= 4) bf[buf][f - 1] = tr_read(sB, wb, f - 1, s);
+    else af[buf][f - 4] = tr_read(sA, wa, f - 4, s);
+  };
+  f32x16 acc[4][4];
+  auto mfma2 = [&](int buf, int p) {
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq) {
+      const int idx = 2 * p + qq, a = idx >> 2, b = idx & 3;
+      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
+    }
+  };
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  };
+
+  typename Epi::State st;
+  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
+
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_b(i);
+  loader_advance();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+  zero_acc();
+  __builtin_amdgcn_s_waitcnt(0x0F78);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
+
+  int cs = 0;
+  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
+    for (int c_kt = 0; c_kt < nk; ++c_kt) {
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+          mfma2(s & 1, p);
+          dsr(cs, s + 1, (s + 1) & 1, p);
+          if (s == 0) load_b(p);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (s == 0) loader_advance();
+      }
+      __builtin_amdgcn_s_waitcnt(0x0070);
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        mfma2(1, p);
+        dsr(cs ^ 1, 0, 0, p);
+        load_a(p);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      cs ^= 1;
+    }
+    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
+    zero_acc();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Epilogues. Each is a template on EDGE: the interior of the tile grid (every tile fully inside
 // M x N) runs the EDGE = false instance, which carries no bounds predicates; ragged last tiles
 // are launched separately with EDGE = true. Keeping one variant per kernel keeps the
@@ -433,9 +614,13 @@ struct FwdParams {
   float* ws;          // [NSTAT][P][T]
   int P;              // total partial slots
   int slot_base;      // first slot written by this launch
+  // SAVE: e[t][v] = exp2(c2 * x[t][v] - ref[v / 128][t]) in bf16, ref = c2 * (maximum of the
+  // 128 logits of the block); columns [V, ldv) are written as zero.
+  u16* probs; int64_t ldv;
+  float* probs_ref;   // [ceil(V / 128)][T]
 };
 
-template <bool EDGE, bool AFFINE, bool MOMENTS>
+template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
 struct FwdEpi {
   typedef FwdParams Params;
   struct State {
@@ -453,7 +638,7 @@ struct FwdEpi {
     }
   }
 
-  static DEVI void tile(State& st, const Params& p, const f32x16 (&acc)[4][4], int v0, int, int lane) {
+  static DEVI void tile(State& st, const Params& p, const f32x16 (&acc)[4][4], int v0, int t0, int lane) {
     const int vl = v0 + 4 * (lane >> 5);
     auto vidx = [&](int a, int r) { return vl + a * 32 + 8 * (r >> 2) + (r & 3); };
     auto logit = [&](int a, int b, int r) -> float {
@@ -481,6 +666,8 @@ struct FwdEpi {
         }
       st.mn[b] = fminf(st.mn[b], tmin);
       if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
+      // SAVE: both lanes of a token (lane, lane ^ 32) use the maximum of all 128 logits
+      if (SAVE) tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
       const float m_old = st.m[b];
       const float m_new = fmaxf(m_old, tmax);
       // rescale the running sums to the new maximum; on the first tile m_old = -inf and
@@ -491,14 +678,56 @@ struct FwdEpi {
       q = alpha * fmaf(dl, s, q);
       s = alpha * s;
       const float mc = (!EDGE || m_new > neg_inf()) ? m_new * p.c2 : 0.f;
+      if (!SAVE) {
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float t = fmaf(logit(a, b, r), p.c2, -mc);
-          const float e = fast_exp2(t);
-          if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
+          for (int r = 0; r < 16; ++r) {
+            const float t = fmaf(logit(a, b, r), p.c2, -mc);
+            const float e = fast_exp2(t);
+            if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
+          }
+      } else {
+        // exponentials relative to the block maximum (what is stored), folded into the
+        // running sums with the factor 2^(block max - running max) <= 1
+        const bool any = !EDGE || tmax > neg_inf();  // false: every row of the block is >= V
+        const float rc = any ? tmax * p.c2 : 0.f;
+        const int tok = t0 + b * 32 + (lane & 31);
+        u16* row = p.probs + (int64_t)tok * p.ldv;
+        float ts = 0.f, tq = 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
+            const int vq = vl + a * 32 + 8 * rq;
+            u16 d[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const float t = fmaf(logit(a, b, rq * 4 + k), p.c2, -rc);
+              float e = fast_exp2(t);
+              if (EDGE && vq + k >= p.V) e = 0.f;
+              else { ts += e; tq = fmaf(t, e, tq); }
+              d[k] = f32_to_bf16_bits(e);
+            }
+            if (!EDGE || (tok < p.T && vq < p.ldv)) {
+              u32x2 pk;
+              pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
+              pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+              *(u32x2*)(row + vq) = pk;
+            }
+          }
+          // pins the partial sums here: without it the compiler sinks the whole summation
+          // chain below the stores of all four token blocks and spills every term
+          asm volatile("" : "+v"(ts), "+v"(tq));
+          __builtin_amdgcn_sched_barrier(0);
         }
+        const float db = any ? rc - mc : 0.f;  // <= 0
+        const float beta = fast_exp2(db);
+        s = fmaf(beta, ts, s);
+        q = fmaf(beta, fmaf(db, ts, tq), q);
+        if ((lane >> 5) == 0 && (!EDGE || (tok < p.T && v0 < p.V)))
+          p.probs_ref[(int64_t)(v0 >> 7) * p.T + tok] = rc;
+      }
       st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
       const int lab = st.lab[b];
       const bool hit = (lab >= v0) && (lab < v0 + 128);
@@ -527,10 +756,14 @@ struct FwdEpi {
     }
   }
 };
-template <bool E> using FwdPlain = FwdEpi<E, false, false>;
-template <bool E> using FwdPlainMom = FwdEpi<E, false, true>;
-template <bool E> using FwdAffine = FwdEpi<E, true, false>;
-template <bool E> using FwdAffineMom = FwdEpi<E, true, true>;
+template <bool E> using FwdPlain = FwdEpi<E, false, false, false>;
+template <bool E> using FwdPlainMom = FwdEpi<E, false, true, false>;
+template <bool E> using FwdAffine = FwdEpi<E, true, false, false>;
+template <bool E> using FwdAffineMom = FwdEpi<E, true, true, false>;
+template <bool E> using FwdPlainSave = FwdEpi<E, false, false, true>;
+template <bool E> using FwdPlainMomSave = FwdEpi<E, false, true, true>;
+template <bool E> using FwdAffineSave = FwdEpi<E, true, false, true>;
+template <bool E> using FwdAffineMomSave = FwdEpi<E, true, true, true>;
 
 // Merge the partial statistics of one token over all slots.
 __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, int V,
@@ -587,7 +820,7 @@ struct BwdParams {
   u16* dlT; int64_t ldt;     // ldt = T rounded up to 64; columns [T, ldt) are written as zero
 };
 
-template <bool EDGE, bool AFFINE>
+template <bool EDGE, bool AFFINE, bool WT>  // WT: also write the token-contiguous copy dlT
 struct BwdEpi {
   typedef BwdParams Params;
   struct State {
@@ -646,7 +879,7 @@ struct BwdEpi {
             pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
             *(u32x2*)(row + vq) = pk;
           }
-          if (!EDGE || t < p.ldt) {
+          if (WT && (!EDGE || t < p.ldt)) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               if (!EDGE || vq + e < p.V) col[(int64_t)(vq + e) * p.ldt] = d[e];
@@ -657,8 +890,45 @@ struct BwdEpi {
     }
   }
 };
-template <bool E> using BwdPlain = BwdEpi<E, false>;
-template <bool E> using BwdAffine = BwdEpi<E, true>;
+template <bool E> using BwdPlain = BwdEpi<E, false, false>;
+template <bool E> using BwdAffine = BwdEpi<E, true, false>;
+template <bool E> using BwdPlainT = BwdEpi<E, false, true>;
+template <bool E> using BwdAffineT = BwdEpi<E, true, true>;
+
+// dlogits from the exponentials the forward saved, in place:
+//   dl[t][v] = g[t] * invT * scale * (onehot(v == label[t]) - e[t][v] * 2^(ref[v/128][t] - lse2[t]))
+// with lse2 = c2 * row_max + log2(sum_exp). The label's entry is taken from the fp32 label
+// log-probability, -expm1(logprob), so that 1 - p keeps its precision when p is close to 1.
+// Rows [T, Tpad) are written as zero. One thread per 8 columns; grid (ceil(ldv / 2048), Tpad).
+__global__ __launch_bounds__(256) void dlogits_from_saved_kernel(
+    u16* __restrict__ probs, int64_t ldv, const float* __restrict__ ref,
+    const int64_t* __restrict__ labels, const float* __restrict__ row_max,
+    const float* __restrict__ sum_exp, const float* __restrict__ grad,
+    const float* __restrict__ logprobs, int T, int V, float c2, float gscale) {
+  const int t = blockIdx.y;
+  const int64_t v = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (v >= ldv) return;
+  u32x4* ptr = (u32x4*)(probs + (int64_t)t * ldv + v);
+  if (t >= T) { *ptr = u32x4{0u, 0u, 0u, 0u}; return; }
+  const float lse2 = fmaf(row_max[t], c2, fast_log2(sum_exp[t]));
+  const float gs = grad[t] * gscale;
+  int64_t lab = labels[t];
+  if (lab >= V) lab = -1;
+  // blocks past the vocabulary (only padding columns, stored as zero) have no reference
+  const float r = (v < V) ? ref[(v >> 7) * T + t] : lse2;
+  const float f = -gs * fast_exp2(r - lse2);
+  const u32x4 in = *ptr;
+  u32x4 out;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float lo = bf16_bits_to_f32((u16)(in[k] & 0xffffu)) * f;
+    float hi = bf16_bits_to_f32((u16)(in[k] >> 16)) * f;
+    if (v + 2 * k == lab) lo = logprobs ? -gs * expm1f(logprobs[t]) : lo + gs;
+    if (v + 2 * k + 1 == lab) hi = logprobs ? -gs * expm1f(logprobs[t]) : hi + gs;
+    out[k] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  }
+  *ptr = out;
+}
 
 // dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ldd. 64x64 tiles.
 __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __restrict__ src,
@@ -702,15 +972,20 @@ int pick_splits(int nbj, int nai, int target_wgs) {
   return S;
 }
 
-template <class Epi, bool FAST>
+enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2 };
+
+template <class Epi, int KERNEL>
 int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
                   const typename Epi::Params& ep, hipStream_t stream) {
   if (nbj <= 0 || nai <= 0) return AREAL_OK;
   if (S > nai) S = nai;
   if (S < 1) S = 1;
   const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
-  if (FAST)
+  if constexpr (KERNEL == KERNEL_NT)
     hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
+                       sc, ep);
+  else if constexpr (KERNEL == KERNEL_TN)
+    hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
   else
     hipLaunchKernelGGL((gemm_nt_generic<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
@@ -746,20 +1021,20 @@ Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixe
 
 // EpiT<EDGE>; ep_edge_a is the parameter block of the ragged-A launch (it may differ from ep in
 // where it writes its partial results).
-template <template <bool> class EpiT, class P>
+template <template <bool> class EpiT, class P, int FAST_KERNEL = KERNEL_NT>
 int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_edge_a,
                 hipStream_t stream) {
   int rc;
   if (!r.fast)
-    return launch_region<EpiT<true>, false>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
-  if ((rc = launch_region<EpiT<false>, true>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+    return launch_region<EpiT<true>, KERNEL_GENERIC>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
+  if ((rc = launch_region<EpiT<false>, FAST_KERNEL>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_b &&
-      (rc = launch_region<EpiT<true>, true>(g, r.nbj_full, 1, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+      (rc = launch_region<EpiT<true>, FAST_KERNEL>(g, r.nbj_full, 1, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_a &&
-      (rc = launch_region<EpiT<true>, true>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
-                                            ep_edge_a, stream)) != AREAL_OK)
+      (rc = launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
+                                                   ep_edge_a, stream)) != AREAL_OK)
     return rc;
   return AREAL_OK;
 }
@@ -794,7 +1069,7 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   if ((rc = check_operand(B, ldb)) != AREAL_OK) return rc;
   if (out_mode == 0 ? (ldo % 4 != 0 || ((uintptr_t)out & 7)) : (ldo % 4 != 0 || !aligned16(out)))
     return AREAL_ERR_ALIGNMENT;
-  GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K};
+  GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0, 0};
   const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
   const StoreParams ep{out, ldo, (int)M, (int)N};
   if (out_mode == 0) return launch_gemm<StoreBf16>(g, r, ep, ep, stream);
@@ -813,13 +1088,19 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // a label logit of 0). Outputs are fp32 [T]; any output pointer other than row_max / sum_exp
 // may be null; vocab_mean and vocab_norm cost two extra operations per logit and are computed
 // only when one of them is requested.
+//
+// probs / probs_ref (both null or both set) keep the exponentials of the softmax for
+// areal_lmhead_bwd_saved: probs bf16 [round_up(T, 64)][round_up(V, 64)] (rows >= T are not
+// written), probs_ref fp32 [ceil(V / 128)][T].
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
-                     float* row_max, float* sum_exp, void* workspace, size_t workspace_bytes,
-                     hipStream_t stream) {
+                     float* row_max, float* sum_exp, void* probs, float* probs_ref,
+                     void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0 || labels == nullptr) return AREAL_ERR_BAD_ARG;
+  if ((probs == nullptr) != (probs_ref == nullptr)) return AREAL_ERR_BAD_ARG;
+  if (probs != nullptr && !aligned16(probs)) return AREAL_ERR_ALIGNMENT;
   if (!(inv_temperature > 0.f) || !(logit_scale > 0.f)) return AREAL_ERR_BAD_ARG;
   if (T == 0) return AREAL_OK;
   if (T > (1 << 30) || V > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
@@ -830,17 +1111,24 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   if (workspace == nullptr || workspace_bytes < need) return AREAL_ERR_WORKSPACE;
   const Regions r = fwd_regions(T, H, V);
   const int P = fwd_slots(r);
-  GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H};
+  GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H, 0, 0, 0};
   FwdParams ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
-               (float*)workspace, P, 0};
+               (float*)workspace, P, 0, (u16*)probs, round_up_i64(V, BK), probs_ref};
   FwdParams ep_a = ep;
   ep_a.slot_base = 4 * r.S;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
   const bool moments = (vocab_mean != nullptr) || (vocab_norm != nullptr);
-  if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
-  else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
-  else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
-  else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
+  if (probs == nullptr) {
+    if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
+    else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
+    else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
+    else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
+  } else {
+    if (!affine && !moments) rc = launch_gemm<FwdPlainSave>(g, r, ep, ep_a, stream);
+    else if (!affine) rc = launch_gemm<FwdPlainMomSave>(g, r, ep, ep_a, stream);
+    else if (!moments) rc = launch_gemm<FwdAffineSave>(g, r, ep, ep_a, stream);
+    else rc = launch_gemm<FwdAffineMomSave>(g, r, ep, ep_a, stream);
+  }
   if (rc != AREAL_OK) return rc;
   const int threads = 256;
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, threads)), dim3(threads),
@@ -910,36 +1198,115 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     const int64_t Tc = (T - t0) < Tc_max ? (T - t0) : Tc_max;
     const int64_t ldt_c = round_up_i64(Tc, BK);
     const u16* hid_c = (const u16*)hidden + t0 * H;
-    // 1. recompute logits of the chunk, emit dlogits in both layouts
+    // dWeight reads dl and hidden k-major (no transposed copies) when the chunk is a multiple
+    // of 64 tokens; otherwise it goes through dlT and hidden^T.
+    const bool tn = (Tc % BK == 0) && dweight_f32 != nullptr;
+    const bool need_dlT = dweight_f32 != nullptr && !tn;
+    // 1. recompute logits of the chunk, emit dlogits
     {
-      GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H};
+      GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H, 0, 0, 0};
       BwdParams ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
                    (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
       const Regions r = plan_regions(V, Tc, H, 512, 0);
-      rc = affine ? launch_gemm<BwdAffine>(g, r, ep, ep, stream)
-                  : launch_gemm<BwdPlain>(g, r, ep, ep, stream);
+      if (need_dlT)
+        rc = affine ? launch_gemm<BwdAffineT>(g, r, ep, ep, stream)
+                    : launch_gemm<BwdPlainT>(g, r, ep, ep, stream);
+      else
+        rc = affine ? launch_gemm<BwdAffine>(g, r, ep, ep, stream)
+                    : launch_gemm<BwdPlain>(g, r, ep, ep, stream);
       if (rc != AREAL_OK) return rc;
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
-      GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv};
+      GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv, 0, 0, 0};
       const StoreParams ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc};
       const Regions r = plan_regions(H, Tc, ldv, 0, 1 << 20);
       if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
     }
-    // 3. dWeight[v, h] += sum_t dlT[v, t] * hidden^T[h, t]
-    if (dweight_f32 != nullptr) {
+    // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
+    if (tn) {
+      GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv, (int)Tc};
+      const StoreParams ep{dweight_f32, H, (int)H, (int)V};
+      const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
+      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
+                                  : launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
+      if (rc != AREAL_OK) return rc;
+    } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
                          dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldt_c, 64)),
                          dim3(256), 0, stream, hid_c, H, (int)Tc, (int)H, hT, ldt_c);
       AREAL_CHECK_LAUNCH();
-      GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c};
+      GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
       rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32>(g, r, ep, ep, stream)
                                   : launch_gemm<StoreF32>(g, r, ep, ep, stream);
       if (rc != AREAL_OK) return rc;
     }
+  }
+  return AREAL_OK;
+}
+
+// Workspace of the backward from saved exponentials: W^T [H, round_up(V, 64)] bf16.
+size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (T <= 0 || H <= 0 || V <= 0) return 0;
+  return (size_t)(H * round_up_i64(V, BK)) * 2 + 256;
+}
+
+// Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref): no logits are
+// recomputed. probs is overwritten with the bf16 dlogits, so it can be used once. logprobs
+// (nullable) are the label log-probabilities of the forward; with them the label's entry of
+// dlogits is evaluated in fp32.
+int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
+                           const float* row_max, const float* sum_exp, const float* logprobs,
+                           const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
+                           float inv_temperature, float logit_scale, void* probs,
+                           const float* probs_ref, void* dhidden, float* dweight_f32,
+                           int accumulate, void* workspace, size_t workspace_bytes,
+                           hipStream_t stream) {
+  if (T < 0 || H <= 0 || V <= 0) return AREAL_ERR_BAD_ARG;
+  if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr ||
+      probs == nullptr || probs_ref == nullptr)
+    return AREAL_ERR_BAD_ARG;
+  if (dhidden == nullptr && dweight_f32 == nullptr) return AREAL_ERR_BAD_ARG;
+  if (T == 0) return AREAL_OK;
+  if (T > (1 << 30) || V > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  int rc;
+  if ((rc = check_operand(hidden, H)) != AREAL_OK) return rc;
+  if ((rc = check_operand(weight, H)) != AREAL_OK) return rc;
+  if (!aligned16(probs)) return AREAL_ERR_ALIGNMENT;
+  if (dhidden != nullptr && !aligned16(dhidden)) return AREAL_ERR_ALIGNMENT;
+  if (dweight_f32 != nullptr && !aligned16(dweight_f32)) return AREAL_ERR_ALIGNMENT;
+  if (dhidden != nullptr &&
+      (workspace == nullptr || workspace_bytes < areal_lmhead_bwd_saved_workspace_bytes(T, H, V)))
+    return AREAL_ERR_WORKSPACE;
+  const int64_t ldv = round_up_i64(V, BK), Tpad = round_up_i64(T, BK);
+  u16* dl = (u16*)probs;
+  hipLaunchKernelGGL(dlogits_from_saved_kernel,
+                     dim3((unsigned)ceil_div_i64(ldv, 2048), (unsigned)Tpad), dim3(256), 0, stream,
+                     dl, ldv, probs_ref, labels, row_max, sum_exp, grad_logprobs, logprobs, (int)T,
+                     (int)V, inv_temperature * LOG2E, inv_temperature * logit_scale);
+  AREAL_CHECK_LAUNCH();
+  if (dhidden != nullptr) {
+    u16* wT = (u16*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    hipLaunchKernelGGL(transpose_pad_bf16_kernel,
+                       dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
+                       dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
+    AREAL_CHECK_LAUNCH();
+    // dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
+    GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
+    const StoreParams ep{dhidden, H, (int)H, (int)T};
+    const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
+    if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+  }
+  if (dweight_f32 != nullptr) {
+    // dWeight[v, h] += sum_t dl[t, v] * hidden[t, h], k-major over the Tpad rows of dl
+    GemmArgs g{(const u16*)hidden, H, (int)H, dl, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
+    const StoreParams ep{dweight_f32, H, (int)H, (int)V};
+    const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
+    rc = accumulate ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
+                    : launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
+    if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;
 }

@@ -3,9 +3,19 @@
 Host-side counterpart of the reference's chunked LM head
 (``areal/models/mcore/vocab_parallel_head.py:560-938`` and its wrapper
 ``chunked_lm_head_logprobs_entropy`` at ``:941-982``): same outputs
-(``ChunkedLMHeadOutput``), same saved state (row max and sum of exponentials per token, never
-a ``[T, V]`` tensor), same error behaviour.  The arithmetic runs in the HIP kernels of
+(``ChunkedLMHeadOutput``), same error behaviour.  The arithmetic runs in the HIP kernels of
 ``csrc/lmhead.hip`` through the C ABI.
+
+Two ways of carrying state to the backward:
+
+* ``save_probs=False``: what the reference does -- row max and sum of exponentials per token,
+  never a ``[T, V]`` tensor; the backward recomputes the logits chunk by chunk
+  (``vocab_parallel_head.py:806-829``).
+* ``save_probs=True``: the forward also writes the softmax exponentials as a bf16 ``[T, V]``
+  tensor (2 bytes per logit), the backward turns them into dlogits in place and skips the
+  recomputation, a quarter of the step's matrix work.  The reference's logits-in path saves
+  the same amount through autograd; 288 GB of HBM make it the default while it fits
+  ``SAVE_PROBS_BYTES_LIMIT``.
 """
 
 from __future__ import annotations
@@ -21,6 +31,13 @@ from areal_amd import _lib
 # plus transposed operands).  An MI355X has 288 GB of HBM, so one chunk normally covers the
 # whole micro-batch.
 DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
+
+# save_probs=None keeps the exponentials when the bf16 [T, V] buffer is at most this large.
+SAVE_PROBS_BYTES_LIMIT = 24 << 30
+
+
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
 
 
 class ChunkedLMHeadOutput(NamedTuple):
@@ -48,7 +65,9 @@ def default_token_chunk(T: int, H: int, V: int, budget: int = DEFAULT_BWD_WORKSP
 
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, bias, labels, temperature, logit_scale, token_chunk):
+    def forward(
+        ctx, hidden, weight, bias, labels, temperature, logit_scale, token_chunk, save_probs
+    ):
         lib = _lib.load()
         dev = _lib.require_gpu(hidden, weight, labels, bias)
         H = hidden.size(-1)
@@ -62,6 +81,15 @@ class _FusedLMHead(torch.autograd.Function):
         outs = [torch.empty(labels.shape, dtype=torch.float32, device=dev) for _ in range(6)]
         outs += [torch.empty(T, dtype=torch.float32, device=dev) for _ in range(2)]
         logprobs, entropy, vmin, vmax, vmean, vnorm, row_max, sum_exp = outs
+        needs_grad = any(ctx.needs_input_grad[:2])
+        if save_probs is None:
+            save_probs = 2 * _round_up(T, 64) * _round_up(V, 64) <= SAVE_PROBS_BYTES_LIMIT
+        probs = probs_ref = None
+        if save_probs and needs_grad and T > 0:
+            probs = torch.empty(
+                (_round_up(T, 64), _round_up(V, 64)), dtype=torch.bfloat16, device=dev
+            )
+            probs_ref = torch.empty(((V + 127) // 128, T), dtype=torch.float32, device=dev)
         if T > 0:
             nbytes = lib.areal_lmhead_fwd_workspace_bytes(T, H, V)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -69,11 +97,16 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(bias_f), _lib.ptr(labels_1d),
                 T, H, V, 1.0 / temperature, logit_scale,
                 *[_lib.ptr(o) for o in outs],
+                _lib.ptr(probs), _lib.ptr(probs_ref),
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_fwd")
 
         ctx.save_for_backward(hidden_2d, weight_c, labels_1d, row_max, sum_exp)
+        # Plain attributes, not saved tensors: the backward overwrites probs in place.
+        ctx.probs = probs
+        ctx.probs_ref = probs_ref
+        ctx.label_logprobs = logprobs.detach().reshape(-1).clone() if probs is not None else None
         ctx.bias_f = bias_f
         ctx.temperature = temperature
         ctx.logit_scale = logit_scale
@@ -91,7 +124,7 @@ class _FusedLMHead(torch.autograd.Function):
         if need_b:
             raise NotImplementedError("gradient of the lm_head bias is not implemented")
         if grad_logprobs is None or not (need_h or need_w):
-            return (None,) * 7
+            return (None,) * 8
         lib = _lib.load()
         dev = hidden_2d.device
         T, H = hidden_2d.shape
@@ -99,9 +132,24 @@ class _FusedLMHead(torch.autograd.Function):
         g = grad_logprobs.reshape(-1).to(torch.float32).contiguous()
         dh = torch.empty_like(hidden_2d) if need_h else None
         dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if need_w else None
+        probs, probs_ref = ctx.probs, ctx.probs_ref
+        ctx.probs = ctx.probs_ref = None  # consumed; a second backward recomputes the logits
         if T == 0:
             if dw32 is not None:
                 dw32.zero_()
+        elif probs is not None:
+            nbytes = lib.areal_lmhead_bwd_saved_workspace_bytes(T, H, V) if need_h else 0
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if need_h else None
+            rc = lib.areal_lmhead_bwd_saved(
+                _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(labels_1d),
+                _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),
+                T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
+                _lib.ptr(probs), _lib.ptr(probs_ref),
+                _lib.ptr(dh), _lib.ptr(dw32), 0,
+                _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+            )
+            _lib.check(rc, "areal_lmhead_bwd_saved")
+            del probs, probs_ref
         else:
             chunk = ctx.token_chunk or default_token_chunk(T, H, V)
             nbytes = lib.areal_lmhead_bwd_workspace_bytes(T, H, V, chunk)
@@ -126,7 +174,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.check(rc, "areal_cast_f32_to_bf16")
         if dh is not None:
             dh = dh.view(ctx.hidden_shape)
-        return dh, dw, None, None, None, None, None
+        return dh, dw, None, None, None, None, None, None
 
 
 def fused_lm_head_logprobs_entropy(
@@ -139,6 +187,7 @@ def fused_lm_head_logprobs_entropy(
     logit_scale: float = 1.0,
     bias: torch.Tensor | None = None,
     token_chunk: int | None = None,
+    save_probs: bool | None = None,
 ) -> ChunkedLMHeadOutput:
     """Label log-probabilities, entropy and vocabulary statistics of ``hidden @ weight.T``.
 
@@ -153,6 +202,8 @@ def fused_lm_head_logprobs_entropy(
         bias: optional ``[V]`` bias added to the logits.
         token_chunk: tokens per backward chunk (bounds the bf16 dlogits workspace);
             ``None`` picks the largest chunk within ``DEFAULT_BWD_WORKSPACE_BYTES``.
+        save_probs: keep the bf16 softmax exponentials for the backward instead of recomputing
+            the logits; ``None`` decides by ``SAVE_PROBS_BYTES_LIMIT``.
 
     Gradient flows through ``logprobs`` only (to ``hidden`` and ``weight``), as in the
     reference (``vocab_parallel_head.py:732-734``).
@@ -186,6 +237,7 @@ def fused_lm_head_logprobs_entropy(
     if bias is not None and bias.shape != (weight.size(0),):
         raise ValueError(f"bias must have shape ({weight.size(0)},), got {tuple(bias.shape)}")
     values = _FusedLMHead.apply(
-        hidden, weight, bias, labels, float(temperature), float(logit_scale), token_chunk
+        hidden, weight, bias, labels, float(temperature), float(logit_scale), token_chunk,
+        save_probs,
     )
     return ChunkedLMHeadOutput(*values)

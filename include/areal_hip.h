@@ -44,13 +44,19 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
 /* hidden [T,H] bf16, weight [V,H] bf16 (H % 8 == 0, 16-byte aligned), bias [V] fp32 or NULL,
  * labels [T] int64. Outputs fp32 [T]; row_max and sum_exp are the state saved for backward
- * (vocab_parallel_head.py:704-713). logits = (hidden . weight^T + bias) * logit_scale. */
+ * (vocab_parallel_head.py:704-713). logits = (hidden . weight^T + bias) * logit_scale.
+ *
+ * probs / probs_ref (both NULL, or both set) additionally keep the softmax exponentials for
+ * areal_lmhead_bwd_saved, the counterpart of autograd saving the logits in the reference's
+ * logits-in path (_gather_logprobs_entropy, areal/utils/functional/vocab_parallel.py:24-30): probs is bf16
+ * [round_up(T,64)][round_up(V,64)] holding exp((x - m_blk)/T) per 128-wide vocabulary block,
+ * probs_ref is fp32 [ceil(V/128)][T] holding m_blk / T * log2(e). */
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
-                     float* row_max, float* sum_exp, void* workspace, size_t workspace_bytes,
-                     areal_stream_t stream);
+                     float* row_max, float* sum_exp, void* probs, float* probs_ref,
+                     void* workspace, size_t workspace_bytes, areal_stream_t stream);
 
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
 
@@ -63,6 +69,22 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                      float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
                      int accumulate, int64_t token_chunk, void* workspace, size_t workspace_bytes,
                      areal_stream_t stream);
+
+size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
+
+/* Backward from the exponentials the forward kept (probs, probs_ref): the logits are not
+ * recomputed (vocab_parallel_head.py:806-829 recomputes them chunk by chunk to save memory; an
+ * MI355X has the HBM to keep them). probs is overwritten with the bf16 dlogits and can be
+ * used once. logprobs (NULL allowed) are the forward's label log-probabilities: with them the
+ * label's dlogit is -expm1(logprob) in fp32. Other arguments as areal_lmhead_bwd; bias does
+ * not enter (it is part of the saved exponentials). workspace may be NULL if dhidden is. */
+int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
+                           const float* row_max, const float* sum_exp, const float* logprobs,
+                           const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
+                           float inv_temperature, float logit_scale, void* probs,
+                           const float* probs_ref, void* dhidden, float* dweight_f32,
+                           int accumulate, void* workspace, size_t workspace_bytes,
+                           areal_stream_t stream);
 
 /* out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]  (bf16 in, fp32 accumulate).
  * out_mode 0: bf16 store, 1: fp32 store, 2: fp32 accumulate. The contraction used by the

@@ -51,8 +51,9 @@ SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("save_probs", [False, True], ids=["recompute", "saved"])
 @pytest.mark.parametrize("T,H,V,temp,scale,use_bias,chunk", SHAPES)
-def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, chunk):
+def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, chunk, save_probs):
     g = torch.Generator().manual_seed(T * 7 + V)
     hidden = torch.randn(T, H, generator=g).bfloat16()
     weight = (torch.randn(V, H, generator=g) * (0.5 if V < 10000 else 0.02)).bfloat16()
@@ -63,7 +64,8 @@ def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, ch
     h = hidden.to(dev).requires_grad_(True)
     w = weight.to(dev).requires_grad_(True)
     out = fused_lm_head_logprobs_entropy(h, w, labels.to(dev), temperature=temp, logit_scale=scale,
-                                         bias=bias.to(dev) if use_bias else None, token_chunk=chunk)
+                                         bias=bias.to(dev) if use_bias else None, token_chunk=chunk,
+                                         save_probs=save_probs)
     want = L.lm_head_logprobs_entropy(hidden, weight, labels, temp, scale, bias)
     names = ["logprobs", "entropy", "vocab_min", "vocab_max", "vocab_mean", "vocab_norm"]
     for name, a, b in zip(names, out, want):
@@ -88,9 +90,68 @@ def test_no_vocab_sized_tensor_is_saved(dev):
     h = torch.randn(T, H, device=dev).bfloat16().requires_grad_(True)
     w = torch.randn(V, H, device=dev).bfloat16().requires_grad_(True)
     y = torch.randint(0, V, (T,), device=dev)
-    out = fused_lm_head_logprobs_entropy(h, w, y)
+    out = fused_lm_head_logprobs_entropy(h, w, y, save_probs=False)
     for t in out.logprobs.grad_fn.saved_tensors:
         assert tuple(t.shape) != (T, V) and t.numel() <= max(T * H, V * H)
+
+
+def test_saved_exponentials_are_bf16_and_used_once(dev):
+    # save_probs=True keeps one bf16 [T, V] buffer (padded to 64), consumed by the first
+    # backward; a second backward over a retained graph recomputes the logits instead.
+    T, H, V = 100, 64, 1000
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * 0.3).bfloat16().to(dev)
+    y = torch.randint(0, V, (T,), generator=g).to(dev)
+    grad = torch.randn(T, generator=g).to(dev)
+    h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, y, save_probs=True)
+    fn = out.logprobs.grad_fn
+    assert fn.probs.dtype == torch.bfloat16 and tuple(fn.probs.shape) == (128, 1024)
+    assert tuple(fn.probs_ref.shape) == (8, T)
+    loss = (out.logprobs * grad).sum()
+    loss.backward(retain_graph=True)
+    assert fn.probs is None
+    g1h, g1w = h.grad.clone(), w.grad.clone()
+    h.grad = None
+    w.grad = None
+    loss.backward()
+    assert _rel(h.grad.float(), g1h.float()) < 1e-2 and _rel(w.grad.float(), g1w.float()) < 1e-2
+    with torch.no_grad():  # nothing is kept when no gradient can flow
+        out = fused_lm_head_logprobs_entropy(hidden, weight, y, save_probs=True)
+    assert out.logprobs.grad_fn is None
+
+
+def test_saved_path_confident_tokens_and_invalid_labels(dev):
+    # Tokens whose label probability is ~1: 1 - p must not be lost to the bf16 rounding of p
+    # (the label's dlogit comes from the fp32 log-probability). Labels outside [0, V) get no
+    # one-hot term, as in the recompute path.
+    T, H, V = 192, 64, 777
+    g = torch.Generator().manual_seed(9)
+    weight = (torch.randn(V, H, generator=g) * 0.3).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    hidden = (weight[labels].float() * 4.0).bfloat16()  # logit of the label dominates
+    grad = torch.randn(T, generator=g)
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels.to(dev), save_probs=True)
+    assert out.logprobs.max().item() > -1e-3
+    (out.logprobs * grad.to(dev)).sum().backward()
+    dh_want, dw_want = L.lm_head_backward(hidden, weight, labels, grad)
+    assert _rel(h.grad.cpu().float(), dh_want) < 1e-2
+    assert _rel(w.grad.cpu().float(), dw_want) < 1e-2
+    bad = labels.clone()
+    bad[::2] = -100
+    bad[1::4] = V + 3
+    res = []
+    for save in (False, True):
+        h2 = hidden.to(dev).requires_grad_(True)
+        w2 = weight.to(dev).requires_grad_(True)
+        o = fused_lm_head_logprobs_entropy(h2, w2, bad.to(dev), save_probs=save)
+        (o.logprobs * grad.to(dev)).sum().backward()
+        res.append((o.logprobs.detach(), h2.grad.float(), w2.grad.float()))
+    torch.testing.assert_close(res[0][0], res[1][0], rtol=0, atol=1e-4)
+    assert _rel(res[1][1], res[0][1]) < 1e-2 and _rel(res[1][2], res[0][2]) < 1e-2
 
 
 def test_chunking_and_repeat_runs_are_bit_identical(dev):
@@ -103,7 +164,7 @@ def test_chunking_and_repeat_runs_are_bit_identical(dev):
     res = []
     for chunk in (None, None, 256):
         h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
-        out = fused_lm_head_logprobs_entropy(h, w, y, token_chunk=chunk)
+        out = fused_lm_head_logprobs_entropy(h, w, y, token_chunk=chunk, save_probs=False)
         (out.logprobs * grad).sum().backward()
         res.append((out.logprobs.detach(), out.entropy, h.grad, w.grad))
     for a, b in zip(res[0], res[1]):
