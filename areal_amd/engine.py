@@ -56,8 +56,12 @@ def compute_logprobs_and_loss(
     temperature: float = 1.0,
     pad_length: int = 0,
     loss_multiplier: float = 1.0,
+    save_probs: bool | None = None,
 ) -> torch.Tensor:
     """Scaled loss of one micro-batch (``fsdp_engine.py:2147-2217``).
+
+    ``save_probs`` is handed to ``fused_lm_head_logprobs_entropy`` (keep the bf16 softmax
+    exponentials for the backward, or recompute the logits there).
 
     ``loss_fn(logprobs, entropy, mb_input, vocab_min_logits=..., vocab_max_logits=...)`` is
     the actor loss (normally a ``functools.partial`` of ``grpo_loss_fn``).  The per-token
@@ -69,7 +73,8 @@ def compute_logprobs_and_loss(
     if hidden.ndim == 3 and hidden.shape[0] == 1:
         hidden = hidden.squeeze(0)
     out = fused_lm_head_logprobs_entropy(
-        hidden, lm_head_weight, _labels(model_inputs), temperature=temperature
+        hidden, lm_head_weight, _labels(model_inputs), temperature=temperature,
+        save_probs=save_probs,
     )
     logprobs, entropy = out.logprobs, out.entropy
     vmin, vmax = out.vocab_min_logits, out.vocab_max_logits

@@ -81,7 +81,7 @@ class _FusedLMHead(torch.autograd.Function):
         outs = [torch.empty(labels.shape, dtype=torch.float32, device=dev) for _ in range(6)]
         outs += [torch.empty(T, dtype=torch.float32, device=dev) for _ in range(2)]
         logprobs, entropy, vmin, vmax, vmean, vnorm, row_max, sum_exp = outs
-        needs_grad = any(ctx.needs_input_grad[:2])
+        needs_grad = any(ctx.needs_input_grad[:2])  # the caller has ruled out no_grad mode
         if save_probs is None:
             save_probs = 2 * _round_up(T, 64) * _round_up(V, 64) <= SAVE_PROBS_BYTES_LIMIT
         probs = probs_ref = None
@@ -236,6 +236,8 @@ def fused_lm_head_logprobs_entropy(
         raise ValueError(f"hidden size must be a multiple of 8, got {hidden.size(-1)}")
     if bias is not None and bias.shape != (weight.size(0),):
         raise ValueError(f"bias must have shape ({weight.size(0)},), got {tuple(bias.shape)}")
+    if not torch.is_grad_enabled():
+        save_probs = False  # no backward will come: keep nothing
     values = _FusedLMHead.apply(
         hidden, weight, bias, labels, float(temperature), float(logit_scale), token_chunk,
         save_probs,

@@ -178,6 +178,9 @@ def main() -> None:
     ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true")
+    ap.add_argument("--recompute", action="store_true",
+                    help="backward recomputes the logits (save_probs=False) instead of using the "
+                         "bf16 exponentials kept by the forward")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -211,15 +214,20 @@ def main() -> None:
                                                    lower=0.5, upper=2.0),
     )
 
+    # None: keep the exponentials if the bf16 [T, V] buffer fits the library's default limit
+    save_probs = False if args.recompute else None
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
     t_fwd = t_loss = t_bwd = 0.0
+    saved = False
 
     def step(timed: bool):
-        nonlocal t_fwd, t_loss, t_bwd
+        nonlocal t_fwd, t_loss, t_bwd, saved
         hidden.grad = None
         weight.grad = None
         ev[0].record()
-        out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0)
+        out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0,
+                                             save_probs=save_probs)
+        saved = out.logprobs.grad_fn.probs is not None
         ev[1].record()
         loss = loss_fn(out.logprobs, out.entropy, input_data,
                        vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
@@ -244,15 +252,30 @@ def main() -> None:
     ms_per_step = wall * 1e3 / args.steps
     tokens_per_s = T * args.steps / wall
 
-    # Roofline of the MFMA contraction kernel (gemm_nt_sweep): one step launches it four times
-    # (forward, recompute, dHidden, dWeight) for 3 algorithmic GEMMs = 6*T*H*V flops; the
-    # recompute launch carries no algorithmic flops.  Durations are the HIP-event times of the
-    # forward and backward library calls (they also contain the merge, transpose and cast
+    # Roofline of the MFMA contraction kernels (gemm_nt_sweep / gemm_tn_sweep): one step runs
+    # 3 algorithmic GEMMs = 6*T*H*V flops (forward with the softmax epilogue, dHidden, dWeight);
+    # with --recompute a fourth launch recomputes the logits and carries no algorithmic flops.
+    # Durations are the HIP-event times of the forward and backward library calls on the
+    # stream they are launched on (they also contain the merge, dlogits, transpose and cast
     # kernels, which makes the figure slightly pessimistic).
     gemm_ms = (t_fwd + t_bwd) / args.steps
     algo_flops = 6.0 * T * H * V
     achieved = algo_flops / (gemm_ms * 1e-3) / 1e12
     fwd_tflops = 2.0 * T * H * V / (t_fwd / args.steps * 1e-3) / 1e12
+
+    # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+    # command (KiB per dispatch, scaled by the factors the same counters show for the fp32->bf16
+    # cast kernel of known size: fetch x2.0, write x1.0). Only measured for the default workload.
+    traffic = None
+    traffic_detail = None
+    if args.workload == "qwen3-8b" and saved:
+        kib = 1024.0
+        traffic_detail = {
+            "gemm_nt_sweep<FwdEpi> forward": 3.19194e7 * kib * 2.0 + 1.12812e7 * kib,
+            "gemm_nt_sweep<StoreEpi> dHidden": 2.91944e7 * kib * 2.0 + 3.072e5 * kib,
+            "gemm_tn_sweep<StoreEpi> dWeight": 2.96736e7 * kib * 2.0 + 2.42893e6 * kib,
+        }
+        traffic = sum(traffic_detail.values()) / 3.0
 
     result = {
         "metric": "packed tokens/sec, logprob+entropy+PPO loss fwd+bwd; % bf16 MFMA peak",
@@ -272,16 +295,20 @@ def main() -> None:
             "tokens": T, "hidden": H, "vocab": V,
             "loss": "PPO clip eps=0.2, rejection sampling ratio in [0.5, 2.0] (token, mask)",
             "final_loss": float(loss.detach().item()),
+            "backward": "saved bf16 exponentials" if saved else "recompute logits",
         },
         "pct_bf16_mfma_peak": 100.0 * (algo_flops / (ms_per_step * 1e-3) / 1e12) / PEAK_BF16_TFLOPS,
         "roofline": {
-            "kernel": "gemm_nt_sweep (4 launches/step: forward, recompute, dHidden, dWeight)",
+            "kernel": ("gemm_nt_sweep<FwdEpi>, gemm_nt_sweep<StoreEpi> (dHidden), "
+                       "gemm_tn_sweep<StoreEpi> (dWeight)"
+                       + ("" if saved else ", gemm_nt_sweep<BwdEpi> (recompute)")),
             "bound": "mfma",
             "achieved": achieved,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_BF16_TFLOPS,
-            "traffic": None,
+            "traffic": traffic,
+            "traffic_bytes_per_launch": traffic_detail,
             "forward_only_tflops": fwd_tflops,
             "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},

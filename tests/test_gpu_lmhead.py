@@ -118,7 +118,7 @@ def test_saved_exponentials_are_bf16_and_used_once(dev):
     loss.backward()
     assert _rel(h.grad.float(), g1h.float()) < 1e-2 and _rel(w.grad.float(), g1w.float()) < 1e-2
     with torch.no_grad():  # nothing is kept when no gradient can flow
-        out = fused_lm_head_logprobs_entropy(hidden, weight, y, save_probs=True)
+        out = fused_lm_head_logprobs_entropy(h, w, y, save_probs=True)
     assert out.logprobs.grad_fn is None
 
 
