@@ -142,6 +142,18 @@ def hbm_rooflines(dev):
     m = (torch.rand(T, device=dev) > 0.25).float()
     add("gae_block_total+gae_carry+gae_apply", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
         20 * T, timed(lambda: compute_gae_packed(r, v, m, cu, None, 1.0, 0.95)))
+    # the padded drop-in signature on the same batch: [1024, 8192] (8.39 M slots)
+    from areal_amd.ppo.gae import _compute_token_level_gae
+
+    rp = torch.zeros(1024, 8192, device=dev)
+    rp[torch.arange(1024, device=dev), (lens.to(dev) - 2).clamp(min=0)] = 1.0
+    vp = torch.randn(1024, 8192, device=dev)
+    pos = torch.arange(8192, device=dev)[None, :]
+    mp = ((pos >= (lens.to(dev) // 4)[:, None]) & (pos < (lens.to(dev) - 1)[:, None])).float()
+    no_eos = torch.zeros(1024, dtype=torch.bool, device=dev)
+    add("gae_block_total+gae_carry+gae_apply", "config 3 padded form: [1024, 8192] slots, 20 B/slot",
+        20 * rp.numel(), timed(lambda: _compute_token_level_gae(rp, vp, mp, no_eos, 1.0, 0.95)))
+    del rp, vp, mp
     x = torch.randn(1024, 1600, device=dev)
     mk = (torch.rand(1024, 1600, device=dev) > 0.25).float()
     norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
@@ -160,8 +172,32 @@ def hbm_rooflines(dev):
         loss, _ = ppo_actor_loss_fn(lp, prox, old, adv, 0.2, mask, rejection_sampling=rs)
         loss.backward()
 
-    add("loss_token+loss_finalize+loss_grad_scale", "PPO + IcePop, 4 Mi tokens, fwd+bwd, 47 B/token + 8 B/token grad scale",
+    add("ppo_actor_loss_fn + backward (API level)",
+        "PPO + IcePop, 4 Mi tokens, fwd+bwd through the Python API: includes the one device-to-host copy "
+        "of the counters per call (the reference has 1-3 .item() syncs), 47 B/token + 8 B/token grad scale",
         55 * Tl, timed(loss_step))
+
+    # the same kernels through the C ABI without the host copy, back to back on the stream
+    from areal_amd import _lib
+    from areal_amd.functional import functional as F
+
+    lib = _lib.load()
+    cfg = _lib.LossConfig()
+    cfg.loss_kind = F.LOSS_PPO
+    cfg.clip_lo, cfg.clip_hi = 0.8, 1.2
+    F._fill_rs(cfg, rs)
+    lp32, mask_b = lp.detach(), mask.bool().contiguous()
+    gout = torch.ones(1, device=dev)
+    grad = torch.empty(Tl, device=dev)
+
+    def loss_kernels():
+        o = F._run_loss_kernel(cfg, lp32.shape, lp32, prox, old, adv, mask_b, None, True)
+        rc = lib.areal_actor_loss_grad(_lib.ptr(o["dlp"]), _lib.ptr(gout), _lib.ptr(o["counters_dev"]),
+                                       _lib.ptr(grad), Tl, _lib.stream_ptr(dev))
+        _lib.check(rc, "areal_actor_loss_grad")
+
+    add("loss_token+loss_finalize+loss_grad_scale", "PPO + IcePop, 4 Mi tokens, fwd+bwd kernels through the C ABI, "
+        "47 B/token + 8 B/token grad scale", 55 * Tl, timed(loss_kernels, iters=50))
     lg = torch.randn(4096, V_QWEN, device=dev).bfloat16()
     lab = torch.randint(0, V_QWEN, (4096,), device=dev)
     add("rows_fwd_kernel", "config 1: [4096, 151936] bf16 logits, logprob + entropy forward",
