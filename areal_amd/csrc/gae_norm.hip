@@ -27,12 +27,14 @@ struct Map {
 DEVI Map map_identity() { return Map{1.0, 0.0, 1.0, 0.0, 0.0}; }
 // (f o g): apply g first, then f.
 DEVI Map compose(const Map& f, const Map& g) {
+  // explicit fma: this file is compiled without contraction (the normalisation kernels follow
+  // the reference's fp32 rounding), but the fp64 maps are more exact with it and cost half
   Map r;
   r.a11 = f.a11 * g.a11;
-  r.a12 = f.a11 * g.a12 + f.a12 * g.a22;
+  r.a12 = fma(f.a11, g.a12, f.a12 * g.a22);
   r.a22 = f.a22 * g.a22;
-  r.b1 = f.a11 * g.b1 + f.a12 * g.b2 + f.b1;
-  r.b2 = f.a22 * g.b2 + f.b2;
+  r.b1 = fma(f.a11, g.b1, fma(f.a12, g.b2, f.b1));
+  r.b2 = fma(f.a22, g.b2, f.b2);
   return r;
 }
 DEVI Map shfl_down_map(const Map& m, int d) {
@@ -57,6 +59,7 @@ struct GaeArgs {
   float lam;
   float* adv;
   float* ret;
+  int block_per_seq;         // single-pass kernel, padded rows of at least a tile: block = row
 };
 
 DEVI int gae_seq_of(const GaeArgs& g, int64_t t) {
@@ -197,8 +200,8 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_carry_kernel(const Map* total
     carry[2 * b] = A;
     carry[2 * b + 1] = nv;
     const Map f = totals[b];
-    const double A2 = f.a11 * A + f.a12 * nv + f.b1;
-    const double nv2 = f.a22 * nv + f.b2;
+    const double A2 = fma(f.a11, A, fma(f.a12, nv, f.b1));
+    const double nv2 = fma(f.a22, nv, f.b2);
     A = A2; nv = nv2;
   }
 }
@@ -223,12 +226,240 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_apply_kernel(GaeArgs g, const
     const int64_t t = t0 + i;
     if (t >= g.n) continue;
     const Map& f = mp[i];
-    const double A2 = f.a11 * A + f.a12 * nv + f.b1;
-    const double nv2 = f.a22 * nv + f.b2;
+    const double A2 = fma(f.a11, A, fma(f.a12, nv, f.b1));
+    const double nv2 = fma(f.a22, nv, f.b2);
     A = A2; nv = nv2;
     const float a = (float)A;
     g.adv[t] = a;
     g.ret[t] = a + v[i];
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Single-pass GAE. Sequences are independent, so a block that starts at the end of a sequence
+// needs no carry from its right. Block b owns the sequences whose END lies in the token range
+// (b*TILE, (b+1)*TILE] and walks from the end of its last owned sequence down to the start of
+// its first one, tile by tile (tiles are absolute multiples of TILE, so the vector loads stay
+// aligned), carrying (A, nv) across its tiles. Every token is read once and written once:
+// 20 B/token, one launch, no dependency between blocks. A sequence much longer than a tile is
+// walked by one block; the host picks the three-launch scan above when the average sequence
+// is very long.
+// ---------------------------------------------------------------------------------------
+
+// #{i in [0, n) : ends[i] <= x} for a non-decreasing array, by one wave: every round probes 64
+// positions and keeps the gap after the last probe that is <= x.
+DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
+  int base = 0, len = n;
+  while (len > 0) {
+    const int step = (len + 63) >> 6;
+    const int idx = base + lane * step;
+    const bool le = (idx < base + len) && ((int64_t)ends[idx] <= x);
+    const int cnt = __popcll(__builtin_amdgcn_ballot_w64(le));
+    if (cnt == 0) break;  // ends[base] > x
+    const int hit = base + (cnt - 1) * step;  // last probe <= x
+    const int lim = base + len;
+    base = hit + 1;
+    len = step - 1;
+    if (base + len > lim) len = lim - base;
+  }
+  return base;
+}
+
+__global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
+  __shared__ Map smem[4];
+  __shared__ Map all[GAE_THREADS];
+  __shared__ int32_t s_cu[GAE_TILE + 2];
+  __shared__ int s_own[2];
+  const int tid = threadIdx.x;
+  // Workgroups go to the 8 XCDs round-robin by id. Giving XCD x the x-th eighth of the token
+  // ranges keeps the work even when only every k-th range owns a sequence end (padded rows).
+  const int64_t per_xcd = (gridDim.x + 7) >> 3;
+  const int64_t range = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  // padded rows of at least a tile: only every (L / TILE)-th range would own a row, so the grid
+  // is one block per row instead (lo, hi] = the range holding the row's end
+  const int64_t lo = g.block_per_seq ? ((int64_t)(blockIdx.x + 1) * g.uniform_len - 1)
+                                     : range * GAE_TILE;
+  if (!g.block_per_seq && (range >= per_xcd * 8 || lo >= g.n)) return;
+  const int64_t hi = g.block_per_seq ? lo + 1 : (lo + GAE_TILE < g.n ? lo + GAE_TILE : g.n);
+  const bool uniform = g.uniform_len > 0;
+
+  // tokens outside every sequence (none in a well-formed batch) are written as zero
+  {
+    const int64_t cov_lo = uniform ? 0 : (int64_t)g.cu[0];
+    const int64_t cov_hi = uniform ? g.n : (int64_t)g.cu[g.n_seqs];
+    if (lo < cov_lo || hi > cov_hi) {
+      for (int64_t t = lo + tid; t < hi; t += GAE_THREADS)
+        if (t < cov_lo || t >= cov_hi) { g.adv[t] = 0.f; g.ret[t] = 0.f; }
+    }
+  }
+
+  // owned sequences [s_first, s_last]: lo < end(s) <= hi
+  int s_first, s_last;
+  if (uniform) {
+    s_first = (int)(lo / g.uniform_len);
+    s_last = (int)(hi / g.uniform_len) - 1;
+  } else {
+    if (tid < 64) {
+      const int a = wave_count_le(g.cu + 1, g.n_seqs, lo, tid);
+      const int b = wave_count_le(g.cu + 1, g.n_seqs, hi, tid);
+      if (tid == 0) { s_own[0] = a; s_own[1] = b - 1; }
+    }
+    __syncthreads();
+    s_first = s_own[0];
+    s_last = s_own[1];
+  }
+  if (s_first > s_last) return;  // uniform for the block
+
+  const int n_own = s_last - s_first + 1;
+  const int32_t* cu_own = nullptr;  // cu_own[i] = cu[s_first + i], i in [0, n_own]
+  if (!uniform) {
+    if (n_own <= GAE_TILE + 1) {
+      for (int i = tid; i <= n_own; i += GAE_THREADS) s_cu[i] = g.cu[s_first + i];
+      __syncthreads();
+      cu_own = s_cu;
+    } else {
+      cu_own = g.cu + s_first;  // only with many empty sequences
+    }
+  }
+  const int64_t t_begin = uniform ? (int64_t)s_first * g.uniform_len : (int64_t)cu_own[0];
+  const int64_t t_end = uniform ? (int64_t)(s_last + 1) * g.uniform_len : (int64_t)cu_own[n_own];
+  if (t_end <= t_begin) return;
+
+  double A0 = 0.0, nv0 = 0.0;  // state entering the current tile from its right
+  for (int64_t tile = (t_end - 1) / GAE_TILE; tile >= t_begin / GAE_TILE; --tile) {
+    const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
+    // The thread keeps its 8 tokens as raw inputs plus two bit masks and rebuilds a token's map
+    // where it is needed (twice): holding 8 fp64 maps would halve the occupancy.
+    float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS], lm[GAE_ITEMS];
+    unsigned valid = 0, ends = 0, boot = 0;  // bit i: token owned / last of its sequence / no_eos
+    // owned tokens of this thread: local indices [i_lo, i_hi)
+    const int64_t d_lo = t_begin - t0, d_hi = t_end - t0;
+    const int i_lo = d_lo > 0 ? (d_lo < GAE_ITEMS ? (int)d_lo : GAE_ITEMS) : 0;
+    const int i_hi = d_hi < GAE_ITEMS ? (d_hi > 0 ? (int)d_hi : 0) : GAE_ITEMS;
+    const bool any = i_lo < i_hi;
+#pragma unroll
+    for (int i = 0; i < GAE_ITEMS; ++i) { rw[i] = 0.f; v[i] = 0.f; ms[i] = 0.f; lm[i] = g.lam; }
+    if (any) {
+      if (t0 + GAE_ITEMS <= g.n) {
+#pragma unroll
+        for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+          const f32x4 a = *(const f32x4*)(g.rewards + t0 + 4 * q);
+          const f32x4 b = *(const f32x4*)(g.values + t0 + 4 * q);
+          const f32x4 c = *(const f32x4*)(g.mask + t0 + 4 * q);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { rw[4 * q + e] = a[e]; v[4 * q + e] = b[e]; ms[4 * q + e] = c[e]; }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < GAE_ITEMS; ++i) {
+          const bool in = t0 + i < g.n;
+          rw[i] = in ? g.rewards[t0 + i] : 0.f;
+          v[i] = in ? g.values[t0 + i] : 0.f;
+          ms[i] = in ? g.mask[t0 + i] : 0.f;
+        }
+      }
+      // sequence of the first owned token of this thread (index relative to s_first)
+      const int64_t tf = t0 + i_lo;
+      int sq;
+      int e_loc;  // local index one past the last token of sequence sq (clamped)
+      if (uniform) {
+        sq = (int)(tf / g.uniform_len) - s_first;
+        const int64_t e = (int64_t)(sq + s_first + 1) * g.uniform_len - t0;
+        e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+      } else {
+        int a = 0, b = n_own;  // cu_own[a] <= tf < cu_own[b]
+        while (b - a > 1) {
+          const int mid = (a + b) >> 1;
+          if ((int64_t)cu_own[mid] <= tf) a = mid; else b = mid;
+        }
+        sq = a;
+        const int64_t e = (int64_t)cu_own[sq + 1] - t0;
+        e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+      }
+      valid = ((1u << i_hi) - 1u) & ~((1u << i_lo) - 1u);
+      if (e_loc > i_hi && g.lam_seq == nullptr) {
+        // common case: all owned tokens inside one sequence, none of them its last
+      } else {
+        // a sequence ends among these tokens (or lambda is per sequence): walk them
+        for (int i = i_lo; i < i_hi; ++i) {
+          while (i >= e_loc && sq + 1 < n_own) {
+            ++sq;
+            const int64_t e = (uniform ? (int64_t)(sq + s_first + 1) * g.uniform_len
+                                       : (int64_t)cu_own[sq + 1]) - t0;
+            e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+          }
+          if (g.lam_seq != nullptr) {
+            const float l = g.lam_seq[s_first + sq];
+#pragma unroll
+            for (int k = 0; k < GAE_ITEMS; ++k) if (k == i) lm[k] = l;
+          }
+          if (i == e_loc - 1) {
+            ends |= 1u << i;
+            if (g.no_eos != nullptr && g.no_eos[s_first + sq] != 0) boot |= 1u << i;
+          }
+        }
+      }
+    }
+    const double gam = (double)g.discount;
+    auto token_map = [&](int i) -> Map {
+      const double val = (double)v[i];
+      // not owned: identity (m = 0 with no offsets); last token of a sequence: constant map
+      const double m = ((valid >> i) & 1u) ? (double)ms[i] : 0.0;
+      const double c = gam * (double)lm[i];
+      Map f;
+      f.a11 = fma(c, m, 1.0 - m);
+      f.a12 = gam * m;
+      f.a22 = 1.0 - m;
+      f.b1 = ((double)rw[i] - val) * m;
+      f.b2 = val * m;
+      if ((ends >> i) & 1u) f = Map{0.0, 0.0, 0.0, 0.0, ((boot >> i) & 1u) ? val : 0.0};
+      return f;
+    };
+    Map mine = token_map(GAE_ITEMS - 1);
+#pragma unroll
+    for (int i = GAE_ITEMS - 2; i >= 0; --i) {
+      mine = compose(token_map(i), mine);
+      if (i & 1) __builtin_amdgcn_sched_barrier(0);  // two maps in flight, not eight
+    }
+    Map total;
+    const Map incl = block_suffix_scan(mine, smem, total);
+    all[tid] = incl;
+    __syncthreads();
+    const Map excl = tid + 1 < GAE_THREADS ? all[tid + 1] : map_identity();
+    double A = fma(excl.a11, A0, fma(excl.a12, nv0, excl.b1));
+    double nv = fma(excl.a22, nv0, excl.b2);
+    if (any) {
+      // opaque to the optimiser: otherwise it keeps the 8 maps of the first use alive
+#pragma unroll
+      for (int i = 0; i < GAE_ITEMS; ++i)
+        asm volatile("" : "+v"(rw[i]), "+v"(v[i]), "+v"(ms[i]), "+v"(lm[i]));
+      float oa[GAE_ITEMS], orr[GAE_ITEMS];
+#pragma unroll
+      for (int i = GAE_ITEMS - 1; i >= 0; --i) {
+        const Map f = token_map(i);
+        const double A2 = fma(f.a11, A, fma(f.a12, nv, f.b1));
+        const double nv2 = fma(f.a22, nv, f.b2);
+        A = A2; nv = nv2;
+        oa[i] = (float)A;
+        orr[i] = oa[i] + v[i];
+        if (i & 1) __builtin_amdgcn_sched_barrier(0);
+      }
+      if (valid == (1u << GAE_ITEMS) - 1u) {
+#pragma unroll
+        for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+          *(f32x4*)(g.adv + t0 + 4 * q) = f32x4{oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};
+          *(f32x4*)(g.ret + t0 + 4 * q) = f32x4{orr[4 * q], orr[4 * q + 1], orr[4 * q + 2], orr[4 * q + 3]};
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < GAE_ITEMS; ++i)
+          if ((valid >> i) & 1u) { g.adv[t0 + i] = oa[i]; g.ret[t0 + i] = orr[i]; }
+      }
+    }
+    // state entering the next tile on the left
+    const double A1 = fma(total.a11, A0, fma(total.a12, nv0, total.b1));
+    const double nv1 = fma(total.a22, nv0, total.b2);
+    A0 = A1; nv0 = nv1;
   }
 }
 
@@ -275,12 +506,13 @@ DEVI void split_range(const NormArgs& a, int g, int sp, int64_t& lo, int64_t& hi
   if (lo > g1) lo = g1;
 }
 
-// Sum of one partial array over all splits of group g (fixed order).
-DEVI double group_partial(const NormArgs& a, int which, int g) {
+// Sum of one partial array over all splits of group g, computed cooperatively by the block
+// (fixed order: the same tree whatever the launch).
+DEVI double group_partial(const NormArgs& a, int which, int g, double* smem) {
   double r = 0.0;
   const double* p = a.part + ((int64_t)which * a.G + g) * a.nsplit;
-  for (int i = 0; i < a.nsplit; ++i) r += p[i];
-  return r;
+  for (int i = threadIdx.x; i < a.nsplit; i += blockDim.x) r += p[i];
+  return block_sum_d(r, smem);
 }
 // Sum over every group and split, computed cooperatively by the block.
 DEVI double batch_partial(const NormArgs& a, int which, double* smem) {
@@ -309,8 +541,8 @@ DEVI MeanCtx make_mean_ctx(const NormArgs& a, int g, double* smem) {
   } else if (a.mean_level == LEVEL_GROUP) {
     if (g == a.tail_group) { c.zero = true; return c; }
     if (a.grows[g] == 1 && c.loo) { c.identity = true; return c; }
-    c.cnt = group_partial(a, 0, g);
-    c.sum = group_partial(a, 1, g);
+    c.cnt = group_partial(a, 0, g, smem);
+    c.sum = group_partial(a, 1, g, smem);
   } else {
     c.zero = true;
     return c;
@@ -409,8 +641,8 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_apply_kernel(NormArgs a) {
     if (g == a.tail_group) std_d = 0.0;
     else if (a.grows[g] == 1 && a.unbiased) std_d = 1.0;
     else {
-      const double cnt = group_partial(a, 0, g);
-      const double ss = group_partial(a, 2, g);
+      const double cnt = group_partial(a, 0, g, smem);
+      const double ss = group_partial(a, 2, g, smem);
       if (a.unbiased) std_d = cnt <= 1.0 ? 1.0 : sqrt(ss / (cnt - 1.0));
       else std_d = cnt == 0.0 ? 1.0 : sqrt(ss / cnt);
     }
@@ -509,7 +741,16 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
   Map* totals = (Map*)wp;
   double* carry = (double*)(wp + (size_t)nb * sizeof(Map));
   GaeArgs g{rewards, values, loss_mask, cu_seqlens, no_eos, lambda_seq, n_tokens, (int)n_seqs,
-            uniform_len, discount, gae_lambda, advantages, returns};
+            uniform_len, discount, gae_lambda, advantages, returns, 0};
+  // sequences of ordinary length: single pass, one launch. Very long sequences on average (few
+  // blocks would own any work): reduce-then-scan over all tokens.
+  if (n_tokens / n_seqs <= 64 * GAE_TILE) {
+    g.block_per_seq = uniform_len >= GAE_TILE;
+    const int64_t grid = g.block_per_seq ? n_seqs : ceil_div_i64(nb, 8) * 8;
+    hipLaunchKernelGGL(gae_owned_kernel, dim3((unsigned)grid), dim3(GAE_THREADS), 0, stream, g);
+    AREAL_CHECK_LAUNCH();
+    return AREAL_OK;
+  }
   hipLaunchKernelGGL(gae_block_total_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g,
                      totals);
   AREAL_CHECK_LAUNCH();
@@ -521,16 +762,19 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
   return AREAL_OK;
 }
 
-static int norm_nsplit(int64_t max_group_len) {
-  int64_t s = ceil_div_i64(max_group_len, 16384);
+// Blocks per group: about 4096 elements per block, and at most 2048 partials per array in all
+// (every block of the later passes sums them) unless there are more groups than that.
+static int norm_nsplit(int64_t n_groups, int64_t max_group_len) {
+  int64_t s = ceil_div_i64(max_group_len, 4096);
+  const int64_t cap = n_groups >= 2048 ? 1 : 2048 / n_groups;
+  if (s > cap) s = cap;
   if (s < 1) s = 1;
-  if (s > 512) s = 512;
   return (int)s;
 }
 
 size_t areal_group_norm_workspace_bytes(int64_t n_groups, int64_t max_group_len) {
   if (n_groups <= 0) return 0;
-  return (size_t)3 * n_groups * norm_nsplit(max_group_len) * sizeof(double) + 256;
+  return (size_t)3 * n_groups * norm_nsplit(n_groups, max_group_len) * sizeof(double) + 256;
 }
 
 // Normalization(x, mask, groups): levels 0 = none, 1 = batch, 2 = group.
@@ -553,7 +797,7 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
     return AREAL_ERR_WORKSPACE;
   NormArgs a;
   a.x = x; a.mask = mask; a.n = n; a.goff = group_offsets; a.grows = group_rows;
-  a.G = (int)n_groups; a.tail_group = tail_group; a.nsplit = norm_nsplit(max_group_len);
+  a.G = (int)n_groups; a.tail_group = tail_group; a.nsplit = norm_nsplit(n_groups, max_group_len);
   a.mean_level = mean_level; a.std_level = std_level; a.leave1out = leave_one_out;
   a.unbiased = unbiased; a.eps = eps;
   a.part = (double*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);

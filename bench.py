@@ -140,7 +140,7 @@ def hbm_rooflines(dev):
     r[cu[1:].long() - 2] = 1.0
     v = torch.randn(T, device=dev)
     m = (torch.rand(T, device=dev) > 0.25).float()
-    add("gae_block_total+gae_carry+gae_apply", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
+    add("gae_owned_kernel", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
         20 * T, timed(lambda: compute_gae_packed(r, v, m, cu, None, 1.0, 0.95)))
     # the padded drop-in signature on the same batch: [1024, 8192] (8.39 M slots)
     from areal_amd.ppo.gae import _compute_token_level_gae
@@ -151,7 +151,7 @@ def hbm_rooflines(dev):
     pos = torch.arange(8192, device=dev)[None, :]
     mp = ((pos >= (lens.to(dev) // 4)[:, None]) & (pos < (lens.to(dev) - 1)[:, None])).float()
     no_eos = torch.zeros(1024, dtype=torch.bool, device=dev)
-    add("gae_block_total+gae_carry+gae_apply", "config 3 padded form: [1024, 8192] slots, 20 B/slot",
+    add("gae_owned_kernel", "config 3 padded form: [1024, 8192] slots, 20 B/slot",
         20 * rp.numel(), timed(lambda: _compute_token_level_gae(rp, vp, mp, no_eos, 1.0, 0.95)))
     del rp, vp, mp
     x = torch.randn(1024, 1600, device=dev)

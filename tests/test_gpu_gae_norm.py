@@ -82,6 +82,48 @@ def test_gae_packed_matches_oracle_and_edge_cases(dev):
     assert a0.numel() == 0 and r0.numel() == 0
 
 
+@pytest.mark.parametrize("lens", [
+    [140_000],                                   # one very long sequence: the reduce-then-scan launches
+    [1] * 5000,                                  # one-token sequences: thousands of ends per tile
+    [0, 3, 0, 0, 2500, 0, 7, 0],                 # empty sequences between real ones
+    [5, 70_000, 1, 2049, 2047, 4096, 1, 30_000], # ends on and around tile edges, long next to short
+    [2048] * 9,                                  # every end exactly on a tile edge
+], ids=["one-long", "unit", "empty", "mixed", "tile-aligned"])
+def test_gae_packed_sequence_layouts(dev, lens):
+    g = torch.Generator().manual_seed(len(lens) * 13 + lens[0])
+    lens = torch.tensor(lens)
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    T = int(cu[-1])
+    r = torch.randn(T, generator=g) * (torch.rand(T, generator=g) > 0.8)
+    v = torch.randn(T, generator=g)
+    m = (torch.rand(T, generator=g) > 0.3).float()
+    ne = torch.rand(lens.numel(), generator=g) > 0.5
+    lam = torch.rand(lens.numel(), generator=g) * 0.2 + 0.8
+    for lam_arg in (0.95, lam):
+        want_a, want_r = G.gae_packed(r, v, m, cu, ne, 0.999, lam_arg)
+        a, rt = compute_gae_packed(r.to(dev), v.to(dev), m.to(dev), cu.to(dev), ne.to(dev), 0.999,
+                                   lam_arg.to(dev) if isinstance(lam_arg, torch.Tensor) else lam_arg)
+        scale = max(want_a.abs().max().item(), 1.0)
+        torch.testing.assert_close(a.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
+        torch.testing.assert_close(rt.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
+
+
+def test_gae_padded_long_rows(dev):
+    # rows longer than a tile, and far longer (takes the reduce-then-scan launches)
+    for bs, L in ((7, 8192), (2, 140_000)):
+        g = torch.Generator().manual_seed(L)
+        r = torch.randn(bs, L, generator=g) * (torch.rand(bs, L, generator=g) > 0.95)
+        v = torch.randn(bs, L, generator=g)
+        m = (torch.rand(bs, L, generator=g) > 0.1).float()
+        m[:, -1] = 0
+        ne = torch.tensor([i % 2 == 0 for i in range(bs)])
+        want_a, want_r = G.gae_padded(r, v, m, ne, 1.0, 0.95)
+        a, rt = _compute_token_level_gae(r.to(dev), v.to(dev), m.to(dev), ne.to(dev), 1.0, 0.95)
+        scale = max(want_a.abs().max().item(), 1.0)
+        torch.testing.assert_close(a.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
+        torch.testing.assert_close(rt.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
+
+
 def test_gae_sequences_are_independent(dev):
     """Changing one sequence must not change any other (the scan's reset maps)."""
     g = torch.Generator().manual_seed(3)
