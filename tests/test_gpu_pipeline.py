@@ -211,3 +211,163 @@ def test_config4_full_size_masks_bit_exact(dev):
         assert sg["n_valid_tokens"] == so["n_valid_tokens"]
         assert sg["filtered_fraction"] == so["filtered_fraction"]
         torch.testing.assert_close(lg.cpu(), lo, rtol=1e-4, atol=1e-8)
+
+
+# ---------------------------------------------------------------------------------------
+# Full-size forward + backward (BASELINE configs 2, 4, 5). The oracle cannot run [T, V] on
+# the CPU in seconds, so the gradients are checked three ways: the loss stage against the
+# oracle fed the GPU's log-probs (elementwise, any size); dHidden rows and dWeight rows of
+# sampled tokens / vocabulary ids against a plain fp32 PyTorch evaluation of the closed form
+# on the GPU (torch.matmul + logsumexp in token chunks: an independent implementation of
+# the same mathematics); and the size-independent identity sum_v dWeight[v, :] = 0 (every
+# token's dlogits sum to zero over the vocabulary).
+# ---------------------------------------------------------------------------------------
+def _make_lm_inputs(T, H, V, seed, dev):
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    for i in range(0, T, 16384):
+        n = min(16384, T - i)
+        hidden[i:i + n] = torch.randn(n, H, generator=g).bfloat16().to(dev)
+    weight = torch.empty(V, H, dtype=torch.bfloat16, device=dev)
+    for i in range(0, V, 32768):
+        n = min(32768, V - i)
+        weight[i:i + n] = (torch.randn(n, H, generator=g) * 0.02).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    return g, hidden, weight, labels
+
+
+def _torch_lse(hidden, wf, chunk=4096):
+    """logsumexp over the vocabulary of hidden @ weight.T in fp32 (wf = weight.float()), in
+    token chunks."""
+    out = torch.empty(hidden.shape[0], dtype=torch.float32, device=hidden.device)
+    for i in range(0, hidden.shape[0], chunk):
+        out[i:i + chunk] = torch.logsumexp(hidden[i:i + chunk].float() @ wf.T, dim=-1)
+    return out
+
+
+def _check_lm_gradients(hidden, weight, labels, dlogp, dh, dw, n_rows=96, n_cols=128):
+    """dh [T,H], dw [V,H] against the closed form on sampled rows / vocabulary ids."""
+    T, V = hidden.shape[0], weight.shape[0]
+    dev = hidden.device
+    wf = weight.float()
+    lse = _torch_lse(hidden, wf)
+    # dHidden[t] = g_t (W[label_t] - sum_v p_tv W[v]) on sampled tokens with g_t != 0
+    nz = dlogp.nonzero().flatten()
+    rows = nz[torch.linspace(0, nz.numel() - 1, n_rows).long()]
+    p = torch.exp(hidden[rows].float() @ wf.T - lse[rows, None])
+    p = (-p)
+    p[torch.arange(rows.numel(), device=dev), labels[rows]] += 1.0
+    dl = (p * dlogp[rows, None]).bfloat16().float()
+    dh_want = dl @ wf
+    rel = (dh[rows].float() - dh_want).norm() / dh_want.norm()
+    assert rel < 1e-2, f"dHidden rel err {rel}"
+    assert (dh[dlogp == 0] == 0).all()
+    # dWeight[v] = sum_t g_t (1[v = label_t] - p_tv) h_t on sampled vocabulary ids (half of them
+    # ids that occur as labels)
+    cols = torch.cat([labels[rows[: n_cols // 2]], torch.randint(0, V, (n_cols // 2,), device=dev)]).unique()
+    dw_want = torch.zeros(cols.numel(), hidden.shape[1], device=dev)
+    for i in range(0, T, 8192):
+        h = hidden[i:i + 8192]
+        pc = -torch.exp(h.float() @ wf[cols].T - lse[i:i + 8192, None])
+        pc += (labels[i:i + 8192, None] == cols[None, :]).float()
+        dlc = (pc * dlogp[i:i + 8192, None]).bfloat16().float()
+        dw_want += dlc.T @ h.float()
+    rel = (dw[cols].float() - dw_want).norm() / dw_want.norm()
+    assert rel < 1e-2, f"dWeight rel err {rel}"
+    # every token's dlogits sum to zero over the vocabulary
+    colsum = dw.float().sum(dim=0)
+    scale = dw.float().abs().sum(dim=0)
+    assert (colsum.abs() <= 2e-2 * scale + 1e-6).all()
+
+
+def _segments(T, n_seqs, g):
+    cuts = torch.sort(torch.randperm(T - 1, generator=g)[: n_seqs - 1] + 1).values
+    return torch.cat([torch.zeros(1, dtype=torch.long), cuts, torch.tensor([T])]).to(torch.int32)
+
+
+@pytest.mark.parametrize("save_probs", [True, False], ids=["saved", "recompute"])
+def test_config4_full_size_forward_backward(dev, save_probs):
+    T, H, V = 32768, 4096, 151936
+    g, hidden, weight, labels = _make_lm_inputs(T, H, V, 3, dev)
+    h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels, save_probs=save_probs)
+    lp = out.logprobs.detach()
+    torch.manual_seed(3)
+    old = lp + torch.distributions.Laplace(0.0, 0.1).sample((T,)).to(dev)
+    adv = torch.randn(T, generator=g).to(dev)
+    mask = (torch.rand(T, generator=g) > 0.1).to(dev)
+    rs = dict(level="token", action="mask", metric="ratio", lower=0.5, upper=2.0)
+    loss, stat = ppo_actor_loss_fn(out.logprobs, lp, old, adv, 0.2, mask,
+                                   rejection_sampling=RejectionSamplingConfig(**rs))
+    lp_cpu = lp.cpu().requires_grad_(True)
+    lo, so = O.ppo_actor_loss(lp_cpu, lp.cpu(), old.cpu(), adv.cpu(), 0.2, mask.cpu(), rejection_sampling_cfg=rs)
+    lo.backward()
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-8)
+    loss.backward()
+    _check_lm_gradients(hidden, weight, labels, lp_cpu.grad.to(dev), h.grad, w.grad)
+
+
+def test_config2_full_size_decoupled_ppo(dev):
+    """T=16384, H=1536, 64 sequences; proximal and behaviour log-probs drawn independently."""
+    T, H, V = 16384, 1536, 151936
+    g, hidden, weight, labels = _make_lm_inputs(T, H, V, 1, dev)
+    h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels)
+    lp = out.logprobs.detach()
+    prox = lp + 0.1 * torch.randn(T, generator=g).to(dev)
+    old = lp + 0.1 * torch.randn(T, generator=g).to(dev)
+    adv = torch.randn(T, generator=g).to(dev)
+    mask = (torch.rand(T, generator=g) > 0.2).to(dev)
+    rs = dict(level="token", action="clamp", metric="ratio", upper=5.0, lower=0.0)
+    cfg = RejectionSamplingConfig(level="token", action="clamp", metric="ratio", upper=5.0)  # lower -> 0.0
+    loss, stat = ppo_actor_loss_fn(out.logprobs, prox, old, adv, 0.2, mask, eps_clip_higher=0.28, c_clip=3.0,
+                                   rejection_sampling=cfg)
+    lp_cpu = lp.cpu().requires_grad_(True)
+    lo, so = O.ppo_actor_loss(lp_cpu, prox.cpu(), old.cpu(), adv.cpu(), 0.2, mask.cpu(), eps_clip_higher=0.28,
+                              c_clip=3.0, rejection_sampling_cfg=rs)
+    lo.backward()
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-8)
+    torch.testing.assert_close(stat["behave_imp_weight"].cpu(), so["behave_imp_weight"], rtol=1e-6, atol=0)
+    loss.backward()
+    _check_lm_gradients(hidden, weight, labels, lp_cpu.grad.to(dev), h.grad, w.grad)
+
+
+def test_config5_full_size_cispo_sequence_rejection(dev):
+    """T=131072, H=5120: CISPO (eps 1.0 / 4.0) with sequence-level mean-ratio rejection (upper
+    5.0) over 4 x 32 packed sequences. The bf16 [T, V] buffer would be 39.8 GB, above the
+    default limit, so the backward recomputes the logits in token chunks; peak memory of the
+    step stays under 64 GB."""
+    from areal_amd.functional import cispo_loss_fn
+
+    T, H, V = 131072, 5120, 151936
+    g, hidden, weight, labels = _make_lm_inputs(T, H, V, 4, dev)
+    cu = _segments(T, 128, g)
+    h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    out = fused_lm_head_logprobs_entropy(h, w, labels)
+    assert out.logprobs.grad_fn.probs is None  # recompute mode was chosen
+    lp = out.logprobs.detach()
+    prox = lp + 0.2 * torch.randn(T, generator=g).to(dev)
+    # a few sequences far off-policy so that the sequence filter rejects some
+    seq_shift = (torch.rand(128, generator=g) < 0.1).float() * 2.0
+    lens = (cu[1:] - cu[:-1]).long()
+    old = prox - torch.repeat_interleave(seq_shift, lens).to(dev) + 0.05 * torch.randn(T, generator=g).to(dev)
+    adv = torch.randn(T, generator=g).to(dev)
+    mask = (torch.rand(T, generator=g) > 0.2).to(dev)
+    rs = dict(level="sequence", action="mask", metric="ratio", agg="mean", upper=5.0)
+    loss, stat = cispo_loss_fn(out.logprobs, prox, adv, 1.0, mask, eps_clip_higher=4.0, old_logprobs=old,
+                               rejection_sampling=RejectionSamplingConfig(**rs), cu_seqlens=cu.to(dev))
+    loss.backward()
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - base
+    assert peak < 64e9, f"peak step memory {peak / 1e9:.1f} GB"
+    lp_cpu = lp.cpu().requires_grad_(True)
+    lo, so = O.cispo_loss(lp_cpu, prox.cpu(), adv.cpu(), 1.0, mask.cpu(), eps_clip_higher=4.0,
+                          old_logprobs=old.cpu(), rejection_sampling_cfg=rs, cu_seqlens=cu)
+    lo.backward()
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-8)
+    assert torch.equal(stat["behave_mask"].cpu(), so["behave_mask"])
+    assert 0.0 < stat["filtered_fraction"] < 0.5
+    _check_lm_gradients(hidden, weight, labels, lp_cpu.grad.to(dev), h.grad, w.grad)
