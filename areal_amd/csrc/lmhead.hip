@@ -966,9 +966,13 @@ __global__ void cast_f32_to_bf16_kernel(const float* __restrict__ src, u16* __re
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// Splits of the A range per B tile: enough workgroups to fill the chip, and at least 4 so that
+// the 32 workgroups sharing an XCD's L2 form an 8 x 4 block (12 distinct operand tiles per sweep
+// step) rather than 32 x 1 (33 tiles: with many B tiles that re-reads every B tile from HBM for
+// every A tile).
 int pick_splits(int nbj, int nai, int target_wgs) {
   int S = 1;
-  while (nbj * S < target_wgs && S * 2 <= nai && S < 64) S *= 2;
+  while ((nbj * S < target_wgs || S < 4) && S * 2 <= nai && S < 64) S *= 2;
   return S;
 }
 
@@ -1139,13 +1143,16 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   return AREAL_OK;
 }
 
-// Backward workspace: W^T [H, ldv] + per token chunk: hidden^T [H, ldt], dl [Tc, ldv],
-// dlT [V, ldt], all bf16.
+// Backward workspace (bf16): W^T [H, ldv] + dl [Tc, ldv] per token chunk; chunks that are not a
+// multiple of 64 tokens also need hidden^T [H, ldt] and dlT [V, ldt] (token_chunk a multiple of
+// 64 and T a multiple of 64 avoid them).
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk) {
   if (T <= 0 || H <= 0 || V <= 0 || token_chunk <= 0) return 0;
   const int64_t Tc = token_chunk < T ? token_chunk : T;
   const int64_t ldv = round_up_i64(V, BK), ldt = round_up_i64(Tc, BK);
-  int64_t elems = H * ldv + H * ldt + Tc * ldv + V * ldt;
+  int64_t elems = H * ldv + Tc * ldv;
+  const bool ragged = (Tc % BK != 0) || (T % Tc) % BK != 0;  // some chunk is not a multiple of 64
+  if (ragged) elems += H * ldt + V * ldt;
   return (size_t)elems * 2 + 4 * 256;  // slack for 256-byte sub-buffer alignment
 }
 
@@ -1180,10 +1187,11 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     return (u16*)r;
   };
   char* wp = (char*)workspace;
+  const bool ragged = (Tc_max % BK != 0) || (T % Tc_max) % BK != 0;
   u16* wT = carve(wp, H * ldv * 2);
-  u16* hT = carve(wp, H * ldt * 2);
   u16* dl = carve(wp, Tc_max * ldv * 2);
-  u16* dlT = carve(wp, V * ldt * 2);
+  u16* hT = ragged ? carve(wp, H * ldt * 2) : nullptr;
+  u16* dlT = ragged ? carve(wp, V * ldt * 2) : nullptr;
 
   const float c2 = inv_temperature * LOG2E;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);

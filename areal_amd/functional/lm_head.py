@@ -33,7 +33,7 @@ from areal_amd import _lib
 DEFAULT_BWD_WORKSPACE_BYTES = 24 << 30
 
 # save_probs=None keeps the exponentials when the bf16 [T, V] buffer is at most this large.
-SAVE_PROBS_BYTES_LIMIT = 24 << 30
+SAVE_PROBS_BYTES_LIMIT = 40 << 30
 
 
 def _round_up(x: int, m: int) -> int:
@@ -55,9 +55,12 @@ class ChunkedLMHeadOutput(NamedTuple):
 
 
 def default_token_chunk(T: int, H: int, V: int, budget: int = DEFAULT_BWD_WORKSPACE_BYTES) -> int:
-    """Largest token chunk (multiple of 256) whose backward workspace fits ``budget``."""
-    per_token = 2 * (2 * V + H) + 64
-    fixed = 2 * H * (V + 8)
+    """Largest token chunk (multiple of 256) whose backward workspace fits ``budget``: bf16
+    dlogits of the chunk plus the transposed weight (and, when ``T`` is not a multiple of 64,
+    transposed copies of the last chunk's hidden states and dlogits)."""
+    ragged = T % 64 != 0
+    per_token = 2 * V + 64 + (2 * (V + H) if ragged else 0)
+    fixed = 2 * H * (V + 64)
     chunk = max((budget - fixed) // per_token, 256)
     chunk = (chunk // 256) * 256
     return int(min(max(chunk, 256), max(T, 1)))

@@ -29,6 +29,9 @@ WORKLOADS = {
                      desc="BASELINE config 4: Qwen3-8B shape fwd+bwd, IcePop ratio bounds [0.5, 2.0]"),
     "qwen2.5-1.5b": dict(T=16384, H=1536, n_seqs=64, lo=32, hi=2048, seed=1,
                          desc="BASELINE config 2: Qwen2.5-1.5B shape fwd+bwd, decoupled PPO"),
+    "qwen3-14b-128k": dict(T=131072, H=5120, n_seqs=4, lo=32768, hi=32768, seed=4,
+                           desc="BASELINE config 5 shape: 4 x 32768 tokens, H=5120, fwd+bwd (39.8 GB of bf16 "
+                                "exponentials kept for the backward)"),
     "qwen2.5-0.5b": dict(T=4096, H=896, n_seqs=16, lo=64, hi=512, seed=0,
                          desc="BASELINE config 1 shape (run fwd+bwd here)"),
 }
