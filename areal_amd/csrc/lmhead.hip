@@ -1264,19 +1264,21 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref): no logits are
 // recomputed. probs is overwritten with the bf16 dlogits, so it can be used once. logprobs
 // (nullable) are the label log-probabilities of the forward; with them the label's entry of
-// dlogits is evaluated in fp32.
+// dlogits is evaluated in fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32
+// accumulate, 2 = bf16 store (the whole batch is one contraction, so no fp32 staging is needed).
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
-                           const float* probs_ref, void* dhidden, float* dweight_f32,
-                           int accumulate, void* workspace, size_t workspace_bytes,
+                           const float* probs_ref, void* dhidden, void* dweight,
+                           int dweight_mode, void* workspace, size_t workspace_bytes,
                            hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0) return AREAL_ERR_BAD_ARG;
   if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr ||
       probs == nullptr || probs_ref == nullptr)
     return AREAL_ERR_BAD_ARG;
-  if (dhidden == nullptr && dweight_f32 == nullptr) return AREAL_ERR_BAD_ARG;
+  if (dhidden == nullptr && dweight == nullptr) return AREAL_ERR_BAD_ARG;
+  if (dweight_mode < 0 || dweight_mode > 2) return AREAL_ERR_BAD_ARG;
   if (T == 0) return AREAL_OK;
   if (T > (1 << 30) || V > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
   int rc;
@@ -1284,7 +1286,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   if ((rc = check_operand(weight, H)) != AREAL_OK) return rc;
   if (!aligned16(probs)) return AREAL_ERR_ALIGNMENT;
   if (dhidden != nullptr && !aligned16(dhidden)) return AREAL_ERR_ALIGNMENT;
-  if (dweight_f32 != nullptr && !aligned16(dweight_f32)) return AREAL_ERR_ALIGNMENT;
+  if (dweight != nullptr && !aligned16(dweight)) return AREAL_ERR_ALIGNMENT;
   if (dhidden != nullptr &&
       (workspace == nullptr || workspace_bytes < areal_lmhead_bwd_saved_workspace_bytes(T, H, V)))
     return AREAL_ERR_WORKSPACE;
@@ -1307,13 +1309,14 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
     if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
   }
-  if (dweight_f32 != nullptr) {
+  if (dweight != nullptr) {
     // dWeight[v, h] += sum_t dl[t, v] * hidden[t, h], k-major over the Tpad rows of dl
     GemmArgs g{(const u16*)hidden, H, (int)H, dl, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
-    const StoreParams ep{dweight_f32, H, (int)H, (int)V};
+    const StoreParams ep{dweight, H, (int)H, (int)V};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
-    rc = accumulate ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
-                    : launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
+    rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
+         : dweight_mode == 0 ? launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
+                             : launch_gemm<StoreBf16, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
     if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;

@@ -134,8 +134,12 @@ class _FusedLMHead(torch.autograd.Function):
         V = weight_c.size(0)
         g = grad_logprobs.reshape(-1).to(torch.float32).contiguous()
         dh = torch.empty_like(hidden_2d) if need_h else None
-        dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if need_w else None
         probs, probs_ref = ctx.probs, ctx.probs_ref
+        # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
+        # the chunked recompute mode accumulates in fp32 and casts at the end
+        direct = probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
+        dw_direct = torch.empty((V, H), dtype=torch.bfloat16, device=dev) if (need_w and direct) else None
+        dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if (need_w and not direct) else None
         ctx.probs = ctx.probs_ref = None  # consumed; a second backward recomputes the logits
         if T == 0:
             if dw32 is not None:
@@ -148,7 +152,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
                 _lib.ptr(probs), _lib.ptr(probs_ref),
-                _lib.ptr(dh), _lib.ptr(dw32), 0,
+                _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32), 2 if direct else 0,
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd_saved")
@@ -165,7 +169,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd")
-        dw = None
+        dw = dw_direct
         if dw32 is not None:
             if ctx.weight_dtype == torch.float32:
                 dw = dw32

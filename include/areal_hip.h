@@ -76,14 +76,15 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * recomputed (vocab_parallel_head.py:806-829 recomputes them chunk by chunk to save memory; an
  * MI355X has the HBM to keep them). probs is overwritten with the bf16 dlogits and can be
  * used once. logprobs (NULL allowed) are the forward's label log-probabilities: with them the
- * label's dlogit is -expm1(logprob) in fp32. Other arguments as areal_lmhead_bwd; bias does
- * not enter (it is part of the saved exponentials). workspace may be NULL if dhidden is. */
+ * label's dlogit is -expm1(logprob) in fp32. dweight [V,H]: dweight_mode 0 = fp32 store,
+ * 1 = fp32 accumulate, 2 = bf16 store. Other arguments as areal_lmhead_bwd; bias does not enter
+ * (it is part of the saved exponentials). workspace may be NULL if dhidden is. */
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
-                           const float* probs_ref, void* dhidden, float* dweight_f32,
-                           int accumulate, void* workspace, size_t workspace_bytes,
+                           const float* probs_ref, void* dhidden, void* dweight,
+                           int dweight_mode, void* workspace, size_t workspace_bytes,
                            areal_stream_t stream);
 
 /* out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]  (bf16 in, fp32 accumulate).
