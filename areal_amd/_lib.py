@@ -60,6 +60,14 @@ SIGNATURES: dict[str, tuple] = {
         [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
     "areal_actor_loss_grad": (I, [P, P, P, P, I64, P]),
+    "areal_aux_loss_workspace_bytes": (SZ, [I64, I64]),
+    "areal_sapo_loss": (
+        I,
+        [P, P, P, P, P, I64, I64, I64, F, F, I, P, P, P, P, P, P, P, P, P, P, SZ, P],
+    ),
+    "areal_critic_loss": (I, [P, P, P, P, I64, F, I, P, P, P, P, P, P, SZ, P]),
+    "areal_dpo_seq_logps": (I, [P, P, P, P, I64, I64, P, P, P]),
+    "areal_dpo_seq_logps_grad": (I, [P, P, P, I64, I64, P, P]),
     "areal_gae_workspace_bytes": (SZ, [I64]),
     "areal_gae_packed": (
         I,

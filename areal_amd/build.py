@@ -30,7 +30,7 @@ HIPCC_FLAGS = [
 # Elementwise kernels whose boolean outputs are compared bit-for-bit with a CPU evaluation of
 # the same formulas are compiled without floating-point contraction, so a*b+c rounds twice as
 # it does in the reference's separate tensor ops.
-NO_CONTRACT = {"ppo_loss.hip", "gae_norm.hip"}
+NO_CONTRACT = {"ppo_loss.hip", "gae_norm.hip", "aux_loss.hip"}
 
 
 def _hipcc() -> str:

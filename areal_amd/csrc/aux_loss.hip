@@ -1,0 +1,389 @@
+// Losses that share the actor loss's data layout: SAPO soft-gate policy loss, the clipped PPO
+// critic loss, and the per-sequence log-probability sums of DPO.
+//
+// Follows areal/utils/functional/functional.py: sapo_loss_fn (:599-675) with
+// _compute_sequence_level_ratio_and_advantages (:56-149), ppo_critic_loss_fn (:869-933) with
+// _huber_loss / _mse_loss (:859-866), dpo_pair_logratios (:796-841).
+//
+// fp32 per-token arithmetic in the order of the reference's tensor expressions (compiled with
+// -ffp-contract=off); sums are fp64 block partials reduced in a fixed order. Forward and the
+// closed-form gradient come out of the same pass.
+#include "common.hpp"
+
+namespace {
+
+constexpr int AUX_THREADS = 256;
+constexpr int AUX_MAX_BLOCKS = 1024;
+
+template <typename T>
+DEVI T block_sum(T v, T* smem) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[w] = v;
+  __syncthreads();
+  T r = 0;
+  const int nw = (blockDim.x + 63) >> 6;
+  for (int i = 0; i < nw; ++i) r += smem[i];
+  return r;
+}
+
+int aux_grid(int64_t n) {
+  int64_t b = ceil_div_i64(n, AUX_THREADS);
+  if (b > AUX_MAX_BLOCKS) b = AUX_MAX_BLOCKS;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+struct SeqLayout {
+  const int32_t* cu;    // [n_seqs + 1] or null
+  int n_seqs;
+  int64_t uniform_len;  // > 0: sequence s covers [s*uniform_len, (s+1)*uniform_len)
+};
+DEVI int seq_of(const SeqLayout& q, int64_t t) {
+  if (q.uniform_len > 0) return (int)(t / q.uniform_len);
+  int lo = 0, hi = q.n_seqs;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)q.cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+DEVI void seq_range(const SeqLayout& q, int s, int64_t n, int64_t& t0, int64_t& t1) {
+  if (q.uniform_len > 0) { t0 = (int64_t)s * q.uniform_len; t1 = t0 + q.uniform_len; }
+  else { t0 = q.cu[s]; t1 = q.cu[s + 1]; }
+  if (t1 > n) t1 = n;
+}
+
+struct SumCount {
+  double sum;
+  long long n_valid, n_clip;
+};
+
+// counters: [0] loss sum [1] masked-token count [4] clipped count [7] loss; the layout of the
+// actor loss, so that its gradient-scaling entry point serves these losses too.
+// denom_mode 0: sum / max(count, 1); 1: sum / count (0/0 = NaN, as torch); 2: sum / n_total.
+__global__ void aux_finalize_kernel(const SumCount* parts, int nparts, int denom_mode,
+                                    double n_total, float* loss_out, double* counters) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double s = 0.0;
+  long long nv = 0, nc = 0;
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    s += parts[i].sum; nv += parts[i].n_valid; nc += parts[i].n_clip;
+  }
+  s = block_sum(s, sm_d);
+  nv = block_sum(nv, sm_l);
+  nc = block_sum(nc, sm_l);
+  if (threadIdx.x == 0) {
+    for (int k = 0; k < 8; ++k) counters[k] = 0.0;
+    counters[0] = s;
+    float loss;
+    if (denom_mode == 0) {
+      counters[1] = (double)nv;
+      loss = (float)s / (float)(nv > 0 ? nv : 1);
+    } else if (denom_mode == 1) {
+      // the gradient scaling divides by max(counters[1], 1): an empty mask gives NaN loss and
+      // zero gradient times NaN upstream, as 0/0 does in the reference
+      counters[1] = (double)nv;
+      loss = (float)s / (float)nv;
+    } else {
+      counters[1] = n_total;
+      loss = (float)s / (float)n_total;
+    }
+    counters[4] = (double)nc;
+    counters[7] = (double)loss;
+    if (loss_out) *loss_out = loss;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// SAPO
+// ---------------------------------------------------------------------------------------
+struct SapoIO {
+  const float* lp;
+  const float* old;
+  const float* adv;
+  const uint8_t* mask;
+  SeqLayout seq;
+  int64_t n;
+  float tau_pos, tau_neg;
+  int seq_level;
+  const float* seq_stat;  // [n_seqs][3]: ratio_s, mean advantage, count
+  float* dlp;
+  float* stat_loss;
+  float* stat_ratio;
+  float* stat_kl;
+  float* soft_gate;
+  float* gate_pos;
+  float* gate_neg;
+};
+
+// Per-sequence geometric-mean ratio and mean advantage over the mask (one block per sequence).
+__global__ __launch_bounds__(AUX_THREADS) void sapo_seq_kernel(SapoIO io, float* seq_stat) {
+  __shared__ double sm_d[8];
+  const int s = blockIdx.x;
+  int64_t t0, t1;
+  seq_range(io.seq, s, io.n, t0, t1);
+  double sum_lr = 0.0, sum_adv = 0.0, cnt = 0.0;
+  for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
+    if (io.mask[t] == 0) continue;
+    cnt += 1.0;
+    sum_lr += (double)(io.lp[t] - io.old[t]);
+    sum_adv += (double)io.adv[t];
+  }
+  sum_lr = block_sum(sum_lr, sm_d);
+  sum_adv = block_sum(sum_adv, sm_d);
+  cnt = block_sum(cnt, sm_d);
+  if (threadIdx.x == 0) {
+    const float denom = (float)(cnt > 0.0 ? cnt : 1.0);
+    seq_stat[3 * s + 0] = expf((float)sum_lr / denom);
+    seq_stat[3 * s + 1] = (float)sum_adv / denom;
+    seq_stat[3 * s + 2] = (float)cnt;
+  }
+}
+
+DEVI float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__global__ __launch_bounds__(AUX_THREADS) void sapo_token_kernel(SapoIO io, SumCount* parts) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double loss_sum = 0.0;
+  long long n_valid = 0;
+  const float scale_pos = 4.0f / io.tau_pos, scale_neg = 4.0f / io.tau_neg;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < io.n;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const bool m = io.mask[t] != 0;
+    const float kl = io.lp[t] - io.old[t];
+    float ratio, a, dscale;  // d ratio / d lp[t] = ratio * dscale (summed over the sequence)
+    if (io.seq_level) {
+      const int s = seq_of(io.seq, t);
+      ratio = m ? io.seq_stat[3 * s] : 0.0f;
+      a = m ? io.seq_stat[3 * s + 1] : 0.0f;
+      // every masked token of the sequence carries the same term; the sum over them of
+      // d ratio_s / d lp[t] = ratio_s / count is ratio_s
+      dscale = 1.0f;
+    } else {
+      ratio = expf(kl);
+      a = io.adv[t];
+      dscale = 1.0f;
+    }
+    const float gp = sigmoidf(io.tau_pos * (ratio - 1.0f));
+    const float gn = sigmoidf(io.tau_neg * (ratio - 1.0f));
+    const float sp = gp * scale_pos, sn = gn * scale_neg;
+    const bool pos = a > 0.0f;
+    const float gate = pos ? sp : sn;
+    const float pg = (-gate) * a;
+    // d gate / d ratio = scale * tau * g (1 - g) = 4 g (1 - g)
+    const float g = pos ? gp : gn;
+    const float dgate = 4.0f * g * (1.0f - g);
+    const float d = m ? ((-dgate) * a) * (ratio * dscale) : 0.0f;
+    if (m) { loss_sum += (double)pg; n_valid += 1; }
+    if (io.dlp) io.dlp[t] = d;
+    if (io.stat_loss) io.stat_loss[t] = pg;
+    if (io.stat_ratio) io.stat_ratio[t] = ratio;
+    if (io.stat_kl) io.stat_kl[t] = kl;
+    if (io.soft_gate) io.soft_gate[t] = gate;
+    if (io.gate_pos) io.gate_pos[t] = sp;
+    if (io.gate_neg) io.gate_neg[t] = sn;
+  }
+  loss_sum = block_sum(loss_sum, sm_d);
+  n_valid = block_sum(n_valid, sm_l);
+  if (threadIdx.x == 0) parts[blockIdx.x] = SumCount{loss_sum, n_valid, 0};
+}
+
+// ---------------------------------------------------------------------------------------
+// Critic loss
+// ---------------------------------------------------------------------------------------
+DEVI float value_loss(float x, float y, int huber, float& dx) {
+  if (huber) {
+    const float delta = 10.0f;
+    const float diff = fabsf(x - y);
+    if (diff < delta) { dx = x - y; return (0.5f * diff) * diff; }
+    dx = (x > y ? delta : (x < y ? -delta : 0.0f));
+    return delta * (diff - 0.5f * delta);
+  }
+  const float e = x - y;
+  dx = e;
+  return (0.5f * e) * e;
+}
+
+__global__ __launch_bounds__(AUX_THREADS) void critic_token_kernel(
+    const float* value, const float* old_value, const float* target, const uint8_t* mask, int64_t n,
+    float eps, int huber, float* dvalue, float* stat_loss, uint8_t* clip_mask, SumCount* parts) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double loss_sum = 0.0;
+  long long n_valid = 0, n_clip = 0;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const bool m = mask ? mask[t] != 0 : true;
+    const float v = value[t], ov = old_value[t], tg = target[t];
+    float d_orig, d_clip;
+    const float l_orig = value_loss(v, tg, huber, d_orig);
+    const float dv = v - ov;
+    const float dc = dv != dv ? dv : (dv < -eps ? -eps : (dv > eps ? eps : dv));
+    const float vc = ov + dc;
+    const float l_clip = value_loss(vc, tg, huber, d_clip);
+    // clamp passes the gradient inside the closed band; torch.max splits ties evenly
+    const float pass = (dv >= -eps && dv <= eps) ? 1.0f : 0.0f;
+    const float w_orig = l_orig > l_clip ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
+    const float w_clip = l_clip > l_orig ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
+    const float l = (l_orig != l_orig || l_clip != l_clip) ? __builtin_nanf("")
+                                                             : (l_orig > l_clip ? l_orig : l_clip);
+    const bool clip = (l_clip > l_orig) && m;
+    if (m) { loss_sum += (double)l; n_valid += 1; }
+    n_clip += clip;
+    if (dvalue) dvalue[t] = m ? (w_orig * d_orig + w_clip * (d_clip * pass)) : 0.0f;
+    if (stat_loss) stat_loss[t] = l;
+    if (clip_mask) clip_mask[t] = clip;
+  }
+  loss_sum = block_sum(loss_sum, sm_d);
+  n_valid = block_sum(n_valid, sm_l);
+  n_clip = block_sum(n_clip, sm_l);
+  if (threadIdx.x == 0) parts[blockIdx.x] = SumCount{loss_sum, n_valid, n_clip};
+}
+
+// ---------------------------------------------------------------------------------------
+// DPO: per-sequence sums of the shifted-mask log-probabilities (fp64), one block per sequence.
+// shifted_mask[t] = loss_mask[t + 1] (0 at the very end), and 0 at the last token of every
+// non-empty sequence. out[s] = {sum policy, sum reference, count}.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AUX_THREADS) void dpo_seq_kernel(const float* lp, const float* ref,
+                                                              const uint8_t* mask, SeqLayout seq,
+                                                              int64_t n, double* out,
+                                                              uint8_t* shifted_mask) {
+  __shared__ double sm_d[8];
+  const int s = blockIdx.x;
+  int64_t t0, t1;
+  seq_range(seq, s, n, t0, t1);
+  double sp = 0.0, sr = 0.0, cnt = 0.0;
+  for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
+    const bool m = (t + 1 < t1) && (mask[t + 1] != 0);
+    if (shifted_mask) shifted_mask[t] = m;
+    if (!m) continue;
+    // the reference multiplies in the log-probs' dtype and then widens
+    sp += (double)(lp[t] * 1.0f);
+    sr += (double)(ref[t] * 1.0f);
+    cnt += 1.0;
+  }
+  sp = block_sum(sp, sm_d);
+  sr = block_sum(sr, sm_d);
+  cnt = block_sum(cnt, sm_d);
+  if (threadIdx.x == 0) { out[3 * s] = sp; out[3 * s + 1] = sr; out[3 * s + 2] = cnt; }
+}
+
+// grad_lp[t] = shifted_mask[t] * grad_seq[seq(t)]  (fp64 upstream, fp32 out)
+__global__ __launch_bounds__(AUX_THREADS) void dpo_seq_grad_kernel(const double* grad_seq,
+                                                                   const uint8_t* shifted_mask,
+                                                                   SeqLayout seq, int64_t n,
+                                                                   float* grad_lp) {
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
+       t += (int64_t)gridDim.x * blockDim.x)
+    grad_lp[t] = shifted_mask[t] ? (float)grad_seq[seq_of(seq, t)] : 0.0f;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t areal_aux_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
+  (void)n_tokens;
+  if (n_seqs < 0) n_seqs = 0;
+  return (size_t)AUX_MAX_BLOCKS * sizeof(SumCount) + (size_t)n_seqs * 3 * sizeof(float) + 256;
+}
+
+// SAPO policy loss: forward, closed-form d(loss sum)/d logprobs (to be scaled with
+// areal_actor_loss_grad), per-token statistics. seq_level != 0 uses the geometric-mean ratio
+// and the mean advantage of each sequence (cu_seqlens or uniform_len).
+int areal_sapo_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
+                    const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
+                    int64_t n_seqs, int64_t uniform_len, float tau_pos, float tau_neg,
+                    int seq_level, float* loss, float* dlogprobs, float* stat_loss,
+                    float* stat_ratio, float* stat_approx_kl, float* soft_gate, float* gate_pos,
+                    float* gate_neg, double* counters, void* workspace, size_t workspace_bytes,
+                    hipStream_t stream) {
+  if (n_tokens < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
+  if (!(tau_pos > 0.f) || !(tau_neg > 0.f)) return AREAL_ERR_BAD_ARG;
+  if (n_tokens > 0 && (!logprobs || !old_logprobs || !advantages || !loss_mask))
+    return AREAL_ERR_BAD_ARG;
+  if (seq_level && n_tokens > 0 && (n_seqs <= 0 || (uniform_len <= 0 && cu_seqlens == nullptr)))
+    return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_aux_loss_workspace_bytes(n_tokens, n_seqs))
+    return AREAL_ERR_WORKSPACE;
+  char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  SumCount* parts = (SumCount*)wp;
+  float* seq_stat = (float*)(wp + (size_t)AUX_MAX_BLOCKS * sizeof(SumCount));
+  SapoIO io{logprobs, old_logprobs, advantages, loss_mask,
+            SeqLayout{cu_seqlens, (int)n_seqs, uniform_len}, n_tokens, tau_pos, tau_neg,
+            seq_level, seq_stat, dlogprobs, stat_loss, stat_ratio, stat_approx_kl, soft_gate,
+            gate_pos, gate_neg};
+  const int grid = aux_grid(n_tokens);
+  if (seq_level && n_tokens > 0) {
+    hipLaunchKernelGGL(sapo_seq_kernel, dim3((unsigned)n_seqs), dim3(AUX_THREADS), 0, stream, io,
+                       seq_stat);
+    AREAL_CHECK_LAUNCH();
+  }
+  hipLaunchKernelGGL(sapo_token_kernel, dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid, 0,
+                     0.0, loss, counters);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// Clipped PPO critic loss (mse or huber with delta 10). loss_mask may be null (plain mean).
+int areal_critic_loss(const float* value, const float* old_value, const float* target_value,
+                      const uint8_t* loss_mask, int64_t n, float value_eps_clip, int huber,
+                      float* loss, float* dvalue, float* stat_loss, uint8_t* clip_mask,
+                      double* counters, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
+  if (n < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
+  if (n > 0 && (!value || !old_value || !target_value)) return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_aux_loss_workspace_bytes(n, 0))
+    return AREAL_ERR_WORKSPACE;
+  SumCount* parts = (SumCount*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  const int grid = aux_grid(n);
+  hipLaunchKernelGGL(critic_token_kernel, dim3(grid), dim3(AUX_THREADS), 0, stream, value,
+                     old_value, target_value, loss_mask, n, value_eps_clip, huber, dvalue,
+                     stat_loss, clip_mask, parts);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid,
+                     loss_mask ? 1 : 2, (double)n, loss, counters);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// DPO: seq_sums [n_seqs][3] fp64 = {sum of policy log-probs, sum of reference log-probs,
+// token count} over the shifted mask of each packed sequence; shifted_mask [n] is written for
+// the backward.
+int areal_dpo_seq_logps(const float* logprobs, const float* ref_logprobs, const uint8_t* loss_mask,
+                        const int32_t* cu_seqlens, int64_t n_tokens, int64_t n_seqs,
+                        double* seq_sums, uint8_t* shifted_mask, hipStream_t stream) {
+  if (n_tokens < 0 || n_seqs < 0) return AREAL_ERR_BAD_ARG;
+  if (n_seqs == 0) return AREAL_OK;
+  if (!logprobs || !ref_logprobs || !loss_mask || !cu_seqlens || !seq_sums)
+    return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(dpo_seq_kernel, dim3((unsigned)n_seqs), dim3(AUX_THREADS), 0, stream, logprobs,
+                     ref_logprobs, loss_mask, SeqLayout{cu_seqlens, (int)n_seqs, 0}, n_tokens,
+                     seq_sums, shifted_mask);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// grad_logprobs[t] = shifted_mask[t] * grad_seq[sequence of t]
+int areal_dpo_seq_logps_grad(const double* grad_seq, const uint8_t* shifted_mask,
+                             const int32_t* cu_seqlens, int64_t n_tokens, int64_t n_seqs,
+                             float* grad_logprobs, hipStream_t stream) {
+  if (n_tokens < 0 || n_seqs < 0) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!grad_seq || !shifted_mask || !cu_seqlens || !grad_logprobs || n_seqs == 0)
+    return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(dpo_seq_grad_kernel, dim3(aux_grid(n_tokens)), dim3(AUX_THREADS), 0, stream,
+                     grad_seq, shifted_mask, SeqLayout{cu_seqlens, (int)n_seqs, 0}, n_tokens,
+                     grad_logprobs);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+}  // extern "C"

@@ -7,6 +7,12 @@ from areal_amd.functional.functional import (
     masked_normalization,
     ppo_actor_loss_fn,
 )
+from areal_amd.functional.aux_losses import (
+    dpo_pair_logratios,
+    dpo_preference_loss,
+    ppo_critic_loss_fn,
+    sapo_loss_fn,
+)
 from areal_amd.functional.lm_head import (
     ChunkedLMHeadOutput,
     fused_lm_head_logprobs_entropy,
@@ -22,6 +28,10 @@ __all__ = [
     "cispo_loss_fn",
     "masked_normalization",
     "ppo_actor_loss_fn",
+    "sapo_loss_fn",
+    "ppo_critic_loss_fn",
+    "dpo_pair_logratios",
+    "dpo_preference_loss",
     "gather_logprobs",
     "gather_logprobs_entropy",
     "ChunkedLMHeadOutput",

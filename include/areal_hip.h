@@ -168,6 +168,46 @@ int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const d
                           float* grad_logprobs, int64_t n_tokens, areal_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------
+ * SAPO policy loss, PPO critic loss, DPO sequence sums (same per-token layout as the actor loss)
+ * replace sapo_loss_fn (areal/utils/functional/functional.py:599-675), ppo_critic_loss_fn
+ * (:869-933) and the scatter-adds of dpo_pair_logratios (:796-841).
+ * counters [8] double use the actor loss's layout ([0] loss sum, [1] denominator, [4] clipped
+ * count, [7] loss), so areal_actor_loss_grad turns the d(loss sum) output into the gradient.
+ * ------------------------------------------------------------------------------------- */
+size_t areal_aux_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs);
+
+/* seq_level != 0: geometric-mean ratio and mean advantage per sequence (functional.py:56-149;
+ * cu_seqlens [n_seqs+1] or uniform_len > 0). Per-token outputs may be NULL. */
+int areal_sapo_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
+                    const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
+                    int64_t n_seqs, int64_t uniform_len, float tau_pos, float tau_neg,
+                    int seq_level, float* loss, float* dlogprobs, float* stat_loss,
+                    float* stat_ratio, float* stat_approx_kl, float* soft_gate, float* gate_pos,
+                    float* gate_neg, double* counters, void* workspace, size_t workspace_bytes,
+                    areal_stream_t stream);
+
+/* loss = mean over the mask (or over all n when loss_mask is NULL) of
+ * max(l(value, target), l(old + clamp(value - old, +-eps), target)); l = mse or huber(10). */
+int areal_critic_loss(const float* value, const float* old_value, const float* target_value,
+                      const uint8_t* loss_mask, int64_t n, float value_eps_clip, int huber,
+                      float* loss, float* dvalue, float* stat_loss, uint8_t* clip_mask,
+                      double* counters, void* workspace, size_t workspace_bytes,
+                      areal_stream_t stream);
+
+/* seq_sums [n_seqs][3] double = {sum policy log-probs, sum reference log-probs, count} over
+ * shifted_mask[t] = loss_mask[t+1] inside each packed sequence (its last token excluded);
+ * shifted_mask [n_tokens] is written for the backward. */
+int areal_dpo_seq_logps(const float* logprobs, const float* ref_logprobs,
+                        const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
+                        int64_t n_seqs, double* seq_sums, uint8_t* shifted_mask,
+                        areal_stream_t stream);
+
+/* grad_logprobs[t] = shifted_mask[t] * grad_seq[sequence of t]. */
+int areal_dpo_seq_logps_grad(const double* grad_seq, const uint8_t* shifted_mask,
+                             const int32_t* cu_seqlens, int64_t n_tokens, int64_t n_seqs,
+                             float* grad_logprobs, areal_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------
  * GAE over packed sequences
  * replaces _compute_token_level_gae (areal/trainer/ppo/gae.py:10-36); per-sequence lambda as
  * produced by areal/trainer/ppo/lambda_fn.py:50-112.

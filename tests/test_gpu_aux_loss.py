@@ -1,0 +1,134 @@
+"""HIP SAPO / critic / DPO kernels through the C ABI against the reference's literals and the
+CPU oracle (loss <= 1e-4 rel, masks bit-exact, gradients against the oracle's autograd)."""
+
+import pytest
+import torch
+
+from areal_amd.functional import (
+    dpo_pair_logratios,
+    dpo_preference_loss,
+    ppo_critic_loss_fn,
+    sapo_loss_fn,
+)
+from oracle import aux_loss as A
+
+pytestmark = pytest.mark.gpu
+
+
+def test_sapo_reference_literals(dev):
+    # tests/test_functional.py:923-954 and :1160-1195 of the reference
+    lp = torch.tensor([[1.0, 1.0]], device=dev)
+    loss, stat = sapo_loss_fn(lp, lp.clone(), torch.ones(1, 2, device=dev), 1.0, 1.0,
+                              torch.ones(1, 2, dtype=torch.bool, device=dev))
+    assert loss.ndim == 0 and loss.dtype == torch.float32
+    assert abs(loss.item() + 2.0) < 1e-5
+    assert torch.allclose(stat["sapo_soft_gate"].cpu(), torch.tensor([[2.0, 2.0]]), atol=1e-5)
+    grads = []
+    for tau in (1.0, 2.0):
+        x = torch.zeros(1, 1, device=dev, requires_grad=True)
+        l, _ = sapo_loss_fn(x, torch.zeros(1, 1, device=dev), torch.ones(1, 1, device=dev), tau, tau,
+                            torch.ones(1, 1, dtype=torch.bool, device=dev))
+        l.backward()
+        grads.append(x.grad.item())
+    assert abs(grads[0] - grads[1]) < 1e-6 and abs(grads[0] + 1.0) < 1e-6
+    with pytest.raises(ValueError, match="must be positive"):
+        sapo_loss_fn(lp, lp, lp, 0.0, 1.0, torch.ones(1, 2, dtype=torch.bool, device=dev))
+    with pytest.raises(ValueError, match="Invalid importance_sampling_level"):
+        sapo_loss_fn(lp, lp, lp, 1.0, 1.0, torch.ones(1, 2, dtype=torch.bool, device=dev), "turn")
+    with pytest.raises(ValueError, match="cu_seqlens is required"):
+        sapo_loss_fn(lp[0], lp[0], lp[0], 1.0, 1.0, torch.ones(2, dtype=torch.bool, device=dev), "sequence")
+
+
+@pytest.mark.parametrize("level", ["token", "sequence"])
+@pytest.mark.parametrize("layout", ["packed", "padded"])
+def test_sapo_matches_oracle(dev, level, layout):
+    g = torch.Generator().manual_seed(11)
+    if layout == "packed":
+        lens = torch.randint(1, 400, (37,), generator=g)
+        cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+        shape = (int(cu[-1]),)
+    else:
+        cu, shape = None, (24, 300)
+    lp = (torch.randn(shape, generator=g) * 0.3 - 1.0)
+    old = lp + torch.randn(shape, generator=g) * 0.2
+    adv = torch.randn(shape, generator=g)
+    adv.view(-1)[::17] = 0.0
+    mask = torch.rand(shape, generator=g) > 0.25
+    if layout == "padded":
+        mask[3] = False  # an all-masked row
+    lp_c = lp.clone().requires_grad_(True)
+    want, ws = A.sapo_loss(lp_c, old, adv, 1.0, 1.05, mask, level, cu)
+    want.backward()
+    x = lp.to(dev).requires_grad_(True)
+    loss, stat = sapo_loss_fn(x, old.to(dev), adv.to(dev), 1.0, 1.05, mask.to(dev), level,
+                              cu.to(dev) if cu is not None else None)
+    loss.backward()
+    torch.testing.assert_close(loss.detach().cpu(), want.detach(), rtol=1e-4, atol=1e-7)
+    for key, okey in (("loss", "loss"), ("importance_weight", "importance_weight"), ("approx_kl", "approx_kl"),
+                      ("sapo_soft_gate", "sapo_soft_gate"), ("sapo_scaled_gate_pos", "sapo_scaled_gate_pos"),
+                      ("sapo_scaled_gate_neg", "sapo_scaled_gate_neg")):
+        assert stat[key].shape == shape
+        torch.testing.assert_close(stat[key].cpu(), ws[okey], rtol=2e-5, atol=1e-6)
+    assert not stat["clip_mask"].any() and not stat["dual_clip_mask"].any()
+    torch.testing.assert_close(x.grad.cpu(), lp_c.grad, rtol=1e-4, atol=1e-8)
+
+
+@pytest.mark.parametrize("kind", ["mse", "huber"])
+@pytest.mark.parametrize("masked", [True, False])
+def test_critic_loss_matches_oracle(dev, kind, masked):
+    g = torch.Generator().manual_seed(5)
+    shape = (19, 257)
+    old = torch.randn(shape, generator=g) * 3
+    value = old + torch.randn(shape, generator=g) * 0.5
+    target = old + torch.randn(shape, generator=g) * (15.0 if kind == "huber" else 1.0)
+    value.view(-1)[:50] = old.view(-1)[:50]          # ties: zero step
+    value.view(-1)[50:80] = old.view(-1)[50:80] + 0.2  # exactly on the clip bound
+    mask = (torch.rand(shape, generator=g) > 0.3) if masked else None
+    v_c = value.clone().requires_grad_(True)
+    want, ws = A.critic_loss(v_c, old, target, 0.2, mask, kind)
+    want.backward()
+    v = value.to(dev).requires_grad_(True)
+    loss, stat = ppo_critic_loss_fn(v, old.to(dev), target.to(dev), 0.2, mask.to(dev) if masked else None, kind)
+    loss.backward()
+    torch.testing.assert_close(loss.detach().cpu(), want.detach(), rtol=1e-4, atol=1e-7)
+    assert torch.equal(stat["clip_mask"].cpu(), ws["clip_mask"])
+    torch.testing.assert_close(stat["loss"].cpu(), ws["loss"], rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(v.grad.cpu(), v_c.grad, rtol=1e-4, atol=1e-9)
+    with pytest.raises(NotImplementedError):
+        ppo_critic_loss_fn(v, old.to(dev), target.to(dev), 0.2, None, "l1")
+    with pytest.raises(AssertionError):
+        ppo_critic_loss_fn(v.double(), old.to(dev), target.to(dev), 0.2)
+
+
+def test_critic_loss_hand_cases(dev):
+    value = torch.tensor([0.6, 0.9, 0.1], device=dev, requires_grad=True)
+    loss, stat = ppo_critic_loss_fn(value, torch.full((3,), 0.5, device=dev), torch.ones(3, device=dev), 0.2)
+    assert stat["clip_mask"].tolist() == [False, True, False]
+    loss.backward()
+    torch.testing.assert_close(value.grad.cpu(), torch.tensor([(0.6 - 1.0) / 3, 0.0, (0.1 - 1.0) / 3]),
+                               rtol=1e-6, atol=1e-8)
+
+
+def test_dpo_pair_logratios_matches_oracle(dev):
+    g = torch.Generator().manual_seed(8)
+    lens = torch.cat([torch.tensor([1, 2, 0, 5]), torch.randint(1, 3000, (36,), generator=g)])
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    n = int(cu[-1])
+    lp, ref = -torch.rand(n, generator=g) * 3, -torch.rand(n, generator=g) * 3
+    mask = torch.rand(n, generator=g) > 0.4
+    valid = torch.rand(20, generator=g) > 0.2
+    lp_c = lp.clone().requires_grad_(True)
+    wp, wr, wl = A.dpo_pair_logratios(lp_c, ref, cu, mask, valid)
+    x = lp.to(dev).requires_grad_(True)
+    p, r, l = dpo_pair_logratios(x, ref.to(dev), cu.to(dev), mask.to(dev), valid.to(dev))
+    assert p.dtype == torch.float64 and p.shape == wp.shape
+    torch.testing.assert_close(p.detach().cpu(), wp.detach(), rtol=1e-12, atol=1e-9)
+    torch.testing.assert_close(r.cpu(), wr, rtol=1e-12, atol=1e-9)
+    assert torch.equal(l.cpu(), wl)
+    # sigmoid DPO loss on the pair deltas, backward to the log-probs
+    def dpo(pp, rr):
+        logits = (pp[:, 0] - pp[:, 1]) - (rr[:, 0] - rr[:, 1])
+        return dpo_preference_loss(logits, beta=0.1).mean()
+    dpo(wp, wr).backward()
+    dpo(p, r).backward()
+    torch.testing.assert_close(x.grad.cpu(), lp_c.grad, rtol=1e-5, atol=1e-9)
