@@ -73,6 +73,8 @@ SIGNATURES: dict[str, tuple] = {
         I,
         [P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, SZ, P],
     ),
+    "areal_turn_gae_workspace_bytes": (SZ, [I64, I64]),
+    "areal_turn_gae": (I, [P, P, P, P, P, P, I64, I64, F, F, P, P, P, P, SZ, P]),
     "areal_group_norm_workspace_bytes": (SZ, [I64, I64]),
     "areal_group_norm": (
         I,

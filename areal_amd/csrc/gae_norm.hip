@@ -708,6 +708,211 @@ __global__ __launch_bounds__(NORM_THREADS) void masked_norm_apply_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Turn-level GAE (areal/trainer/ppo/gae.py:82-163): every generated turn is one timestep.
+// One block per padded row. Active tokens carry non-decreasing turn ids (checked; a violation
+// sets *status), so a turn starts at the first active token whose id exceeds every active id on
+// its left. Pass 1 compacts the turns: start position's value, and the fp64 prefix sum of the
+// active rewards taken just before the start (turn reward = difference of consecutive
+// prefixes). Thread 0 then runs the recurrence over the compact turns right to left, and pass
+// 2 hands every token its turn's advantage and return.
+// Per row workspace: prefix [L+1] double, value/adv/ret [L] float each.
+// ---------------------------------------------------------------------------------------
+constexpr int TURN_THREADS = 256;
+constexpr int TURN_ITEMS = 4;
+
+struct TurnArgs {
+  const float* rewards;
+  const float* values;
+  const float* mask;       // float loss mask, nonzero = active
+  const int32_t* turn_ids;
+  const uint8_t* no_eos;   // [bs] or null
+  const float* lam_seq;    // [bs] or null
+  int64_t bs, L;
+  float discount, lam;
+  float* adv;
+  float* ret;
+  double* ws_prefix;       // [bs][L + 1]
+  float* ws_val;           // [bs][L]
+  float* ws_adv;           // [bs][L]
+  float* ws_ret;           // [bs][L]
+  int* status;             // bit 0: negative id, bit 1: id >= L, bit 2: ids go backwards
+};
+
+struct TurnCarry { int count; int maxid; double sum; };
+
+// Exclusive scan over the block of (start count, running max id, reward sum), chunk carry
+// included. smem: [TURN_THREADS] of each.
+DEVI TurnCarry turn_block_exclusive(int cnt, int mx, double sm, const TurnCarry& carry, int* s_cnt,
+                                    int* s_max, double* s_sum, TurnCarry& chunk_total) {
+  const int tid = threadIdx.x;
+  __syncthreads();
+  s_cnt[tid] = cnt; s_max[tid] = mx; s_sum[tid] = sm;
+  __syncthreads();
+  // Hillis-Steele inclusive scan (256 threads, 8 steps)
+  for (int d = 1; d < TURN_THREADS; d <<= 1) {
+    int c = 0, m = -1; double v = 0.0;
+    if (tid >= d) { c = s_cnt[tid - d]; m = s_max[tid - d]; v = s_sum[tid - d]; }
+    __syncthreads();
+    if (tid >= d) {
+      s_cnt[tid] += c;
+      s_max[tid] = s_max[tid] > m ? s_max[tid] : m;
+      s_sum[tid] += v;
+    }
+    __syncthreads();
+  }
+  TurnCarry ex = carry;
+  if (tid > 0) {
+    ex.count += s_cnt[tid - 1];
+    ex.maxid = ex.maxid > s_max[tid - 1] ? ex.maxid : s_max[tid - 1];
+    ex.sum += s_sum[tid - 1];
+  }
+  chunk_total.count = carry.count + s_cnt[TURN_THREADS - 1];
+  chunk_total.maxid = carry.maxid > s_max[TURN_THREADS - 1] ? carry.maxid : s_max[TURN_THREADS - 1];
+  chunk_total.sum = carry.sum + s_sum[TURN_THREADS - 1];
+  return ex;
+}
+
+__global__ __launch_bounds__(TURN_THREADS) void turn_gae_kernel(TurnArgs a) {
+  __shared__ int s_cnt[TURN_THREADS];
+  __shared__ int s_max[TURN_THREADS];
+  __shared__ double s_sum[TURN_THREADS];
+  __shared__ int s_k;
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x, L = a.L;
+  const float* rw = a.rewards + row * L;
+  const float* vl = a.values + row * L;
+  const float* ms = a.mask + row * L;
+  const int32_t* id = a.turn_ids + row * L;
+  double* prefix = a.ws_prefix + row * (L + 1);
+  float* tval = a.ws_val + row * L;
+  float* tadv = a.ws_adv + row * L;
+  float* tret = a.ws_ret + row * L;
+  int bad = 0;
+
+  // ---- pass 1: compact the turns
+  TurnCarry carry{0, -1, 0.0};
+  for (int64_t base = 0; base < L; base += TURN_THREADS * TURN_ITEMS) {
+    const int64_t t0 = base + (int64_t)tid * TURN_ITEMS;
+    int ids[TURN_ITEMS]; bool act[TURN_ITEMS]; float r[TURN_ITEMS];
+    int cnt = 0, mx = -1; double sm = 0.0;
+    // thread-local: starts relative to the maximum seen inside the thread's own items
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      const int64_t t = t0 + i;
+      act[i] = t < L && ms[t] != 0.0f;
+      ids[i] = act[i] ? id[t] : -1;
+      r[i] = act[i] ? rw[t] : 0.0f;
+      if (act[i]) {
+        if (ids[i] < 0) bad |= 1;
+        if ((int64_t)ids[i] >= L) bad |= 2;
+        mx = mx > ids[i] ? mx : ids[i];
+        sm += (double)r[i];
+      }
+    }
+    (void)cnt;
+    // the number of starts in a thread depends on the maximum to its left, so scan the maximum
+    // and the reward sums first, then count starts, then scan the counts
+    TurnCarry tot1;
+    const TurnCarry ex1 = turn_block_exclusive(0, mx, sm, carry, s_cnt, s_max, s_sum, tot1);
+    int run_max = ex1.maxid;
+    bool start[TURN_ITEMS];
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      start[i] = act[i] && ids[i] > run_max;
+      if (act[i] && ids[i] < run_max) bad |= 4;
+      if (act[i]) run_max = run_max > ids[i] ? run_max : ids[i];
+      cnt += start[i];
+    }
+    TurnCarry tot2;
+    const TurnCarry ex2 = turn_block_exclusive(cnt, -1, 0.0, TurnCarry{carry.count, -1, 0.0}, s_cnt,
+                                               s_max, s_sum, tot2);
+    int k = ex2.count;
+    double run_sum = ex1.sum;
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      if (start[i]) {
+        prefix[k] = run_sum;            // active rewards strictly before this turn
+        tval[k] = vl[t0 + i];           // the turn's state value: value at its first token
+        ++k;
+      }
+      run_sum += (double)r[i];
+    }
+    carry.count = tot2.count; carry.maxid = tot1.maxid; carry.sum = tot1.sum;
+  }
+  if (tid == 0) { prefix[carry.count] = carry.sum; s_k = carry.count; }
+  if (bad) atomicOr(a.status, bad);
+  __syncthreads();
+  __threadfence_block();
+  const int K = s_k;
+
+  // ---- recurrence over the turns, right to left (gae.py:139-150)
+  if (tid == 0) {
+    const float gam = a.discount;
+    const float lam = a.lam_seq ? a.lam_seq[row] : a.lam;
+    const float c = gam * lam;
+    float nextv = (a.no_eos && a.no_eos[row]) ? vl[L - 1] : 0.0f;
+    float last = 0.0f;
+    for (int k = K - 1; k >= 0; --k) {
+      const float R = (float)(prefix[k + 1] - prefix[k]);
+      const float V = tval[k];
+      const float delta = (R + gam * nextv) - V;
+      const float g = delta + c * last;
+      tadv[k] = g;
+      tret[k] = g + V;
+      nextv = V;
+      last = g;
+    }
+  }
+  __syncthreads();
+  __threadfence_block();
+
+  // ---- pass 2: every token takes the result of its turn (gae.py:152-157)
+  TurnCarry carry2{0, -1, 0.0};
+  for (int64_t base = 0; base < L; base += TURN_THREADS * TURN_ITEMS) {
+    const int64_t t0 = base + (int64_t)tid * TURN_ITEMS;
+    int ids[TURN_ITEMS]; bool act[TURN_ITEMS]; float m[TURN_ITEMS];
+    int mx = -1;
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      const int64_t t = t0 + i;
+      m[i] = t < L ? ms[t] : 0.0f;
+      act[i] = m[i] != 0.0f;
+      ids[i] = act[i] ? id[t] : -1;
+      if (act[i]) mx = mx > ids[i] ? mx : ids[i];
+    }
+    TurnCarry tot1;
+    const TurnCarry ex1 = turn_block_exclusive(0, mx, 0.0, carry2, s_cnt, s_max, s_sum, tot1);
+    int run_max = ex1.maxid, cnt = 0;
+    bool start[TURN_ITEMS];
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      start[i] = act[i] && ids[i] > run_max;
+      if (act[i]) run_max = run_max > ids[i] ? run_max : ids[i];
+      cnt += start[i];
+    }
+    TurnCarry tot2;
+    const TurnCarry ex2 = turn_block_exclusive(cnt, -1, 0.0, TurnCarry{carry2.count, -1, 0.0}, s_cnt,
+                                               s_max, s_sum, tot2);
+    int k = ex2.count;  // turns started strictly before this thread's first token
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      const int64_t t = t0 + i;
+      if (start[i]) ++k;
+      if (t >= L) continue;
+      if (act[i] && k > 0) {
+        const float mm = m[i];
+        a.adv[row * L + t] = tadv[k - 1] * mm;
+        a.ret[row * L + t] = tret[k - 1] * mm + vl[t] * (1.0f - mm);
+      } else {
+        a.adv[row * L + t] = 0.0f;
+        a.ret[row * L + t] = vl[t];
+      }
+    }
+    carry2.count = tot2.count; carry2.maxid = tot1.maxid;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -758,6 +963,42 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
                      carry);
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(gae_apply_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g, carry);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+size_t areal_turn_gae_workspace_bytes(int64_t bs, int64_t max_seqlen) {
+  if (bs <= 0 || max_seqlen <= 0) return 0;
+  return (size_t)bs * ((size_t)(max_seqlen + 1) * sizeof(double) + (size_t)max_seqlen * 3 * sizeof(float)) + 256;
+}
+
+// Turn-level GAE on padded [bs, max_seqlen] tensors: rewards, values, loss_mask fp32, turn_ids
+// int32 (-1 in prompt / tool gaps), no_eos [bs] (nullable), lambda_seq [bs] (nullable, else the
+// scalar). status (device int, zeroed by the caller) receives a bit mask of malformed turn ids
+// at active tokens: 1 negative, 2 not smaller than max_seqlen, 4 decreasing.
+int areal_turn_gae(const float* rewards, const float* values, const float* loss_mask,
+                   const int32_t* turn_ids, const uint8_t* no_eos, const float* lambda_seq,
+                   int64_t bs, int64_t max_seqlen, float discount, float gae_lambda,
+                   float* advantages, float* returns, int* status, void* workspace,
+                   size_t workspace_bytes, hipStream_t stream) {
+  if (bs < 0 || max_seqlen < 0) return AREAL_ERR_BAD_ARG;
+  if (bs == 0 || max_seqlen == 0) return AREAL_OK;
+  if (!rewards || !values || !loss_mask || !turn_ids || !advantages || !returns || !status)
+    return AREAL_ERR_BAD_ARG;
+  if (bs > (1 << 30) || max_seqlen > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  if (workspace == nullptr || workspace_bytes < areal_turn_gae_workspace_bytes(bs, max_seqlen))
+    return AREAL_ERR_WORKSPACE;
+  char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  TurnArgs a;
+  a.rewards = rewards; a.values = values; a.mask = loss_mask; a.turn_ids = turn_ids;
+  a.no_eos = no_eos; a.lam_seq = lambda_seq; a.bs = bs; a.L = max_seqlen;
+  a.discount = discount; a.lam = gae_lambda; a.adv = advantages; a.ret = returns;
+  a.ws_prefix = (double*)wp;
+  a.ws_val = (float*)(wp + (size_t)bs * (size_t)(max_seqlen + 1) * sizeof(double));
+  a.ws_adv = a.ws_val + (size_t)bs * max_seqlen;
+  a.ws_ret = a.ws_adv + (size_t)bs * max_seqlen;
+  a.status = status;
+  hipLaunchKernelGGL(turn_gae_kernel, dim3((unsigned)bs), dim3(TURN_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

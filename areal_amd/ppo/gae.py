@@ -94,3 +94,69 @@ def compute_gae_packed(
         loss_mask.to(torch.float32).contiguous(),
         cu, no_eos, lam_seq, n_seqs, 0, discount, lam,
     )
+
+
+_TURN_ID_ERRORS = (
+    (1, "turn_ids must be non-negative at every active loss token"),
+    (2, "turn_ids at active loss tokens must be smaller than the sequence length"),
+    (4, "turn_ids at active loss tokens must be temporally nondecreasing"),
+)
+
+
+def _compute_turn_level_gae(
+    rewards: torch.Tensor,
+    values: torch.Tensor,
+    loss_mask: torch.Tensor,
+    turn_ids: torch.Tensor,
+    seq_no_eos_mask: torch.Tensor,
+    discount: float,
+    gae_lambda: float | torch.Tensor,
+    validate: bool = True,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """GAE with each generated turn treated as one timestep, on padded ``[bs, max_seqlen]``
+    tensors (``areal/trainer/ppo/gae.py:82-163``).
+
+    Shape, device and dtype errors are raised as in the reference.  Malformed turn ids at
+    active tokens (negative, too large, going backwards) are found by the kernel; with
+    ``validate=True`` the flag is read back (one host synchronisation) and raised as the
+    reference's ``RuntimeError``; the reference uses device-side asserts there, which on a GPU
+    would abort the process.  ``validate=False`` skips the read-back.
+    """
+    if turn_ids.shape != loss_mask.shape:
+        raise ValueError(f"turn_ids must have shape {loss_mask.shape}, got {turn_ids.shape}")
+    if turn_ids.device != loss_mask.device:
+        raise ValueError(
+            "turn_ids and loss_mask must be on the same device, got "
+            f"{turn_ids.device} and {loss_mask.device}"
+        )
+    if turn_ids.dtype not in (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64):
+        raise ValueError(f"turn_ids must use an integer dtype, got {turn_ids.dtype}")
+    lib = _lib.load()
+    bs, max_seqlen = rewards.shape
+    r = rewards.to(torch.float32).contiguous()
+    v = values.to(torch.float32).contiguous()
+    m = loss_mask.to(torch.float32).contiguous()
+    # ids beyond int32 cannot be valid (they must be smaller than the sequence length)
+    ids = turn_ids.clamp(min=-1, max=2**31 - 1).to(torch.int32).contiguous()
+    dev = _lib.require_gpu(r, v, m, ids)
+    lam_seq, lam = _split_lambda(gae_lambda, bs, dev)
+    no_eos = seq_no_eos_mask.to(device=dev, dtype=torch.bool).contiguous()
+    adv = torch.empty((bs, max_seqlen), dtype=torch.float32, device=dev)
+    ret = torch.empty((bs, max_seqlen), dtype=torch.float32, device=dev)
+    if bs == 0 or max_seqlen == 0:
+        return adv, ret
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    nbytes = lib.areal_turn_gae_workspace_bytes(bs, max_seqlen)
+    ws = _lib.workspace(nbytes, dev)
+    rc = lib.areal_turn_gae(
+        _lib.ptr(r), _lib.ptr(v), _lib.ptr(m), _lib.ptr(ids), _lib.ptr(no_eos), _lib.ptr(lam_seq),
+        bs, max_seqlen, float(discount), float(lam), _lib.ptr(adv), _lib.ptr(ret),
+        _lib.ptr(status), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_turn_gae")
+    if validate:
+        flags = int(status.item())
+        for bit, message in _TURN_ID_ERRORS:
+            if flags & bit:
+                raise RuntimeError(message)
+    return adv, ret

@@ -220,6 +220,18 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
                      float gae_lambda, float* advantages, float* returns, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
 
+/* Turn-level GAE (areal/trainer/ppo/gae.py:82-163) on padded [bs, max_seqlen] tensors: every
+ * generated turn is one timestep. turn_ids int32 (-1 in prompt / tool gaps; non-decreasing over
+ * the active tokens of a row), loss_mask fp32 (nonzero = active). *status (device int, zeroed
+ * by the caller) receives a bit mask of malformed ids at active tokens: 1 negative, 2 not
+ * smaller than max_seqlen, 4 decreasing (the conditions _validate_turn_ids asserts, :39-79). */
+size_t areal_turn_gae_workspace_bytes(int64_t bs, int64_t max_seqlen);
+int areal_turn_gae(const float* rewards, const float* values, const float* loss_mask,
+                   const int32_t* turn_ids, const uint8_t* no_eos, const float* lambda_seq,
+                   int64_t bs, int64_t max_seqlen, float discount, float gae_lambda,
+                   float* advantages, float* returns, int* status, void* workspace,
+                   size_t workspace_bytes, areal_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * Normalisation
  * replaces Normalization.__call__ / _compute_mean / _compute_std

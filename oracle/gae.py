@@ -50,3 +50,50 @@ def gae_packed(rewards, values, loss_mask, cu_seqlens, seq_no_eos_mask, discount
         )
         adv[s:e] = a[0]
     return adv, adv + values
+
+
+def gae_turn_level(rewards, values, loss_mask, turn_ids, seq_no_eos_mask, discount, gae_lambda):
+    """Turn-level GAE (``areal/trainer/ppo/gae.py:82-163``): every generated turn is one
+    timestep; its reward is the sum of its active tokens' rewards, its value the value at its
+    first active token; the turn's advantage is broadcast to its tokens.
+
+    Pinned by the reference's literals (tests/test_ppo_gae.py:81-151): [[2,2,2,2]] for lambda
+    0.5 over two turns; gaps / unused ids with bootstrap giving advantages
+    [[3.75,3.75,0,6,6]] and returns [[4.75,4.75,9,8,8]]; per-sample lambda [[2,2,2,2],[1,1,2,2]].
+    Validation raises as the reference does on the CPU (RuntimeError from the asserts)."""
+    if turn_ids.shape != loss_mask.shape:
+        raise ValueError(f"turn_ids must have shape {loss_mask.shape}, got {turn_ids.shape}")
+    if turn_ids.dtype not in (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64):
+        raise ValueError(f"turn_ids must use an integer dtype, got {turn_ids.dtype}")
+    bs, width = rewards.shape
+    valid = loss_mask.bool()
+    if not torch.all(~valid | (turn_ids >= 0)):
+        raise RuntimeError("turn_ids must be non-negative at every active loss token")
+    if not torch.all(~valid | (turn_ids < width)):
+        raise RuntimeError("turn_ids at active loss tokens must be smaller than the sequence length")
+    active = torch.where(valid, turn_ids, torch.full_like(turn_ids, -1))
+    if not torch.all(~valid | (turn_ids >= torch.cummax(active, dim=1).values)):
+        raise RuntimeError("turn_ids at active loss tokens must be temporally nondecreasing")
+    safe = torch.clamp(turn_ids.long(), min=0, max=width - 1)
+    turn_rewards = torch.zeros_like(rewards).scatter_add_(1, safe, rewards * valid.to(rewards.dtype))
+    pos = torch.arange(width).expand(bs, -1)
+    first = torch.full_like(safe, width).scatter_reduce_(
+        1, safe, torch.where(valid, pos, torch.full_like(pos, width)), reduce="amin", include_self=True
+    )
+    valid_turn = first < width
+    turn_values = values.gather(1, first.clamp(max=width - 1)) * valid_turn.to(values.dtype)
+    turn_adv = torch.zeros(bs, width, dtype=torch.float32)
+    last = torch.zeros(bs, dtype=torch.float32)
+    nxt = values[:, width - 1] * seq_no_eos_mask
+    c = discount * gae_lambda
+    for k in reversed(range(width)):
+        delta = turn_rewards[:, k] + discount * nxt - turn_values[:, k]
+        new = delta + c * last
+        m = valid_turn[:, k]
+        turn_adv[:, k] = torch.where(m, new, torch.zeros_like(last))
+        nxt = torch.where(m, turn_values[:, k], nxt)
+        last = torch.where(m, new, last)
+    turn_ret = turn_adv + turn_values
+    adv = torch.gather(turn_adv, 1, safe) * loss_mask
+    ret = torch.gather(turn_ret, 1, safe) * loss_mask + values * (1 - loss_mask)
+    return adv, ret

@@ -208,3 +208,73 @@ def test_masked_normalization_matches_oracle(dev):
         torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-6)
     want = N.masked_normalization(x, None)
     torch.testing.assert_close(masked_normalization(x.to(dev)).cpu(), want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- turn-level GAE
+def test_turn_level_gae_reference_literals(dev):
+    from areal_amd.ppo.gae import _compute_turn_level_gae
+
+    r = _t([[0.0, 1.0, 0.0, 2.0]], dev)
+    a, rt = _compute_turn_level_gae(r, torch.zeros_like(r), torch.ones_like(r),
+                                    torch.tensor([[0, 0, 1, 1]], dtype=torch.int32, device=dev),
+                                    torch.tensor([False], device=dev), 1.0, 0.5)
+    assert torch.equal(a.cpu(), torch.tensor([[2.0, 2.0, 2.0, 2.0]])) and torch.equal(rt, a)
+    r = _t([[0.0, 3.0, 0.0, 0.0, 4.0]], dev)
+    v = _t([[1.0, 5.0, 9.0, 2.0, 8.0]], dev)
+    a, rt = _compute_turn_level_gae(r, v, _t([[1.0, 1.0, 0.0, 1.0, 1.0]], dev),
+                                    torch.tensor([[0, 0, -1, 2, 2]], device=dev),
+                                    torch.tensor([True], device=dev), 0.5, 0.25)
+    assert torch.equal(a.cpu(), torch.tensor([[3.75, 3.75, 0.0, 6.0, 6.0]]))
+    assert torch.equal(rt.cpu(), torch.tensor([[4.75, 4.75, 9.0, 8.0, 8.0]]))
+    r = _t([[0.0, 1.0, 0.0, 2.0]] * 2, dev)
+    a, _ = _compute_turn_level_gae(r, torch.zeros_like(r), torch.ones_like(r),
+                                   torch.tensor([[0, 0, 1, 1]] * 2, dtype=torch.int32, device=dev),
+                                   torch.tensor([False, False], device=dev), 1.0, _t([0.5, 0.0], dev))
+    assert torch.equal(a.cpu(), torch.tensor([[2.0, 2.0, 2.0, 2.0], [1.0, 1.0, 2.0, 2.0]]))
+
+
+@pytest.mark.parametrize("ids,message", [([-1, 0, 0, 1], "non-negative"), ([0, 0, 4, 4], "smaller than the sequence length"),
+                                         ([0, 1, 0, 2], "temporally nondecreasing")])
+def test_turn_level_gae_rejects_malformed_ids(dev, ids, message):
+    from areal_amd.ppo.gae import _compute_turn_level_gae
+
+    r = torch.zeros(1, 4, device=dev)
+    with pytest.raises(RuntimeError, match=message):
+        _compute_turn_level_gae(r, r, torch.ones_like(r), torch.tensor([ids], device=dev),
+                                torch.tensor([False], device=dev), 1.0, 1.0)
+    with pytest.raises(ValueError, match="integer dtype"):
+        _compute_turn_level_gae(r, r, torch.ones_like(r), torch.zeros(1, 4, device=dev),
+                                torch.tensor([False], device=dev), 1.0, 1.0)
+    with pytest.raises(ValueError, match="must have shape"):
+        _compute_turn_level_gae(r, r, torch.ones_like(r), torch.zeros(1, 3, dtype=torch.long, device=dev),
+                                torch.tensor([False], device=dev), 1.0, 1.0)
+
+
+@pytest.mark.parametrize("bs,L,max_turn_len", [(5, 37, 4), (16, 3000, 200), (3, 9000, 3000), (4, 1500, 1)])
+def test_turn_level_gae_matches_oracle(dev, bs, L, max_turn_len):
+    from areal_amd.ppo.gae import _compute_turn_level_gae
+
+    g = torch.Generator().manual_seed(bs * 7 + L)
+    ids = torch.full((bs, L), -1, dtype=torch.int64)
+    mask = torch.zeros(bs, L)
+    for b in range(bs):
+        t, k = int(torch.randint(0, 5, (1,), generator=g)), 0
+        while t < L:
+            n = int(torch.randint(1, max_turn_len + 1, (1,), generator=g))
+            ids[b, t:t + n] = k
+            mask[b, t:t + n] = (torch.rand(min(n, L - t), generator=g) > 0.1).float()
+            t += n + int(torch.randint(0, 6, (1,), generator=g))  # a gap (prompt / tool output)
+            k += int(torch.randint(1, 3, (1,), generator=g))      # ids may skip
+        ids[b][ids[b] >= L] = -1
+        mask[b][ids[b] < 0] = 0
+    r = torch.randn(bs, L, generator=g) * (torch.rand(bs, L, generator=g) > 0.7)
+    v = torch.randn(bs, L, generator=g)
+    ne = torch.rand(bs, generator=g) > 0.5
+    lam = torch.rand(bs, generator=g) * 0.3 + 0.7
+    for lam_arg in (0.9, lam):
+        want_a, want_r = G.gae_turn_level(r, v, mask, ids, ne, 0.97, lam_arg)
+        a, rt = _compute_turn_level_gae(r.to(dev), v.to(dev), mask.to(dev), ids.to(dev), ne.to(dev), 0.97,
+                                        lam_arg.to(dev) if isinstance(lam_arg, torch.Tensor) else lam_arg)
+        scale = max(want_a.abs().max().item(), 1.0)
+        torch.testing.assert_close(a.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
+        torch.testing.assert_close(rt.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)

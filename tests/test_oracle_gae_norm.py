@@ -184,3 +184,49 @@ def test_masked_normalization_closed_form():
     act = x[m.bool()].double()
     want = ((x.double() * m.double()) - act.mean()) / (act.std(unbiased=False) + 1e-5)
     torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- turn-level GAE
+def test_turn_level_gae_reference_literals():
+    # reference tests/test_ppo_gae.py:81-151 (inputs and expected values re-typed)
+    r = torch.tensor([[0.0, 1.0, 0.0, 2.0]])
+    a, rt = G.gae_turn_level(r, torch.zeros_like(r), torch.ones_like(r), torch.tensor([[0, 0, 1, 1]], dtype=torch.int32),
+                             torch.tensor([False]), 1.0, 0.5)
+    assert torch.equal(a, torch.tensor([[2.0, 2.0, 2.0, 2.0]])) and torch.equal(rt, a)
+    r = torch.tensor([[0.0, 3.0, 0.0, 0.0, 4.0]])
+    v = torch.tensor([[1.0, 5.0, 9.0, 2.0, 8.0]])
+    a, rt = G.gae_turn_level(r, v, torch.tensor([[1.0, 1.0, 0.0, 1.0, 1.0]]), torch.tensor([[0, 0, -1, 2, 2]]),
+                             torch.tensor([True]), 0.5, 0.25)
+    assert torch.equal(a, torch.tensor([[3.75, 3.75, 0.0, 6.0, 6.0]]))
+    assert torch.equal(rt, torch.tensor([[4.75, 4.75, 9.0, 8.0, 8.0]]))
+    r = torch.tensor([[0.0, 1.0, 0.0, 2.0], [0.0, 1.0, 0.0, 2.0]])
+    a, _ = G.gae_turn_level(r, torch.zeros_like(r), torch.ones_like(r),
+                            torch.tensor([[0, 0, 1, 1], [0, 0, 1, 1]], dtype=torch.int32),
+                            torch.tensor([False, False]), 1.0, torch.tensor([0.5, 0.0]))
+    assert torch.equal(a, torch.tensor([[2.0, 2.0, 2.0, 2.0], [1.0, 1.0, 2.0, 2.0]]))
+
+
+@pytest.mark.parametrize("ids,message", [([-1, 0, 0, 1], "non-negative"), ([0, 0, 4, 4], "smaller than the sequence length"),
+                                         ([0, 1, 0, 2], "temporally nondecreasing")])
+def test_turn_level_gae_rejects_malformed_ids(ids, message):
+    # reference tests/test_ppo_gae.py:511-532
+    r = torch.zeros(1, 4)
+    with pytest.raises(RuntimeError, match=message):
+        G.gae_turn_level(r, r, torch.ones_like(r), torch.tensor([ids]), torch.tensor([False]), 1.0, 1.0)
+    with pytest.raises(ValueError, match="integer dtype"):
+        G.gae_turn_level(r, r, torch.ones_like(r), torch.zeros(1, 4), torch.tensor([False]), 1.0, 1.0)
+
+
+def test_turn_level_gae_with_one_token_turns_is_token_level_gae():
+    # every active token its own turn: the turn recurrence is the token recurrence over the
+    # active tokens (value of the next ACTIVE token), which gae_padded computes as well
+    g = torch.Generator().manual_seed(4)
+    bs, L = 3, 40
+    r, v = torch.randn(bs, L, generator=g), torch.randn(bs, L, generator=g)
+    m = (torch.rand(bs, L, generator=g) > 0.3).float()
+    m[:, -1] = 0
+    ids = torch.arange(L).expand(bs, -1).clone()
+    ne = torch.tensor([True, False, True])
+    a, _ = G.gae_turn_level(r, v, m, ids, ne, 0.9, 0.8)
+    want, _ = G.gae_padded(r, v, m, ne, 0.9, 0.8)
+    torch.testing.assert_close(a, want * m, rtol=1e-5, atol=1e-6)
