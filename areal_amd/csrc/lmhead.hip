@@ -1025,12 +1025,20 @@ Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixe
 
 // EpiT<EDGE>; ep_edge_a is the parameter block of the ragged-A launch (it may differ from ep in
 // where it writes its partial results).
-template <template <bool> class EpiT, class P, int FAST_KERNEL = KERNEL_NT>
+// MERGE_EDGES: epilogues whose bounds predicates are cheap (plain stores) run ONE launch of the
+// EDGE = true instance over all tiles when any tile is ragged: a separate launch for the last
+// row of tiles has too few workgroups to fill the chip and each walks the whole K range.
+template <template <bool> class EpiT, class P, int FAST_KERNEL = KERNEL_NT, bool MERGE_EDGES = false>
 int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_edge_a,
                 hipStream_t stream) {
   int rc;
   if (!r.fast)
     return launch_region<EpiT<true>, KERNEL_GENERIC>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
+  if (MERGE_EDGES && (r.ragged_a || r.ragged_b)) {
+    const int nai = r.nai_full + (r.ragged_a ? 1 : 0);
+    return launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), 0, nai,
+                                                  r.S == r.nai_full ? nai : r.S, ep, stream);
+  }
   if ((rc = launch_region<EpiT<false>, FAST_KERNEL>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_b &&
@@ -1076,9 +1084,9 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0, 0};
   const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
   const StoreParams ep{out, ldo, (int)M, (int)N};
-  if (out_mode == 0) return launch_gemm<StoreBf16>(g, r, ep, ep, stream);
-  if (out_mode == 1) return launch_gemm<StoreF32>(g, r, ep, ep, stream);
-  return launch_gemm<AccumF32>(g, r, ep, ep, stream);
+  if (out_mode == 0) return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  if (out_mode == 1) return launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  return launch_gemm<AccumF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
 }
 
 static Regions fwd_regions(int64_t T, int64_t H, int64_t V) { return plan_regions(V, T, H, 512, 0); }
@@ -1229,15 +1237,15 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv, 0, 0, 0};
       const StoreParams ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc};
       const Regions r = plan_regions(H, Tc, ldv, 0, 1 << 20);
-      if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+      if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
     }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
     if (tn) {
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv, (int)Tc};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
-      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
-                                  : launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
+      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
+                                  : launch_gemm<StoreF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream);
       if (rc != AREAL_OK) return rc;
     } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -1247,8 +1255,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
-      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32>(g, r, ep, ep, stream)
-                                  : launch_gemm<StoreF32>(g, r, ep, ep, stream);
+      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)
+                                  : launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
       if (rc != AREAL_OK) return rc;
     }
   }
@@ -1307,16 +1315,16 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
     const StoreParams ep{dhidden, H, (int)H, (int)T};
     const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
-    if ((rc = launch_gemm<StoreBf16>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+    if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
   }
   if (dweight != nullptr) {
     // dWeight[v, h] += sum_t dl[t, v] * hidden[t, h], k-major over the Tpad rows of dl
     GemmArgs g{(const u16*)hidden, H, (int)H, dl, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
     const StoreParams ep{dweight, H, (int)H, (int)V};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
-    rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
-         : dweight_mode == 0 ? launch_gemm<StoreF32, StoreParams, KERNEL_TN>(g, r, ep, ep, stream)
-                             : launch_gemm<StoreBf16, StoreParams, KERNEL_TN>(g, r, ep, ep, stream);
+    rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
+         : dweight_mode == 0 ? launch_gemm<StoreF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
+                             : launch_gemm<StoreBf16, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream);
     if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;
