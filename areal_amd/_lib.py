@@ -73,6 +73,12 @@ SIGNATURES: dict[str, tuple] = {
         I,
         [P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, SZ, P],
     ),
+    "areal_seqlens_from_mask": (I, [P, I64, I64, P, P, P, P]),
+    "areal_pack_padded": (I, [P, P, P, I64, I64, I64, I64, P]),
+    "areal_unpack_to_padded": (I, [P, P, P, P, I64, I64, I64, P, I, P]),
+    "areal_realign_packed": (I, [P, P, P, I64, P, I64, I64, P, I, I, I64, P]),
+    "areal_masked_stats_workspace_bytes": (SZ, [I]),
+    "areal_masked_stats": (I, [P, P, I, I64, P, P, SZ, P]),
     "areal_turn_gae_workspace_bytes": (SZ, [I64, I64]),
     "areal_turn_gae": (I, [P, P, P, P, P, P, I64, I64, F, F, P, P, P, P, SZ, P]),
     "areal_group_norm_workspace_bytes": (SZ, [I64, I64]),

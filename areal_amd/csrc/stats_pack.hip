@@ -1,0 +1,331 @@
+// Data movement and logging reductions either side of the loss: packing padded [B, S] batches
+// into the packed layout by cu_seqlens and back, re-aligning a packed batch, and the masked
+// sum / count / min / max of many per-token statistics in one launch.
+//
+// Follows areal/utils/data.py: pack_tensor_dict (:496-545), pad_packed_tensor_dict (:822-982),
+// unpack_sequence + pad_and_stack_tensors_along_first_dim as used by reorder_and_pad_outputs
+// (areal/engine/core/train_engine.py:110-144); and areal/utils/stats_tracker.py: _avg_of,
+// _min_of, _max_of (:455-560), which reduce every logged tensor under its denominator mask.
+#include "common.hpp"
+
+namespace {
+
+constexpr int PK_THREADS = 256;
+
+DEVI int seq_of_cu(const int32_t* cu, int n_seqs, int64_t t) {
+  int lo = 0, hi = n_seqs;  // last s with cu[s] <= t
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if ((int64_t)cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// Copies `eb` bytes (one token's trailing dimensions) with the widest aligned access.
+DEVI void copy_elem(char* dst, const char* src, int64_t eb) {
+  if (((eb | (uintptr_t)dst | (uintptr_t)src) & 15) == 0) {
+    for (int64_t i = 0; i < eb; i += 16) *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
+  } else if (((eb | (uintptr_t)dst | (uintptr_t)src) & 3) == 0) {
+    for (int64_t i = 0; i < eb; i += 4) *(uint32_t*)(dst + i) = *(const uint32_t*)(src + i);
+  } else {
+    for (int64_t i = 0; i < eb; ++i) dst[i] = src[i];
+  }
+}
+DEVI void fill_elem(char* dst, const char* pattern, int pb, int64_t eb) {
+  for (int64_t i = 0; i < eb; ++i) dst[i] = pattern[i % pb];
+}
+
+// lens[b] = number of nonzero entries of mask row b (one block per row).
+__global__ __launch_bounds__(PK_THREADS) void rowlens_kernel(const uint8_t* mask, int64_t S,
+                                                             int32_t* lens) {
+  __shared__ int sm[4];
+  const uint8_t* row = mask + (int64_t)blockIdx.x * S;
+  int len = 0;
+  for (int64_t s = threadIdx.x; s < S; s += blockDim.x) len += row[s] != 0;
+  len = wave_sum(len);
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = len;
+  __syncthreads();
+  if (threadIdx.x == 0) lens[blockIdx.x] = sm[0] + sm[1] + sm[2] + sm[3];
+}
+// cu = exclusive prefix sums of lens, *max_len = max(lens) (one block).
+__global__ __launch_bounds__(PK_THREADS) void cu_scan_kernel(const int32_t* lens, int64_t B,
+                                                             int32_t* cu, int32_t* max_len) {
+  __shared__ int sm[PK_THREADS];
+  __shared__ int carry, mx;
+  if (threadIdx.x == 0) { carry = 0; mx = 0; cu[0] = 0; }
+  __syncthreads();
+  for (int64_t b0 = 0; b0 < B; b0 += PK_THREADS) {
+    const int64_t b = b0 + threadIdx.x;
+    const int len = b < B ? lens[b] : 0;
+    sm[threadIdx.x] = len;
+    __syncthreads();
+    for (int d = 1; d < PK_THREADS; d <<= 1) {
+      const int v = threadIdx.x >= d ? sm[threadIdx.x - d] : 0;
+      __syncthreads();
+      sm[threadIdx.x] += v;
+      __syncthreads();
+    }
+    if (b < B) {
+      cu[b + 1] = carry + sm[threadIdx.x];
+      atomicMax(&mx, len);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) carry += sm[PK_THREADS - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *max_len = mx;
+}
+
+// packed[cu[b] + j] = padded[b][j] for j < cu[b+1] - cu[b]   (pack = true)
+// padded[b][j] = j < len_b ? packed[cu[b] + j] : fill         (pack = false)
+__global__ __launch_bounds__(PK_THREADS) void pack_kernel(const char* padded, char* packed,
+                                                          const int32_t* cu, int n_seqs, int64_t S,
+                                                          int64_t eb, int64_t total) {
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int b = seq_of_cu(cu, n_seqs, t);
+    const int64_t j = t - cu[b];
+    copy_elem(packed + t * eb, padded + ((int64_t)b * S + j) * eb, eb);
+  }
+}
+struct Fill { char bytes[16]; int n; };
+__global__ __launch_bounds__(PK_THREADS) void unpack_kernel(const char* packed, char* padded,
+                                                            const int32_t* cu, const int32_t* row_seq,
+                                                            int64_t B, int64_t S, int64_t eb,
+                                                            Fill fill) {
+  const int64_t total = B * S;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / S, j = i - row * S;
+    const int64_t b = row_seq ? row_seq[row] : row;  // packed sequence shown in this row
+    const int64_t len = (int64_t)cu[b + 1] - cu[b];
+    if (j < len) copy_elem(padded + i * eb, packed + ((int64_t)cu[b] + j) * eb, eb);
+    else fill_elem(padded + i * eb, fill.bytes, fill.n, eb);
+  }
+}
+
+// dst[cu_new[s] + j] = j < old length of s ? src[cu_old[s] + j] : fill; sequences of cu_new
+// beyond n_old (a trailing pad segment) are all fill. arange != 0: dst is int64 position ids,
+// and the fill is j (position inside the new sequence) instead.
+__global__ __launch_bounds__(PK_THREADS) void realign_kernel(const char* src, char* dst,
+                                                             const int32_t* cu_old, int n_old,
+                                                             const int32_t* cu_new, int n_new,
+                                                             int64_t eb, Fill fill, int arange,
+                                                             int64_t total_new) {
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total_new;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int s = seq_of_cu(cu_new, n_new, t);
+    const int64_t j = t - cu_new[s];
+    const int64_t len = s < n_old ? (int64_t)cu_old[s + 1] - cu_old[s] : 0;
+    char* d = dst + t * eb;
+    if (j < len && src != nullptr) {
+      copy_elem(d, src + ((int64_t)cu_old[s] + j) * eb, eb);
+    } else if (arange) {
+      const int64_t v = (src == nullptr) ? j : j - len;  // whole-sequence arange, or pad arange
+      for (int64_t k = 0; k < eb; k += 8) *(int64_t*)(d + k) = v;
+    } else {
+      fill_elem(d, fill.bytes, fill.n, eb);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Masked statistics of K tensors in one launch.
+// ---------------------------------------------------------------------------------------
+constexpr int STATS_MAX_K = 32;
+constexpr int STATS_BLOCKS = 256;
+struct StatsArgs {
+  const float* v[STATS_MAX_K];
+  const uint8_t* m[STATS_MAX_K];  // denominator mask of tensor k (null: all ones)
+  int K;
+  int64_t n;
+};
+struct StatPart { double sum, cnt; float mn, mx; };
+
+DEVI double block_sum_d(double v, double* smem) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[w] = v;
+  __syncthreads();
+  double r = 0.0;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i];
+  return r;
+}
+DEVI float block_minmax(float v, float* smem, bool is_min) {
+  v = is_min ? wave_min(v) : wave_max(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) smem[w] = v;
+  __syncthreads();
+  float r = smem[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = is_min ? fminf(r, smem[i]) : fmaxf(r, smem[i]);
+  return r;
+}
+
+// grid (STATS_BLOCKS, K): partial over a slice of tensor blockIdx.y
+__global__ __launch_bounds__(PK_THREADS) void stats_partial_kernel(StatsArgs a, StatPart* parts) {
+  __shared__ double sm_d[4];
+  __shared__ float sm_f[4];
+  const int k = blockIdx.y;
+  const float* v = a.v[k];
+  const uint8_t* m = a.m[k];
+  double sum = 0.0, cnt = 0.0;
+  float mn = pos_inf(), mx = neg_inf();
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    if (m != nullptr && m[i] == 0) continue;
+    const float x = v[i];
+    sum += (double)x; cnt += 1.0;
+    mn = fminf(mn, x); mx = fmaxf(mx, x);
+  }
+  sum = block_sum_d(sum, sm_d);
+  cnt = block_sum_d(cnt, sm_d);
+  mn = block_minmax(mn, sm_f, true);
+  mx = block_minmax(mx, sm_f, false);
+  if (threadIdx.x == 0) parts[(int64_t)k * gridDim.x + blockIdx.x] = StatPart{sum, cnt, mn, mx};
+}
+// out[k] = {sum, count, min, max} (min = +inf, max = -inf when the mask is empty)
+__global__ __launch_bounds__(PK_THREADS) void stats_final_kernel(const StatPart* parts, int nparts,
+                                                                 double* out) {
+  __shared__ double sm_d[4];
+  __shared__ float sm_f[4];
+  const int k = blockIdx.x;
+  double sum = 0.0, cnt = 0.0;
+  float mn = pos_inf(), mx = neg_inf();
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    const StatPart p = parts[(int64_t)k * nparts + i];
+    sum += p.sum; cnt += p.cnt; mn = fminf(mn, p.mn); mx = fmaxf(mx, p.mx);
+  }
+  sum = block_sum_d(sum, sm_d);
+  cnt = block_sum_d(cnt, sm_d);
+  mn = block_minmax(mn, sm_f, true);
+  mx = block_minmax(mx, sm_f, false);
+  if (threadIdx.x == 0) {
+    out[4 * k] = sum; out[4 * k + 1] = cnt; out[4 * k + 2] = (double)mn; out[4 * k + 3] = (double)mx;
+  }
+}
+
+int pk_grid(int64_t n) {
+  int64_t b = ceil_div_i64(n, PK_THREADS);
+  if (b > 65535) b = 65535;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+bool make_fill(const void* fill, int fill_bytes, Fill& f) {
+  if (fill_bytes < 0 || fill_bytes > 16) return false;
+  f.n = fill_bytes > 0 ? fill_bytes : 1;
+  for (int i = 0; i < 16; ++i) f.bytes[i] = 0;
+  if (fill_bytes > 0 && fill != nullptr)
+    for (int i = 0; i < fill_bytes; ++i) f.bytes[i] = ((const char*)fill)[i];
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+// attention_mask [B, S] bytes (nonzero = token) -> lens [B], cu_seqlens [B+1], *max_len, all
+// int32 on the device (data.py:513-517).
+int areal_seqlens_from_mask(const uint8_t* attention_mask, int64_t B, int64_t S, int32_t* lens,
+                            int32_t* cu_seqlens, int32_t* max_len, hipStream_t stream) {
+  if (B < 0 || S < 0) return AREAL_ERR_BAD_ARG;
+  if (!cu_seqlens || !max_len || (B > 0 && (!attention_mask || !lens))) return AREAL_ERR_BAD_ARG;
+  if (B > (1 << 30) || B * S >= ((int64_t)1 << 31)) return AREAL_ERR_UNSUPPORTED;
+  if (B > 0) {
+    hipLaunchKernelGGL(rowlens_kernel, dim3((unsigned)B), dim3(PK_THREADS), 0, stream,
+                       attention_mask, S, lens);
+    AREAL_CHECK_LAUNCH();
+  }
+  hipLaunchKernelGGL(cu_scan_kernel, dim3(1), dim3(PK_THREADS), 0, stream, lens, B, cu_seqlens,
+                     max_len);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// packed [total, E] <- the first len_b tokens of every row of padded [B, S, E]; elem_bytes = bytes
+// of one token's trailing dimensions (data.py:535-541).
+int areal_pack_padded(const void* padded, void* packed, const int32_t* cu_seqlens, int64_t B,
+                      int64_t S, int64_t elem_bytes, int64_t total, hipStream_t stream) {
+  if (B < 0 || S < 0 || elem_bytes <= 0 || total < 0) return AREAL_ERR_BAD_ARG;
+  if (total == 0) return AREAL_OK;
+  if (!padded || !packed || !cu_seqlens || B == 0) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(pack_kernel, dim3(pk_grid(total)), dim3(PK_THREADS), 0, stream,
+                     (const char*)padded, (char*)packed, cu_seqlens, (int)B, S, elem_bytes, total);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// padded [B, S, E] <- packed sequences, the rest filled with the fill pattern (fill_bytes <= 16
+// bytes repeated over the element; NULL = zero bytes): unpack_sequence + reorder_list +
+// pad_and_stack. row_seq [B] (nullable): row r shows packed sequence row_seq[r].
+int areal_unpack_to_padded(const void* packed, void* padded, const int32_t* cu_seqlens,
+                           const int32_t* row_seq, int64_t B, int64_t S, int64_t elem_bytes,
+                           const void* fill, int fill_bytes, hipStream_t stream) {
+  if (B < 0 || S < 0 || elem_bytes <= 0) return AREAL_ERR_BAD_ARG;
+  if (B == 0 || S == 0) return AREAL_OK;
+  if (!padded || !cu_seqlens) return AREAL_ERR_BAD_ARG;
+  Fill f;
+  if (!make_fill(fill, fill_bytes, f)) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(unpack_kernel, dim3(pk_grid(B * S)), dim3(PK_THREADS), 0, stream,
+                     (const char*)packed, (char*)padded, cu_seqlens, row_seq, B, S, elem_bytes, f);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// Re-layout of a packed batch (data.py:848-911, :927-969): sequence s moves from cu_old to
+// cu_new (new length >= old length, the tail filled); cu_new may hold extra trailing
+// sequences (the batch pad), filled entirely. position_ids != 0: elem_bytes is a multiple of 8
+// (int64 channels); src == NULL writes 0..len-1 per new sequence, otherwise the pads continue
+// with 0, 1, 2, ... after the copied part.
+int areal_realign_packed(const void* src, void* dst, const int32_t* cu_old, int64_t n_old,
+                         const int32_t* cu_new, int64_t n_new, int64_t elem_bytes,
+                         const void* fill, int fill_bytes, int position_ids, int64_t total_new,
+                         hipStream_t stream) {
+  if (n_old < 0 || n_new < 0 || elem_bytes <= 0 || total_new < 0) return AREAL_ERR_BAD_ARG;
+  if (total_new == 0) return AREAL_OK;
+  if (!dst || !cu_new || n_new == 0 || (n_old > 0 && !cu_old)) return AREAL_ERR_BAD_ARG;
+  if (position_ids && (elem_bytes % 8 != 0 || ((uintptr_t)dst & 7))) return AREAL_ERR_ALIGNMENT;
+  if (!position_ids && src == nullptr && n_old > 0) return AREAL_ERR_BAD_ARG;
+  Fill f;
+  if (!make_fill(fill, fill_bytes, f)) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(realign_kernel, dim3(pk_grid(total_new)), dim3(PK_THREADS), 0, stream,
+                     (const char*)src, (char*)dst, cu_old, (int)n_old, cu_new, (int)n_new,
+                     elem_bytes, f, position_ids, total_new);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+size_t areal_masked_stats_workspace_bytes(int K) {
+  if (K <= 0) return 0;
+  return (size_t)K * STATS_BLOCKS * sizeof(StatPart) + 256;
+}
+
+// out [K][4] double = {sum, count, min, max} of values[k][i] over mask[k][i] != 0 (mask[k] NULL:
+// every element). values / masks are HOST arrays of K device pointers, K <= 32.
+int areal_masked_stats(const float* const* values, const uint8_t* const* masks, int K, int64_t n,
+                       double* out, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (K < 0 || K > STATS_MAX_K || n < 0) return AREAL_ERR_BAD_ARG;
+  if (K == 0) return AREAL_OK;
+  if (!values || !masks || !out) return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_masked_stats_workspace_bytes(K))
+    return AREAL_ERR_WORKSPACE;
+  StatsArgs a;
+  a.K = K; a.n = n;
+  for (int k = 0; k < STATS_MAX_K; ++k) { a.v[k] = nullptr; a.m[k] = nullptr; }
+  for (int k = 0; k < K; ++k) {
+    if (values[k] == nullptr && n > 0) return AREAL_ERR_BAD_ARG;
+    a.v[k] = values[k]; a.m[k] = masks[k];
+  }
+  StatPart* parts = (StatPart*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  int blocks = (int)ceil_div_i64(n > 0 ? n : 1, PK_THREADS * 8);
+  if (blocks > STATS_BLOCKS) blocks = STATS_BLOCKS;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(stats_partial_kernel, dim3(blocks, K), dim3(PK_THREADS), 0, stream, a, parts);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(stats_final_kernel, dim3(K), dim3(PK_THREADS), 0, stream, parts, blocks, out);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+}  // extern "C"

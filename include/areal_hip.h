@@ -251,6 +251,37 @@ size_t areal_masked_norm_workspace_bytes(int64_t n);
 int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased, double eps,
                       float* out, void* workspace, size_t workspace_bytes, areal_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Packing / padding by cu_seqlens and masked logging statistics (the steps either side of the
+ * loss). Replace the per-sequence Python loops of pack_tensor_dict (areal/utils/data.py:496-545),
+ * pad_packed_tensor_dict (:822-982), unpack_sequence + reorder_list +
+ * pad_and_stack_tensors_along_first_dim as composed by reorder_and_pad_outputs
+ * (areal/engine/core/train_engine.py:110-144), and the per-tensor torch.where(...).sum() / min /
+ * max of stats_tracker (areal/utils/stats_tracker.py:455-560).
+ * elem_bytes = bytes of one token's trailing dimensions; fill = up to 16 bytes repeated over an
+ * element (NULL = zeros).
+ * ------------------------------------------------------------------------------------- */
+int areal_seqlens_from_mask(const uint8_t* attention_mask, int64_t B, int64_t S, int32_t* lens,
+                            int32_t* cu_seqlens, int32_t* max_len, areal_stream_t stream);
+int areal_pack_padded(const void* padded, void* packed, const int32_t* cu_seqlens, int64_t B,
+                      int64_t S, int64_t elem_bytes, int64_t total, areal_stream_t stream);
+int areal_unpack_to_padded(const void* packed, void* padded, const int32_t* cu_seqlens,
+                           const int32_t* row_seq, int64_t B, int64_t S, int64_t elem_bytes,
+                           const void* fill, int fill_bytes, areal_stream_t stream);
+/* Sequence s moves from cu_old to cu_new (new length >= old, tail filled); sequences of cu_new
+ * beyond n_old are all fill. position_ids != 0 (int64 elements): src NULL writes 0..len-1 per
+ * new sequence, otherwise the filled parts count 0, 1, 2, ... */
+int areal_realign_packed(const void* src, void* dst, const int32_t* cu_old, int64_t n_old,
+                         const int32_t* cu_new, int64_t n_new, int64_t elem_bytes,
+                         const void* fill, int fill_bytes, int position_ids, int64_t total_new,
+                         areal_stream_t stream);
+size_t areal_masked_stats_workspace_bytes(int K);
+/* out [K][4] double = {sum, count, min, max} of values[k] where masks[k] != 0 (NULL mask: all).
+ * values / masks are HOST arrays of K <= 32 device pointers. */
+int areal_masked_stats(const float* const* values, const uint8_t* const* masks, int K, int64_t n,
+                       double* out, void* workspace, size_t workspace_bytes,
+                       areal_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
