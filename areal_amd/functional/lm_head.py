@@ -15,7 +15,7 @@ Two ways of carrying state to the backward:
   tensor (2 bytes per logit), the backward turns them into dlogits in place and skips the
   recomputation, a quarter of the step's matrix work.  The reference's logits-in path saves
   the same amount through autograd; 288 GB of HBM make it the default while it fits
-  ``SAVE_PROBS_BYTES_LIMIT``.
+  ``SAVE_PROBS_BYTES_LIMIT`` and 60 % of the memory still available.
 """
 
 from __future__ import annotations
@@ -38,6 +38,13 @@ SAVE_PROBS_BYTES_LIMIT = 40 << 30
 
 def _round_up(x: int, m: int) -> int:
     return (x + m - 1) // m * m
+
+
+def _available_bytes(dev: torch.device) -> int:
+    """Device memory the allocator can still hand out: free on the device plus what the caching
+    allocator holds but has not given to a tensor."""
+    free, _ = torch.cuda.mem_get_info(dev)
+    return free + torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
 
 
 class ChunkedLMHeadOutput(NamedTuple):
@@ -86,7 +93,8 @@ class _FusedLMHead(torch.autograd.Function):
         logprobs, entropy, vmin, vmax, vmean, vnorm, row_max, sum_exp = outs
         needs_grad = any(ctx.needs_input_grad[:2])  # the caller has ruled out no_grad mode
         if save_probs is None:
-            save_probs = 2 * _round_up(T, 64) * _round_up(V, 64) <= SAVE_PROBS_BYTES_LIMIT
+            need = 2 * _round_up(T, 64) * _round_up(V, 64)
+            save_probs = need <= SAVE_PROBS_BYTES_LIMIT and need <= 0.6 * _available_bytes(dev)
         probs = probs_ref = None
         if save_probs and needs_grad and T > 0:
             probs = torch.empty(
