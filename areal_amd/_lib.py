@@ -66,6 +66,8 @@ SIGNATURES: dict[str, tuple] = {
         [P, P, P, P, P, I64, I64, I64, F, F, I, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
     "areal_critic_loss": (I, [P, P, P, P, I64, F, I, P, P, P, P, P, P, SZ, P]),
+    "areal_m2po_mask_workspace_bytes": (SZ, [I64]),
+    "areal_m2po_mask": (I, [P, P, P, I64, F, P, P, SZ, P]),
     "areal_dpo_seq_logps": (I, [P, P, P, P, I64, I64, P, P, P]),
     "areal_dpo_seq_logps_grad": (I, [P, P, P, I64, I64, P, P]),
     "areal_gae_workspace_bytes": (SZ, [I64]),

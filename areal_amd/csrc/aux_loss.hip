@@ -283,6 +283,156 @@ __global__ __launch_bounds__(AUX_THREADS) void dpo_seq_grad_kernel(const double*
     grad_lp[t] = shifted_mask[t] ? (float)grad_seq[seq_of(seq, t)] : 0.0f;
 }
 
+
+// ---------------------------------------------------------------------------------------
+// M2PO second-moment mask (areal/trainer/ppo/actor.py:933-1014): among the tokens of the loss
+// mask, drop the tokens with the largest m2 = (old - prox)^2 until the mean m2 of the rest is
+// below the threshold (always keeping at least one). The reference sorts; here the cut is found
+// by a 4 x 8-bit radix select over the bit patterns of m2 (non-negative floats order like
+// unsigned integers): every pass builds a 256-bin (count, sum) histogram of the still undecided
+// tokens and a single thread walks the bins upwards, keeping whole bins while the running mean
+// stays below the threshold and descending into the first bin that would break it. The mean of
+// the j smallest values is non-decreasing in j, so the kept set is a prefix of the ascending
+// order. Ties at the cut value are kept in index order.
+// ---------------------------------------------------------------------------------------
+constexpr int M2_BLOCKS = 512;
+struct M2State {
+  unsigned int prefix;          // decided high bits of the cut value
+  int all_kept;                 // every token kept: nothing to cut
+  unsigned long long kept;      // tokens strictly below the undecided range
+  double kept_sum;
+  unsigned long long group;     // after the last pass: tokens equal to the cut value
+  unsigned long long take;      // ... and how many of them are kept
+};
+DEVI unsigned int m2_key(const float* old, const float* prox, int64_t t) {
+  const float d = old[t] - prox[t];
+  return __float_as_uint(d * d) & 0x7fffffffu;
+}
+__global__ void m2_init_kernel(M2State* st) {
+  st->prefix = 0; st->all_kept = 0; st->kept = 0; st->kept_sum = 0.0; st->group = 0; st->take = 0;
+}
+// pass with `shift` in {24, 16, 8, 0}: histogram of bits [shift, shift+8) over the tokens whose
+// higher bits equal the prefix
+__global__ __launch_bounds__(AUX_THREADS) void m2_hist_kernel(const float* old, const float* prox,
+                                                              const uint8_t* mask, int64_t n, int shift,
+                                                              const M2State* st, unsigned int* part_cnt,
+                                                              double* part_sum) {
+  __shared__ unsigned int h_cnt[256];
+  __shared__ double h_sum[256];
+  h_cnt[threadIdx.x] = 0; h_sum[threadIdx.x] = 0.0;
+  __syncthreads();
+  const unsigned int prefix = st->prefix;
+  const bool skip = st->all_kept != 0;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n && !skip;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    if (mask[t] == 0) continue;
+    const unsigned int key = m2_key(old, prox, t);
+    if (shift < 24 && (key >> (shift + 8)) != (prefix >> (shift + 8))) continue;
+    const unsigned int b = (key >> shift) & 255u;
+    atomicAdd(&h_cnt[b], 1u);
+    atomicAdd(&h_sum[b], (double)__uint_as_float(key));
+  }
+  __syncthreads();
+  part_cnt[(int64_t)blockIdx.x * 256 + threadIdx.x] = h_cnt[threadIdx.x];
+  part_sum[(int64_t)blockIdx.x * 256 + threadIdx.x] = h_sum[threadIdx.x];
+}
+__global__ __launch_bounds__(AUX_THREADS) void m2_select_kernel(const unsigned int* part_cnt,
+                                                                const double* part_sum, int nparts,
+                                                                int shift, double thr, M2State* st) {
+  __shared__ unsigned long long cnt[256];
+  __shared__ double sum[256];
+  unsigned long long c = 0; double s = 0.0;
+  for (int i = 0; i < nparts; ++i) {
+    c += part_cnt[(int64_t)i * 256 + threadIdx.x];
+    s += part_sum[(int64_t)i * 256 + threadIdx.x];
+  }
+  cnt[threadIdx.x] = c; sum[threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.x != 0 || st->all_kept) return;
+  unsigned long long C = st->kept; double S = st->kept_sum;
+  int cut = -1;
+  for (int b = 0; b < 256; ++b) {
+    if (cnt[b] == 0) continue;
+    const double mean = (S + sum[b]) / (double)(C + cnt[b]);
+    if (mean < thr) { C += cnt[b]; S += sum[b]; }
+    else { cut = b; break; }
+  }
+  if (cut < 0) { st->all_kept = 1; return; }
+  st->kept = C; st->kept_sum = S;
+  st->prefix |= (unsigned int)cut << shift;
+  if (shift == 0) {
+    // tokens equal to the cut value v: keep the largest r with (S + r v) / (C + r) < thr
+    const unsigned long long g = cnt[cut];
+    const double v = (double)__uint_as_float(st->prefix);
+    unsigned long long r = 0;
+    for (unsigned long long lo = 0, hi = g; lo < hi;) {  // bisection on r (the mean is monotone in r)
+      const unsigned long long mid = lo + (hi - lo + 1) / 2;
+      if ((S + (double)mid * v) / (double)(C + mid) < thr) { lo = mid; r = mid; } else { hi = mid - 1; }
+    }
+    if (C + r == 0) r = 1;  // the reference keeps one token when no suffix mean is below
+    st->group = g; st->take = r;
+  }
+}
+// rank of the tokens equal to the cut value, in index order: per-block counts, then offsets
+__global__ __launch_bounds__(AUX_THREADS) void m2_tie_count_kernel(const float* old, const float* prox,
+                                                                   const uint8_t* mask, int64_t n,
+                                                                   int64_t per_block, const M2State* st,
+                                                                   unsigned long long* block_eq) {
+  __shared__ unsigned long long sm[8];
+  const int64_t t0 = (int64_t)blockIdx.x * per_block;
+  const int64_t t1 = t0 + per_block < n ? t0 + per_block : n;
+  unsigned long long c = 0;
+  if (!st->all_kept)
+    for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x)
+      c += (mask[t] != 0 && m2_key(old, prox, t) == st->prefix);
+  c = block_sum(c, sm);
+  if (threadIdx.x == 0) block_eq[blockIdx.x] = c;
+}
+__global__ __launch_bounds__(AUX_THREADS) void m2_apply_kernel(const float* old, const float* prox,
+                                                               const uint8_t* mask, int64_t n,
+                                                               int64_t per_block, int nblocks,
+                                                               const M2State* st,
+                                                               const unsigned long long* block_eq,
+                                                               uint8_t* new_mask) {
+  __shared__ unsigned long long sm_scan[AUX_THREADS];
+  const int64_t t0 = (int64_t)blockIdx.x * per_block;
+  const int64_t t1 = t0 + per_block < n ? t0 + per_block : n;
+  if (st->all_kept) {
+    for (int64_t t = t0 + threadIdx.x; t < t1; t += blockDim.x) new_mask[t] = mask[t] != 0;
+    return;
+  }
+  const unsigned int vstar = st->prefix;
+  const unsigned long long take = st->take;
+  unsigned long long before = 0;  // equal tokens in earlier blocks
+  for (int i = 0; i < (int)blockIdx.x; ++i) before += block_eq[i];
+  // each thread owns a contiguous slice of the block's range, so ranks follow the index order
+  const int64_t len = t1 - t0;
+  const int64_t per_thread = (len + blockDim.x - 1) / blockDim.x;
+  const int64_t a = t0 + (int64_t)threadIdx.x * per_thread;
+  const int64_t b = a + per_thread < t1 ? a + per_thread : t1;
+  unsigned long long mine = 0;
+  for (int64_t t = a; t < b; ++t) mine += (mask[t] != 0 && m2_key(old, prox, t) == vstar);
+  sm_scan[threadIdx.x] = mine;
+  __syncthreads();
+  for (int d = 1; d < AUX_THREADS; d <<= 1) {
+    const unsigned long long v = (int)threadIdx.x >= d ? sm_scan[threadIdx.x - d] : 0;
+    __syncthreads();
+    sm_scan[threadIdx.x] += v;
+    __syncthreads();
+  }
+  unsigned long long rank = before + sm_scan[threadIdx.x] - mine;
+  for (int64_t t = a; t < b; ++t) {
+    bool keep = false;
+    if (mask[t] != 0) {
+      const unsigned int key = m2_key(old, prox, t);
+      if (key < vstar) keep = true;
+      else if (key == vstar) { keep = rank < take; ++rank; }
+    }
+    new_mask[t] = keep;
+  }
+  (void)nblocks;
+}
+
 }  // namespace
 
 extern "C" {
@@ -382,6 +532,53 @@ int areal_dpo_seq_logps_grad(const double* grad_seq, const uint8_t* shifted_mask
   hipLaunchKernelGGL(dpo_seq_grad_kernel, dim3(aux_grid(n_tokens)), dim3(AUX_THREADS), 0, stream,
                      grad_seq, shifted_mask, SeqLayout{cu_seqlens, (int)n_seqs, 0}, n_tokens,
                      grad_logprobs);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+size_t areal_m2po_mask_workspace_bytes(int64_t n_tokens) {
+  (void)n_tokens;
+  return sizeof(M2State) + (size_t)M2_BLOCKS * 256 * (sizeof(unsigned int) + sizeof(double)) +
+         (size_t)M2_BLOCKS * sizeof(unsigned long long) + 1024;
+}
+
+// new_mask[t] = loss_mask[t] and token t is not among the largest-m2 tokens that have to go for
+// the mean of m2 = (old - prox)^2 over the rest to fall below m2_threshold (at least one token
+// of a non-empty mask is kept).
+int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
+                    const uint8_t* loss_mask, int64_t n_tokens, float m2_threshold,
+                    uint8_t* new_mask, void* workspace, size_t workspace_bytes,
+                    hipStream_t stream) {
+  if (n_tokens < 0) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!old_logprobs || !proximal_logprobs || !loss_mask || !new_mask) return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_m2po_mask_workspace_bytes(n_tokens))
+    return AREAL_ERR_WORKSPACE;
+  char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  M2State* st = (M2State*)wp;
+  double* part_sum = (double*)(wp + 256);
+  unsigned int* part_cnt = (unsigned int*)(part_sum + (size_t)M2_BLOCKS * 256);
+  unsigned long long* block_eq = (unsigned long long*)(part_cnt + (size_t)M2_BLOCKS * 256);
+  int blocks = (int)ceil_div_i64(n_tokens, AUX_THREADS * 4);
+  if (blocks > M2_BLOCKS) blocks = M2_BLOCKS;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(m2_init_kernel, dim3(1), dim3(1), 0, stream, st);
+  AREAL_CHECK_LAUNCH();
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    hipLaunchKernelGGL(m2_hist_kernel, dim3(blocks), dim3(AUX_THREADS), 0, stream, old_logprobs,
+                       proximal_logprobs, loss_mask, n_tokens, shift, st, part_cnt, part_sum);
+    AREAL_CHECK_LAUNCH();
+    hipLaunchKernelGGL(m2_select_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, part_cnt, part_sum,
+                       blocks, shift, (double)m2_threshold, st);
+    AREAL_CHECK_LAUNCH();
+  }
+  const int64_t per_block = ceil_div_i64(n_tokens, blocks);
+  hipLaunchKernelGGL(m2_tie_count_kernel, dim3(blocks), dim3(AUX_THREADS), 0, stream, old_logprobs,
+                     proximal_logprobs, loss_mask, n_tokens, per_block, st, block_eq);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(m2_apply_kernel, dim3(blocks), dim3(AUX_THREADS), 0, stream, old_logprobs,
+                     proximal_logprobs, loss_mask, n_tokens, per_block, blocks, st, block_eq,
+                     new_mask);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

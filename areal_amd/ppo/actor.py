@@ -16,6 +16,8 @@ import torch
 
 from areal_amd.config import RejectionSamplingConfig
 from areal_amd.data import KLEstimator, Normalization
+from areal_amd import _lib
+from areal_amd.functional.aux_losses import sapo_loss_fn
 from areal_amd.functional.functional import cispo_loss_fn, ppo_actor_loss_fn
 from areal_amd.ppo.gae import _compute_token_level_gae
 
@@ -51,16 +53,7 @@ def grpo_loss_fn(
     ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``:
     bool denominators and fp32 statistics, all of the micro-batch's token shape.
     """
-    del current_version, sapo_tau_pos, sapo_tau_neg, use_decoupled_loss
-    if m2_threshold is not None:
-        raise NotImplementedError("M2PO masking is not part of this path")
-    if use_sapo_loss:
-        if use_cispo_loss:
-            raise ValueError(
-                "CISPO and SAPO are mutually exclusive surrogates. "
-                "Set at most one of use_cispo_loss / use_sapo_loss."
-            )
-        raise NotImplementedError("the SAPO surrogate is not part of this path")
+    del current_version
     if input_data.get("teacher_logp") is not None:
         raise NotImplementedError("distillation terms are not part of this path")
 
@@ -85,7 +78,15 @@ def grpo_loss_fn(
             "This indicates computation failed."
         )
 
+    if m2_threshold is not None:
+        loss_mask = _apply_m2po_masking(old_logp, prox_logp, loss_mask, m2_threshold)
+
     if use_cispo_loss:
+        if use_sapo_loss:
+            raise ValueError(
+                "CISPO and SAPO are mutually exclusive surrogates. "
+                "Set at most one of use_cispo_loss / use_sapo_loss."
+            )
         if importance_sampling_level != "token":
             raise ValueError(
                 "CISPO only supports importance_sampling_level='token'. "
@@ -100,6 +101,22 @@ def grpo_loss_fn(
             loss_mask=loss_mask,
             old_logprobs=old_logp,
             rejection_sampling=rejection_sampling,
+            cu_seqlens=input_data.get("cu_seqlens"),
+        )
+    elif use_sapo_loss:
+        if use_decoupled_loss:
+            raise ValueError(
+                "SAPO is not compatible with `use_decoupled_loss=True`. "
+                "Please set `actor.use_decoupled_loss=false` in your configuration."
+            )
+        loss, stat = sapo_loss_fn(
+            logprobs=logprobs,
+            old_logprobs=old_logp,
+            advantages=advantages,
+            tau_pos=sapo_tau_pos,
+            tau_neg=sapo_tau_neg,
+            loss_mask=loss_mask,
+            importance_sampling_level=importance_sampling_level,
             cu_seqlens=input_data.get("cu_seqlens"),
         )
     else:
@@ -149,11 +166,46 @@ def grpo_loss_fn(
             stats["scalar/rs_filtered_fraction"] = stat["filtered_fraction"]
         if vocab_min_logits is not None and vocab_max_logits is not None:
             stats.update(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits)
+        if use_sapo_loss:
+            stats.update(
+                sapo_soft_gate=stat["sapo_soft_gate"],
+                sapo_scaled_gate_pos=stat["sapo_scaled_gate_pos"],
+                sapo_scaled_gate_neg=stat["sapo_scaled_gate_neg"],
+            )
         if vocab_mean_logits is not None:
             stats["vocab_mean_logits"] = vocab_mean_logits
         if vocab_norm_logits is not None:
             stats["vocab_norm_logits"] = vocab_norm_logits
     return loss
+
+
+def _apply_m2po_masking(
+    old_logp: torch.Tensor,
+    prox_logp: torch.Tensor,
+    loss_mask: torch.Tensor,
+    m2_threshold: float,
+) -> torch.Tensor:
+    """M2PO (second-moment PPO) masking: drop the tokens with the largest
+    ``(old_logp - prox_logp)**2`` until the mean over the remaining masked tokens is below
+    ``m2_threshold``; at least one token of a non-empty mask stays
+    (``areal/trainer/ppo/actor.py:933-1014``).  The reference sorts; the kernel finds the cut
+    with a radix select, and keeps tokens that tie at the cut value in index order."""
+    lib = _lib.load()
+    mask_bool = loss_mask.detach().bool().contiguous().view(-1)
+    old = old_logp.detach().to(torch.float32).contiguous().view(-1)
+    prox = prox_logp.detach().to(torch.float32).contiguous().view(-1)
+    dev = _lib.require_gpu(old, prox, mask_bool)
+    n = int(mask_bool.numel())
+    out = torch.empty(n, dtype=torch.bool, device=dev)
+    if n > 0:
+        nbytes = lib.areal_m2po_mask_workspace_bytes(n)
+        ws = _lib.workspace(nbytes, dev)
+        rc = lib.areal_m2po_mask(
+            _lib.ptr(old), _lib.ptr(prox), _lib.ptr(mask_bool), n, float(m2_threshold),
+            _lib.ptr(out), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_m2po_mask")
+    return out.view_as(loss_mask)
 
 
 def compute_advantages(

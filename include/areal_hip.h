@@ -194,6 +194,16 @@ int areal_critic_loss(const float* value, const float* old_value, const float* t
                       double* counters, void* workspace, size_t workspace_bytes,
                       areal_stream_t stream);
 
+/* M2PO second-moment mask (_apply_m2po_masking, areal/trainer/ppo/actor.py:933-1014): new_mask =
+ * loss_mask minus the largest-m2 tokens (m2 = (old - prox)^2) that have to go for the mean m2 of
+ * the rest to fall below m2_threshold; one token of a non-empty mask always stays. Found by a
+ * radix select over the bit patterns of m2 instead of the reference's sort. */
+size_t areal_m2po_mask_workspace_bytes(int64_t n_tokens);
+int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
+                    const uint8_t* loss_mask, int64_t n_tokens, float m2_threshold,
+                    uint8_t* new_mask, void* workspace, size_t workspace_bytes,
+                    areal_stream_t stream);
+
 /* seq_sums [n_seqs][3] double = {sum policy log-probs, sum reference log-probs, count} over
  * shifted_mask[t] = loss_mask[t+1] inside each packed sequence (its last token excluded);
  * shifted_mask [n_tokens] is written for the backward. */

@@ -111,3 +111,32 @@ def dpo_preference_loss(logits, *, beta, loss_type="sigmoid"):
     if loss_type == "ipo":
         return (logits.float() - 1.0 / (2.0 * beta)) ** 2
     raise ValueError(f"Unsupported DPO loss_type: {loss_type!r}")
+
+
+def m2po_mask(old_logp, prox_logp, loss_mask, m2_threshold):
+    """_apply_m2po_masking + _get_m2po_loss_mask (areal/trainer/ppo/actor.py:933-1014): sort the
+    masked tokens by m2 = (old - prox)^2 descending and drop the largest until the mean of the
+    rest is below the threshold (at least one token stays).
+
+    The reference has no test for it ("parity unpinned" against the reference). Pinned by
+    hand-computed cases (tests/test_oracle_aux_loss.py) and by the defining property checked
+    with brute force: the kept set is the largest set of smallest-m2 tokens whose mean is below
+    the threshold, or the single smallest token when no such set exists."""
+    delta = old_logp - prox_logp
+    m2 = delta * delta
+    flat = loss_mask.reshape(-1).bool()
+    sel = m2.reshape(-1)[flat]
+    if sel.numel() == 0:
+        return loss_mask
+    sorted_m2, indices = torch.sort(sel, descending=True)
+    restored = torch.argsort(indices)
+    n = sorted_m2.numel()
+    suffix = sorted_m2.flip(0).cumsum(0).flip(0)
+    counts = torch.arange(n, 0, -1, dtype=sorted_m2.dtype)
+    below = torch.where(suffix / counts < m2_threshold)[0]
+    num_to_mask = int(below[0]) if len(below) > 0 else n - 1
+    keep_sorted = torch.ones(n, dtype=torch.bool)
+    keep_sorted[:num_to_mask] = False
+    full = torch.zeros_like(flat)
+    full[flat] = keep_sorted[restored]
+    return full.view_as(loss_mask)

@@ -132,3 +132,56 @@ def test_dpo_pair_logratios_matches_oracle(dev):
     dpo(wp, wr).backward()
     dpo(p, r).backward()
     torch.testing.assert_close(x.grad.cpu(), lp_c.grad, rtol=1e-5, atol=1e-9)
+
+
+# ---------------------------------------------------------------- M2PO mask
+def test_m2po_mask_hand_cases(dev):
+    from areal_amd.ppo.actor import _apply_m2po_masking
+
+    old = torch.zeros(5, device=dev)
+    prox = torch.tensor([1.0, 2.0, 3.0, 0.5, 9.0], device=dev)
+    mask = torch.tensor([True, True, True, True, False], device=dev)
+    for thr, want in ((4.0, [1, 1, 1, 1, 0]), (2.0, [1, 1, 0, 1, 0]), (0.7, [1, 0, 0, 1, 0]),
+                      (0.3, [0, 0, 0, 1, 0]), (0.1, [0, 0, 0, 1, 0])):
+        out = _apply_m2po_masking(old, prox, mask, thr)
+        assert out.dtype == torch.bool and out.tolist() == [bool(w) for w in want], thr
+    none = torch.zeros(5, dtype=torch.bool, device=dev)
+    assert not _apply_m2po_masking(old, prox, none, 1.0).any()
+
+
+@pytest.mark.parametrize("n,thr", [(37, 0.02), (5000, 0.005), (300_000, 0.02), (300_000, 0.0001), (300_000, 5.0)])
+def test_m2po_mask_matches_oracle(dev, n, thr):
+    from areal_amd.ppo.actor import _apply_m2po_masking
+
+    g = torch.Generator().manual_seed(n)
+    old = torch.randn(n, generator=g) * 0.2
+    prox = old + torch.randn(n, generator=g) * 0.15
+    prox[::7] = old[::7]                       # many exact zeros of m2
+    mask = torch.rand(n, generator=g) > 0.3
+    want = A.m2po_mask(old, prox, mask, thr)
+    got = _apply_m2po_masking(old.to(dev), prox.to(dev), mask.to(dev), thr).cpu()
+    # the kept count may differ by the few tokens whose suffix mean is within rounding of the
+    # threshold (the oracle accumulates in fp32, the kernel in fp64); the sets are nested
+    assert not (got & ~mask).any()
+    diff = int((got != want).sum())
+    assert diff <= max(2, n // 100_000), diff
+    m2 = (old - prox) ** 2
+    if (mask & ~got).any():
+        assert m2[got].max() <= m2[mask & ~got].min()
+    kept_mean = m2[got].double().mean().item()
+    assert kept_mean < thr or int(got.sum()) == 1
+
+
+def test_m2po_ties_at_the_cut_are_kept_in_index_order(dev):
+    from areal_amd.ppo.actor import _apply_m2po_masking
+
+    # values 1 (x6) and 0 (x2): threshold 0.7 keeps the zeros and four of the ones
+    old = torch.zeros(8, device=dev)
+    prox = torch.tensor([1.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0, 1.0], device=dev)
+    mask = torch.ones(8, dtype=torch.bool, device=dev)
+    out = _apply_m2po_masking(old, prox, mask, 0.7)
+    # kept sets of size j have mean (j - 2) / j: below 0.7 up to j = 6
+    assert out.tolist() == [True, True, True, True, True, True, False, False]
+    # 2-D shapes keep their shape
+    out2 = _apply_m2po_masking(old.view(2, 4), prox.view(2, 4), mask.view(2, 4), 0.7)
+    assert out2.shape == (2, 4) and out2.view(-1).tolist() == out.tolist()

@@ -162,8 +162,10 @@ def test_kl_estimator_values():
 def test_grpo_loss_fn_rejects_out_of_scope_options():
     z = torch.zeros(4)
     data = dict(logprobs=z, advantages=z, loss_mask=torch.ones(4), prox_logp=z)
-    with pytest.raises(NotImplementedError, match="M2PO"):
-        grpo_loss_fn(z, z, data, 0.2, None, None, m2_threshold=0.1)
+    with pytest.raises(ValueError, match="not compatible with `use_decoupled_loss=True`"):
+        grpo_loss_fn(z, z, data, 0.2, None, None, use_sapo_loss=True, use_decoupled_loss=True)
+    with pytest.raises(NotImplementedError, match="distillation"):
+        grpo_loss_fn(z, z, dict(data, teacher_logp=z), 0.2, None, None)
     with pytest.raises(ValueError, match="mutually exclusive"):
         grpo_loss_fn(z, z, data, 0.2, 4.0, None, use_cispo_loss=True, use_sapo_loss=True)
     with pytest.raises(ValueError, match="CISPO only supports"):

@@ -159,3 +159,37 @@ def test_dpo_preference_loss_closed_forms():
     torch.testing.assert_close(A.dpo_preference_loss(x, beta=0.5, loss_type="ipo"), (x - 1.0) ** 2)
     with pytest.raises(ValueError):
         A.dpo_preference_loss(x, beta=0.5, loss_type="hinge")
+
+
+# ---------------------------------------------------------------- M2PO mask
+def test_m2po_mask_hand_cases():
+    old = torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0])
+    prox = torch.tensor([1.0, 2.0, 3.0, 0.5, 9.0])   # m2 = 1, 4, 9, 0.25, 81
+    mask = torch.tensor([True, True, True, True, False])
+    # means of the suffixes (descending 9, 4, 1, 0.25): 3.5625, 1.75, 0.625, 0.25
+    assert A.m2po_mask(old, prox, mask, 4.0).tolist() == [True, True, True, True, False]
+    assert A.m2po_mask(old, prox, mask, 2.0).tolist() == [True, True, False, True, False]
+    assert A.m2po_mask(old, prox, mask, 0.7).tolist() == [True, False, False, True, False]
+    assert A.m2po_mask(old, prox, mask, 0.3).tolist() == [False, False, False, True, False]
+    # no suffix mean below the threshold: all but the smallest are dropped
+    assert A.m2po_mask(old, prox, mask, 0.1).tolist() == [False, False, False, True, False]
+    none = torch.zeros(5, dtype=torch.bool)
+    assert A.m2po_mask(old, prox, none, 1.0) is none
+
+
+def test_m2po_mask_is_the_largest_prefix_with_mean_below_threshold():
+    g = torch.Generator().manual_seed(2)
+    for thr in (0.005, 0.02, 0.05, 1.0):
+        old = torch.randn(4, 50, generator=g) * 0.2
+        prox = old + torch.randn(4, 50, generator=g) * 0.15
+        mask = torch.rand(4, 50, generator=g) > 0.3
+        out = A.m2po_mask(old, prox, mask, thr)
+        assert out.shape == mask.shape and not (out & ~mask).any()
+        m2 = ((old - prox) ** 2)[mask].double().sort().values
+        means = m2.cumsum(0) / torch.arange(1, m2.numel() + 1)
+        ok = (means < thr).nonzero()
+        want_kept = int(ok[-1]) + 1 if len(ok) else 1
+        assert int(out.sum()) == want_kept
+        kept = ((old - prox) ** 2)[out]
+        dropped = ((old - prox) ** 2)[mask & ~out]
+        assert dropped.numel() == 0 or kept.max() <= dropped.min()
