@@ -68,6 +68,8 @@ SIGNATURES: dict[str, tuple] = {
     "areal_critic_loss": (I, [P, P, P, P, I64, F, I, P, P, P, P, P, P, SZ, P]),
     "areal_m2po_mask_workspace_bytes": (SZ, [I64]),
     "areal_m2po_mask": (I, [P, P, P, I64, F, P, P, SZ, P]),
+    "areal_prox_logp_approx": (I, [P, P, P, I64, I, I, P, P]),
+    "areal_distill_terms": (I, [P, P, P, P, I64, I, P, P, P, P, P, SZ, P]),
     "areal_dpo_seq_logps": (I, [P, P, P, P, I64, I64, P, P, P]),
     "areal_dpo_seq_logps_grad": (I, [P, P, P, I64, I64, P, P]),
     "areal_gae_workspace_bytes": (SZ, [I64]),

@@ -433,6 +433,73 @@ __global__ __launch_bounds__(AUX_THREADS) void m2_apply_kernel(const float* old,
   (void)nblocks;
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Proximal log-prob approximations (compute_prox_logp_approximations,
+// areal/trainer/ppo/actor.py:768-848): version-aware interpolation between the behaviour and
+// the current policy. method 0: log-linear, 1: linear in probability space, 2: rollout.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AUX_THREADS) void prox_approx_kernel(const float* old, const float* lp,
+                                                                  const int64_t* versions, int64_t n,
+                                                                  int current_version, int method,
+                                                                  float* out) {
+  const float v_theta = (float)current_version;
+  const float v_prox = (float)(current_version - 1);
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t ver = versions[t];
+    const float v_behave = (float)ver;
+    const float diff = v_theta - v_behave, gap = v_prox - v_behave;
+    float alpha = (diff > 0.0f && ver >= 0) ? gap / diff : 0.0f;
+    alpha = alpha != alpha ? alpha : (alpha < 0.0f ? 0.0f : (alpha > 1.0f ? 1.0f : alpha));
+    const float o = old[t], l = lp[t];
+    float r;
+    if (method == 0) r = o + alpha * (l - o);
+    else if (method == 1) r = logf(((1.0f - alpha) * expf(o) + alpha * expf(l)) + 1e-10f);
+    else r = o;
+    out[t] = r;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Distillation terms of the actor loss (areal/trainer/ppo/actor.py:629-658), masked sums with
+// the closed-form gradient w.r.t. the current log-probs.
+//   mode 0 (joint KD + RL): term = (lp - teacher) * mask
+//   mode 1 (pure KD, reverse KL with importance weight): term = exp(lp - old) * (teacher - lp)
+//          * mask, the reward (teacher - lp) treated as a constant
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(AUX_THREADS) void distill_token_kernel(const float* lp, const float* old,
+                                                                    const float* teacher,
+                                                                    const uint8_t* mask, int64_t n,
+                                                                    int mode, float* dlp, float* term_out,
+                                                                    SumCount* parts) {
+  __shared__ double sm_d[8];
+  __shared__ long long sm_l[8];
+  double sum = 0.0;
+  long long cnt = 0;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
+       t += (int64_t)gridDim.x * blockDim.x) {
+    const float m = mask[t] != 0 ? 1.0f : 0.0f;
+    float term, d;
+    if (mode == 0) {
+      term = (lp[t] - teacher[t]) * m;
+      d = m;
+    } else {
+      const float reward = teacher[t] - lp[t];
+      const float iw = expf(lp[t] - old[t]);
+      term = (iw * reward) * m;
+      d = term;  // d iw / d lp = iw
+    }
+    sum += (double)term;
+    cnt += mask[t] != 0;
+    if (dlp) dlp[t] = d;
+    if (term_out) term_out[t] = term;
+  }
+  sum = block_sum(sum, sm_d);
+  cnt = block_sum(cnt, sm_l);
+  if (threadIdx.x == 0) parts[blockIdx.x] = SumCount{sum, cnt, 0};
+}
+
 }  // namespace
 
 extern "C" {
@@ -579,6 +646,44 @@ int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
   hipLaunchKernelGGL(m2_apply_kernel, dim3(blocks), dim3(AUX_THREADS), 0, stream, old_logprobs,
                      proximal_logprobs, loss_mask, n_tokens, per_block, blocks, st, block_eq,
                      new_mask);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// out[t] = approximation of the proximal policy's log-prob from the behaviour policy's
+// (old_logprobs, generated at versions[t], negative for prompt tokens) and the current one's.
+// method 0 log-linear, 1 linear in probability space, 2 rollout (= old_logprobs).
+int areal_prox_logp_approx(const float* old_logprobs, const float* logprobs, const int64_t* versions,
+                           int64_t n_tokens, int current_version, int method, float* out,
+                           hipStream_t stream) {
+  if (n_tokens < 0 || method < 0 || method > 2) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!old_logprobs || !logprobs || !versions || !out) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(prox_approx_kernel, dim3(aux_grid(n_tokens)), dim3(AUX_THREADS), 0, stream,
+                     old_logprobs, logprobs, versions, n_tokens, current_version, method, out);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// value = sum(term) / max(count(mask), 1), dlogprobs = d(sum)/d logprobs, term per token; mode 0:
+// (logprobs - teacher) * mask; mode 1: exp(logprobs - old) * (teacher - logprobs) * mask with the
+// second factor held constant. counters as in areal_sapo_loss.
+int areal_distill_terms(const float* logprobs, const float* old_logprobs, const float* teacher_logprobs,
+                        const uint8_t* loss_mask, int64_t n_tokens, int mode, float* value,
+                        float* dlogprobs, float* term, double* counters, void* workspace,
+                        size_t workspace_bytes, hipStream_t stream) {
+  if (n_tokens < 0 || counters == nullptr || mode < 0 || mode > 1) return AREAL_ERR_BAD_ARG;
+  if (n_tokens > 0 && (!logprobs || !teacher_logprobs || !loss_mask || (mode == 1 && !old_logprobs)))
+    return AREAL_ERR_BAD_ARG;
+  if (workspace == nullptr || workspace_bytes < areal_aux_loss_workspace_bytes(n_tokens, 0))
+    return AREAL_ERR_WORKSPACE;
+  SumCount* parts = (SumCount*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  const int grid = aux_grid(n_tokens);
+  hipLaunchKernelGGL(distill_token_kernel, dim3(grid), dim3(AUX_THREADS), 0, stream, logprobs,
+                     old_logprobs, teacher_logprobs, loss_mask, n_tokens, mode, dlogprobs, term, parts);
+  AREAL_CHECK_LAUNCH();
+  hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid, 0, 0.0,
+                     value, counters);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

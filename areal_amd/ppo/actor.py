@@ -17,12 +17,24 @@ import torch
 from areal_amd.config import RejectionSamplingConfig
 from areal_amd.data import KLEstimator, Normalization
 from areal_amd import _lib
-from areal_amd.functional.aux_losses import sapo_loss_fn
+from areal_amd.functional.aux_losses import _Launch, _ScaledLoss, sapo_loss_fn
 from areal_amd.functional.functional import cispo_loss_fn, ppo_actor_loss_fn
 from areal_amd.ppo.gae import _compute_token_level_gae
 
+# areal/utils/constants.py:36-92
 PROX_LOGP_METHOD_RECOMPUTE = "recompute"
+PROX_LOGP_METHOD_LOGLINEAR = "loglinear"
+PROX_LOGP_METHOD_METRICS = "metrics"
 PROX_LOGP_METHOD_REUSE_TRAIN_LOGP = "reuse_train_logp"
+PROX_LOGP_METHODS_ALL = [
+    PROX_LOGP_METHOD_RECOMPUTE, PROX_LOGP_METHOD_LOGLINEAR, PROX_LOGP_METHOD_METRICS,
+    PROX_LOGP_METHOD_REUSE_TRAIN_LOGP,
+]
+PROX_APPROX_METHOD_LOGLINEAR = "loglinear"
+PROX_APPROX_METHOD_LINEAR = "linear"
+PROX_APPROX_METHOD_ROLLOUT = "rollout"
+PROX_APPROX_METHODS_ALL = [PROX_APPROX_METHOD_LOGLINEAR, PROX_APPROX_METHOD_LINEAR, PROX_APPROX_METHOD_ROLLOUT]
+_APPROX_ID = {PROX_APPROX_METHOD_LOGLINEAR: 0, PROX_APPROX_METHOD_LINEAR: 1, PROX_APPROX_METHOD_ROLLOUT: 2}
 
 
 def grpo_loss_fn(
@@ -53,30 +65,24 @@ def grpo_loss_fn(
     ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``:
     bool denominators and fp32 statistics, all of the micro-batch's token shape.
     """
-    del current_version
-    if input_data.get("teacher_logp") is not None:
-        raise NotImplementedError("distillation terms are not part of this path")
-
+    if prox_logp_method not in PROX_LOGP_METHODS_ALL:
+        raise ValueError(f"'{prox_logp_method}' is not a valid ProxLogpMethod")
     old_logp = input_data["logprobs"]
     advantages = input_data["advantages"]
     loss_mask = input_data["loss_mask"].bool()
-    prox_logp = input_data.get("prox_logp")
+    prox_logp_gt = input_data.get("prox_logp")
     entropy = entropy.detach()
 
     if prox_logp_method == PROX_LOGP_METHOD_REUSE_TRAIN_LOGP:
-        prox_logp = logprobs.detach()
-    elif prox_logp_method != PROX_LOGP_METHOD_RECOMPUTE:
-        raise NotImplementedError(f"prox_logp_method='{prox_logp_method}' is not part of this path")
-    if prox_logp is None:
-        raise ValueError(
-            f"prox_logp is None but prox_logp_method='{prox_logp_method}'. "
-            "This indicates compute_logp() was skipped incorrectly."
-        )
-    if torch.isnan(prox_logp).any() or torch.isinf(prox_logp).any():
-        raise RuntimeError(
-            f"prox_logp contains NaN or Inf with prox_logp_method='{prox_logp_method}'. "
-            "This indicates computation failed."
-        )
+        prox_logp_gt = logprobs.detach()
+    prox_logp = _resolve_proximal_logp(
+        prox_logp_gt=prox_logp_gt,
+        prox_logp_method=prox_logp_method,
+        old_logp=old_logp,
+        logprobs=logprobs.detach(),
+        versions=input_data.get("versions"),
+        current_version=current_version,
+    )
 
     if m2_threshold is not None:
         loss_mask = _apply_m2po_masking(old_logp, prox_logp, loss_mask, m2_threshold)
@@ -134,6 +140,21 @@ def grpo_loss_fn(
             cu_seqlens=input_data.get("cu_seqlens"),
         )
 
+    # joint distillation (actor.py:629-658)
+    teacher_logp = input_data.get("teacher_logp")
+    rkl_stat = None
+    if teacher_logp is not None:
+        rl_loss_weight = input_data.get("rl_loss_weight", 1.0)
+        distill_loss_weight = input_data.get("distill_loss_weight", 0.005)
+        pure_kd = rl_loss_weight == 0
+        value, term = _distill_term(logprobs, old_logp, teacher_logp.detach(), loss_mask, pure_kd)
+        if pure_kd:
+            loss = (-1 * distill_loss_weight) * value
+            rkl_stat = -1 * term
+        else:
+            loss = rl_loss_weight * loss + distill_loss_weight * value
+            rkl_stat = term
+
     if stats is not None:
         lp = logprobs.detach()
         logp_diff = (old_logp - lp) * loss_mask
@@ -166,17 +187,200 @@ def grpo_loss_fn(
             stats["scalar/rs_filtered_fraction"] = stat["filtered_fraction"]
         if vocab_min_logits is not None and vocab_max_logits is not None:
             stats.update(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits)
+        if rkl_stat is not None:
+            stats["rkl_loss"] = rkl_stat
         if use_sapo_loss:
             stats.update(
                 sapo_soft_gate=stat["sapo_soft_gate"],
                 sapo_scaled_gate_pos=stat["sapo_scaled_gate_pos"],
                 sapo_scaled_gate_neg=stat["sapo_scaled_gate_neg"],
             )
+        compute_logp_mask = stat.get("behave_mask", loss_mask)
+        _collect_proximal_approximation_stats(
+            stats, prox_logp_method, prox_logp_gt, old_logp, lp, input_data.get("versions"),
+            current_version, compute_logp_mask,
+        )
+        if "versions" in input_data and current_version is not None:
+            _collect_version_staleness_stats(stats, input_data["versions"], current_version, compute_logp_mask)
         if vocab_mean_logits is not None:
             stats["vocab_mean_logits"] = vocab_mean_logits
         if vocab_norm_logits is not None:
             stats["vocab_norm_logits"] = vocab_norm_logits
     return loss
+
+
+def compute_prox_logp_approximations(
+    old_logp: torch.Tensor,
+    logprobs: torch.Tensor,
+    versions: torch.Tensor,
+    current_version: int,
+    method: str | None = None,
+) -> dict[str, torch.Tensor]:
+    """Version-aware approximations of the proximal policy's log-probs (``actor.py:768-848``):
+    one key if ``method`` is given, all three methods otherwise."""
+    lib = _lib.load()
+    shape = old_logp.shape
+    old = old_logp.detach().to(torch.float32).contiguous().view(-1)
+    lp = logprobs.detach().to(torch.float32).contiguous().view(-1)
+    ver = versions.detach().to(torch.int64).contiguous().view(-1)
+    dev = _lib.require_gpu(old, lp, ver)
+    out = {}
+    for m in ([method] if method else PROX_APPROX_METHODS_ALL):
+        if m not in _APPROX_ID:
+            continue
+        res = torch.empty(old.numel(), dtype=torch.float32, device=dev)
+        rc = lib.areal_prox_logp_approx(
+            _lib.ptr(old), _lib.ptr(lp), _lib.ptr(ver), old.numel(), int(current_version),
+            _APPROX_ID[m], _lib.ptr(res), _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_prox_logp_approx")
+        out[m] = res.view(shape)
+    return out
+
+
+def _resolve_proximal_logp(prox_logp_gt, prox_logp_method, old_logp, logprobs, versions, current_version):
+    """Proximal log-probs to train with: the recomputed ones, or the log-linear approximation
+    when the forward pass was skipped (``actor.py:851-930``; same errors)."""
+    prox_logp_is_none = prox_logp_gt is None
+    if prox_logp_is_none:
+        if prox_logp_method not in (PROX_LOGP_METHOD_LOGLINEAR, PROX_LOGP_METHOD_REUSE_TRAIN_LOGP):
+            raise ValueError(
+                f"prox_logp is None but prox_logp_method='{prox_logp_method}'. "
+                "This indicates compute_logp() was skipped incorrectly."
+            )
+        if versions is None:
+            raise ValueError(
+                f"prox_logp is None with prox_logp_method='{prox_logp_method}' "
+                "but versions not available. "
+                "Cannot proceed without either ground truth or approximation."
+            )
+    prox_logp = prox_logp_gt
+    if prox_logp_method == PROX_LOGP_METHOD_LOGLINEAR:
+        if prox_logp_is_none and versions is not None and current_version is not None:
+            prox_logp = compute_prox_logp_approximations(
+                old_logp, logprobs, versions, current_version, PROX_APPROX_METHOD_LOGLINEAR
+            )[PROX_APPROX_METHOD_LOGLINEAR]
+    if prox_logp is None:
+        raise RuntimeError(
+            f"prox_logp is None after handling prox_logp_method='{prox_logp_method}'. "
+            "This indicates configuration or computation error."
+        )
+    if torch.isnan(prox_logp).any() or torch.isinf(prox_logp).any():
+        raise RuntimeError(
+            f"prox_logp contains NaN or Inf with prox_logp_method='{prox_logp_method}'. "
+            "This indicates computation failed."
+        )
+    return prox_logp
+
+
+def _distill_term(logprobs, old_logp, teacher_logp, loss_mask, pure_kd: bool):
+    """``sum(term) / max(count, 1)`` (differentiable w.r.t. ``logprobs``) and the per-token term:
+    ``(logprobs - teacher) * mask`` for the joint loss, ``exp(logprobs - old) * (teacher -
+    logprobs.detach()) * mask`` for pure distillation (``actor.py:640-656``)."""
+    lib = _lib.load()
+    shape = logprobs.shape
+    f32 = lambda t: t.detach().to(torch.float32).contiguous().view(-1)  # noqa: E731
+    old, teacher = f32(old_logp), f32(teacher_logp)
+    mask_bool = loss_mask.detach().bool().contiguous().view(-1)
+    dev = _lib.require_gpu(logprobs, old, teacher, mask_bool)
+    n = int(mask_bool.numel())
+
+    def launch(want_grad: bool):
+        out = {
+            "loss": torch.empty((), dtype=torch.float32, device=dev),
+            "dsum": torch.empty(n, dtype=torch.float32, device=dev) if want_grad else None,
+            "term": torch.empty(n, dtype=torch.float32, device=dev),
+            "counters": torch.empty(8, dtype=torch.float64, device=dev),
+        }
+        nbytes = lib.areal_aux_loss_workspace_bytes(n, 0)
+        ws = _lib.workspace(nbytes, dev)
+        rc = lib.areal_distill_terms(
+            _lib.ptr(f32(logprobs)), _lib.ptr(old), _lib.ptr(teacher), _lib.ptr(mask_bool), n,
+            int(pure_kd), _lib.ptr(out["loss"]), _lib.ptr(out["dsum"]), _lib.ptr(out["term"]),
+            _lib.ptr(out["counters"]), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_distill_terms")
+        return out
+
+    runner = _Launch(launch)
+    value = _ScaledLoss.apply(logprobs, runner)
+    return value, runner.out["term"].view(shape)
+
+
+_EPSILON = 1e-8
+
+
+def _approximation_errors(ground_truth, approximation):
+    diff = ground_truth - approximation
+    return {
+        "abs_error": torch.abs(diff).float(),
+        "rel_error": torch.abs(diff / (torch.abs(ground_truth) + _EPSILON)).float(),
+        "squared_error": (diff * diff).float(),
+    }
+
+
+def _collect_proximal_approximation_stats(
+    stats, prox_logp_method, prox_logp_gt, old_logp, logprobs, versions, current_version, mask
+):
+    """What ``_log_proximal_approximation_stats`` (``actor.py:1138-1226``) hands to the tracker's
+    ``compute_logp`` scope, as ``compute_logp/<key>`` entries of ``stats`` (logging only)."""
+    pre = "compute_logp/"
+    stats[pre + "n_valid_tokens"] = mask.bool()
+    if prox_logp_gt is not None:
+        stats[pre + "prox_logp_gt"] = prox_logp_gt.float()
+    if versions is None or current_version is None:
+        return
+    gt = None
+    if prox_logp_method == PROX_LOGP_METHOD_LOGLINEAR:
+        approximations = compute_prox_logp_approximations(
+            old_logp, logprobs, versions, current_version, PROX_APPROX_METHOD_LOGLINEAR
+        )
+    elif prox_logp_method == PROX_LOGP_METHOD_METRICS and prox_logp_gt is not None:
+        approximations = compute_prox_logp_approximations(old_logp, logprobs, versions, current_version, None)
+        gt = prox_logp_gt
+    else:
+        approximations = {}
+    for name, approx in approximations.items():
+        behave_w = torch.exp(approx - old_logp).float()
+        imp_w = torch.exp(logprobs - approx).float()
+        stats[f"{pre}{name}/approx_logp"] = approx.float()
+        stats[f"{pre}{name}/behave_imp_weight"] = behave_w
+        stats[f"{pre}{name}/importance_weight"] = imp_w
+        if gt is not None:
+            for k, v in _approximation_errors(gt, approx).items():
+                stats[f"{pre}{name}/{k}"] = v
+            be = _approximation_errors(torch.exp(gt - old_logp).float(), behave_w)
+            ie = _approximation_errors(torch.exp(logprobs - gt).float(), imp_w)
+            stats[f"{pre}{name}/behave_imp_weight_abs_error"] = be["abs_error"]
+            stats[f"{pre}{name}/behave_imp_weight_rel_error"] = be["rel_error"]
+            stats[f"{pre}{name}/importance_weight_abs_error"] = ie["abs_error"]
+            stats[f"{pre}{name}/importance_weight_rel_error"] = ie["rel_error"]
+    log_ratio = (logprobs.float() - old_logp.float()).detach()
+    stats[pre + "kl_div_direct"] = -log_ratio
+    stats[pre + "kl_div_taylor"] = log_ratio**2 / 2.0
+    stats[pre + "kl_div_dual"] = log_ratio.exp() - 1 - log_ratio
+
+
+def _collect_version_staleness_stats(stats, versions, current_version, mask):
+    """The scalars of ``_log_version_staleness_stats`` (``actor.py:1229-1272``) as
+    ``scalar/version_stats/<key>`` entries of ``stats``: one reduction launch, one host copy."""
+    from areal_amd.stats import masked_stats
+
+    v_behave = versions.float()
+    generated = mask.bool() & (versions >= 0)
+    res = masked_stats(
+        {"proximal": (current_version - 1) - v_behave, "theta": current_version - v_behave},
+        {"proximal": generated, "theta": generated},
+    )
+    if res["proximal"]["count"] == 0:
+        return
+    pre = "scalar/version_stats/"
+    for name in ("proximal", "theta"):
+        for k in ("avg", "max", "min"):
+            stats[f"{pre}sample_staleness_{name}_{k}"] = res[name][k]
+    stats[pre + "v_theta"] = current_version
+    stats[pre + "v_proximal"] = current_version - 1
+    stats[pre + "n_valid_generated_tokens"] = int(res["proximal"]["count"])
 
 
 def _apply_m2po_masking(

@@ -204,6 +204,22 @@ int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
                     uint8_t* new_mask, void* workspace, size_t workspace_bytes,
                     areal_stream_t stream);
 
+/* Proximal log-prob approximation (compute_prox_logp_approximations,
+ * areal/trainer/ppo/actor.py:768-848). versions [n] int64 (negative = prompt token). method 0
+ * log-linear, 1 linear in probability space, 2 rollout. */
+int areal_prox_logp_approx(const float* old_logprobs, const float* logprobs,
+                           const int64_t* versions, int64_t n_tokens, int current_version,
+                           int method, float* out, areal_stream_t stream);
+
+/* Distillation terms of grpo_loss_fn (actor.py:629-658): value = sum(term) / max(count(mask), 1).
+ * mode 0: term = (logprobs - teacher) * mask (joint KD + RL penalty); mode 1: term =
+ * exp(logprobs - old) * (teacher - logprobs) * mask with the second factor held constant (pure
+ * KD). dlogprobs = d(sum)/d logprobs; scale it with areal_actor_loss_grad. */
+int areal_distill_terms(const float* logprobs, const float* old_logprobs,
+                        const float* teacher_logprobs, const uint8_t* loss_mask, int64_t n_tokens,
+                        int mode, float* value, float* dlogprobs, float* term, double* counters,
+                        void* workspace, size_t workspace_bytes, areal_stream_t stream);
+
 /* seq_sums [n_seqs][3] double = {sum policy log-probs, sum reference log-probs, count} over
  * shifted_mask[t] = loss_mask[t+1] inside each packed sequence (its last token excluded);
  * shifted_mask [n_tokens] is written for the backward. */

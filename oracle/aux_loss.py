@@ -140,3 +140,44 @@ def m2po_mask(old_logp, prox_logp, loss_mask, m2_threshold):
     full = torch.zeros_like(flat)
     full[flat] = keep_sorted[restored]
     return full.view_as(loss_mask)
+
+
+def prox_logp_approximations(old_logp, logprobs, versions, current_version, method=None):
+    """compute_prox_logp_approximations (areal/trainer/ppo/actor.py:768-848).
+
+    Pinned by the reference's literals (tests/test_prox_approx.py:24-211): log-linear
+    [-1.25, -2.25, -3.25] at alpha 0.5, mixed versions [-1.375, -2.1], alpha 0 when the behaviour
+    version is the proximal one or equals the current one, prompt tokens (version < 0) unchanged,
+    linear log(0.375), rollout = old."""
+    v_prox = current_version - 1
+    v_behave = versions.float()
+    v_theta = float(current_version)
+    generated = versions >= 0
+    diff = v_theta - v_behave
+    gap = v_prox - v_behave
+    alpha = torch.where((diff > 0) & generated, gap / diff, torch.zeros_like(v_behave)).clamp(0.0, 1.0)
+    out = {}
+    for m in ([method] if method else ["loglinear", "linear", "rollout"]):
+        if m == "loglinear":
+            out[m] = old_logp + alpha * (logprobs - old_logp)
+        elif m == "linear":
+            out[m] = torch.log((1 - alpha) * torch.exp(old_logp) + alpha * torch.exp(logprobs) + 1e-10)
+        elif m == "rollout":
+            out[m] = old_logp.clone()
+    return out
+
+
+def distill_loss(loss, logprobs, old_logp, teacher_logp, loss_mask, rl_loss_weight=1.0, distill_loss_weight=0.005):
+    """The joint-distillation tail of grpo_loss_fn (actor.py:629-658): returns (loss, rkl_stat).
+
+    No reference test covers it ("parity unpinned"): pinned by hand-computed two-token cases of
+    both branches and by autograd of these same expressions."""
+    teacher_logp = teacher_logp.detach()
+    if rl_loss_weight == 0:
+        reward = teacher_logp - logprobs.detach()
+        iw = torch.exp(logprobs - old_logp)
+        term = iw * reward * loss_mask
+        return -1 * distill_loss_weight * term.sum() / loss_mask.sum().clamp(min=1), -1 * term
+    per_token = (logprobs - teacher_logp) * loss_mask
+    penalty = per_token.sum() / loss_mask.sum().clamp(min=1)
+    return rl_loss_weight * loss + distill_loss_weight * penalty, per_token

@@ -164,8 +164,10 @@ def test_grpo_loss_fn_rejects_out_of_scope_options():
     data = dict(logprobs=z, advantages=z, loss_mask=torch.ones(4), prox_logp=z)
     with pytest.raises(ValueError, match="not compatible with `use_decoupled_loss=True`"):
         grpo_loss_fn(z, z, data, 0.2, None, None, use_sapo_loss=True, use_decoupled_loss=True)
-    with pytest.raises(NotImplementedError, match="distillation"):
-        grpo_loss_fn(z, z, dict(data, teacher_logp=z), 0.2, None, None)
+    with pytest.raises(ValueError, match="not a valid ProxLogpMethod"):
+        grpo_loss_fn(z, z, data, 0.2, None, None, prox_logp_method="guess")
+    with pytest.raises(ValueError, match="versions not available"):
+        grpo_loss_fn(z, z, dict(data, prox_logp=None), 0.2, None, None, prox_logp_method="loglinear")
     with pytest.raises(ValueError, match="mutually exclusive"):
         grpo_loss_fn(z, z, data, 0.2, 4.0, None, use_cispo_loss=True, use_sapo_loss=True)
     with pytest.raises(ValueError, match="CISPO only supports"):

@@ -193,3 +193,46 @@ def test_m2po_mask_is_the_largest_prefix_with_mean_below_threshold():
         kept = ((old - prox) ** 2)[out]
         dropped = ((old - prox) ** 2)[mask & ~out]
         assert dropped.numel() == 0 or kept.max() <= dropped.min()
+
+
+# ---------------------------------------------------------------- proximal approximations
+def test_prox_approximation_reference_literals():
+    # reference tests/test_prox_approx.py:24-186
+    old = torch.tensor([[-1.0, -2.0, -3.0]])
+    new = torch.tensor([[-1.5, -2.5, -3.5]])
+    a = A.prox_logp_approximations(old, new, torch.tensor([[0, 0, 0]], dtype=torch.int32), 2)
+    torch.testing.assert_close(a["loglinear"], torch.tensor([[-1.25, -2.25, -3.25]]), rtol=1e-4, atol=1e-4)
+    assert torch.equal(a["rollout"], old) and set(a) == {"loglinear", "linear", "rollout"}
+    a = A.prox_logp_approximations(torch.tensor([[-1.0], [-2.0]]), torch.tensor([[-1.5], [-2.2]]),
+                                   torch.tensor([[0], [2]], dtype=torch.int32), 4)
+    torch.testing.assert_close(a["loglinear"], torch.tensor([[-1.375], [-2.1]]), rtol=1e-4, atol=1e-4)
+    one = torch.tensor([[-1.0]])
+    for ver, cur in ((4, 5), (3, 3)):   # behaviour == proximal; behaviour == current (0/0)
+        a = A.prox_logp_approximations(one, torch.tensor([[-2.0]]), torch.tensor([[ver]], dtype=torch.int32), cur)
+        torch.testing.assert_close(a["loglinear"], one, rtol=1e-4, atol=1e-4)
+    a = A.prox_logp_approximations(torch.tensor([[-0.693]]), torch.tensor([[-1.386]]),
+                                   torch.tensor([[0]], dtype=torch.int32), 2)
+    torch.testing.assert_close(a["linear"], torch.log(torch.tensor([[0.375]])), rtol=1e-3, atol=1e-3)
+    a = A.prox_logp_approximations(old, new, torch.tensor([[-1, 0, 1]], dtype=torch.int32), 3, "loglinear")
+    assert a["loglinear"][0, 0] == old[0, 0] and torch.isfinite(a["loglinear"]).all() and list(a) == ["loglinear"]
+
+
+def test_distill_loss_hand_cases():
+    lp = torch.tensor([-1.0, -2.0, -0.5], requires_grad=True)
+    old = torch.tensor([-1.0, -1.5, -0.5])
+    teacher = torch.tensor([-0.5, -1.0, -9.0])
+    mask = torch.tensor([True, True, False])
+    base = (lp * torch.tensor([1.0, 0.0, 0.0])).sum()          # a stand-in RL loss: -1.0
+    loss, stat = A.distill_loss(base, lp, old, teacher, mask, 2.0, 0.1)
+    # penalty = ((-1 + 0.5) + (-2 + 1)) / 2 = -0.75; loss = 2 * (-1) + 0.1 * (-0.75)
+    assert abs(loss.item() - (-2.075)) < 1e-6 and stat.tolist() == [-0.5, -1.0, 0.0]
+    loss.backward()
+    torch.testing.assert_close(lp.grad, torch.tensor([2.0 + 0.05, 0.05, 0.0]))
+    lp.grad = None
+    loss, stat = A.distill_loss(base, lp, old, teacher, mask, 0, 0.1)
+    # term = exp(lp - old) * (teacher - lp): [1 * 0.5, exp(-0.5) * 1.0]
+    t1 = math.exp(-0.5)
+    assert abs(loss.item() - (-0.1 * (0.5 + t1) / 2)) < 1e-6
+    torch.testing.assert_close(stat, torch.tensor([-0.5, -t1, 0.0]))
+    loss.backward()
+    torch.testing.assert_close(lp.grad, torch.tensor([-0.1 * 0.5 / 2, -0.1 * t1 / 2, 0.0]))
