@@ -85,6 +85,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_masked_stats": (I, [P, P, I, I64, P, P, SZ, P]),
     "areal_turn_gae_workspace_bytes": (SZ, [I64, I64]),
     "areal_turn_gae": (I, [P, P, P, P, P, P, I64, I64, F, F, P, P, P, P, SZ, P]),
+    "areal_gae_lambda_context": (I, [P, P, I64, I64, P, P, P, P]),
     "areal_group_norm_workspace_bytes": (SZ, [I64, I64]),
     "areal_group_norm": (
         I,

@@ -913,6 +913,66 @@ __global__ __launch_bounds__(TURN_THREADS) void turn_gae_kernel(TurnArgs a) {
   }
 }
 
+// Per-row lengths for the per-sample lambda functions (_build_gae_lambda_context,
+// areal/trainer/ppo/gae.py:166-205): number of active tokens, and number of distinct turn ids
+// among them (= turn starts, ids being non-decreasing over the active tokens; violations are
+// reported through *status as in turn_gae_kernel). turn_ids may be null (turn count 0).
+__global__ __launch_bounds__(TURN_THREADS) void gae_context_kernel(const float* mask,
+                                                                   const int32_t* turn_ids, int64_t L,
+                                                                   int64_t* token_len,
+                                                                   int64_t* turn_cnt, int* status) {
+  __shared__ int s_cnt[TURN_THREADS];
+  __shared__ int s_max[TURN_THREADS];
+  __shared__ double s_sum[TURN_THREADS];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const float* ms = mask + row * L;
+  const int32_t* id = turn_ids ? turn_ids + row * L : nullptr;
+  int bad = 0;
+  TurnCarry carry{0, -1, 0.0};
+  int64_t starts = 0;
+  for (int64_t base = 0; base < L; base += TURN_THREADS * TURN_ITEMS) {
+    const int64_t t0 = base + (int64_t)tid * TURN_ITEMS;
+    int ids[TURN_ITEMS]; bool act[TURN_ITEMS];
+    int mx = -1, nact = 0;
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      const int64_t t = t0 + i;
+      act[i] = t < L && ms[t] != 0.0f;
+      ids[i] = (act[i] && id) ? id[t] : -1;
+      nact += act[i];
+      if (act[i] && id) {
+        if (ids[i] < 0) bad |= 1;
+        if ((int64_t)ids[i] >= L) bad |= 2;
+        mx = mx > ids[i] ? mx : ids[i];
+      }
+    }
+    TurnCarry tot;
+    // count: active tokens; max: running turn id; sum unused
+    const TurnCarry ex = turn_block_exclusive(nact, mx, 0.0, carry, s_cnt, s_max, s_sum, tot);
+    int run_max = ex.maxid;
+#pragma unroll
+    for (int i = 0; i < TURN_ITEMS; ++i) {
+      if (!act[i] || !id) continue;
+      if (ids[i] > run_max) ++starts;
+      if (ids[i] < run_max) bad |= 4;
+      run_max = run_max > ids[i] ? run_max : ids[i];
+    }
+    carry = tot;
+  }
+  // total of the per-thread start counts
+  __syncthreads();
+  s_cnt[tid] = (int)starts;
+  __syncthreads();
+  if (tid == 0) {
+    long long tot = 0;
+    for (int i = 0; i < TURN_THREADS; ++i) tot += s_cnt[i];
+    token_len[row] = carry.count;
+    turn_cnt[row] = tot;
+  }
+  if (bad) atomicOr(status, bad);
+}
+
 }  // namespace
 
 extern "C" {
@@ -999,6 +1059,20 @@ int areal_turn_gae(const float* rewards, const float* values, const float* loss_
   a.ws_ret = a.ws_adv + (size_t)bs * max_seqlen;
   a.status = status;
   hipLaunchKernelGGL(turn_gae_kernel, dim3((unsigned)bs), dim3(TURN_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// token_lengths[b] = active tokens of row b; turn_counts[b] = distinct turn ids among them (0
+// when turn_ids is null). status as in areal_turn_gae.
+int areal_gae_lambda_context(const float* loss_mask, const int32_t* turn_ids, int64_t bs,
+                             int64_t max_seqlen, int64_t* token_lengths, int64_t* turn_counts,
+                             int* status, hipStream_t stream) {
+  if (bs < 0 || max_seqlen < 0) return AREAL_ERR_BAD_ARG;
+  if (bs == 0) return AREAL_OK;
+  if (!loss_mask || !token_lengths || !turn_counts || !status) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(gae_context_kernel, dim3((unsigned)bs), dim3(TURN_THREADS), 0, stream,
+                     loss_mask, turn_ids, max_seqlen, token_lengths, turn_counts, status);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

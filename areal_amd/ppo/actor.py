@@ -1,10 +1,11 @@
 """PPO actor-side callers of the kernels: the GRPO loss wrapper and advantage computation.
 
-``grpo_loss_fn`` mirrors the call shape of ``areal/trainer/ppo/actor.py:527-760`` (which keys
-it reads from ``input_data``, ``entropy.detach()``, pass-through of the vocabulary statistics)
-and ``compute_advantages`` mirrors ``PPOActor._compute_advantages`` (``actor.py:178-323``).
-Features of the reference that are not on this path (M2PO masking, SAPO, distillation terms,
-proximal-logp approximation, turn-level GAE) raise ``NotImplementedError``.
+``grpo_loss_fn`` mirrors ``areal/trainer/ppo/actor.py:527-760`` (which keys it reads from
+``input_data``, ``entropy.detach()``, pass-through of the vocabulary statistics, every loss
+branch and the logging helpers of ``:1020-1272``) and ``compute_advantages`` mirrors
+``PPOActor._compute_advantages`` (``actor.py:178-323``), including turn-level GAE, per-sample
+lambda functions and the overlong-response penalty.  Statistics go to an optional ``stats``
+dict instead of the reference's process-wide ``stats_tracker``.
 """
 
 from __future__ import annotations
@@ -19,7 +20,7 @@ from areal_amd.data import KLEstimator, Normalization
 from areal_amd import _lib
 from areal_amd.functional.aux_losses import _Launch, _ScaledLoss, sapo_loss_fn
 from areal_amd.functional.functional import cispo_loss_fn, ppo_actor_loss_fn
-from areal_amd.ppo.gae import _compute_token_level_gae
+from areal_amd.ppo.gae import _compute_token_level_gae, _compute_turn_level_gae, compute_gae_lambda
 
 # areal/utils/constants.py:36-92
 PROX_LOGP_METHOD_RECOMPUTE = "recompute"
@@ -428,15 +429,35 @@ def compute_advantages(
     use_decoupled_loss: bool = False,
     recompute_logprob: bool = False,
     group_sizes: list[int] | None = None,
+    gae_timestep_unit: str = "token",
+    gae_lambda_fn=None,
+    gae_lambda_kwargs: dict | None = None,
+    overlong_reward_penalty: bool = False,
+    overlong_tokens: int | None = None,
+    overlong_penalty_factor: float | None = None,
+    max_new_tokens: int | None = None,
 ) -> dict[str, Any]:
-    """Reward shaping, KL-regularised rewards, token-level GAE and advantage normalisation on a
-    padded ``[bs, L]`` batch; writes ``returns, advantages, kl_rewards, tot_rewards, loss_mask,
-    logprobs`` back into ``data`` exactly as ``actor.py:178-323`` does."""
+    """Reward shaping, KL-regularised rewards, token- or turn-level GAE and advantage
+    normalisation on a padded ``[bs, L]`` batch; writes ``returns, advantages, kl_rewards,
+    tot_rewards, loss_mask, logprobs`` back into ``data`` exactly as ``actor.py:178-323`` does.
+    ``gae_lambda_fn`` (with ``gae_lambda_kwargs``) is a per-sample lambda function as resolved by
+    ``areal_amd.ppo.lambda_fn.resolve_gae_lambda_fn``; without it ``gae_lambda`` is used."""
+    if gae_timestep_unit not in ("token", "turn"):
+        raise ValueError(f"gae_timestep_unit must be 'token' or 'turn', got {gae_timestep_unit!r}")
     if kl_estimator is None:
         kl_estimator = KLEstimator("k1")
     bs = data["input_ids"].shape[0]
     dev = data["input_ids"].device
     batch_indices = torch.arange(bs, device=dev, dtype=torch.long)
+
+    if overlong_reward_penalty:
+        assert overlong_tokens is not None
+        assert overlong_penalty_factor is not None
+        # reward_overlong_penalty (functional.py:937-959), without its per-sample loop
+        response_lengths = data["loss_mask"].sum(dim=-1).long()
+        exceed = response_lengths - (max_new_tokens - overlong_tokens)
+        penalty = torch.clamp(-exceed / overlong_tokens * overlong_penalty_factor, max=0)
+        data["rewards"] = data["rewards"] + penalty.to(data["rewards"].dtype)
 
     reward_score = (data["rewards"] + reward_bias) * reward_scaling
     reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)
@@ -444,6 +465,17 @@ def compute_advantages(
         reward_score = reward_norm(reward_score, group_sizes=group_sizes)
 
     loss_mask = torch.roll(data["loss_mask"].float(), shifts=-1, dims=-1)
+
+    # structural turn ids follow the same next-token convention as the mask and the log-probs
+    turn_ids = data.get("turn_ids")
+    if turn_ids is not None:
+        turn_ids = torch.roll(turn_ids, shifts=-1, dims=-1)
+        turn_ids[:, -1] = -1
+    elif gae_timestep_unit == "turn":
+        raise ValueError(
+            "actor.gae_timestep_unit='turn' requires rollout data to "
+            "include 'turn_ids'."
+        )
 
     if not use_decoupled_loss and recompute_logprob:
         prox = data["prox_logp"]
@@ -478,21 +510,36 @@ def compute_advantages(
         )
     else:
         gae_outcome_rewards[batch_indices, indices] = reward_score
-    rewards = gae_kl_rewards + gae_outcome_rewards
+    # turn mode keeps the token KL as a local actor penalty instead of summing it into turns
+    rewards = gae_outcome_rewards if gae_timestep_unit == "turn" else gae_kl_rewards + gae_outcome_rewards
 
     values = data["values"] if "values" in data else torch.zeros_like(rewards)
-    if not isinstance(gae_lambda, torch.Tensor):
+    if gae_lambda_fn is not None:
+        gae_lambda = compute_gae_lambda(gae_lambda_fn, gae_lambda_kwargs, loss_mask, turn_ids, gae_timestep_unit)
+    elif not isinstance(gae_lambda, torch.Tensor):
         gae_lambda = float(gae_lambda)
         if not math.isfinite(gae_lambda):
             raise ValueError(f"Static gae_lambda must be finite, got {gae_lambda}")
-    advantages, returns = _compute_token_level_gae(
-        rewards=rewards,
-        values=values,
-        loss_mask=loss_mask,
-        seq_no_eos_mask=seq_no_eos_mask,
-        discount=discount,
-        gae_lambda=gae_lambda,
-    )
+    if gae_timestep_unit == "turn":
+        advantages, returns = _compute_turn_level_gae(
+            rewards=rewards,
+            values=values,
+            loss_mask=loss_mask,
+            turn_ids=turn_ids,
+            seq_no_eos_mask=seq_no_eos_mask,
+            discount=discount,
+            gae_lambda=gae_lambda,
+        )
+        advantages = advantages + gae_kl_rewards
+    else:
+        advantages, returns = _compute_token_level_gae(
+            rewards=rewards,
+            values=values,
+            loss_mask=loss_mask,
+            seq_no_eos_mask=seq_no_eos_mask,
+            discount=discount,
+            gae_lambda=gae_lambda,
+        )
     data["returns"] = returns
     if adv_norm is not None:
         advantages = adv_norm(advantages, loss_mask, group_sizes=group_sizes)

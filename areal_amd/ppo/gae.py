@@ -155,8 +155,84 @@ def _compute_turn_level_gae(
     )
     _lib.check(rc, "areal_turn_gae")
     if validate:
-        flags = int(status.item())
-        for bit, message in _TURN_ID_ERRORS:
-            if flags & bit:
-                raise RuntimeError(message)
+        _raise_turn_id_errors(status)
     return adv, ret
+
+
+def _raise_turn_id_errors(status: torch.Tensor) -> None:
+    flags = int(status.item())
+    for bit, message in _TURN_ID_ERRORS:
+        if flags & bit:
+            raise RuntimeError(message)
+
+
+def _build_gae_lambda_context(
+    loss_mask: torch.Tensor,
+    turn_ids: torch.Tensor | None,
+    *,
+    gae_timestep_unit: str,
+    validate: bool = True,
+) -> dict[str, torch.Tensor]:
+    """Per-sample lengths from the GAE eligibility mask (``areal/trainer/ppo/gae.py:166-205``):
+    ``effective_token_lengths`` (active tokens), ``turn_counts`` (distinct active turn ids, zero
+    without ``turn_ids``) and ``timestep_lengths`` (the one ``gae_timestep_unit`` selects)."""
+    if turn_ids is None and gae_timestep_unit == "turn":
+        raise ValueError("Turn-level GAE requires rollout data to include 'turn_ids'.")
+    if turn_ids is not None:
+        if turn_ids.shape != loss_mask.shape:
+            raise ValueError(f"turn_ids must have shape {loss_mask.shape}, got {turn_ids.shape}")
+        if turn_ids.device != loss_mask.device:
+            raise ValueError(
+                "turn_ids and loss_mask must be on the same device, got "
+                f"{turn_ids.device} and {loss_mask.device}"
+            )
+        if turn_ids.dtype not in (torch.uint8, torch.int8, torch.int16, torch.int32, torch.int64):
+            raise ValueError(f"turn_ids must use an integer dtype, got {turn_ids.dtype}")
+    lib = _lib.load()
+    bs, max_seqlen = loss_mask.shape
+    m = loss_mask.to(torch.float32).contiguous()
+    ids = turn_ids.clamp(min=-1, max=2**31 - 1).to(torch.int32).contiguous() if turn_ids is not None else None
+    dev = _lib.require_gpu(m, ids)
+    token_lengths = torch.zeros(bs, dtype=torch.int64, device=dev)
+    turn_counts = torch.zeros(bs, dtype=torch.int64, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    rc = lib.areal_gae_lambda_context(
+        _lib.ptr(m), _lib.ptr(ids), bs, max_seqlen, _lib.ptr(token_lengths), _lib.ptr(turn_counts),
+        _lib.ptr(status), _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_gae_lambda_context")
+    if validate and turn_ids is not None:
+        _raise_turn_id_errors(status)
+    return {
+        "effective_token_lengths": token_lengths,
+        "turn_counts": turn_counts,
+        "timestep_lengths": token_lengths if gae_timestep_unit == "token" else turn_counts,
+    }
+
+
+def compute_gae_lambda(gae_lambda_fn, gae_lambda_kwargs, loss_mask, turn_ids, gae_timestep_unit):
+    """One lambda per local trajectory from a custom function, with the reference's checks of
+    its output (``areal/trainer/ppo/actor.py:325-362``)."""
+    context = _build_gae_lambda_context(loss_mask, turn_ids, gae_timestep_unit=gae_timestep_unit)
+    gae_lambda = gae_lambda_fn(context, **(gae_lambda_kwargs or {}))
+    if not isinstance(gae_lambda, torch.Tensor):
+        raise TypeError(
+            "gae_lambda function must return a torch.Tensor with shape "
+            f"[{loss_mask.shape[0]}], got {type(gae_lambda).__name__}"
+        )
+    expected_shape = torch.Size([loss_mask.shape[0]])
+    if gae_lambda.shape != expected_shape:
+        raise ValueError(
+            "gae_lambda function must return one value per local trajectory: "
+            f"expected shape {expected_shape}, got {gae_lambda.shape}"
+        )
+    if gae_lambda.device != loss_mask.device:
+        raise ValueError(
+            "gae_lambda output and loss_mask must be on the same device, got "
+            f"{gae_lambda.device} and {loss_mask.device}"
+        )
+    if not torch.is_floating_point(gae_lambda):
+        raise TypeError(f"gae_lambda function must return a floating-point tensor, got {gae_lambda.dtype}")
+    if not bool(torch.all(torch.isfinite(gae_lambda))):
+        raise RuntimeError("gae_lambda function returned a non-finite value")
+    return gae_lambda.detach().float()

@@ -258,6 +258,13 @@ int areal_turn_gae(const float* rewards, const float* values, const float* loss_
                    float* advantages, float* returns, int* status, void* workspace,
                    size_t workspace_bytes, areal_stream_t stream);
 
+/* Per-row lengths for per-sample lambda functions (_build_gae_lambda_context,
+ * areal/trainer/ppo/gae.py:166-205): active tokens, and distinct turn ids among them (turn_ids
+ * may be NULL: turn counts 0). status as in areal_turn_gae. */
+int areal_gae_lambda_context(const float* loss_mask, const int32_t* turn_ids, int64_t bs,
+                             int64_t max_seqlen, int64_t* token_lengths, int64_t* turn_counts,
+                             int* status, areal_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * Normalisation
  * replaces Normalization.__call__ / _compute_mean / _compute_std

@@ -278,3 +278,89 @@ def test_turn_level_gae_matches_oracle(dev, bs, L, max_turn_len):
         scale = max(want_a.abs().max().item(), 1.0)
         torch.testing.assert_close(a.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
         torch.testing.assert_close(rt.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
+
+
+# ---------------------------------------------------------------- per-sample lambda, turn-mode advantages
+def test_gae_lambda_context_reference_literals(dev):
+    # reference tests/test_ppo_gae.py:279-341, :436-480
+    from areal_amd.ppo.gae import _build_gae_lambda_context, compute_gae_lambda
+    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda, vapo_length_adaptive_gae
+
+    mask = _t([[1, 1, 1, 1, 0], [1, 1, 0, 0, 0], [0, 0, 0, 0, 0]], dev)
+    ids = torch.tensor([[0, 0, 1, 1, -1], [0, 1, -1, -1, -1], [-1, -1, -1, -1, -1]], dtype=torch.int32, device=dev)
+    c = _build_gae_lambda_context(mask, ids, gae_timestep_unit="token")
+    assert c["effective_token_lengths"].tolist() == [4, 2, 0] and c["turn_counts"].tolist() == [2, 2, 0]
+    lam = compute_gae_lambda(vapo_length_adaptive_gae, {"alpha": 1.0}, mask, ids, "token")
+    assert torch.equal(lam.cpu(), torch.tensor([0.75, 0.5, 0.0]))
+    mask2 = _t([[1, 1, 0, 1, 1], [1, 1, 1, 1, 0], [0, 0, 0, 0, 0]], dev)
+    ids2 = torch.tensor([[0, 0, -1, 2, 2], [0, 0, 0, 0, -1], [-1, -1, -1, -1, -1]], dtype=torch.int32, device=dev)
+    lam = compute_gae_lambda(vapo_length_adaptive_gae, {"alpha": 1.0}, mask2, ids2, "turn")
+    assert torch.equal(lam.cpu(), torch.tensor([0.5, 0.0, 0.0]))
+    lam = compute_gae_lambda(relative_position_gae_lambda, {"q": 0.3}, torch.ones(2, 6, device=dev),
+                             torch.tensor([[0, 0, 1, 1, 2, 2], [0] * 6], dtype=torch.int32, device=dev), "turn")
+    torch.testing.assert_close(lam.cpu(), torch.tensor([0.3 ** 0.5, 1.0]), rtol=1e-6, atol=1e-7)
+    lam = compute_gae_lambda(vapo_length_adaptive_gae, {"alpha": 1.0}, _t([[1, 1], [1, 0]], dev), None, "token")
+    assert torch.equal(lam.cpu(), torch.tensor([0.5, 0.0]))
+    with pytest.raises(ValueError, match="one value per local trajectory"):
+        compute_gae_lambda(lambda context: torch.tensor(0.5, device=dev), {}, torch.ones(2, 2, device=dev),
+                           torch.zeros(2, 2, dtype=torch.int32, device=dev), "token")
+    with pytest.raises(ValueError, match="requires rollout data to include 'turn_ids'"):
+        _build_gae_lambda_context(mask, None, gae_timestep_unit="turn")
+    # long rows: counts over several chunks of the row
+    g = torch.Generator().manual_seed(0)
+    m = (torch.rand(7, 5000, generator=g) > 0.4).float()
+    tid = (torch.arange(5000) // 37).expand(7, -1).to(torch.int32)
+    c = _build_gae_lambda_context(m.to(dev), tid.to(dev), gae_timestep_unit="turn")
+    assert torch.equal(c["effective_token_lengths"].cpu(), m.sum(1).long())
+    want_turns = torch.tensor([len(set(tid[b][m[b] > 0].tolist())) for b in range(7)])
+    assert torch.equal(c["timestep_lengths"].cpu(), want_turns)
+
+
+def test_compute_advantages_relative_position_lambda_main_path(dev):
+    # reference tests/test_ppo_gae.py:406-433: a terminal reward decays as q^((L-k)/(L-1))
+    from areal_amd.ppo.actor import compute_advantages
+    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda
+
+    q, L = 0.3, 10
+    batch = {
+        "input_ids": torch.zeros(1, L + 1, dtype=torch.long, device=dev),
+        "loss_mask": torch.tensor([[0] + [1] * L], dtype=torch.float32, device=dev),
+        "logprobs": torch.zeros(1, L + 1, device=dev),
+        "attention_mask": torch.ones(1, L + 1, dtype=torch.bool, device=dev),
+        "rewards": torch.tensor([1.0], device=dev),
+    }
+    out = compute_advantages(batch, gae_lambda_fn=relative_position_gae_lambda, gae_lambda_kwargs={"q": q})
+    want = torch.tensor([[q ** ((L - k) / (L - 1)) for k in range(1, L + 1)] + [0.0]])
+    torch.testing.assert_close(out["advantages"].cpu(), want, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(out["returns"].cpu(), want, rtol=1e-6, atol=1e-7)
+
+
+def test_compute_advantages_turn_mode_keeps_kl_token_local(dev):
+    # reference tests/test_ppo_gae.py:551-583 in spirit: turn advantages broadcast, the token
+    # KL penalty added per token, returns carry the task reward only
+    from areal_amd.ppo.actor import compute_advantages
+    from areal_amd.data import KLEstimator
+
+    L = 6
+    batch = {
+        "input_ids": torch.zeros(1, L, dtype=torch.long, device=dev),
+        "loss_mask": torch.tensor([[0, 1, 1, 1, 1, 0]], dtype=torch.float32, device=dev),
+        "logprobs": torch.tensor([[0.0, -1.0, -2.0, -1.0, -3.0, 0.0]], device=dev),
+        "ref_logp": torch.tensor([[-1.5, -1.0, -1.0, -2.5, 0.0, 0.0]], device=dev),
+        "attention_mask": torch.tensor([[1, 1, 1, 1, 1, 0]], dtype=torch.bool, device=dev),
+        "rewards": torch.tensor([2.0], device=dev),
+        "turn_ids": torch.tensor([[-1, 0, 0, 1, 1, -1]], device=dev),
+    }
+    out = compute_advantages(dict(batch), kl_ctl=0.1, kl_estimator=KLEstimator("k1"), gae_timestep_unit="turn",
+                             gae_lambda=0.5)
+    # rolled mask [1,1,1,1,0,0], rolled ids [0,0,1,1,-1,-1]; reward 2 at position seqlen-2 = 3
+    # turns: R = [0, 2], V = 0: A_1 = 2, A_0 = 0 + 0.5 * 2 = 1
+    kl = out["kl_rewards"].cpu()
+    want_adv = torch.tensor([[1.0, 1.0, 2.0, 2.0, 0.0, 0.0]]) + kl * torch.tensor([[1, 1, 1, 1, 0, 0.0]])
+    want_adv[0, 4] = 0.0
+    torch.testing.assert_close(out["advantages"].cpu(), want_adv, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(out["returns"].cpu(), torch.tensor([[1.0, 1.0, 2.0, 2.0, 0.0, 0.0]]), rtol=1e-6, atol=1e-7)
+    with pytest.raises(ValueError, match="requires rollout data to"):
+        b2 = dict(batch)
+        del b2["turn_ids"]
+        compute_advantages(b2, gae_timestep_unit="turn")
