@@ -930,6 +930,25 @@ __global__ __launch_bounds__(256) void dlogits_from_saved_kernel(
   *ptr = out;
 }
 
+// out[v] (+)= sum over rows of dl[row][v], fp32: the lm_head bias gradient. One block per 64
+// columns: 4 row lanes x 64 columns per pass (128-byte row pieces), LDS reduce over the lanes.
+__global__ __launch_bounds__(256) void colsum_bf16_kernel(const u16* __restrict__ dl, int64_t ld,
+                                                          int64_t rows, int V, int accumulate,
+                                                          float* __restrict__ out) {
+  __shared__ float sm[4][64];
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int lane_row = threadIdx.x >> 6;
+  float acc = 0.f;
+  if (c < V)
+    for (int64_t r = lane_row; r < rows; r += 4) acc += bf16_bits_to_f32(dl[r * ld + c]);
+  sm[lane_row][threadIdx.x & 63] = acc;
+  __syncthreads();
+  if (lane_row == 0 && c < V) {
+    const float s = (sm[0][threadIdx.x] + sm[1][threadIdx.x]) + (sm[2][threadIdx.x] + sm[3][threadIdx.x]);
+    out[c] = accumulate ? out[c] + s : s;
+  }
+}
+
 // dst[c][r] = src[r][c] for r < R, c < C; dst[c][r] = 0 for R <= r < ldd. 64x64 tiles.
 __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __restrict__ src,
                                                                  int64_t lds_, int R, int C,
@@ -1170,8 +1189,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, const float* row_max, const float* sum_exp,
                      const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
-                     int accumulate, int64_t token_chunk, void* workspace, size_t workspace_bytes,
-                     hipStream_t stream) {
+                     float* dbias, int accumulate, int64_t token_chunk, void* workspace,
+                     size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0 || token_chunk <= 0) return AREAL_ERR_BAD_ARG;
   if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr)
     return AREAL_ERR_BAD_ARG;
@@ -1239,6 +1258,12 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       const Regions r = plan_regions(H, Tc, ldv, 0, 1 << 20);
       if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
     }
+    // dBias[v] += sum_t dl[t, v]
+    if (dbias != nullptr) {
+      hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
+                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, dbias);
+      AREAL_CHECK_LAUNCH();
+    }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
     if (tn) {
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv, (int)Tc};
@@ -1279,8 +1304,8 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
                            const float* probs_ref, void* dhidden, void* dweight,
-                           int dweight_mode, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream) {
+                           int dweight_mode, float* dbias, void* workspace,
+                           size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0) return AREAL_ERR_BAD_ARG;
   if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr ||
       probs == nullptr || probs_ref == nullptr)
@@ -1316,6 +1341,11 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     const StoreParams ep{dhidden, H, (int)H, (int)T};
     const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
     if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+  }
+  if (dbias != nullptr) {
+    hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
+                       dl, ldv, T, (int)V, dweight_mode == 1 ? 1 : 0, dbias);
+    AREAL_CHECK_LAUNCH();
   }
   if (dweight != nullptr) {
     // dWeight[v, h] += sum_t dl[t, v] * hidden[t, h], k-major over the Tpad rows of dl

@@ -124,6 +124,7 @@ class _FusedLMHead(torch.autograd.Function):
         ctx.token_chunk = token_chunk
         ctx.hidden_shape = hidden.shape
         ctx.weight_dtype = weight.dtype
+        ctx.bias_dtype = bias.dtype if bias is not None else None
         ctx.set_materialize_grads(False)
         ctx.mark_non_differentiable(entropy, vmin, vmax, vmean, vnorm)
         return tuple(outs[:6])
@@ -132,16 +133,18 @@ class _FusedLMHead(torch.autograd.Function):
     def backward(ctx, grad_logprobs, *unused):
         hidden_2d, weight_c, labels_1d, row_max, sum_exp = ctx.saved_tensors
         need_h, need_w, need_b = ctx.needs_input_grad[:3]
-        if need_b:
-            raise NotImplementedError("gradient of the lm_head bias is not implemented")
-        if grad_logprobs is None or not (need_h or need_w):
+        want_h = need_h
+        if grad_logprobs is None or not (need_h or need_w or need_b):
             return (None,) * 8
         lib = _lib.load()
         dev = hidden_2d.device
         T, H = hidden_2d.shape
         V = weight_c.size(0)
         g = grad_logprobs.reshape(-1).to(torch.float32).contiguous()
+        # the kernels need one of dHidden / dWeight as an output; a bias-only request computes dHidden
+        need_h = need_h or (need_b and not need_w)
         dh = torch.empty_like(hidden_2d) if need_h else None
+        db32 = torch.empty(V, dtype=torch.float32, device=dev) if need_b else None
         probs, probs_ref = ctx.probs, ctx.probs_ref
         # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
         # the chunked recompute mode accumulates in fp32 and casts at the end
@@ -152,6 +155,8 @@ class _FusedLMHead(torch.autograd.Function):
         if T == 0:
             if dw32 is not None:
                 dw32.zero_()
+            if db32 is not None:
+                db32.zero_()
         elif probs is not None:
             nbytes = lib.areal_lmhead_bwd_saved_workspace_bytes(T, H, V) if need_h else 0
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if need_h else None
@@ -161,7 +166,7 @@ class _FusedLMHead(torch.autograd.Function):
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
                 _lib.ptr(probs), _lib.ptr(probs_ref),
                 _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32), 2 if direct else 0,
-                _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+                _lib.ptr(db32), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd_saved")
             del probs, probs_ref
@@ -173,7 +178,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(ctx.bias_f),
                 _lib.ptr(labels_1d), _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
-                _lib.ptr(dh), _lib.ptr(dw32), 0, chunk,
+                _lib.ptr(dh), _lib.ptr(dw32), _lib.ptr(db32), 0, chunk,
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd")
@@ -187,9 +192,9 @@ class _FusedLMHead(torch.autograd.Function):
                     _lib.ptr(dw32), _lib.ptr(dw), dw32.numel(), _lib.stream_ptr(dev)
                 )
                 _lib.check(rc, "areal_cast_f32_to_bf16")
-        if dh is not None:
-            dh = dh.view(ctx.hidden_shape)
-        return dh, dw, None, None, None, None, None, None
+        dh = dh.view(ctx.hidden_shape) if (dh is not None and want_h) else None
+        db = db32.to(ctx.bias_dtype) if db32 is not None else None
+        return dh, dw, db, None, None, None, None, None
 
 
 def fused_lm_head_logprobs_entropy(

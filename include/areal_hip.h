@@ -61,14 +61,15 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
 
 /* grad_logprobs [T] fp32. Writes dhidden [T,H] bf16 (NULL to skip) and dweight_f32 [V,H] fp32
- * (NULL to skip; added to when accumulate != 0). dlogits are rounded to bf16 before the two
- * gradient contractions, as in vocab_parallel_head.py:830-839. */
+ * (NULL to skip; added to when accumulate != 0); dbias [V] fp32 (NULL to skip) = column sums of
+ * dlogits (vocab_parallel_head.py:862-863). dlogits are rounded to bf16 before the gradient
+ * contractions, as in vocab_parallel_head.py:830-839. */
 int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, const float* row_max, const float* sum_exp,
                      const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
-                     int accumulate, int64_t token_chunk, void* workspace, size_t workspace_bytes,
-                     areal_stream_t stream);
+                     float* dbias, int accumulate, int64_t token_chunk, void* workspace,
+                     size_t workspace_bytes, areal_stream_t stream);
 
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
@@ -77,15 +78,16 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * MI355X has the HBM to keep them). probs is overwritten with the bf16 dlogits and can be
  * used once. logprobs (NULL allowed) are the forward's label log-probabilities: with them the
  * label's dlogit is -expm1(logprob) in fp32. dweight [V,H]: dweight_mode 0 = fp32 store,
- * 1 = fp32 accumulate, 2 = bf16 store. Other arguments as areal_lmhead_bwd; bias does not enter
- * (it is part of the saved exponentials). workspace may be NULL if dhidden is. */
+ * 1 = fp32 accumulate, 2 = bf16 store; dbias [V] fp32 or NULL (added to in mode 1). Other
+ * arguments as areal_lmhead_bwd; the bias itself does not enter (it is part of the saved
+ * exponentials). workspace may be NULL if dhidden is. */
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
                            const float* probs_ref, void* dhidden, void* dweight,
-                           int dweight_mode, void* workspace, size_t workspace_bytes,
-                           areal_stream_t stream);
+                           int dweight_mode, float* dbias, void* workspace,
+                           size_t workspace_bytes, areal_stream_t stream);
 
 /* out[j*ldo + i] = sum_k A[i*lda + k] * B[j*ldb + k]  (bf16 in, fp32 accumulate).
  * out_mode 0: bf16 store, 1: fp32 store, 2: fp32 accumulate. The contraction used by the

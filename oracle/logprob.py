@@ -73,13 +73,15 @@ def lm_head_logprobs_entropy(
 
 def lm_head_backward(
     hidden, weight, labels, grad_logprobs, temperature=1.0, logit_scale=1.0, bias=None,
-    round_dlogits_to=torch.bfloat16, row_chunk: int = 1024,
+    round_dlogits_to=torch.bfloat16, row_chunk: int = 1024, with_bias_grad: bool = False,
 ):
-    """Closed-form dHidden [T,H] and dWeight [V,H] (fp32) for upstream dLoss/dlogprobs."""
+    """Closed-form dHidden [T,H] and dWeight [V,H] (fp32) for upstream dLoss/dlogprobs; with
+    ``with_bias_grad`` also dBias [V] = column sums of dlogits (vocab_parallel_head.py:862-863)."""
     inv_t = 1.0 / temperature
     w = weight.float()
     d_hidden = torch.zeros(hidden.shape, dtype=torch.float32)
     d_weight = torch.zeros(weight.shape, dtype=torch.float32)
+    d_bias = torch.zeros(weight.shape[0], dtype=torch.float32)
     for i in range(0, hidden.shape[0], row_chunk):
         h = hidden[i : i + row_chunk].float()
         x = lm_head_logits(hidden[i : i + row_chunk], weight, bias, logit_scale)
@@ -92,6 +94,9 @@ def lm_head_backward(
             d = d.to(round_dlogits_to).float()
         d_hidden[i : i + row_chunk] = d @ w
         d_weight += d.T @ h
+        d_bias += d.sum(dim=0)
+    if with_bias_grad:
+        return d_hidden, d_weight, d_bias
     return d_hidden, d_weight
 
 

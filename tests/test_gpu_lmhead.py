@@ -58,14 +58,14 @@ def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, ch
     hidden = torch.randn(T, H, generator=g).bfloat16()
     weight = (torch.randn(V, H, generator=g) * (0.5 if V < 10000 else 0.02)).bfloat16()
     bias = (torch.randn(V, generator=g) * 0.1).bfloat16() if use_bias else None
+    b_dev = bias.to(dev).requires_grad_(True) if use_bias else None
     labels = torch.randint(0, V, (T,), generator=g)
     grad = torch.randn(T, generator=g)
     grad[::3] = 0
     h = hidden.to(dev).requires_grad_(True)
     w = weight.to(dev).requires_grad_(True)
     out = fused_lm_head_logprobs_entropy(h, w, labels.to(dev), temperature=temp, logit_scale=scale,
-                                         bias=bias.to(dev) if use_bias else None, token_chunk=chunk,
-                                         save_probs=save_probs)
+                                         bias=b_dev, token_chunk=chunk, save_probs=save_probs)
     want = L.lm_head_logprobs_entropy(hidden, weight, labels, temp, scale, bias)
     names = ["logprobs", "entropy", "vocab_min", "vocab_max", "vocab_mean", "vocab_norm"]
     for name, a, b in zip(names, out, want):
@@ -75,7 +75,11 @@ def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, ch
         assert err < tol, f"{name}: max abs err {err}"
     assert out.logprobs.requires_grad and not out.entropy.requires_grad
     (out.logprobs * grad.to(dev)).sum().backward()
-    dh_want, dw_want = L.lm_head_backward(hidden, weight, labels, grad, temp, scale, bias)
+    dh_want, dw_want, db_want = L.lm_head_backward(hidden, weight, labels, grad, temp, scale, bias,
+                                                   with_bias_grad=True)
+    if use_bias:  # column sums of the bf16 dlogits (vocab_parallel_head.py:862-863)
+        assert b_dev.grad.dtype == torch.bfloat16
+        assert _rel(b_dev.grad.cpu().float(), db_want) < 1e-2
     assert h.grad.dtype == torch.bfloat16 and w.grad.dtype == torch.bfloat16
     assert _rel(h.grad.cpu().float(), dh_want) < 1e-2
     assert _rel(w.grad.cpu().float(), dw_want) < 1e-2

@@ -55,9 +55,10 @@ def test_lm_head_against_float64_and_autograd(temp, scale, use_bias):
     y = torch.randint(0, V, (T,))
     out = L.lm_head_logprobs_entropy(h, w, y, temp, scale, b)
     hd, wd = h.double().requires_grad_(True), w.double().requires_grad_(True)
+    bd = b.double().requires_grad_(True) if b is not None else None
     logits = hd @ wd.T
     if b is not None:
-        logits = logits + b.double()
+        logits = logits + bd
     logits = logits * scale
     lsm = torch.log_softmax(logits / temp, -1)
     lp = lsm.gather(-1, y[:, None])[:, 0]
@@ -70,7 +71,9 @@ def test_lm_head_against_float64_and_autograd(temp, scale, use_bias):
     g = torch.randn(T)
     g[::3] = 0
     (lp * g.double()).sum().backward()
-    dh, dw = L.lm_head_backward(h, w, y, g, temp, scale, b, round_dlogits_to=None)
+    dh, dw, db = L.lm_head_backward(h, w, y, g, temp, scale, b, round_dlogits_to=None, with_bias_grad=True)
+    if b is not None:
+        torch.testing.assert_close(db.double(), bd.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(dh.double(), hd.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(dw.double(), wd.grad, rtol=1e-4, atol=1e-5)
     assert (dh[::3] == 0).all()  # zero upstream gradient -> exactly zero rows
