@@ -32,6 +32,11 @@ struct GemmArgs {
   int K;                              // multiple of 8
   int acols, bcols;                   // k-major (TN) form only: readable columns of A and B
   int akrows;                         // k-major form only: rows of A that may be read (<= K)
+  // split-K (gemm_nt_sweep with a store epilogue only): the grid is ksplit copies of the tile
+  // schedule; copy z contracts k-tiles [z*kt_per_split, (z+1)*kt_per_split) and writes its
+  // partial result zstride bytes after the previous copy's. ksplit <= 1: off.
+  int ksplit, kt_per_split;
+  int64_t zstride;
 };
 
 // Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
@@ -228,12 +233,24 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
                                                           typename Epi::Params ep) {
   __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
   int bj, split, ai_begin, ai_end;
-  if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
+  int wg = blockIdx.x, nk = g.K / BK;
+  if (g.ksplit > 1) {
+    const int per_copy = gridDim.x / g.ksplit;
+    const int z = wg / per_copy;
+    wg -= z * per_copy;
+    const int kt0 = z * g.kt_per_split;
+    nk -= kt0;
+    nk = nk < g.kt_per_split ? nk : g.kt_per_split;
+    g.A += (int64_t)kt0 * BK;
+    g.B += (int64_t)kt0 * BK;
+    Epi::split_output(ep, (int64_t)z * g.zstride);
+    if (nk <= 0) return;
+  }
+  if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave >> 1, wb = wave & 1;
-  const int nk = g.K / BK;
 
   // ---- loader: lane -> (row of the wave's 64-row slice, swizzled chunk)
   const u16* ga[8];
@@ -562,6 +579,7 @@ struct StoreEpi {
   struct State {};
   static DEVI void begin(State&, const Params&, int, int, int, int) {}
   static DEVI void end(State&, const Params&, int, int, int, int) {}
+  static DEVI void split_output(Params& p, int64_t bytes) { p.out = (char*)p.out + bytes; }
   static DEVI void tile(State&, const Params& p, f32x16 (&acc)[4][4], int i0, int j0, int lane) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -627,6 +645,7 @@ struct FwdEpi {
     float m[4], s[4], q[4], xl[4], mn[4], sx[4], sx2[4];
     int lab[4];
   };
+  static DEVI void split_output(Params&, int64_t) {}
   static DEVI void begin(State& st, const Params& p, int t0, int, int, int lane) {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -842,6 +861,7 @@ struct BwdEpi {
     }
   }
   static DEVI void end(State&, const Params&, int, int, int, int) {}
+  static DEVI void split_output(Params&, int64_t) {}
 
   static DEVI void tile(State& st, const Params& p, const f32x16 (&acc)[4][4], int v0, int t0, int lane) {
     const int vl = v0 + 4 * (lane >> 5);
@@ -968,6 +988,24 @@ __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __re
   }
 }
 
+// out[i] = bf16(sum_z part[z * zstride + i]): the split-K partial results of dHidden.
+__global__ void splitk_reduce_bf16_kernel(const float* __restrict__ part, int Z, int64_t zstride,
+                                          int64_t n, u16* __restrict__ out) {
+  int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
+  for (; i < n; i += stride) {  // n % 4 == 0
+    f32x4 a = *(const f32x4*)(part + i);
+    for (int z = 1; z < Z; ++z) {
+      const f32x4 b = *(const f32x4*)(part + (int64_t)z * zstride + i);
+      a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+    }
+    u32x2 o;
+    o[0] = (uint32_t)f32_to_bf16_bits(a[0]) | ((uint32_t)f32_to_bf16_bits(a[1]) << 16);
+    o[1] = (uint32_t)f32_to_bf16_bits(a[2]) | ((uint32_t)f32_to_bf16_bits(a[3]) << 16);
+    *(u32x2*)(out + i) = o;
+  }
+}
+
 __global__ void cast_f32_to_bf16_kernel(const float* __restrict__ src, u16* __restrict__ dst,
                                         int64_t n) {
   int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
@@ -1005,8 +1043,8 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
   if (S < 1) S = 1;
   const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
   if constexpr (KERNEL == KERNEL_NT)
-    hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
-                       sc, ep);
+    hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
+                       dim3(NTHREADS), 0, stream, g, sc, ep);
   else if constexpr (KERNEL == KERNEL_TN)
     hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
@@ -1078,6 +1116,54 @@ int check_operand(const void* p, int64_t ld) {
 
 // Slots of partial softmax statistics per token written by the forward launches.
 int fwd_slots(const Regions& r) { return 4 * r.S + (r.ragged_a ? 4 : 0); }
+
+// dHidden [T, H] has few output tiles when the model is small (H / 256 x T / 256). When the
+// tile count does not fill whole rounds of 256 workgroups, the vocabulary (K) range is split
+// over copies of the schedule, each writing an fp32 partial result that
+// splitk_reduce_bf16_kernel sums.
+int dh_ksplit(int64_t H, int64_t T, int64_t K) {
+  const int64_t tiles = ceil_div_i64(H, TILE) * ceil_div_i64(T, TILE);
+  if (tiles >= 2048 || K % BK != 0) return 1;
+  const int64_t nk = K / BK;
+  // rounds of 256 workgroups per unit of K, plus a small charge per split for the reduction
+  int best = 1;
+  double best_cost = (double)ceil_div_i64(tiles, 256);
+  for (int z = 2; z <= 16 && z <= nk / 8; ++z) {
+    const double cost = (double)ceil_div_i64(tiles * z, 256) / z + 0.03 * (z - 1);
+    if (cost < best_cost - 1e-9) { best_cost = cost; best = z; }
+  }
+  return best;
+}
+size_t dh_partial_bytes(int64_t H, int64_t T, int64_t K) {
+  const int z = dh_ksplit(H, T, K);
+  return z > 1 ? (size_t)z * (size_t)(T * H) * sizeof(float) + 256 : 0;
+}
+
+// dHidden[t, h] = sum_v dl[t, v] * W^T[h, v], bf16 out; split-K through `partial` when it pays.
+int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t T, void* dhidden,
+                   float* partial, hipStream_t stream) {
+  GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
+  const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
+  int z = dh_ksplit(H, T, ldv);
+  const int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
+  if (z > 1) z = (int)ceil_div_i64(ldv / BK, kps);  // no empty split
+  if (z <= 1 || partial == nullptr) {
+    const StoreParams ep{dhidden, H, (int)H, (int)T};
+    return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  }
+  g.ksplit = z;
+  g.kt_per_split = kps;
+  g.zstride = T * H * (int64_t)sizeof(float);
+  const StoreParams ep{partial, H, (int)H, (int)T};
+  int rc = launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  if (rc != AREAL_OK) return rc;
+  int64_t blocks = ceil_div_i64(T * H, 256 * 4);
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial,
+                     z, T * H, T * H, (u16*)dhidden);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
 
 }  // namespace
 
@@ -1180,7 +1266,8 @@ size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t
   int64_t elems = H * ldv + Tc * ldv;
   const bool ragged = (Tc % BK != 0) || (T % Tc) % BK != 0;  // some chunk is not a multiple of 64
   if (ragged) elems += H * ldt + V * ldt;
-  return (size_t)elems * 2 + 4 * 256;  // slack for 256-byte sub-buffer alignment
+  // slack for 256-byte sub-buffer alignment
+  return (size_t)elems * 2 + dh_partial_bytes(H, Tc, ldv) + 5 * 256;
 }
 
 // Backward. grad_logprobs [T] fp32 = dLoss/dlogprobs. Writes dhidden [T,H] bf16 and adds the
@@ -1219,6 +1306,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   u16* dl = carve(wp, Tc_max * ldv * 2);
   u16* hT = ragged ? carve(wp, H * ldt * 2) : nullptr;
   u16* dlT = ragged ? carve(wp, V * ldt * 2) : nullptr;
+  float* dh_part = dh_partial_bytes(H, Tc_max, ldv) ? (float*)carve(wp, dh_partial_bytes(H, Tc_max, ldv)) : nullptr;
 
   const float c2 = inv_temperature * LOG2E;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
@@ -1253,10 +1341,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
-      GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)Tc, (int)ldv, 0, 0, 0};
-      const StoreParams ep{(u16*)dhidden + t0 * H, H, (int)H, (int)Tc};
-      const Regions r = plan_regions(H, Tc, ldv, 0, 1 << 20);
-      if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+      if ((rc = launch_dhidden(wT, dl, ldv, H, Tc, (u16*)dhidden + t0 * H, dh_part, stream)) != AREAL_OK)
+        return rc;
     }
     // dBias[v] += sum_t dl[t, v]
     if (dbias != nullptr) {
@@ -1291,7 +1377,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 // Workspace of the backward from saved exponentials: W^T [H, round_up(V, 64)] bf16.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
-  return (size_t)(H * round_up_i64(V, BK)) * 2 + 256;
+  return (size_t)(H * round_up_i64(V, BK)) * 2 + dh_partial_bytes(H, T, round_up_i64(V, BK)) + 512;
 }
 
 // Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref): no logits are
@@ -1336,11 +1422,10 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
                        dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
                        dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
     AREAL_CHECK_LAUNCH();
-    // dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
-    GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
-    const StoreParams ep{dhidden, H, (int)H, (int)T};
-    const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
-    if ((rc = launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)) != AREAL_OK) return rc;
+    float* dh_part = dh_partial_bytes(H, T, ldv)
+                         ? (float*)(((uintptr_t)(wT + H * ldv) + 255) & ~(uintptr_t)255)
+                         : nullptr;
+    if ((rc = launch_dhidden(wT, dl, ldv, H, T, dhidden, dh_part, stream)) != AREAL_OK) return rc;
   }
   if (dbias != nullptr) {
     hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
