@@ -36,7 +36,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_lmhead_fwd_workspace_bytes": (SZ, [I64, I64, I64]),
     "areal_lmhead_fwd": (
         I,
-        [P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
+        [P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
     "areal_lmhead_bwd_workspace_bytes": (SZ, [I64, I64, I64, I64]),
     "areal_lmhead_bwd": (

@@ -571,9 +571,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
 // ---------------------------------------------------------------------------------------
 struct StoreParams {
   void* out; int64_t ldo; int M; int N;  // M % 4 == 0
+  const float* jscale;                   // MODE 3: [N] factors of the output rows j
 };
 
-template <bool EDGE, int MODE>  // MODE 0: bf16 store, 1: fp32 store, 2: fp32 accumulate
+// MODE 0: bf16 store, 1: fp32 store, 2: fp32 accumulate, 3: bf16 store of jscale[j] * value
+template <bool EDGE, int MODE>
 struct StoreEpi {
   typedef StoreParams Params;
   struct State {};
@@ -584,16 +586,19 @@ struct StoreEpi {
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int j = j0 + b * 32 + (lane & 31);
+      float js = 1.f;
+      if (MODE == 3) js = (!EDGE || j < p.N) ? p.jscale[j] : 0.f;
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int i = i0 + a * 32 + 8 * rq + 4 * (lane >> 5);
           if (!EDGE || (j < p.N && i < p.M)) {
-            const float x0 = acc[a][b][rq * 4 + 0], x1 = acc[a][b][rq * 4 + 1];
-            const float x2 = acc[a][b][rq * 4 + 2], x3 = acc[a][b][rq * 4 + 3];
+            float x0 = acc[a][b][rq * 4 + 0], x1 = acc[a][b][rq * 4 + 1];
+            float x2 = acc[a][b][rq * 4 + 2], x3 = acc[a][b][rq * 4 + 3];
+            if (MODE == 3) { x0 *= js; x1 *= js; x2 *= js; x3 *= js; }
             const int64_t off = (int64_t)j * p.ldo + i;
-            if (MODE == 0) {
+            if (MODE == 0 || MODE == 3) {
               u32x2 v;
               v[0] = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
               v[1] = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
@@ -614,6 +619,57 @@ struct StoreEpi {
 template <bool E> using StoreBf16 = StoreEpi<E, 0>;
 template <bool E> using StoreF32 = StoreEpi<E, 1>;
 template <bool E> using AccumF32 = StoreEpi<E, 2>;
+template <bool E> using StoreBf16Scaled = StoreEpi<E, 3>;
+
+// Row reference of the saved exponentials e = 2^(c2 x - ref): ref[t] = c2 * (the largest of NREF
+// logits of token t: its label's and a fixed stride sample of the vocabulary) + REF_MARGIN. The
+// estimate never exceeds the row maximum, so the largest exponential of a row is at least
+// 2^-REF_MARGIN and everything within 2^-(126 - REF_MARGIN) of it is a normal bf16 number; the
+// exponentials stay usable while the row maximum is within REF_WINDOW binades above the estimate
+// (largest one 2^(REF_WINDOW - REF_MARGIN), small enough for fp32 accumulation over the
+// vocabulary). lmhead_merge_kernel checks that with the exact row maximum and raises *status
+// otherwise. One wave per token; also clears *status.
+constexpr int NREF = 8;
+constexpr float REF_MARGIN = 60.f;
+constexpr float REF_WINDOW = 150.f;
+
+__global__ __launch_bounds__(256) void lmhead_rowref_kernel(
+    const u16* __restrict__ hidden, const u16* __restrict__ weight, const float* __restrict__ bias,
+    const int64_t* __restrict__ labels, int T, int H, int V, float scale, float c2,
+    float* __restrict__ row_ref, int* __restrict__ status) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) *status = 0;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t >= T) return;
+  int ids[NREF];
+#pragma unroll
+  for (int k = 0; k < NREF; ++k) ids[k] = (int)(((int64_t)k * V) / NREF);
+  const int64_t lab = labels[t];
+  if (lab >= 0 && lab < V) ids[0] = (int)lab;
+  float acc[NREF];
+#pragma unroll
+  for (int k = 0; k < NREF; ++k) acc[k] = 0.f;
+  const u16* hrow = hidden + (int64_t)t * H;
+  for (int h = lane * 8; h < H; h += 512) {  // H % 8 == 0
+    const u32x4 hv = *(const u32x4*)(hrow + h);
+#pragma unroll
+    for (int k = 0; k < NREF; ++k) {
+      const u32x4 wv = *(const u32x4*)(weight + (int64_t)ids[k] * H + h);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[k] = fmaf(bf16_bits_to_f32((u16)(hv[i] & 0xffffu)), bf16_bits_to_f32((u16)(wv[i] & 0xffffu)), acc[k]);
+        acc[k] = fmaf(bf16_bits_to_f32((u16)(hv[i] >> 16)), bf16_bits_to_f32((u16)(wv[i] >> 16)), acc[k]);
+      }
+    }
+  }
+  float mx = neg_inf();
+#pragma unroll
+  for (int k = 0; k < NREF; ++k) {
+    const float x = (wave_sum(acc[k]) + (bias != nullptr ? bias[ids[k]] : 0.f)) * scale;
+    mx = fmaxf(mx, x);
+  }
+  if (lane == 0) row_ref[t] = fmaf(mx, c2, REF_MARGIN);
+}
 
 // ---------------------------------------------------------------------------------------
 // Epilogue 1: online softmax statistics over the vocabulary (forward).
@@ -632,10 +688,10 @@ struct FwdParams {
   float* ws;          // [NSTAT][P][T]
   int P;              // total partial slots
   int slot_base;      // first slot written by this launch
-  // SAVE: e[t][v] = exp2(c2 * x[t][v] - ref[v / 128][t]) in bf16, ref = c2 * (maximum of the
-  // 128 logits of the block); columns [V, ldv) are written as zero.
+  // SAVE: e[t][v] = exp2(c2 * x[t][v] - ref[t]) in bf16, ref = the row reference that
+  // lmhead_rowref_kernel prepared; columns [V, ldv) are written as zero.
   u16* probs; int64_t ldv;
-  float* probs_ref;   // [ceil(V / 128)][T]
+  const float* probs_ref;  // [T]
 };
 
 template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
@@ -671,9 +727,12 @@ struct FwdEpi {
     };
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
+      const int tok = t0 + b * 32 + (lane & 31);
+      float rr = 0.f;  // SAVE: the token's row reference, needed after the statistics pass
+      if (SAVE && (!EDGE || tok < p.T)) rr = p.probs_ref[tok];
       float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+      for (int a = 0; a < 4; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float x = logit(a, b, r);
@@ -683,10 +742,10 @@ struct FwdEpi {
             if (MOMENTS) { sx += x; sx2 = fmaf(x, x, sx2); }
           }
         }
+        if (SAVE) __builtin_amdgcn_sched_barrier(0);  // 16 accumulator reads at a time
+      }
       st.mn[b] = fminf(st.mn[b], tmin);
       if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
-      // SAVE: both lanes of a token (lane, lane ^ 32) use the maximum of all 128 logits
-      if (SAVE) tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
       const float m_old = st.m[b];
       const float m_new = fmaxf(m_old, tmax);
       // rescale the running sums to the new maximum; on the first tile m_old = -inf and
@@ -707,13 +766,13 @@ struct FwdEpi {
             if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
           }
       } else {
-        // exponentials relative to the block maximum (what is stored), folded into the
-        // running sums with the factor 2^(block max - running max) <= 1
-        const bool any = !EDGE || tmax > neg_inf();  // false: every row of the block is >= V
-        const float rc = any ? tmax * p.c2 : 0.f;
-        const int tok = t0 + b * 32 + (lane & 31);
+        // The sums take the exponentials relative to the running maximum, as above (in (0, 1]
+        // whatever the row reference is); what is stored is the same exponential moved to the
+        // row reference by one factor per (token, tile). That factor over- or underflows only
+        // where the stored value is not used: rows outside the reference window, and tiles
+        // whose maximum lies 126 binades below the row's.
+        const float gamma = fast_exp2(mc - rr);
         u16* row = p.probs + (int64_t)tok * p.ldv;
-        float ts = 0.f, tq = 0.f;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
 #pragma unroll
@@ -722,11 +781,12 @@ struct FwdEpi {
             u16 d[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-              const float t = fmaf(logit(a, b, rq * 4 + k), p.c2, -rc);
-              float e = fast_exp2(t);
-              if (EDGE && vq + k >= p.V) e = 0.f;
-              else { ts += e; tq = fmaf(t, e, tq); }
-              d[k] = f32_to_bf16_bits(e);
+              const float t = fmaf(logit(a, b, rq * 4 + k), p.c2, -mc);
+              const float e = fast_exp2(t);
+              float es = e * gamma;
+              if (EDGE && vq + k >= p.V) es = 0.f;
+              else { s += e; q = fmaf(t, e, q); }
+              d[k] = f32_to_bf16_bits(es);
             }
             if (!EDGE || (tok < p.T && vq < p.ldv)) {
               u32x2 pk;
@@ -737,15 +797,9 @@ struct FwdEpi {
           }
           // pins the partial sums here: without it the compiler sinks the whole summation
           // chain below the stores of all four token blocks and spills every term
-          asm volatile("" : "+v"(ts), "+v"(tq));
+          asm volatile("" : "+v"(s), "+v"(q));
           __builtin_amdgcn_sched_barrier(0);
         }
-        const float db = any ? rc - mc : 0.f;  // <= 0
-        const float beta = fast_exp2(db);
-        s = fmaf(beta, ts, s);
-        q = fmaf(beta, fmaf(db, ts, tq), q);
-        if ((lane >> 5) == 0 && (!EDGE || (tok < p.T && v0 < p.V)))
-          p.probs_ref[(int64_t)(v0 >> 7) * p.T + tok] = rc;
       }
       st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
       const int lab = st.lab[b];
@@ -790,7 +844,8 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
                                     float* __restrict__ entropy, float* __restrict__ vmin,
                                     float* __restrict__ vmax, float* __restrict__ vmean,
                                     float* __restrict__ vnorm, float* __restrict__ row_max,
-                                    float* __restrict__ sum_exp) {
+                                    float* __restrict__ sum_exp,
+                                    const float* __restrict__ row_ref, int* __restrict__ status) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const int64_t PT = (int64_t)P * T;
@@ -821,6 +876,8 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
   if (vnorm) vnorm[t] = (float)sqrt(sx2);
   if (row_max) row_max[t] = M;
   if (sum_exp) sum_exp[t] = S;
+  // the saved exponentials of this row are usable if its largest one is at most 2^(window - margin)
+  if (row_ref != nullptr && !(fmaf(M, c2, -row_ref[t]) <= REF_WINDOW - REF_MARGIN)) atomicMax(status, 1);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -915,52 +972,71 @@ template <bool E> using BwdAffine = BwdEpi<E, true, false>;
 template <bool E> using BwdPlainT = BwdEpi<E, false, true>;
 template <bool E> using BwdAffineT = BwdEpi<E, true, true>;
 
-// dlogits from the exponentials the forward saved, in place:
-//   dl[t][v] = g[t] * invT * scale * (onehot(v == label[t]) - e[t][v] * 2^(ref[v/128][t] - lse2[t]))
-// with lse2 = c2 * row_max + log2(sum_exp). The label's entry is taken from the fp32 label
-// log-probability, -expm1(logprob), so that 1 - p keeps its precision when p is close to 1.
-// Rows [T, Tpad) are written as zero. One thread per 8 columns; grid (ceil(ldv / 2048), Tpad).
-__global__ __launch_bounds__(256) void dlogits_from_saved_kernel(
+// Operands of the backward from the exponentials the forward saved, e[t][v] = 2^(c2 x - ref[t]):
+//   dlogits[t][v] = f[t] * e'[t][v],   f[t] = -g[t] * invT * scale * 2^(ref[t] - lse2[t]),
+// with lse2 = c2 * row_max + log2(sum_exp) and e' = e except at the label, where
+// e' = expm1(logprob) * 2^(lse2 - ref) taken from the fp32 label log-probability (so that
+// f * e' = -g' * expm1(logprob) = g' * (1 - p) keeps its precision when p is close to 1).
+// The row factor f never multiplies the [T, V] buffer: dHidden scales its output rows by it and
+// dWeight contracts e' with hs = bf16(f[t] * hidden[t][:]). One block per row of probs:
+// rows < T write f[t], hs[t][:] and the label's entry; rows [T, Tpad) are cleared.
+__global__ __launch_bounds__(256) void saved_prep_kernel(
     u16* __restrict__ probs, int64_t ldv, const float* __restrict__ ref,
     const int64_t* __restrict__ labels, const float* __restrict__ row_max,
     const float* __restrict__ sum_exp, const float* __restrict__ grad,
-    const float* __restrict__ logprobs, int T, int V, float c2, float gscale) {
-  const int t = blockIdx.y;
-  const int64_t v = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
-  if (v >= ldv) return;
-  u32x4* ptr = (u32x4*)(probs + (int64_t)t * ldv + v);
-  if (t >= T) { *ptr = u32x4{0u, 0u, 0u, 0u}; return; }
-  const float lse2 = fmaf(row_max[t], c2, fast_log2(sum_exp[t]));
-  const float gs = grad[t] * gscale;
-  int64_t lab = labels[t];
-  if (lab >= V) lab = -1;
-  // blocks past the vocabulary (only padding columns, stored as zero) have no reference
-  const float r = (v < V) ? ref[(v >> 7) * T + t] : lse2;
-  const float f = -gs * fast_exp2(r - lse2);
-  const u32x4 in = *ptr;
-  u32x4 out;
-#pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    float lo = bf16_bits_to_f32((u16)(in[k] & 0xffffu)) * f;
-    float hi = bf16_bits_to_f32((u16)(in[k] >> 16)) * f;
-    if (v + 2 * k == lab) lo = logprobs ? -gs * expm1f(logprobs[t]) : lo + gs;
-    if (v + 2 * k + 1 == lab) hi = logprobs ? -gs * expm1f(logprobs[t]) : hi + gs;
-    out[k] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    const float* __restrict__ logprobs, const u16* __restrict__ hidden, int T, int H, int V,
+    float c2, float gscale, float* __restrict__ rowfac, u16* __restrict__ hs) {
+  const int t = blockIdx.x;
+  if (t >= T) {
+    u16* row = probs + (int64_t)t * ldv;
+    for (int64_t v = (int64_t)threadIdx.x * 8; v < ldv; v += 2048) *(u32x4*)(row + v) = u32x4{0u, 0u, 0u, 0u};
+    return;
   }
-  *ptr = out;
+  const float lse2 = fmaf(row_max[t], c2, fast_log2(sum_exp[t]));
+  const float f = -(grad[t] * gscale) * fast_exp2(ref[t] - lse2);
+  if (threadIdx.x == 0) {
+    rowfac[t] = f;
+    const int64_t lab = labels[t];
+    if (lab >= 0 && lab < V) {
+      u16* e = probs + (int64_t)t * ldv + lab;
+      const float unit = fast_exp2(lse2 - ref[t]);  // a probability of 1 in the units of e
+      const float el = logprobs ? expm1f(logprobs[t]) * unit : bf16_bits_to_f32(*e) - unit;
+      *e = f32_to_bf16_bits(el);
+    }
+  }
+  if (hs != nullptr) {
+    const u16* src = hidden + (int64_t)t * H;
+    u16* dst = hs + (int64_t)t * H;
+    for (int h = threadIdx.x * 8; h < H; h += 2048) {  // H % 8 == 0
+      const u32x4 in = *(const u32x4*)(src + h);
+      u32x4 out;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float lo = bf16_bits_to_f32((u16)(in[k] & 0xffffu)) * f;
+        const float hi = bf16_bits_to_f32((u16)(in[k] >> 16)) * f;
+        out[k] = (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+      }
+      *(u32x4*)(dst + h) = out;
+    }
+  }
 }
 
-// out[v] (+)= sum over rows of dl[row][v], fp32: the lm_head bias gradient. One block per 64
-// columns: 4 row lanes x 64 columns per pass (128-byte row pieces), LDS reduce over the lanes.
+// out[v] (+)= sum over rows of w[row] * dl[row][v] (w = 1 when null), fp32: the lm_head bias
+// gradient. One block per 64 columns: 4 row lanes x 64 columns per pass (128-byte row pieces),
+// LDS reduce over the lanes.
 __global__ __launch_bounds__(256) void colsum_bf16_kernel(const u16* __restrict__ dl, int64_t ld,
                                                           int64_t rows, int V, int accumulate,
+                                                          const float* __restrict__ w,
                                                           float* __restrict__ out) {
   __shared__ float sm[4][64];
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int lane_row = threadIdx.x >> 6;
   float acc = 0.f;
   if (c < V)
-    for (int64_t r = lane_row; r < rows; r += 4) acc += bf16_bits_to_f32(dl[r * ld + c]);
+    for (int64_t r = lane_row; r < rows; r += 4) {
+      const float x = bf16_bits_to_f32(dl[r * ld + c]);
+      acc = w != nullptr ? fmaf(w[r], x, acc) : acc + x;
+    }
   sm[lane_row][threadIdx.x & 63] = acc;
   __syncthreads();
   if (lane_row == 0 && c < V) {
@@ -988,9 +1064,11 @@ __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __re
   }
 }
 
-// out[i] = bf16(sum_z part[z * zstride + i]): the split-K partial results of dHidden.
+// out[i] = bf16(scale[i / row_len] * sum_z part[z * zstride + i]) (scale = 1 when null): the
+// split-K partial results of dHidden. row_len % 4 == 0.
 __global__ void splitk_reduce_bf16_kernel(const float* __restrict__ part, int Z, int64_t zstride,
-                                          int64_t n, u16* __restrict__ out) {
+                                          int64_t n, const float* __restrict__ scale,
+                                          int64_t row_len, u16* __restrict__ out) {
   int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
   for (; i < n; i += stride) {  // n % 4 == 0
@@ -998,6 +1076,10 @@ __global__ void splitk_reduce_bf16_kernel(const float* __restrict__ part, int Z,
     for (int z = 1; z < Z; ++z) {
       const f32x4 b = *(const f32x4*)(part + (int64_t)z * zstride + i);
       a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+    }
+    if (scale != nullptr) {
+      const float f = scale[i / row_len];
+      a[0] *= f; a[1] *= f; a[2] *= f; a[3] *= f;
     }
     u32x2 o;
     o[0] = (uint32_t)f32_to_bf16_bits(a[0]) | ((uint32_t)f32_to_bf16_bits(a[1]) << 16);
@@ -1139,28 +1221,31 @@ size_t dh_partial_bytes(int64_t H, int64_t T, int64_t K) {
   return z > 1 ? (size_t)z * (size_t)(T * H) * sizeof(float) + 256 : 0;
 }
 
-// dHidden[t, h] = sum_v dl[t, v] * W^T[h, v], bf16 out; split-K through `partial` when it pays.
+// dHidden[t, h] = tscale[t] * sum_v dl[t, v] * W^T[h, v] (tscale = 1 when null), bf16 out;
+// split-K through `partial` when it pays.
 int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t T, void* dhidden,
-                   float* partial, hipStream_t stream) {
+                   float* partial, const float* tscale, hipStream_t stream) {
   GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
   const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
   int z = dh_ksplit(H, T, ldv);
   const int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
   if (z > 1) z = (int)ceil_div_i64(ldv / BK, kps);  // no empty split
   if (z <= 1 || partial == nullptr) {
-    const StoreParams ep{dhidden, H, (int)H, (int)T};
+    const StoreParams ep{dhidden, H, (int)H, (int)T, tscale};
+    if (tscale != nullptr)
+      return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
     return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
   }
   g.ksplit = z;
   g.kt_per_split = kps;
   g.zstride = T * H * (int64_t)sizeof(float);
-  const StoreParams ep{partial, H, (int)H, (int)T};
+  const StoreParams ep{partial, H, (int)H, (int)T, nullptr};
   int rc = launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
   if (rc != AREAL_OK) return rc;
   int64_t blocks = ceil_div_i64(T * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
   hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial,
-                     z, T * H, T * H, (u16*)dhidden);
+                     z, T * H, T * H, tscale, H, (u16*)dhidden);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -1206,17 +1291,22 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // may be null; vocab_mean and vocab_norm cost two extra operations per logit and are computed
 // only when one of them is requested.
 //
-// probs / probs_ref (both null or both set) keep the exponentials of the softmax for
-// areal_lmhead_bwd_saved: probs bf16 [round_up(T, 64)][round_up(V, 64)] (rows >= T are not
-// written), probs_ref fp32 [ceil(V / 128)][T].
+// probs / probs_ref / probs_status (all null or all set) keep the exponentials of the softmax
+// for areal_lmhead_bwd_saved: probs bf16 [round_up(T, 64)][round_up(V, 64)] (rows >= T are not
+// written) holds e = 2^(c2 x - probs_ref[t]); probs_ref fp32 [T] is a per-row reference taken
+// from a few logits of the row before the sweep; *probs_status (one int) is set to 0 when every
+// row's exponentials are in range and to 1 when some row's maximum lies more than 150 binades
+// above its estimate: then probs must not be used and the backward has to recompute.
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
                      float* row_max, float* sum_exp, void* probs, float* probs_ref,
-                     void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                     int* probs_status, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0 || labels == nullptr) return AREAL_ERR_BAD_ARG;
-  if ((probs == nullptr) != (probs_ref == nullptr)) return AREAL_ERR_BAD_ARG;
+  if ((probs == nullptr) != (probs_ref == nullptr) || (probs == nullptr) != (probs_status == nullptr))
+    return AREAL_ERR_BAD_ARG;
   if (probs != nullptr && !aligned16(probs)) return AREAL_ERR_ALIGNMENT;
   if (!(inv_temperature > 0.f) || !(logit_scale > 0.f)) return AREAL_ERR_BAD_ARG;
   if (T == 0) return AREAL_OK;
@@ -1235,6 +1325,12 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   ep_a.slot_base = 4 * r.S;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
   const bool moments = (vocab_mean != nullptr) || (vocab_norm != nullptr);
+  if (probs != nullptr) {
+    hipLaunchKernelGGL(lmhead_rowref_kernel, dim3((unsigned)ceil_div_i64(T, 4)), dim3(256), 0, stream,
+                       (const u16*)hidden, (const u16*)weight, bias, labels, (int)T, (int)H, (int)V,
+                       logit_scale, inv_temperature * LOG2E, probs_ref, probs_status);
+    AREAL_CHECK_LAUNCH();
+  }
   if (probs == nullptr) {
     if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
     else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
@@ -1251,7 +1347,7 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, threads)), dim3(threads),
                      0, stream, (const float*)workspace, P, (int)T, (int)V, inv_temperature,
                      inv_temperature * LOG2E, logprobs, entropy, vocab_min, vocab_max, vocab_mean,
-                     vocab_norm, row_max, sum_exp);
+                     vocab_norm, row_max, sum_exp, (const float*)probs_ref, probs_status);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -1341,13 +1437,13 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
-      if ((rc = launch_dhidden(wT, dl, ldv, H, Tc, (u16*)dhidden + t0 * H, dh_part, stream)) != AREAL_OK)
+      if ((rc = launch_dhidden(wT, dl, ldv, H, Tc, (u16*)dhidden + t0 * H, dh_part, nullptr, stream)) != AREAL_OK)
         return rc;
     }
     // dBias[v] += sum_t dl[t, v]
     if (dbias != nullptr) {
       hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
-                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, dbias);
+                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, nullptr, dbias);
       AREAL_CHECK_LAUNCH();
     }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
@@ -1374,17 +1470,22 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   return AREAL_OK;
 }
 
-// Workspace of the backward from saved exponentials: W^T [H, round_up(V, 64)] bf16.
+// Workspace of the backward from saved exponentials: row factors [T] fp32, scaled hidden states
+// [T, H] bf16, W^T [H, round_up(V, 64)] bf16 and the split-K partials of dHidden.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
-  return (size_t)(H * round_up_i64(V, BK)) * 2 + dh_partial_bytes(H, T, round_up_i64(V, BK)) + 512;
+  return (size_t)T * 4 + (size_t)(T * H) * 2 + (size_t)(H * round_up_i64(V, BK)) * 2 +
+         dh_partial_bytes(H, T, round_up_i64(V, BK)) + 4 * 256;
 }
 
-// Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref): no logits are
-// recomputed. probs is overwritten with the bf16 dlogits, so it can be used once. logprobs
-// (nullable) are the label log-probabilities of the forward; with them the label's entry of
-// dlogits is evaluated in fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32
-// accumulate, 2 = bf16 store (the whole batch is one contraction, so no fp32 staging is needed).
+// Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref, with *probs_status
+// read back as 0): no logits are recomputed and no pass rewrites the [T, V] buffer. Per row,
+// dlogits = f[t] * e' with a row factor f; dHidden scales its output rows by f and dWeight
+// contracts e' with f[t] * hidden[t]. Only the label's entry of each row of probs is rewritten
+// (and rows [T, round_up(T, 64)) are cleared), so probs can be used once. logprobs (nullable)
+// are the label log-probabilities of the forward; with them the label's entry is evaluated in
+// fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store (the
+// whole batch is one contraction, so no fp32 staging is needed).
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
@@ -1406,36 +1507,37 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   if (!aligned16(probs)) return AREAL_ERR_ALIGNMENT;
   if (dhidden != nullptr && !aligned16(dhidden)) return AREAL_ERR_ALIGNMENT;
   if (dweight != nullptr && !aligned16(dweight)) return AREAL_ERR_ALIGNMENT;
-  if (dhidden != nullptr &&
-      (workspace == nullptr || workspace_bytes < areal_lmhead_bwd_saved_workspace_bytes(T, H, V)))
+  if (workspace == nullptr || workspace_bytes < areal_lmhead_bwd_saved_workspace_bytes(T, H, V))
     return AREAL_ERR_WORKSPACE;
   const int64_t ldv = round_up_i64(V, BK), Tpad = round_up_i64(T, BK);
-  u16* dl = (u16*)probs;
-  hipLaunchKernelGGL(dlogits_from_saved_kernel,
-                     dim3((unsigned)ceil_div_i64(ldv, 2048), (unsigned)Tpad), dim3(256), 0, stream,
-                     dl, ldv, probs_ref, labels, row_max, sum_exp, grad_logprobs, logprobs, (int)T,
-                     (int)V, inv_temperature * LOG2E, inv_temperature * logit_scale);
+  auto align256 = [](void* q) { return (void*)(((uintptr_t)q + 255) & ~(uintptr_t)255); };
+  float* rowfac = (float*)align256(workspace);
+  u16* hs = (u16*)align256(rowfac + T);
+  u16* wT = (u16*)align256(hs + T * H);
+  float* dh_part = dh_partial_bytes(H, T, ldv) ? (float*)align256(wT + H * ldv) : nullptr;
+  u16* e = (u16*)probs;
+  hipLaunchKernelGGL(saved_prep_kernel, dim3((unsigned)Tpad), dim3(256), 0, stream, e, ldv, probs_ref,
+                     labels, row_max, sum_exp, grad_logprobs, logprobs, (const u16*)hidden, (int)T,
+                     (int)H, (int)V, inv_temperature * LOG2E, inv_temperature * logit_scale, rowfac,
+                     dweight != nullptr ? hs : nullptr);
   AREAL_CHECK_LAUNCH();
   if (dhidden != nullptr) {
-    u16* wT = (u16*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     hipLaunchKernelGGL(transpose_pad_bf16_kernel,
                        dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
                        dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
     AREAL_CHECK_LAUNCH();
-    float* dh_part = dh_partial_bytes(H, T, ldv)
-                         ? (float*)(((uintptr_t)(wT + H * ldv) + 255) & ~(uintptr_t)255)
-                         : nullptr;
-    if ((rc = launch_dhidden(wT, dl, ldv, H, T, dhidden, dh_part, stream)) != AREAL_OK) return rc;
+    if ((rc = launch_dhidden(wT, e, ldv, H, T, dhidden, dh_part, rowfac, stream)) != AREAL_OK) return rc;
   }
   if (dbias != nullptr) {
     hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
-                       dl, ldv, T, (int)V, dweight_mode == 1 ? 1 : 0, dbias);
+                       e, ldv, T, (int)V, dweight_mode == 1 ? 1 : 0, (const float*)rowfac, dbias);
     AREAL_CHECK_LAUNCH();
   }
   if (dweight != nullptr) {
-    // dWeight[v, h] += sum_t dl[t, v] * hidden[t, h], k-major over the Tpad rows of dl
-    GemmArgs g{(const u16*)hidden, H, (int)H, dl, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
-    const StoreParams ep{dweight, H, (int)H, (int)V};
+    // dWeight[v, h] += sum_t e'[t, v] * hs[t, h], k-major over the Tpad rows of e' (rows of hs
+    // past T are read as row T - 1 and meet the cleared rows of e')
+    GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
+    const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
     rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
          : dweight_mode == 0 ? launch_gemm<StoreF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)

@@ -12,10 +12,13 @@ Two ways of carrying state to the backward:
   never a ``[T, V]`` tensor; the backward recomputes the logits chunk by chunk
   (``vocab_parallel_head.py:806-829``).
 * ``save_probs=True``: the forward also writes the softmax exponentials as a bf16 ``[T, V]``
-  tensor (2 bytes per logit), the backward turns them into dlogits in place and skips the
-  recomputation, a quarter of the step's matrix work.  The reference's logits-in path saves
-  the same amount through autograd; 288 GB of HBM make it the default while it fits
-  ``SAVE_PROBS_BYTES_LIMIT`` and 60 % of the memory still available.
+  tensor (2 bytes per logit), relative to a per-row reference estimated before the sweep; the
+  backward contracts that buffer as it is (the per-row factor of dlogits goes to the output
+  rows of dHidden and to the hidden states for dWeight) and skips the recomputation, a quarter
+  of the step's matrix work.  The reference's logits-in path saves the same amount through
+  autograd; 288 GB of HBM make it the default while it fits ``SAVE_PROBS_BYTES_LIMIT`` and
+  60 % of the memory still available.  If some row's maximum logit lies more than 150 binades
+  above its estimate (the kernel reports it), the backward recomputes instead.
 """
 
 from __future__ import annotations
@@ -95,12 +98,13 @@ class _FusedLMHead(torch.autograd.Function):
         if save_probs is None:
             need = 2 * _round_up(T, 64) * _round_up(V, 64)
             save_probs = need <= SAVE_PROBS_BYTES_LIMIT and need <= 0.6 * _available_bytes(dev)
-        probs = probs_ref = None
+        probs = probs_ref = probs_status = None
         if save_probs and needs_grad and T > 0:
             probs = torch.empty(
                 (_round_up(T, 64), _round_up(V, 64)), dtype=torch.bfloat16, device=dev
             )
-            probs_ref = torch.empty(((V + 127) // 128, T), dtype=torch.float32, device=dev)
+            probs_ref = torch.empty(T, dtype=torch.float32, device=dev)
+            probs_status = torch.empty(1, dtype=torch.int32, device=dev)
         if T > 0:
             nbytes = lib.areal_lmhead_fwd_workspace_bytes(T, H, V)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -108,15 +112,16 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(bias_f), _lib.ptr(labels_1d),
                 T, H, V, 1.0 / temperature, logit_scale,
                 *[_lib.ptr(o) for o in outs],
-                _lib.ptr(probs), _lib.ptr(probs_ref),
+                _lib.ptr(probs), _lib.ptr(probs_ref), _lib.ptr(probs_status),
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_fwd")
 
         ctx.save_for_backward(hidden_2d, weight_c, labels_1d, row_max, sum_exp)
-        # Plain attributes, not saved tensors: the backward overwrites probs in place.
+        # Plain attributes, not saved tensors: the backward rewrites entries of probs in place.
         ctx.probs = probs
         ctx.probs_ref = probs_ref
+        ctx.probs_status = probs_status
         ctx.label_logprobs = logprobs.detach().reshape(-1).clone() if probs is not None else None
         ctx.bias_f = bias_f
         ctx.temperature = temperature
@@ -146,20 +151,23 @@ class _FusedLMHead(torch.autograd.Function):
         dh = torch.empty_like(hidden_2d) if need_h else None
         db32 = torch.empty(V, dtype=torch.float32, device=dev) if need_b else None
         probs, probs_ref = ctx.probs, ctx.probs_ref
+        # one small device-to-host copy: whether every row's saved exponentials are in range
+        if probs is not None and int(ctx.probs_status.item()) != 0:
+            probs = probs_ref = None
         # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
         # the chunked recompute mode accumulates in fp32 and casts at the end
         direct = probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
         dw_direct = torch.empty((V, H), dtype=torch.bfloat16, device=dev) if (need_w and direct) else None
         dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if (need_w and not direct) else None
-        ctx.probs = ctx.probs_ref = None  # consumed; a second backward recomputes the logits
+        ctx.probs = ctx.probs_ref = ctx.probs_status = None  # consumed; a second backward recomputes
         if T == 0:
             if dw32 is not None:
                 dw32.zero_()
             if db32 is not None:
                 db32.zero_()
         elif probs is not None:
-            nbytes = lib.areal_lmhead_bwd_saved_workspace_bytes(T, H, V) if need_h else 0
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if need_h else None
+            nbytes = lib.areal_lmhead_bwd_saved_workspace_bytes(T, H, V)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             rc = lib.areal_lmhead_bwd_saved(
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(labels_1d),
                 _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),

@@ -295,7 +295,7 @@ def main() -> None:
     # 3 algorithmic GEMMs = 6*T*H*V flops (forward with the softmax epilogue, dHidden, dWeight);
     # with --recompute a fourth launch recomputes the logits and carries no algorithmic flops.
     # Durations are the HIP-event times of the forward and backward library calls on the
-    # stream they are launched on (they also contain the merge, dlogits, transpose and cast
+    # stream they are launched on (they also contain the merge, operand-prep, transpose and cast
     # kernels, which makes the figure slightly pessimistic).
     gemm_ms = (t_fwd + t_bwd) / args.steps
     algo_flops = 6.0 * T * H * V

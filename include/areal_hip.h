@@ -46,17 +46,22 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * labels [T] int64. Outputs fp32 [T]; row_max and sum_exp are the state saved for backward
  * (vocab_parallel_head.py:704-713). logits = (hidden . weight^T + bias) * logit_scale.
  *
- * probs / probs_ref (both NULL, or both set) additionally keep the softmax exponentials for
- * areal_lmhead_bwd_saved, the counterpart of autograd saving the logits in the reference's
- * logits-in path (_gather_logprobs_entropy, areal/utils/functional/vocab_parallel.py:24-30): probs is bf16
- * [round_up(T,64)][round_up(V,64)] holding exp((x - m_blk)/T) per 128-wide vocabulary block,
- * probs_ref is fp32 [ceil(V/128)][T] holding m_blk / T * log2(e). */
+ * probs / probs_ref / probs_status (all NULL, or all set) additionally keep the softmax
+ * exponentials for areal_lmhead_bwd_saved, the counterpart of autograd saving the logits in the
+ * reference's logits-in path (_gather_logprobs_entropy,
+ * areal/utils/functional/vocab_parallel.py:24-30): probs is bf16
+ * [round_up(T,64)][round_up(V,64)] holding 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
+ * fp32 [T], a per-row reference estimated from a few logits of the row (its label's among
+ * them) before the sweep; *probs_status (one int32 on the device) is written 0 when every
+ * row's exponentials are in range, 1 when some row's maximum lies more than 150 binades above
+ * its estimate: probs must then not be used and the backward recomputes (areal_lmhead_bwd). */
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
                      float* row_max, float* sum_exp, void* probs, float* probs_ref,
-                     void* workspace, size_t workspace_bytes, areal_stream_t stream);
+                     int* probs_status, void* workspace, size_t workspace_bytes,
+                     areal_stream_t stream);
 
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
 
@@ -73,14 +78,16 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
-/* Backward from the exponentials the forward kept (probs, probs_ref): the logits are not
- * recomputed (vocab_parallel_head.py:806-829 recomputes them chunk by chunk to save memory; an
- * MI355X has the HBM to keep them). probs is overwritten with the bf16 dlogits and can be
- * used once. logprobs (NULL allowed) are the forward's label log-probabilities: with them the
- * label's dlogit is -expm1(logprob) in fp32. dweight [V,H]: dweight_mode 0 = fp32 store,
- * 1 = fp32 accumulate, 2 = bf16 store; dbias [V] fp32 or NULL (added to in mode 1). Other
- * arguments as areal_lmhead_bwd; the bias itself does not enter (it is part of the saved
- * exponentials). workspace may be NULL if dhidden is. */
+/* Backward from the exponentials the forward kept (probs, probs_ref, *probs_status read back as
+ * 0): the logits are not recomputed (vocab_parallel_head.py:806-829 recomputes them chunk by
+ * chunk to save memory; an MI355X has the HBM to keep them) and no pass rewrites the [T, V]
+ * buffer: dlogits[t][:] = f[t] * probs[t][:] with a per-row factor that dHidden applies to its
+ * output rows and dWeight to the hidden states. Only the label's entry of each row of probs is
+ * rewritten, so probs can be used once. logprobs (NULL allowed) are the forward's label
+ * log-probabilities: with them the label's dlogit is -expm1(logprob) in fp32. dweight [V,H]:
+ * dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store; dbias [V] fp32 or NULL
+ * (added to in mode 1). Other arguments as areal_lmhead_bwd; the bias itself does not enter (it
+ * is part of the saved exponentials). */
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,

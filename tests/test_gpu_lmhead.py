@@ -74,6 +74,8 @@ def test_forward_backward_against_oracle(dev, T, H, V, temp, scale, use_bias, ch
         err = (a.cpu() - b).abs().max().item()
         assert err < tol, f"{name}: max abs err {err}"
     assert out.logprobs.requires_grad and not out.entropy.requires_grad
+    if save_probs:  # ordinary logits: the saved exponentials are in range, no recompute fallback
+        assert int(out.logprobs.grad_fn.probs_status.item()) == 0
     (out.logprobs * grad.to(dev)).sum().backward()
     dh_want, dw_want, db_want = L.lm_head_backward(hidden, weight, labels, grad, temp, scale, bias,
                                                    with_bias_grad=True)
@@ -112,7 +114,7 @@ def test_saved_exponentials_are_bf16_and_used_once(dev):
     out = fused_lm_head_logprobs_entropy(h, w, y, save_probs=True)
     fn = out.logprobs.grad_fn
     assert fn.probs.dtype == torch.bfloat16 and tuple(fn.probs.shape) == (128, 1024)
-    assert tuple(fn.probs_ref.shape) == (8, T)
+    assert tuple(fn.probs_ref.shape) == (T,) and int(fn.probs_status.item()) == 0
     loss = (out.logprobs * grad).sum()
     loss.backward(retain_graph=True)
     assert fn.probs is None
@@ -124,6 +126,32 @@ def test_saved_exponentials_are_bf16_and_used_once(dev):
     with torch.no_grad():  # nothing is kept when no gradient can flow
         out = fused_lm_head_logprobs_entropy(h, w, y, save_probs=True)
     assert out.logprobs.grad_fn is None
+
+
+def test_saved_path_falls_back_when_a_row_exceeds_the_exponent_window(dev):
+    # The saved exponentials are relative to a per-row reference estimated from the label's
+    # logit and 7 sampled vocabulary entries. A row whose maximum logit lies more than 150
+    # binades above all of those is reported by the forward, and the backward recomputes the
+    # logits instead of using the buffer: gradients still match the oracle.
+    T, H, V = 96, 64, 1000
+    g = torch.Generator().manual_seed(21)
+    weight = (torch.randn(V, H, generator=g) * 0.3).bfloat16()
+    hot = 777  # not one of the sampled ids k * V / 8 and not a label
+    labels = torch.randint(0, 700, (T,), generator=g)
+    hidden = (torch.randn(T, H, generator=g) * 0.5).bfloat16()
+    hidden[5] = (weight[hot].float() * 40.0).bfloat16()  # logit of `hot` ~ 230 nats above the rest
+    grad = torch.randn(T, generator=g)
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels.to(dev), save_probs=True)
+    assert int(out.logprobs.grad_fn.probs_status.item()) == 1
+    want = L.lm_head_logprobs_entropy(hidden, weight, labels, 1.0, 1.0, None)
+    # the label log-probability of the hot row is about -200: compare relatively
+    torch.testing.assert_close(out.logprobs.cpu(), want[0], rtol=2e-3, atol=2e-3)
+    (out.logprobs * grad.to(dev)).sum().backward()
+    dh_want, dw_want = L.lm_head_backward(hidden, weight, labels, grad, 1.0, 1.0, None)
+    assert _rel(h.grad.cpu().float(), dh_want) < 1e-2
+    assert _rel(w.grad.cpu().float(), dw_want) < 1e-2
 
 
 def test_saved_path_confident_tokens_and_invalid_labels(dev):
