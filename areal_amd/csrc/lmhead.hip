@@ -31,7 +31,7 @@ struct GemmArgs {
   const u16* B; int64_t ldb; int N;   // B rows (index j)
   int K;                              // multiple of 8
   int acols, bcols;                   // k-major (TN) form only: readable columns of A and B
-  int akrows;                         // k-major form only: rows of A that may be read (<= K)
+                                      // (both operands must have K readable rows)
   // split-K (gemm_nt_sweep with a store epilogue only): the grid is ksplit copies of the tile
   // schedule; copy z contracts k-tiles [z*kt_per_split, (z+1)*kt_per_split) and writes its
   // partial result zstride bytes after the previous copy's. ksplit <= 1: off.
@@ -419,8 +419,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
   // stage; lane -> 16-byte piece (lane & 31) of the LDS row, i.e. chunk position cp = piece/4.
   // It fetches the chunk ci = cp ^ (k & 3); k & 3 = ((i & 1) * 2 + (lane >> 5)) & 3.
   const int hl = lane >> 5, piece = lane & 31;
-  const u16* ga = g.A;
-  int a_row[2], a_col[2];  // i even / odd: row inside a 4-row group, first column of the piece
+  const u16* pa[2];  // i even / odd: the lane's piece of its row at k-tile 0
   const u16* gb[2];
   int l_ai = ai_begin, l_kt = 0;
   // global 16-byte piece of instruction parity par for column tile `tile`
@@ -432,22 +431,17 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
     return gp * 8;
   };
   auto set_a_cols = [&](int ai) {
-    a_col[0] = piece_col(ai, g.acols, 0);
-    a_col[1] = piece_col(ai, g.acols, 1);
+#pragma unroll
+    for (int par = 0; par < 2; ++par)
+      pa[par] = g.A + (int64_t)(wave * 16 + 2 * par + hl) * g.lda + piece_col(ai, g.acols, par);
   };
-  a_row[0] = wave * 16 + hl;
-  a_row[1] = wave * 16 + 2 + hl;
   set_a_cols(ai_begin);
   gb[0] = g.B + (int64_t)(wave * 16 + hl) * g.ldb + piece_col(bj, g.bcols, 0);
   gb[1] = g.B + (int64_t)(wave * 16 + 2 + hl) * g.ldb + piece_col(bj, g.bcols, 1);
   int l_stage = 0;
   auto load_a = [&](int i) {
     u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
-    // rows past the last valid one re-read it; the matching rows of B must then be zero
-    const int kb = l_kt * BK + (i >> 1) * 4;
-    const int lim = g.akrows - 1 - kb;
-    const int rl = a_row[i & 1] < lim ? a_row[i & 1] : lim;
-    const u16* src = ga + (int64_t)(kb + rl) * g.lda + a_col[i & 1];
+    const u16* src = pa[i & 1] + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
     lds_dma16(src, __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
   };
   auto load_b = [&](int i) {
@@ -979,7 +973,7 @@ template <bool E> using BwdAffineT = BwdEpi<E, true, true>;
 // f * e' = -g' * expm1(logprob) = g' * (1 - p) keeps its precision when p is close to 1).
 // The row factor f never multiplies the [T, V] buffer: dHidden scales its output rows by it and
 // dWeight contracts e' with hs = bf16(f[t] * hidden[t][:]). One block per row of probs:
-// rows < T write f[t], hs[t][:] and the label's entry; rows [T, Tpad) are cleared.
+// rows < T write f[t], hs[t][:] and the label's entry; rows [T, Tpad) of probs and hs are cleared.
 __global__ __launch_bounds__(256) void saved_prep_kernel(
     u16* __restrict__ probs, int64_t ldv, const float* __restrict__ ref,
     const int64_t* __restrict__ labels, const float* __restrict__ row_max,
@@ -990,6 +984,8 @@ __global__ __launch_bounds__(256) void saved_prep_kernel(
   if (t >= T) {
     u16* row = probs + (int64_t)t * ldv;
     for (int64_t v = (int64_t)threadIdx.x * 8; v < ldv; v += 2048) *(u32x4*)(row + v) = u32x4{0u, 0u, 0u, 0u};
+    if (hs != nullptr)
+      for (int h = threadIdx.x * 8; h < H; h += 2048) *(u32x4*)(hs + (int64_t)t * H + h) = u32x4{0u, 0u, 0u, 0u};
     return;
   }
   const float lse2 = fmaf(row_max[t], c2, fast_log2(sum_exp[t]));
@@ -1225,7 +1221,7 @@ size_t dh_partial_bytes(int64_t H, int64_t T, int64_t K) {
 // split-K through `partial` when it pays.
 int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t T, void* dhidden,
                    float* partial, const float* tscale, hipStream_t stream) {
-  GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0, 0};
+  GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
   const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
   int z = dh_ksplit(H, T, ldv);
   const int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
@@ -1271,7 +1267,7 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   if ((rc = check_operand(B, ldb)) != AREAL_OK) return rc;
   if (out_mode == 0 ? (ldo % 4 != 0 || ((uintptr_t)out & 7)) : (ldo % 4 != 0 || !aligned16(out)))
     return AREAL_ERR_ALIGNMENT;
-  GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0, 0};
+  GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0};
   const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
   const StoreParams ep{out, ldo, (int)M, (int)N};
   if (out_mode == 0) return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
@@ -1318,7 +1314,7 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   if (workspace == nullptr || workspace_bytes < need) return AREAL_ERR_WORKSPACE;
   const Regions r = fwd_regions(T, H, V);
   const int P = fwd_slots(r);
-  GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H, 0, 0, 0};
+  GemmArgs g{(const u16*)weight, H, (int)V, (const u16*)hidden, H, (int)T, (int)H, 0, 0};
   FwdParams ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
                (float*)workspace, P, 0, (u16*)probs, round_up_i64(V, BK), probs_ref};
   FwdParams ep_a = ep;
@@ -1423,7 +1419,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     const bool need_dlT = dweight_f32 != nullptr && !tn;
     // 1. recompute logits of the chunk, emit dlogits
     {
-      GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H, 0, 0, 0};
+      GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H, 0, 0};
       BwdParams ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
                    (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
       const Regions r = plan_regions(V, Tc, H, 512, 0);
@@ -1448,7 +1444,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
     if (tn) {
-      GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv, (int)Tc};
+      GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
       rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
@@ -1459,7 +1455,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                          dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldt_c, 64)),
                          dim3(256), 0, stream, hid_c, H, (int)Tc, (int)H, hT, ldt_c);
       AREAL_CHECK_LAUNCH();
-      GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0, 0};
+      GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
       rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)
@@ -1471,10 +1467,10 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 }
 
 // Workspace of the backward from saved exponentials: row factors [T] fp32, scaled hidden states
-// [T, H] bf16, W^T [H, round_up(V, 64)] bf16 and the split-K partials of dHidden.
+// [round_up(T, 64), H] bf16, W^T [H, round_up(V, 64)] bf16 and the split-K partials of dHidden.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
-  return (size_t)T * 4 + (size_t)(T * H) * 2 + (size_t)(H * round_up_i64(V, BK)) * 2 +
+  return (size_t)T * 4 + (size_t)(round_up_i64(T, BK) * H) * 2 + (size_t)(H * round_up_i64(V, BK)) * 2 +
          dh_partial_bytes(H, T, round_up_i64(V, BK)) + 4 * 256;
 }
 
@@ -1513,7 +1509,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   auto align256 = [](void* q) { return (void*)(((uintptr_t)q + 255) & ~(uintptr_t)255); };
   float* rowfac = (float*)align256(workspace);
   u16* hs = (u16*)align256(rowfac + T);
-  u16* wT = (u16*)align256(hs + T * H);
+  u16* wT = (u16*)align256(hs + Tpad * H);
   float* dh_part = dh_partial_bytes(H, T, ldv) ? (float*)align256(wT + H * ldv) : nullptr;
   u16* e = (u16*)probs;
   hipLaunchKernelGGL(saved_prep_kernel, dim3((unsigned)Tpad), dim3(256), 0, stream, e, ldv, probs_ref,
@@ -1534,9 +1530,9 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     AREAL_CHECK_LAUNCH();
   }
   if (dweight != nullptr) {
-    // dWeight[v, h] += sum_t e'[t, v] * hs[t, h], k-major over the Tpad rows of e' (rows of hs
-    // past T are read as row T - 1 and meet the cleared rows of e')
-    GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv, (int)T};
+    // dWeight[v, h] += sum_t e'[t, v] * hs[t, h], k-major over the Tpad rows of both (rows past
+    // T are cleared)
+    GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv};
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
     rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
