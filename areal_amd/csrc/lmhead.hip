@@ -252,35 +252,44 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave >> 1, wb = wave & 1;
 
-  // ---- loader: lane -> (row of the wave's 64-row slice, swizzled chunk)
-  const u16* ga[8];
-  const u16* gb[8];
+  // ---- loader: lane -> (row of the wave's 64-row slice, swizzled chunk). A load address is a
+  // wave-uniform base (tile origin + k offset, scalar registers) plus a 32-bit byte offset per
+  // lane that is fixed for the tile, so the k loop spends no vector instructions on addresses.
+  // The host keeps 256 * ld * 2 below 2^32.
+  uint32_t oa[8], ob[8];
+  const u16* a_tile;  // origin of the A tile the loader is on
   int l_ai = ai_begin, l_kt = 0;
   auto set_a_rows = [&](int ai) {
+    a_tile = g.A + (int64_t)ai * TILE * g.lda;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int r = wave * 64 + i * 8 + (lane >> 3);
-      int row = ai * TILE + r;
-      row = row < g.M ? row : g.M - 1;  // clamped rows are discarded by the epilogue
-      ga[i] = g.A + (int64_t)row * g.lda + (((lane & 7) ^ swz64(r)) * 8);
+      int rr = ai * TILE + r < g.M ? r : g.M - 1 - ai * TILE;  // clamped rows are discarded by the epilogue
+      oa[i] = 2u * ((uint32_t)rr * (uint32_t)g.lda + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
     }
   };
   set_a_rows(ai_begin);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int r = wave * 64 + i * 8 + (lane >> 3);
-    int row = bj * TILE + r;
-    row = row < g.N ? row : g.N - 1;
-    gb[i] = g.B + (int64_t)row * g.ldb + (((lane & 7) ^ swz64(r)) * 8);
+    int rr = bj * TILE + r < g.N ? r : g.N - 1 - bj * TILE;
+    ob[i] = 2u * ((uint32_t)rr * (uint32_t)g.ldb + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
   }
+  const u16* b_tile = g.B + (int64_t)bj * TILE * g.ldb;
   int l_stage = 0;  // stage the loader fills next
   auto load_a = [&](int i) {
     u16* dst = lds + l_stage * RING_STAGE + wave * 64 * BK + i * 8 * BK;
-    __builtin_amdgcn_global_load_lds(GLB_AS(ga[i] + l_kt * BK), LDS_AS(dst), 16, 0, 0);
+    const char* base = (const char*)(a_tile + l_kt * BK);
+    __builtin_amdgcn_global_load_lds(GLB_AS(base + oa[i]), LDS_AS(dst), 16, 0, 0);
   };
   auto load_b = [&](int i) {
     u16* dst = lds + l_stage * RING_STAGE + RING_OPER + wave * 64 * BK + i * 8 * BK;
-    __builtin_amdgcn_global_load_lds(GLB_AS(gb[i] + l_kt * BK), LDS_AS(dst), 16, 0, 0);
+    const char* base = (const char*)(b_tile + l_kt * BK);
+    // keeps the offset a 32-bit value up to the load, the form that selects the scalar-base
+    // addressing mode (hoisted out of the sweep it would be widened to 64 bits)
+    uint32_t o = ob[i];
+    asm volatile("" : "+v"(o));
+    __builtin_amdgcn_global_load_lds(GLB_AS(base + o), LDS_AS(dst), 16, 0, 0);
   };
   auto loader_advance = [&]() {  // after both halves of a stage were issued
     l_stage ^= 1;
@@ -397,9 +406,11 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // builtin next to ds_read_b64_tr_b16 it cannot prove they do not alias and puts a full
 // vmcnt(0) wait in front of every transposed read, which serialises the prefetch with the
 // math. The kernel orders the two itself with its explicit vmcnt waits and barriers.
-DEVI void lds_dma16(const u16* gptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :: "s"(lds_addr), "v"(gptr) : "memory", "m0");
+// The address is a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset per
+// lane, so advancing along k costs scalar adds only.
+DEVI void lds_dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 DEVI uint32_t lds_addr_of(const u16* p) { return (uint32_t)(uintptr_t)LDS_AS(p); }
 
@@ -419,8 +430,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
   // stage; lane -> 16-byte piece (lane & 31) of the LDS row, i.e. chunk position cp = piece/4.
   // It fetches the chunk ci = cp ^ (k & 3); k & 3 = ((i & 1) * 2 + (lane >> 5)) & 3.
   const int hl = lane >> 5, piece = lane & 31;
-  const u16* pa[2];  // i even / odd: the lane's piece of its row at k-tile 0
-  const u16* gb[2];
+  uint32_t oa[2], ob[2];  // i even / odd: byte offset of the lane's piece of its row at k-tile 0
   int l_ai = ai_begin, l_kt = 0;
   // global 16-byte piece of instruction parity par for column tile `tile`
   auto piece_col = [&](int tile, int ncols, int par) -> int {
@@ -430,24 +440,28 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
     gp = gp < last ? gp : last;  // columns past the end are discarded by the epilogue
     return gp * 8;
   };
+  // offsets stay below 2^32: the host checks 64 * ld * 2 + 2 * cols < 2^32
   auto set_a_cols = [&](int ai) {
 #pragma unroll
     for (int par = 0; par < 2; ++par)
-      pa[par] = g.A + (int64_t)(wave * 16 + 2 * par + hl) * g.lda + piece_col(ai, g.acols, par);
+      oa[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.lda +
+                      (uint32_t)piece_col(ai, g.acols, par));
   };
   set_a_cols(ai_begin);
-  gb[0] = g.B + (int64_t)(wave * 16 + hl) * g.ldb + piece_col(bj, g.bcols, 0);
-  gb[1] = g.B + (int64_t)(wave * 16 + 2 + hl) * g.ldb + piece_col(bj, g.bcols, 1);
+#pragma unroll
+  for (int par = 0; par < 2; ++par)
+    ob[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.ldb +
+                    (uint32_t)piece_col(bj, g.bcols, par));
   int l_stage = 0;
   auto load_a = [&](int i) {
     u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
-    const u16* src = pa[i & 1] + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
-    lds_dma16(src, __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+    const u16* base = g.A + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
+    lds_dma16(base, oa[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
   };
   auto load_b = [&](int i) {
     u16* dst = lds + l_stage * RING_STAGE + RING_OPER + (wave * 16 + i * 2) * TILE;
-    const u16* src = gb[i & 1] + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.ldb;
-    lds_dma16(src, __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+    const u16* base = g.B + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.ldb;
+    lds_dma16(base, ob[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
   };
   auto loader_advance = [&]() {
     l_stage ^= 1;
@@ -1120,12 +1134,18 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
   if (S > nai) S = nai;
   if (S < 1) S = 1;
   const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
-  if constexpr (KERNEL == KERNEL_NT)
+  if constexpr (KERNEL == KERNEL_NT) {
+    // the loader addresses a tile as a 64-bit base plus 32-bit byte offsets per lane
+    if (g.lda > (1 << 22) || g.ldb > (1 << 22)) return AREAL_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
                        dim3(NTHREADS), 0, stream, g, sc, ep);
-  else if constexpr (KERNEL == KERNEL_TN)
+  }
+  else if constexpr (KERNEL == KERNEL_TN) {
+    // the loader addresses a k-tile as a 64-bit base plus 32-bit byte offsets per lane
+    if (g.lda > (1 << 24) || g.ldb > (1 << 24)) return AREAL_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
+  }
   else
     hipLaunchKernelGGL((gemm_nt_generic<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
