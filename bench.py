@@ -311,9 +311,9 @@ def main() -> None:
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            "gemm_nt_sweep<FwdEpi> forward": 4.00787e7 * kib * 2.0 + 1.12821e7 * kib,
-            "gemm_nt_sweep<StoreEpi> dHidden": 2.91945e7 * kib * 2.0 + 3.072e5 * kib,
-            "gemm_tn_sweep<StoreEpi> dWeight": 2.95001e7 * kib * 2.0 + 1.28202e6 * kib,
+            "gemm_nt_sweep<FwdEpi> forward": 4.34454e7 * kib * 2.0 + 1.28786e7 * kib,
+            "gemm_nt_sweep<StoreEpi> dHidden": 3.02432e7 * kib * 2.0 + 2.99008e5 * kib,
+            "gemm_tn_sweep<StoreEpi> dWeight": 3.0399e7 * kib * 2.0 + 1.26301e6 * kib,
         }
         traffic = sum(traffic_detail.values()) / 3.0
 
