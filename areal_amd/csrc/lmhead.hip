@@ -686,6 +686,26 @@ __global__ __launch_bounds__(256) void lmhead_rowref_kernel(
 // sum x^2. One token (its 64 logits in this lane) at a time: the logits are read from the
 // accumulators twice (statistics pass, exponential pass) and never written back.
 // ---------------------------------------------------------------------------------------
+// c2 * m rounded to fp32, and sums / differences with such products, kept out of fma
+// contraction: the softmax sums are relative to this ROUNDED reference (the exponent of a logit
+// is fma(x, c2, -ref): exact product minus the rounded reference), so whatever re-references
+// them has to use the same rounded value or the rounding error of c2 * m (up to ulp(c2 m) / 2
+// binades) enters the result.
+DEVI float ref_of(float m, float c2) {
+#pragma clang fp contract(off)
+  return m * c2;
+}
+DEVI float ref_diff(float a, float b, float c2) {  // fl(a c2) - fl(b c2)
+#pragma clang fp contract(off)
+  const float x = a * c2, y = b * c2;
+  return x - y;
+}
+DEVI float ref_plus(float m, float c2, float add) {  // fl(m c2) + add
+#pragma clang fp contract(off)
+  const float x = m * c2;
+  return x + add;
+}
+
 constexpr int NSTAT = 7;  // m, s, q, xlabel, min, sumx, sumx2
 
 struct FwdParams {
@@ -756,14 +776,14 @@ struct FwdEpi {
       if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
       const float m_old = st.m[b];
       const float m_new = fmaxf(m_old, tmax);
-      // rescale the running sums to the new maximum; on the first tile m_old = -inf and
-      // s = q = 0, so the factor is taken as 2^0 instead of evaluating -inf - x
+      // rescale the running sums to the new reference (see ref_of); on the first tile
+      // m_old = -inf and s = q = 0, so the factor is taken as 2^0 instead of evaluating -inf - x
       float s = st.s[b], q = st.q[b];
-      const float dl = (m_old > neg_inf()) ? (m_old - m_new) * p.c2 : 0.f;
+      const float mc = (!EDGE || m_new > neg_inf()) ? ref_of(m_new, p.c2) : 0.f;
+      const float dl = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
       const float alpha = fast_exp2(dl);
       q = alpha * fmaf(dl, s, q);
       s = alpha * s;
-      const float mc = (!EDGE || m_new > neg_inf()) ? m_new * p.c2 : 0.f;
       if (!SAVE) {
 #pragma unroll
         for (int a = 0; a < 4; ++a)
@@ -856,6 +876,7 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
                                     const float* __restrict__ row_ref, int* __restrict__ status) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
+  (void)inv_temp;  // c2 = inv_temp * log2(e) carries it
   const int64_t PT = (int64_t)P * T;
   const bool moments = vmean != nullptr || vnorm != nullptr;
   float M = neg_inf();
@@ -866,7 +887,7 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
     const float* w = ws + (int64_t)p * T + t;
     const float m = w[0];
     if (m > neg_inf()) {
-      const float dl = (m - M) * c2;
+      const float dl = ref_diff(m, M, c2);  // as in the epilogue
       const float alpha = exp2f(dl);
       S += alpha * w[1 * PT];
       Q += alpha * fmaf(dl, w[1 * PT], w[2 * PT]);
@@ -876,7 +897,13 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
     if (moments) { sx += (double)w[5 * PT]; sx2 += (double)w[6 * PT]; }
   }
   const float logS = logf(S);
-  if (logprobs) logprobs[t] = (xl - M) * inv_temp - logS;
+  // label exponent against the same rounded reference the sums use. For a label inside the
+  // vocabulary (xl <= M) the result is <= 0 in exact arithmetic; the last rounding may leave
+  // +1e-8 when p = 1 to fp32 precision.
+  if (logprobs) {
+    const float lp = fmaf(xl, c2, -ref_of(M, c2)) * LN2 - logS;
+    logprobs[t] = xl <= M ? fminf(lp, 0.f) : lp;
+  }
   if (entropy) entropy[t] = logS - (Q * LN2) / S;
   if (vmin) vmin[t] = mn;
   if (vmax) vmax[t] = M;
@@ -918,7 +945,7 @@ struct BwdEpi {
       if (!EDGE || t < p.T) {
         const int64_t l = p.labels[t];
         st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
-        st.nb[b] = -(p.row_max[t] * p.c2 + fast_log2(p.sum_exp[t]));
+        st.nb[b] = -ref_plus(p.row_max[t], p.c2, fast_log2(p.sum_exp[t]));
         st.gs[b] = p.grad[t] * p.inv_temp * p.scale;
       } else {
         st.lab[b] = -1; st.nb[b] = 0.f; st.gs[b] = 0.f;
@@ -982,7 +1009,7 @@ template <bool E> using BwdAffineT = BwdEpi<E, true, true>;
 
 // Operands of the backward from the exponentials the forward saved, e[t][v] = 2^(c2 x - ref[t]):
 //   dlogits[t][v] = f[t] * e'[t][v],   f[t] = -g[t] * invT * scale * 2^(ref[t] - lse2[t]),
-// with lse2 = c2 * row_max + log2(sum_exp) and e' = e except at the label, where
+// with lse2 = fl(c2 * row_max) + log2(sum_exp) and e' = e except at the label, where
 // e' = expm1(logprob) * 2^(lse2 - ref) taken from the fp32 label log-probability (so that
 // f * e' = -g' * expm1(logprob) = g' * (1 - p) keeps its precision when p is close to 1).
 // The row factor f never multiplies the [T, V] buffer: dHidden scales its output rows by it and
@@ -1002,7 +1029,7 @@ __global__ __launch_bounds__(256) void saved_prep_kernel(
       for (int h = threadIdx.x * 8; h < H; h += 2048) *(u32x4*)(hs + (int64_t)t * H + h) = u32x4{0u, 0u, 0u, 0u};
     return;
   }
-  const float lse2 = fmaf(row_max[t], c2, fast_log2(sum_exp[t]));
+  const float lse2 = ref_plus(row_max[t], c2, fast_log2(sum_exp[t]));
   const float f = -(grad[t] * gscale) * fast_exp2(ref[t] - lse2);
   if (threadIdx.x == 0) {
     rowfac[t] = f;

@@ -133,7 +133,16 @@ __global__ __launch_bounds__(ROW_THREADS) void rows_fwd_kernel(const T* __restri
     const float lse2 = r.m + log2s;
     const int64_t lab = labels[row];
     float lp = 0.f;
-    if (lab >= 0 && lab < V) lp = (Elem<T>::load(x + lab) * c2 - lse2) * LN2_F;
+    if (lab >= 0 && lab < V) {
+      // the label's exponent as the sums saw it: the rounded product, not fused into the
+      // subtraction (lse2 is built from such rounded products)
+      float zl;
+      {
+#pragma clang fp contract(off)
+        zl = Elem<T>::load(x + lab) * c2;
+      }
+      lp = fminf((zl - lse2) * LN2_F, 0.f);
+    }
     if (logprobs) logprobs[row] = lp;
     if (entropy) entropy[row] = (log2s - r.q / r.s) * LN2_F;
     if (lse2_out) lse2_out[row] = lse2;

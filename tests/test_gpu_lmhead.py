@@ -154,6 +154,31 @@ def test_saved_path_falls_back_when_a_row_exceeds_the_exponent_window(dev):
     assert _rel(w.grad.cpu().float(), dw_want) < 1e-2
 
 
+@pytest.mark.parametrize("temp,scale", [(0.7, 2.0), (0.35, 1.0), (1.0, 1.0)])
+def test_logprob_of_saturated_rows_keeps_fp32_resolution(dev, temp, scale):
+    # Logits of magnitude ~65 whose label holds all the probability: c2 * max is ~130, where one
+    # fp32 ulp is 1.5e-5. The kernels keep every softmax sum relative to the rounded product
+    # fl(c2 * max) and merge with that same value, so this rounding cancels: the log-probability
+    # is right to fp32 resolution (not to ulp(c2 * max)) and never positive.
+    T, H, V = 2, 16, 3
+    g = torch.Generator().manual_seed(297)
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * (25.0 * 2.0 / H ** 0.5)).bfloat16()
+    logits = (hidden.double() @ weight.double().T) * scale / temp
+    labels = logits.argmax(dim=1)
+    want = torch.log_softmax(logits, dim=1).gather(1, labels[:, None])[:, 0]
+    for Hp in (16, 64):  # generic kernel and the K % 64 == 0 kernel
+        hd = torch.zeros(T, Hp, dtype=torch.bfloat16)
+        hd[:, :H] = hidden
+        wt = torch.zeros(V, Hp, dtype=torch.bfloat16)
+        wt[:, :H] = weight
+        out = fused_lm_head_logprobs_entropy(hd.to(dev), wt.to(dev), labels.to(dev), temperature=temp,
+                                             logit_scale=scale)
+        lp = out.logprobs.cpu().double()
+        assert (lp <= 0).all()
+        assert (lp - want).abs().max() < 3e-7, (lp, want)
+
+
 def test_saved_path_confident_tokens_and_invalid_labels(dev):
     # Tokens whose label probability is ~1: 1 - p must not be lost to the bf16 rounding of p
     # (the label's dlogit comes from the fp32 log-probability). Labels outside [0, V) get no
