@@ -235,9 +235,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
   int bj, split, ai_begin, ai_end;
   int wg = blockIdx.x, nk = g.K / BK;
   if (g.ksplit > 1) {
-    const int per_copy = gridDim.x / g.ksplit;
+    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
     const int z = wg / per_copy;
     wg -= z * per_copy;
+    // The schedule puts super-block sb on XCD sb % 8 (workgroup id % 8). Copies start on
+    // different XCDs, so that a schedule of fewer than 8 super-blocks still uses all of them.
+    wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);
     const int kt0 = z * g.kt_per_split;
     nk -= kt0;
     nk = nk < g.kt_per_split ? nk : g.kt_per_split;
@@ -1250,11 +1253,29 @@ int dh_ksplit(int64_t H, int64_t T, int64_t K) {
   const int64_t tiles = ceil_div_i64(H, TILE) * ceil_div_i64(T, TILE);
   if (tiles >= 2048 || K % BK != 0) return 1;
   const int64_t nk = K / BK;
-  // rounds of 256 workgroups per unit of K, plus a small charge per split for the reduction
+  // The launch is a schedule of super-blocks of up to 32 workgroups; super-block sb of copy c
+  // runs on XCD (sb + c * n_sb) % 8, whose 32 CUs take its workgroups as they free up. Cost of
+  // z copies = the busiest XCD's rounds of 32 workgroups, each K / z long, plus a small charge
+  // per split for the reduction of the partial results.
+  const int nai = (int)ceil_div_i64(H, TILE), nbj = (int)ceil_div_i64(T, TILE);
+  const Sched sc = make_sched(0, nbj, 0, nai, nai);
+  auto cost_of = [&](int z) {
+    int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int c = 0; c < z; ++c)
+      for (int sb = 0; sb < sc.n_sb; ++sb) {
+        const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
+        const int nb = nbj - sbj * sc.RB < sc.RB ? nbj - sbj * sc.RB : sc.RB;
+        const int ns = sc.S - sbs * sc.RS < sc.RS ? sc.S - sbs * sc.RS : sc.RS;
+        load[(sb + c * sc.n_sb) & 7] += (int64_t)(nb > 0 ? nb : 0) * (ns > 0 ? ns : 0);
+      }
+    int64_t worst = 0;
+    for (int x = 0; x < 8; ++x) worst = load[x] > worst ? load[x] : worst;
+    return (double)ceil_div_i64(worst, 32) / z + 0.03 * (z - 1);
+  };
   int best = 1;
-  double best_cost = (double)ceil_div_i64(tiles, 256);
+  double best_cost = cost_of(1);
   for (int z = 2; z <= 16 && z <= nk / 8; ++z) {
-    const double cost = (double)ceil_div_i64(tiles * z, 256) / z + 0.03 * (z - 1);
+    const double cost = cost_of(z);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = z; }
   }
   return best;
