@@ -869,25 +869,35 @@ template <bool E> using FwdPlainMomSave = FwdEpi<E, false, true, true>;
 template <bool E> using FwdAffineSave = FwdEpi<E, true, false, true>;
 template <bool E> using FwdAffineMomSave = FwdEpi<E, true, true, true>;
 
-// Merge the partial statistics of one token over all slots.
-__global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, int V,
-                                    float inv_temp, float c2, float* __restrict__ logprobs,
-                                    float* __restrict__ entropy, float* __restrict__ vmin,
-                                    float* __restrict__ vmax, float* __restrict__ vmean,
-                                    float* __restrict__ vnorm, float* __restrict__ row_max,
-                                    float* __restrict__ sum_exp,
-                                    const float* __restrict__ row_ref, int* __restrict__ status) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
+// Merge the partial statistics of one token over all slots. A block is 64 tokens (lanes) x
+// MERGE_WAVES waves; wave w takes slots w, w + MERGE_WAVES, ... (loads stay coalesced along the
+// tokens, and a launch with few tokens and many slots still has enough threads in flight), the
+// partial results meet in LDS and wave 0 adds them in a fixed order.
+constexpr int MERGE_WAVES = 8;
+__global__ __launch_bounds__(64 * MERGE_WAVES) void lmhead_merge_kernel(
+    const float* __restrict__ ws, int P, int T, int V, float inv_temp, float c2,
+    float* __restrict__ logprobs, float* __restrict__ entropy, float* __restrict__ vmin,
+    float* __restrict__ vmax, float* __restrict__ vmean, float* __restrict__ vnorm,
+    float* __restrict__ row_max, float* __restrict__ sum_exp, const float* __restrict__ row_ref,
+    int* __restrict__ status) {
+  __shared__ float sh_f[5][MERGE_WAVES][64];   // max, S, Q, label logit, min
+  __shared__ double sh_d[2][MERGE_WAVES][64];  // sum x, sum x^2
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int t = blockIdx.x * 64 + lane;
+  const int tt = t < T ? t : T - 1;  // lanes past the end repeat the last token and write nothing
   (void)inv_temp;  // c2 = inv_temp * log2(e) carries it
   const int64_t PT = (int64_t)P * T;
   const bool moments = vmean != nullptr || vnorm != nullptr;
   float M = neg_inf();
-  for (int p = 0; p < P; ++p) M = fmaxf(M, ws[(int64_t)p * T + t]);
+  for (int p = wv; p < P; p += MERGE_WAVES) M = fmaxf(M, ws[(int64_t)p * T + tt]);
+  sh_f[0][wv][lane] = M;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MERGE_WAVES; ++i) M = fmaxf(M, sh_f[0][i][lane]);
   float S = 0.f, Q = 0.f, xl = 0.f, mn = pos_inf();
   double sx = 0.0, sx2 = 0.0;
-  for (int p = 0; p < P; ++p) {
-    const float* w = ws + (int64_t)p * T + t;
+  for (int p = wv; p < P; p += MERGE_WAVES) {
+    const float* w = ws + (int64_t)p * T + tt;
     const float m = w[0];
     if (m > neg_inf()) {
       const float dl = ref_diff(m, M, c2);  // as in the epilogue
@@ -898,6 +908,17 @@ __global__ void lmhead_merge_kernel(const float* __restrict__ ws, int P, int T, 
     xl += w[3 * PT];
     mn = fminf(mn, w[4 * PT]);
     if (moments) { sx += (double)w[5 * PT]; sx2 += (double)w[6 * PT]; }
+  }
+  sh_f[1][wv][lane] = S; sh_f[2][wv][lane] = Q; sh_f[3][wv][lane] = xl; sh_f[4][wv][lane] = mn;
+  sh_d[0][wv][lane] = sx; sh_d[1][wv][lane] = sx2;
+  __syncthreads();
+  if (wv != 0 || t >= T) return;
+  S = 0.f; Q = 0.f; xl = 0.f; mn = pos_inf(); sx = 0.0; sx2 = 0.0;
+#pragma unroll
+  for (int i = 0; i < MERGE_WAVES; ++i) {
+    S += sh_f[1][i][lane]; Q += sh_f[2][i][lane]; xl += sh_f[3][i][lane];
+    mn = fminf(mn, sh_f[4][i][lane]);
+    sx += sh_d[0][i][lane]; sx2 += sh_d[1][i][lane];
   }
   const float logS = logf(S);
   // label exponent against the same rounded reference the sums use. For a label inside the
@@ -1407,8 +1428,7 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
     else rc = launch_gemm<FwdAffineMomSave>(g, r, ep, ep_a, stream);
   }
   if (rc != AREAL_OK) return rc;
-  const int threads = 256;
-  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, threads)), dim3(threads),
+  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, 64)), dim3(64 * MERGE_WAVES),
                      0, stream, (const float*)workspace, P, (int)T, (int)V, inv_temperature,
                      inv_temperature * LOG2E, logprobs, entropy, vocab_min, vocab_max, vocab_mean,
                      vocab_norm, row_max, sum_exp, (const float*)probs_ref, probs_status);
