@@ -570,6 +570,175 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
 }
 
 // ---------------------------------------------------------------------------------------
+// gemm_mix_sweep: D[i][j] = sum_k A[k][i] * B[j][k]: A stored k-major (row = k, i contiguous,
+// as gemm_tn_sweep reads it), B stored with k contiguous (as gemm_nt_sweep reads it),
+// K % 64 == 0 and A has K readable rows. Used for dHidden[t][h] = sum_v dl[t][v] W[v][h] straight
+// from the [V, H] weight: no transposed copy of the weight is made. The A half of a stage has
+// gemm_tn_sweep's layout and transposed fragment reads, the B half gemm_nt_sweep's; all direct
+// loads are inline assembly for the reason given at lds_dma16. Split-K as in gemm_nt_sweep.
+// ---------------------------------------------------------------------------------------
+template <class Epi>
+__global__ __launch_bounds__(NTHREADS) void gemm_mix_sweep(GemmArgs g, Sched sc,
+                                                           typename Epi::Params ep) {
+  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
+  int bj, split, ai_begin, ai_end;
+  int wg = blockIdx.x, nk = g.K / BK;
+  if (g.ksplit > 1) {
+    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
+    const int z = wg / per_copy;
+    wg -= z * per_copy;
+    wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);  // copies start on different XCDs
+    const int kt0 = z * g.kt_per_split;
+    nk -= kt0;
+    nk = nk < g.kt_per_split ? nk : g.kt_per_split;
+    g.A += (int64_t)kt0 * BK * g.lda;
+    g.B += (int64_t)kt0 * BK;
+    Epi::split_output(ep, (int64_t)z * g.zstride);
+    if (nk <= 0) return;
+  }
+  if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave >> 1, wb = wave & 1;
+
+  // ---- loader, A half (k-major): see gemm_tn_sweep
+  const int hl = lane >> 5, piece = lane & 31;
+  uint32_t oa[2], ob[8];
+  int l_ai = ai_begin, l_kt = 0;
+  auto set_a_cols = [&](int ai) {
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      const int k3 = (par * 2 + hl) & 3;
+      int gp = ai * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + (piece & 3);
+      const int last = g.acols / 8 - 1;
+      gp = gp < last ? gp : last;  // columns past the end are discarded by the epilogue
+      oa[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.lda + (uint32_t)(gp * 8));
+    }
+  };
+  set_a_cols(ai_begin);
+  // ---- loader, B half (k contiguous): see gemm_nt_sweep
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = wave * 64 + i * 8 + (lane >> 3);
+    const int rr = bj * TILE + r < g.N ? r : g.N - 1 - bj * TILE;
+    ob[i] = 2u * ((uint32_t)rr * (uint32_t)g.ldb + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
+  }
+  const u16* b_tile = g.B + (int64_t)bj * TILE * g.ldb;
+  int l_stage = 0;
+  auto load_a = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
+    const u16* base = g.A + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
+    lds_dma16(base, oa[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+  };
+  auto load_b = [&](int i) {
+    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + wave * 64 * BK + i * 8 * BK;
+    lds_dma16(b_tile + l_kt * BK, ob[i], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
+  };
+  auto loader_advance = [&]() {
+    l_stage ^= 1;
+    if (l_kt + 1 < nk) {
+      ++l_kt;
+    } else if (l_ai + 1 < ai_end) {
+      ++l_ai;
+      l_kt = 0;
+      set_a_cols(l_ai);
+    }
+  };
+
+  // ---- fragments: A by transposed reads (gemm_tn_sweep), B by 16-byte reads (gemm_nt_sweep)
+  const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
+  const int frag_row = (G >> 1) * 8 + r4;
+  const int frag_byte = (G & 1) * 32 + (q & 3) * 8;
+  const int rl = lane & 31, ch = lane >> 5;
+  const int sw = swz64(rl);
+  bf16x8 af[2][4], bf[2][4];
+  auto tr_read = [&](const u16* oper, int x, int s) -> bf16x8 {
+    const int ci = wa * 4 + x;
+    const char* base = (const char*)oper + ((ci ^ r4) << 6) + frag_byte;
+    const int k0 = s * 16 + frag_row;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)(base + (k0 << 9)));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)(base + ((k0 + 4) << 9)));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
+  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
+  auto dsr = [&](int st, int s, int buf, int f) {
+    const u16* sA = lds + st * RING_STAGE;
+    const u16* sB = sA + RING_OPER + wb * 128 * BK + rl * BK + ((s * 2 + ch) ^ sw) * 8;
+    if (f == 0) af[buf][0] = tr_read(sA, 0, s);
+    else if (f <= 4) bf[buf][f - 1] = *(const bf16x8*)(sB + (f - 1) * 32 * BK);
+    else af[buf][f - 4] = tr_read(sA, f - 4, s);
+  };
+  f32x16 acc[4][4];
+  auto mfma2 = [&](int buf, int p) {
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq) {
+      const int idx = 2 * p + qq, a = idx >> 2, b = idx & 3;
+      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
+    }
+  };
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  };
+
+  typename Epi::State st;
+  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
+
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_b(i);
+  loader_advance();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_a(i);
+  zero_acc();
+  __builtin_amdgcn_s_waitcnt(0x0F78);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
+
+  int cs = 0;
+  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
+    for (int c_kt = 0; c_kt < nk; ++c_kt) {
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+          mfma2(s & 1, p);
+          dsr(cs, s + 1, (s + 1) & 1, p);
+          if (s == 0) load_b(p);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (s == 0) loader_advance();
+      }
+      __builtin_amdgcn_s_waitcnt(0x0070);
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        mfma2(1, p);
+        dsr(cs ^ 1, 0, 0, p);
+        load_a(p);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      cs ^= 1;
+    }
+    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
+    zero_acc();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Epilogues. Each is a template on EDGE: the interior of the tile grid (every tile fully inside
 // M x N) runs the EDGE = false instance, which carries no bounds predicates; ragged last tiles
 // are launched separately with EDGE = true. Keeping one variant per kernel keeps the
@@ -1176,7 +1345,7 @@ int pick_splits(int nbj, int nai, int target_wgs) {
   return S;
 }
 
-enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2 };
+enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2, KERNEL_MIX = 3 };
 
 template <class Epi, int KERNEL>
 int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
@@ -1191,7 +1360,11 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
     hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
                        dim3(NTHREADS), 0, stream, g, sc, ep);
   }
-  else if constexpr (KERNEL == KERNEL_TN) {
+  else if constexpr (KERNEL == KERNEL_MIX) {
+    if (g.lda > (1 << 24) || g.ldb > (1 << 22)) return AREAL_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((gemm_mix_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
+                       dim3(NTHREADS), 0, stream, g, sc, ep);
+  } else if constexpr (KERNEL == KERNEL_TN) {
     // the loader addresses a k-tile as a 64-bit base plus 32-bit byte offsets per lane
     if (g.lda > (1 << 24) || g.ldb > (1 << 24)) return AREAL_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
@@ -1306,11 +1479,17 @@ size_t dh_partial_bytes(int64_t H, int64_t T, int64_t K) {
   return z > 1 ? (size_t)z * (size_t)(T * H) * sizeof(float) + 256 : 0;
 }
 
-// dHidden[t, h] = tscale[t] * sum_v dl[t, v] * W^T[h, v] (tscale = 1 when null), bf16 out;
-// split-K through `partial` when it pays.
-int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t T, void* dhidden,
-                   float* partial, const float* tscale, hipStream_t stream) {
-  GemmArgs g{wT, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
+// The weight can be contracted as stored ([V, H], k-major for dHidden) when its V rows cover the
+// K = round_up(V, 64) rows the kernel reads; otherwise a zero-padded transposed copy is used.
+bool dh_weight_in_place(int64_t V) { return V % BK == 0; }
+
+// dHidden[t, h] = tscale[t] * sum_v dl[t, v] * W[v, h] (tscale = 1 when null), bf16 out;
+// split-K through `partial` when it pays. w is the weight itself [V, H] when
+// dh_weight_in_place(V), else its transposed copy W^T [H, ldv].
+template <int KERNEL>
+int launch_dhidden_k(const GemmArgs& g0, int64_t H, int64_t T, int64_t ldv, void* dhidden,
+                     float* partial, const float* tscale, hipStream_t stream) {
+  GemmArgs g = g0;
   const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
   int z = dh_ksplit(H, T, ldv);
   const int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
@@ -1318,14 +1497,14 @@ int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t
   if (z <= 1 || partial == nullptr) {
     const StoreParams ep{dhidden, H, (int)H, (int)T, tscale};
     if (tscale != nullptr)
-      return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
-    return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+      return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    return launch_gemm<StoreBf16, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
   }
   g.ksplit = z;
   g.kt_per_split = kps;
   g.zstride = T * H * (int64_t)sizeof(float);
   const StoreParams ep{partial, H, (int)H, (int)T, nullptr};
-  int rc = launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  int rc = launch_gemm<StoreF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
   if (rc != AREAL_OK) return rc;
   int64_t blocks = ceil_div_i64(T * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
@@ -1333,6 +1512,15 @@ int launch_dhidden(const u16* wT, const u16* dl, int64_t ldv, int64_t H, int64_t
                      z, T * H, T * H, tscale, H, (u16*)dhidden);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
+}
+int launch_dhidden(const u16* w, int64_t V, const u16* dl, int64_t ldv, int64_t H, int64_t T,
+                   void* dhidden, float* partial, const float* tscale, hipStream_t stream) {
+  if (dh_weight_in_place(V)) {
+    const GemmArgs g{w, H, (int)H, dl, ldv, (int)T, (int)ldv, (int)H, 0};
+    return launch_dhidden_k<KERNEL_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
+  }
+  const GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
+  return launch_dhidden_k<KERNEL_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
 }
 
 }  // namespace
@@ -1443,7 +1631,7 @@ size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t
   if (T <= 0 || H <= 0 || V <= 0 || token_chunk <= 0) return 0;
   const int64_t Tc = token_chunk < T ? token_chunk : T;
   const int64_t ldv = round_up_i64(V, BK), ldt = round_up_i64(Tc, BK);
-  int64_t elems = H * ldv + Tc * ldv;
+  int64_t elems = (dh_weight_in_place(V) ? 0 : H * ldv) + Tc * ldv;
   const bool ragged = (Tc % BK != 0) || (T % Tc) % BK != 0;  // some chunk is not a multiple of 64
   if (ragged) elems += H * ldt + V * ldt;
   // slack for 256-byte sub-buffer alignment
@@ -1482,7 +1670,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   };
   char* wp = (char*)workspace;
   const bool ragged = (Tc_max % BK != 0) || (T % Tc_max) % BK != 0;
-  u16* wT = carve(wp, H * ldv * 2);
+  const bool w_in_place = dh_weight_in_place(V);
+  u16* wT = w_in_place ? nullptr : carve(wp, H * ldv * 2);
   u16* dl = carve(wp, Tc_max * ldv * 2);
   u16* hT = ragged ? carve(wp, H * ldt * 2) : nullptr;
   u16* dlT = ragged ? carve(wp, V * ldt * 2) : nullptr;
@@ -1490,7 +1679,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 
   const float c2 = inv_temperature * LOG2E;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
-  if (dhidden != nullptr) {
+  if (dhidden != nullptr && !w_in_place) {
     // W^T [H, ldv]: rows = h, columns = v (zero padded to ldv).
     hipLaunchKernelGGL(transpose_pad_bf16_kernel,
                        dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
@@ -1521,7 +1710,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
-      if ((rc = launch_dhidden(wT, dl, ldv, H, Tc, (u16*)dhidden + t0 * H, dh_part, nullptr, stream)) != AREAL_OK)
+      if ((rc = launch_dhidden(w_in_place ? (const u16*)weight : wT, V, dl, ldv, H, Tc,
+                               (u16*)dhidden + t0 * H, dh_part, nullptr, stream)) != AREAL_OK)
         return rc;
     }
     // dBias[v] += sum_t dl[t, v]
@@ -1555,10 +1745,12 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 }
 
 // Workspace of the backward from saved exponentials: row factors [T] fp32, scaled hidden states
-// [round_up(T, 64), H] bf16, W^T [H, round_up(V, 64)] bf16 and the split-K partials of dHidden.
+// [round_up(T, 64), H] bf16, W^T [H, round_up(V, 64)] bf16 (only when V is not a multiple of 64)
+// and the split-K partials of dHidden.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
-  return (size_t)T * 4 + (size_t)(round_up_i64(T, BK) * H) * 2 + (size_t)(H * round_up_i64(V, BK)) * 2 +
+  const size_t wt = dh_weight_in_place(V) ? 0 : (size_t)(H * round_up_i64(V, BK)) * 2;
+  return (size_t)T * 4 + (size_t)(round_up_i64(T, BK) * H) * 2 + wt +
          dh_partial_bytes(H, T, round_up_i64(V, BK)) + 4 * 256;
 }
 
@@ -1597,8 +1789,9 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   auto align256 = [](void* q) { return (void*)(((uintptr_t)q + 255) & ~(uintptr_t)255); };
   float* rowfac = (float*)align256(workspace);
   u16* hs = (u16*)align256(rowfac + T);
+  const bool w_in_place = dh_weight_in_place(V);
   u16* wT = (u16*)align256(hs + Tpad * H);
-  float* dh_part = dh_partial_bytes(H, T, ldv) ? (float*)align256(wT + H * ldv) : nullptr;
+  float* dh_part = dh_partial_bytes(H, T, ldv) ? (float*)align256(wT + (w_in_place ? 0 : H * ldv)) : nullptr;
   u16* e = (u16*)probs;
   hipLaunchKernelGGL(saved_prep_kernel, dim3((unsigned)Tpad), dim3(256), 0, stream, e, ldv, probs_ref,
                      labels, row_max, sum_exp, grad_logprobs, logprobs, (const u16*)hidden, (int)T,
@@ -1606,11 +1799,15 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
                      dweight != nullptr ? hs : nullptr);
   AREAL_CHECK_LAUNCH();
   if (dhidden != nullptr) {
-    hipLaunchKernelGGL(transpose_pad_bf16_kernel,
-                       dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
-                       dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
-    AREAL_CHECK_LAUNCH();
-    if ((rc = launch_dhidden(wT, e, ldv, H, T, dhidden, dh_part, rowfac, stream)) != AREAL_OK) return rc;
+    if (!w_in_place) {
+      hipLaunchKernelGGL(transpose_pad_bf16_kernel,
+                         dim3((unsigned)ceil_div_i64(H, 64), (unsigned)ceil_div_i64(ldv, 64)),
+                         dim3(256), 0, stream, (const u16*)weight, H, (int)V, (int)H, wT, ldv);
+      AREAL_CHECK_LAUNCH();
+    }
+    if ((rc = launch_dhidden(w_in_place ? (const u16*)weight : wT, V, e, ldv, H, T, dhidden, dh_part,
+                             rowfac, stream)) != AREAL_OK)
+      return rc;
   }
   if (dbias != nullptr) {
     hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,

@@ -48,6 +48,9 @@ SHAPES = [
     (300, 64, 1000, 1.5, 1.0, False, 128),
     (700, 128, 5000, 1.0, 2.0, True, None),
     (515, 896, 151936, 1.0, 1.0, False, 256),
+    # V a multiple of 64: dHidden reads the [V, H] weight in place (no transposed copy)
+    (260, 200, 1088, 0.7, 1.0, True, 128),
+    (700, 512, 4096, 1.0, 1.0, False, None),
 ]
 
 
