@@ -303,17 +303,17 @@ def main() -> None:
     fwd_tflops = 2.0 * T * H * V / (t_fwd / args.steps * 1e-3) / 1e12
 
     # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-    # command (KiB per dispatch, scaled by the factors the same counters show for the bf16
-    # transpose kernel of known size: fetch x2.0, write x1.0). Only measured for the default
+    # command (KiB per dispatch, scaled by the factors the same counters show for copy-like
+    # kernels of known size, the operand-prep and the bf16 transpose: fetch x2.0, write x1.0). Only measured for the default
     # workload; the forward's fetch count moves by +-20 % from run to run with L2 hit timing.
     traffic = None
     traffic_detail = None
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            "gemm_nt_sweep<FwdEpi> forward": 4.34454e7 * kib * 2.0 + 1.28786e7 * kib,
-            "gemm_nt_sweep<StoreEpi> dHidden": 3.02432e7 * kib * 2.0 + 2.99008e5 * kib,
-            "gemm_tn_sweep<StoreEpi> dWeight": 3.0399e7 * kib * 2.0 + 1.26301e6 * kib,
+            "gemm_nt_sweep<FwdEpi> forward": 3.38786e7 * kib * 2.0 + 1.29532e7 * kib,
+            "gemm_mix_sweep<StoreEpi> dHidden": 3.46954e7 * kib * 2.0 + 3.01056e5 * kib,
+            "gemm_tn_sweep<StoreEpi> dWeight": 3.05786e7 * kib * 2.0 + 1.26301e6 * kib,
         }
         traffic = sum(traffic_detail.values()) / 3.0
 
@@ -339,7 +339,7 @@ def main() -> None:
         },
         "pct_bf16_mfma_peak": 100.0 * (algo_flops / (ms_per_step * 1e-3) / 1e12) / PEAK_BF16_TFLOPS,
         "roofline": {
-            "kernel": ("gemm_nt_sweep<FwdEpi>, gemm_nt_sweep<StoreEpi> (dHidden), "
+            "kernel": ("gemm_nt_sweep<FwdEpi>, gemm_mix_sweep<StoreEpi> (dHidden), "
                        "gemm_tn_sweep<StoreEpi> (dWeight)"
                        + ("" if saved else ", gemm_nt_sweep<BwdEpi> (recompute)")),
             "bound": "mfma",
