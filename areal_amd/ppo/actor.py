@@ -85,6 +85,14 @@ def grpo_loss_fn(
         current_version=current_version,
     )
 
+    # The reference stops here when the proximal log-probs hold a NaN or Inf (actor.py:924-928),
+    # which costs a host synchronisation before any loss kernel is queued. The same check runs
+    # on the device now and is read after the loss call's own synchronisation: same error, one
+    # idle gap of the GPU less per micro-batch.
+    prox_nonfinite = torch.isfinite(prox_logp).logical_not().any()
+    if not prox_logp.is_cuda:  # nothing to overlap with: report at once
+        _raise_if_nonfinite(prox_nonfinite, prox_logp_method)
+
     if m2_threshold is not None:
         loss_mask = _apply_m2po_masking(old_logp, prox_logp, loss_mask, m2_threshold)
 
@@ -140,6 +148,8 @@ def grpo_loss_fn(
             importance_sampling_level=importance_sampling_level,
             cu_seqlens=input_data.get("cu_seqlens"),
         )
+
+    _raise_if_nonfinite(prox_nonfinite, prox_logp_method)
 
     # joint distillation (actor.py:629-658)
     teacher_logp = input_data.get("teacher_logp")
@@ -239,6 +249,14 @@ def compute_prox_logp_approximations(
     return out
 
 
+def _raise_if_nonfinite(flag: torch.Tensor, prox_logp_method: str) -> None:
+    if bool(flag):
+        raise RuntimeError(
+            f"prox_logp contains NaN or Inf with prox_logp_method='{prox_logp_method}'. "
+            "This indicates computation failed."
+        )
+
+
 def _resolve_proximal_logp(prox_logp_gt, prox_logp_method, old_logp, logprobs, versions, current_version):
     """Proximal log-probs to train with: the recomputed ones, or the log-linear approximation
     when the forward pass was skipped (``actor.py:851-930``; same errors)."""
@@ -265,11 +283,6 @@ def _resolve_proximal_logp(prox_logp_gt, prox_logp_method, old_logp, logprobs, v
         raise RuntimeError(
             f"prox_logp is None after handling prox_logp_method='{prox_logp_method}'. "
             "This indicates configuration or computation error."
-        )
-    if torch.isnan(prox_logp).any() or torch.isinf(prox_logp).any():
-        raise RuntimeError(
-            f"prox_logp contains NaN or Inf with prox_logp_method='{prox_logp_method}'. "
-            "This indicates computation failed."
         )
     return prox_logp
 

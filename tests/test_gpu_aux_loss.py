@@ -243,3 +243,10 @@ def test_grpo_loss_fn_optional_branches_match_oracle(dev, rl_weight):
     with pytest.raises(ValueError, match="versions not available"):
         grpo_loss_fn(x, torch.zeros(n, device=dev), dict(logprobs=old.to(dev), advantages=adv.to(dev),
                      loss_mask=mask.to(dev), prox_logp=None), 0.2, None, None, prox_logp_method="loglinear")
+    # a NaN or Inf among the proximal log-probs is an error, as in the reference (actor.py:924-928)
+    bad = old.clone()
+    bad[3] = float("inf")
+    with pytest.raises(RuntimeError, match="prox_logp contains NaN or Inf"):
+        grpo_loss_fn(x, torch.zeros(n, device=dev), dict(logprobs=old.to(dev), advantages=adv.to(dev),
+                     loss_mask=mask.to(dev), prox_logp=bad.to(dev)), 0.2, None, None)
+
