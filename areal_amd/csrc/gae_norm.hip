@@ -708,6 +708,31 @@ __global__ __launch_bounds__(NORM_THREADS) void masked_norm_apply_kernel(
   }
 }
 
+// The same over each row of a [rows, cols] array (masked_normalization with dim = the trailing
+// dimensions): one block per row, statistics then the apply pass over the row.
+__global__ __launch_bounds__(NORM_THREADS) void masked_norm_rows_kernel(
+    const float* x, const float* mask, int64_t cols, int unbiased, double eps, float* out) {
+  __shared__ double smem[4];
+  const float* xr = x + (int64_t)blockIdx.x * cols;
+  const float* mr = mask ? mask + (int64_t)blockIdx.x * cols : nullptr;
+  float* o = out + (int64_t)blockIdx.x * cols;
+  double cnt = 0.0, s = 0.0, s2 = 0.0;
+  for (int64_t i = threadIdx.x; i < cols; i += blockDim.x) {
+    const double m = mr ? (double)mr[i] : 1.0;
+    const double v = (double)xr[i] * m;
+    cnt += m; s += v; s2 += v * v;
+  }
+  cnt = block_sum_d(cnt, smem); s = block_sum_d(s, smem); s2 = block_sum_d(s2, smem);
+  const double mean = s / cnt;
+  double var = s2 / cnt - mean * mean;
+  if (unbiased) var *= cnt / (cnt - 1.0);
+  const double den = sqrt(var) + eps;
+  for (int64_t i = threadIdx.x; i < cols; i += blockDim.x) {
+    const double v = (double)xr[i] * (mr ? (double)mr[i] : 1.0);
+    o[i] = (float)((v - mean) / den);
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // Turn-level GAE (areal/trainer/ppo/gae.py:82-163): every generated turn is one timestep.
 // One block per padded row. Active tokens carry non-decreasing turn ids (checked; a violation
@@ -1147,6 +1172,18 @@ int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(masked_norm_apply_kernel, dim3((unsigned)nb), dim3(NORM_THREADS), 0, stream, x,
                      mask, n, (const double*)part, (int)nb, unbiased, eps, out);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// masked_normalization over the trailing dimensions: x, mask (nullable), out are [rows, cols].
+int areal_masked_norm_rows(const float* x, const float* mask, int64_t rows, int64_t cols,
+                           int unbiased, double eps, float* out, hipStream_t stream) {
+  if (rows < 0 || cols < 0 || rows > 0x7fffffffLL) return AREAL_ERR_BAD_ARG;
+  if (rows == 0 || cols == 0) return AREAL_OK;
+  if (!x || !out) return AREAL_ERR_BAD_ARG;
+  hipLaunchKernelGGL(masked_norm_rows_kernel, dim3((unsigned)rows), dim3(NORM_THREADS), 0, stream, x,
+                     mask, cols, unbiased, eps, out);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

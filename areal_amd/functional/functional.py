@@ -348,20 +348,43 @@ def masked_normalization(
     reduce_group=None,
 ):
     """Whiten ``x`` over its masked elements (``functional.py:16-53``): fp64 sums,
-    ``var = E[x^2] - E[x]^2``, ``(x * mask - mean) / (sqrt(var) + eps)``.
+    ``var = E[x^2] - E[x]^2``, ``(x * mask - mean) / (sqrt(var) + eps)``, over all dimensions or
+    over the dimensions in ``dim`` (every slice along the others gets its own statistics).
 
-    Only the reduction over all dimensions is implemented (the only use on this path), in fp64
-    whatever ``high_precision`` says; a multi-rank ``all_reduce`` is outside the one-GPU scope.
+    The sums are fp64 whatever ``high_precision`` says; a multi-rank ``all_reduce`` is outside
+    the one-GPU scope.
     """
-    if dim is not None and tuple(sorted(d % x.ndim for d in dim)) != tuple(range(x.ndim)):
-        raise NotImplementedError("masked_normalization reduces over all dimensions only")
     import torch.distributed as dist
 
     if all_reduce and dist.is_initialized() and dist.get_world_size(reduce_group) > 1:
         raise NotImplementedError("masked_normalization runs on one GPU; no all_reduce")
     del high_precision
+    if mask is not None and mask.shape != x.shape:
+        raise ValueError(f"mask must have the shape of x, got {tuple(mask.shape)} and {tuple(x.shape)}")
     lib = _lib.load()
     dev = _lib.require_gpu(x, mask)
+    if dim is not None:
+        dims = sorted({d % x.ndim for d in ((dim,) if isinstance(dim, int) else tuple(dim))})
+    else:
+        dims = list(range(x.ndim))
+    if len(dims) < x.ndim:
+        # reduced dimensions last: [rows, cols], one row per slice along the kept dimensions
+        kept = [d for d in range(x.ndim) if d not in dims]
+        perm = kept + dims
+        xp = x.to(torch.float32).permute(perm).contiguous()
+        mp = mask.to(torch.float32).permute(perm).contiguous() if mask is not None else None
+        rows = 1
+        for d in kept:
+            rows *= x.shape[d]
+        cols = xp.numel() // max(rows, 1)
+        outp = torch.empty_like(xp)
+        rc = lib.areal_masked_norm_rows(
+            _lib.ptr(xp), _lib.ptr(mp), rows, cols, int(bool(unbiased)), float(eps), _lib.ptr(outp),
+            _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_masked_norm_rows")
+        inverse = [perm.index(d) for d in range(x.ndim)]
+        return outp.permute(inverse).contiguous()
     xf = x.to(torch.float32).contiguous()
     mf = mask.to(torch.float32).contiguous() if mask is not None else None
     out = torch.empty_like(xf)

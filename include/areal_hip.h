@@ -293,6 +293,12 @@ size_t areal_masked_norm_workspace_bytes(int64_t n);
 int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased, double eps,
                       float* out, void* workspace, size_t workspace_bytes, areal_stream_t stream);
 
+/* masked_normalization with dim = the trailing dimensions (areal/utils/functional/functional.py:16-53,
+ * the `dim` argument): x, mask (NULL allowed) and out are [rows, cols]; every row is whitened with
+ * its own masked mean and variance. */
+int areal_masked_norm_rows(const float* x, const float* mask, int64_t rows, int64_t cols,
+                           int unbiased, double eps, float* out, areal_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------
  * Packing / padding by cu_seqlens and masked logging statistics (the steps either side of the
  * loss). Replace the per-sequence Python loops of pack_tensor_dict (areal/utils/data.py:496-545),

@@ -122,12 +122,12 @@ def normalization(
     return (centred / (std + eps)).float()
 
 
-def masked_normalization(x, mask=None, unbiased=False, eps=1e-5):
-    """masked_normalization over all dimensions, fp64 sums (functional.py:16-53)."""
+def masked_normalization(x, mask=None, unbiased=False, eps=1e-5, dim=None):
+    """masked_normalization, fp64 sums (functional.py:16-53); dim=None reduces over everything."""
     x = x.to(torch.float64)
-    dims = tuple(range(x.ndim))
+    dims = tuple(range(x.ndim)) if dim is None else ((dim,) if isinstance(dim, int) else tuple(dim))
     if mask is None:
-        factor = torch.tensor(np.prod(x.shape), dtype=torch.float64)
+        factor = torch.tensor(np.prod([x.shape[d] for d in dims]), dtype=torch.float64)
     else:
         mask = mask.to(torch.float64)
         x = x * mask

@@ -208,6 +208,20 @@ def test_masked_normalization_matches_oracle(dev):
         torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-6)
     want = N.masked_normalization(x, None)
     torch.testing.assert_close(masked_normalization(x.to(dev)).cpu(), want, rtol=1e-5, atol=1e-6)
+    # statistics per slice: trailing dimension, leading dimension, and a middle one of a 3-D tensor
+    for dim in (-1, (0,), 1):
+        want = N.masked_normalization(x, m, unbiased=True, dim=dim)
+        got = masked_normalization(x.to(dev), m.to(dev), dim=dim, unbiased=True)
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-6)
+    x3 = torch.randn(6, 50, 7, generator=g)
+    m3 = (torch.rand(6, 50, 7, generator=g) > 0.2).float()
+    for dim in ((1,), (0, 2), (0, 1, 2)):
+        want = N.masked_normalization(x3, m3, dim=dim)
+        got = masked_normalization(x3.to(dev), m3.to(dev), dim=dim)
+        assert got.shape == x3.shape
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-6)
+    want = N.masked_normalization(x3, None, dim=(2,))
+    torch.testing.assert_close(masked_normalization(x3.to(dev), dim=(2,)).cpu(), want, rtol=1e-5, atol=1e-6)
 
 
 # ---------------------------------------------------------------- turn-level GAE

@@ -186,6 +186,24 @@ def test_masked_normalization_closed_form():
     torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-6)
 
 
+def test_masked_normalization_dim_is_per_slice():
+    # dim = the reduced dimensions: each slice along the others is whitened by itself (brute force
+    # per row / per column with torch's own mean and std of the active elements)
+    torch.manual_seed(1)
+    x = torch.randn(5, 40) * 2 + 1
+    m = (torch.rand(5, 40) > 0.3).float()
+    out = N.masked_normalization(x, m, unbiased=True, eps=1e-5, dim=-1)
+    for r in range(5):
+        act = x[r][m[r].bool()].double()
+        want = (x[r].double() * m[r].double() - act.mean()) / (act.std(unbiased=True) + 1e-5)
+        torch.testing.assert_close(out[r].double(), want, rtol=1e-5, atol=1e-6)
+    out0 = N.masked_normalization(x, None, dim=(0,))
+    for c in range(40):
+        col = x[:, c].double()
+        torch.testing.assert_close(out0[:, c].double(), (col - col.mean()) / (col.std(unbiased=False) + 1e-5),
+                                   rtol=1e-5, atol=1e-6)
+
+
 # ---------------------------------------------------------------- turn-level GAE
 def test_turn_level_gae_reference_literals():
     # reference tests/test_ppo_gae.py:81-151 (inputs and expected values re-typed)
