@@ -6,6 +6,7 @@ from areal_amd.functional.functional import (
     cispo_loss_fn,
     masked_normalization,
     ppo_actor_loss_fn,
+    reward_overlong_penalty,
 )
 from areal_amd.functional.aux_losses import (
     dpo_pair_logratios,
@@ -28,6 +29,7 @@ __all__ = [
     "cispo_loss_fn",
     "masked_normalization",
     "ppo_actor_loss_fn",
+    "reward_overlong_penalty",
     "sapo_loss_fn",
     "ppo_critic_loss_fn",
     "dpo_pair_logratios",

@@ -397,3 +397,24 @@ def masked_normalization(
     )
     _lib.check(rc, "areal_masked_norm")
     return out
+
+
+def reward_overlong_penalty(
+    data: dict,
+    overlong_tokens: int,
+    overlong_penalty_factor: float,
+    max_response_length: int,
+) -> dict:
+    """DAPO's soft penalty for responses that run into the last ``overlong_tokens`` tokens of the
+    budget (``functional.py:937-959``): ``rewards[i] += min(-(len_i - (max_response_length -
+    overlong_tokens)) / overlong_tokens * overlong_penalty_factor, 0)`` with ``len_i`` the number
+    of loss-mask tokens of sample ``i``. ``data["rewards"]`` is updated in place, as in the
+    reference; its per-sample Python loop is one vector expression here."""
+    rewards = data["rewards"]
+    response_lengths = data["loss_mask"].sum(dim=-1).long()
+    exceed = response_lengths - (max_response_length - overlong_tokens)
+    penalty = torch.clamp(-exceed / overlong_tokens * overlong_penalty_factor, max=0)
+    rewards += penalty.to(rewards.dtype)
+    data["rewards"] = rewards
+    return data
+

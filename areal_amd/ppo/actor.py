@@ -19,7 +19,11 @@ from areal_amd.config import RejectionSamplingConfig
 from areal_amd.data import KLEstimator, Normalization
 from areal_amd import _lib
 from areal_amd.functional.aux_losses import _Launch, _ScaledLoss, sapo_loss_fn
-from areal_amd.functional.functional import cispo_loss_fn, ppo_actor_loss_fn
+from areal_amd.functional.functional import (
+    cispo_loss_fn,
+    ppo_actor_loss_fn,
+    reward_overlong_penalty,
+)
 from areal_amd.ppo.gae import _compute_token_level_gae, _compute_turn_level_gae, compute_gae_lambda
 
 # areal/utils/constants.py:36-92
@@ -466,11 +470,12 @@ def compute_advantages(
     if overlong_reward_penalty:
         assert overlong_tokens is not None
         assert overlong_penalty_factor is not None
-        # reward_overlong_penalty (functional.py:937-959), without its per-sample loop
-        response_lengths = data["loss_mask"].sum(dim=-1).long()
-        exceed = response_lengths - (max_new_tokens - overlong_tokens)
-        penalty = torch.clamp(-exceed / overlong_tokens * overlong_penalty_factor, max=0)
-        data["rewards"] = data["rewards"] + penalty.to(data["rewards"].dtype)
+        data = reward_overlong_penalty(
+            data,
+            overlong_tokens=overlong_tokens,
+            overlong_penalty_factor=overlong_penalty_factor,
+            max_response_length=max_new_tokens,
+        )
 
     reward_score = (data["rewards"] + reward_bias) * reward_scaling
     reward_score = torch.clip(reward_score, max=reward_clip, min=-reward_clip)

@@ -211,3 +211,24 @@ def test_gae_lambda_functions_reference_literals():
         resolve_gae_lambda_fn(True)
     with pytest.raises(TypeError, match="non-empty dotted function path"):
         resolve_gae_lambda_fn("")
+
+
+def test_reward_overlong_penalty_matches_the_reference_loop():
+    # areal/utils/functional/functional.py:937-959 restated as its per-sample loop (the
+    # reference has no test for it); the vector form must give the same rewards, in place.
+    from areal_amd.functional import reward_overlong_penalty
+
+    loss_mask = torch.zeros(5, 40)
+    for i, n in enumerate([10, 24, 30, 36, 40]):
+        loss_mask[i, :n] = 1
+    rewards = torch.tensor([1.0, 0.0, 1.0, 1.0, 0.5])
+    data = dict(rewards=rewards.clone(), loss_mask=loss_mask, input_ids=torch.zeros(5, 40, dtype=torch.long))
+    held = data["rewards"]
+    out = reward_overlong_penalty(data, overlong_tokens=8, overlong_penalty_factor=1.5, max_response_length=32)
+    want = rewards.clone()
+    for i, n in enumerate([10, 24, 30, 36, 40]):
+        want[i] += min(-(n - (32 - 8)) / 8 * 1.5, 0)
+    assert out is data and data["rewards"] is held  # updated in place
+    torch.testing.assert_close(data["rewards"], want)
+    assert data["rewards"].tolist() == pytest.approx([1.0, 0.0, -0.125, -1.25, -2.5])
+
