@@ -16,6 +16,7 @@ from areal_amd.functional.aux_losses import (
 )
 from areal_amd.functional.lm_head import (
     ChunkedLMHeadOutput,
+    chunked_lm_head_logprobs_entropy,
     fused_lm_head_logprobs_entropy,
 )
 from areal_amd.functional.vocab_parallel import (
@@ -37,5 +38,6 @@ __all__ = [
     "gather_logprobs",
     "gather_logprobs_entropy",
     "ChunkedLMHeadOutput",
+    "chunked_lm_head_logprobs_entropy",
     "fused_lm_head_logprobs_entropy",
 ]

@@ -271,3 +271,49 @@ def fused_lm_head_logprobs_entropy(
         save_probs,
     )
     return ChunkedLMHeadOutput(*values)
+
+
+def chunked_lm_head_logprobs_entropy(
+    output_layer,
+    hidden_states: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    temperature: float,
+    chunk_size: int,
+    logit_scale: float = 1.0,
+) -> ChunkedLMHeadOutput:
+    """The reference's entry point of the same name (``vocab_parallel_head.py:941-982``), for
+    callers that hold an output layer object: the bias comes from ``output_layer.bias`` unless
+    ``output_layer.skip_bias_add`` is set, ``chunk_size`` is validated and otherwise unused (the
+    kernels hold no fp32 logits, so there is nothing to bound by it), and the layer options the
+    fused path cannot honour are refused with the reference's errors. Tensor-parallel layers (a ``tp_group`` of more than one rank) are
+    outside the one-GPU scope."""
+    if not getattr(output_layer, "chunked_loss_supported", True):
+        raise NotImplementedError(
+            "chunked LM Head loss does not support this output-layer forward override"
+        )
+    config = getattr(output_layer, "config", None)
+    if getattr(config, "defer_embedding_wgrad_compute", False):
+        raise NotImplementedError(
+            "chunked LM Head loss is incompatible with defer_embedding_wgrad_compute"
+        )
+    if getattr(output_layer, "gather_output", False):
+        raise NotImplementedError(
+            "chunked LM Head loss requires vocab-parallel (ungathered) output"
+        )
+    tp_group = getattr(output_layer, "tp_group", None)
+    if tp_group is not None:
+        import torch.distributed as dist
+
+        if dist.is_initialized() and dist.get_world_size(tp_group) > 1:
+            raise NotImplementedError("vocab-parallel LM heads over several GPUs are not built here")
+    bias = None
+    if not getattr(output_layer, "skip_bias_add", False):
+        bias = getattr(output_layer, "bias", None)
+    if chunk_size <= 0:
+        raise ValueError(f"chunk_size must be positive, got {chunk_size}")
+    return fused_lm_head_logprobs_entropy(
+        hidden_states, weight, labels, temperature=temperature, logit_scale=logit_scale, bias=bias,
+    )
+

@@ -255,3 +255,27 @@ def test_empty_and_3d_inputs(dev):
     want = L.lm_head_logprobs_entropy(h.cpu().view(10, 16), w.cpu(), y.cpu().view(-1))
     assert out.logprobs.shape == (2, 5)
     torch.testing.assert_close(out.logprobs.cpu().view(-1), want[0], rtol=1e-4, atol=2e-3)
+
+
+def test_chunked_lm_head_wrapper_uses_the_layer_bias(dev):
+    from types import SimpleNamespace
+
+    from areal_amd.functional import chunked_lm_head_logprobs_entropy
+
+    T, H, V = 40, 32, 200
+    g = torch.Generator().manual_seed(3)
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.3).bfloat16()
+    bias = (torch.randn(V, generator=g) * 0.2).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g)
+    layer = SimpleNamespace(bias=bias.to(dev), skip_bias_add=False, gather_output=False, tp_group=None)
+    out = chunked_lm_head_logprobs_entropy(layer, hidden.to(dev), weight.to(dev), labels.to(dev),
+                                           temperature=0.7, chunk_size=16, logit_scale=0.5)
+    want = L.lm_head_logprobs_entropy(hidden, weight, labels, 0.7, 0.5, bias)
+    torch.testing.assert_close(out.logprobs.cpu(), want[0], rtol=0, atol=2e-3)
+    layer.skip_bias_add = True
+    out = chunked_lm_head_logprobs_entropy(layer, hidden.to(dev), weight.to(dev), labels.to(dev),
+                                           temperature=0.7, chunk_size=16, logit_scale=0.5)
+    want = L.lm_head_logprobs_entropy(hidden, weight, labels, 0.7, 0.5, None)
+    torch.testing.assert_close(out.logprobs.cpu(), want[0], rtol=0, atol=2e-3)
+

@@ -232,3 +232,28 @@ def test_reward_overlong_penalty_matches_the_reference_loop():
     torch.testing.assert_close(data["rewards"], want)
     assert data["rewards"].tolist() == pytest.approx([1.0, 0.0, -0.125, -1.25, -2.5])
 
+
+def test_chunked_lm_head_wrapper_refuses_what_the_reference_refuses():
+    # vocab_parallel_head.py:953-966: same exception types and messages; the bias is taken from
+    # the layer unless skip_bias_add
+    from types import SimpleNamespace
+
+    from areal_amd.functional import chunked_lm_head_logprobs_entropy as head
+
+    h, w, y = torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(16, 8, dtype=torch.bfloat16), torch.zeros(4, dtype=torch.long)
+    ok = SimpleNamespace(bias=None, skip_bias_add=False, gather_output=False, tp_group=None,
+                         config=SimpleNamespace(defer_embedding_wgrad_compute=False))
+    with pytest.raises(NotImplementedError, match="forward override"):
+        head(SimpleNamespace(chunked_loss_supported=False), h, w, y, temperature=1.0, chunk_size=4)
+    with pytest.raises(NotImplementedError, match="defer_embedding_wgrad_compute"):
+        head(SimpleNamespace(config=SimpleNamespace(defer_embedding_wgrad_compute=True)), h, w, y,
+             temperature=1.0, chunk_size=4)
+    with pytest.raises(NotImplementedError, match="ungathered"):
+        head(SimpleNamespace(gather_output=True), h, w, y, temperature=1.0, chunk_size=4)
+    with pytest.raises(ValueError, match="chunk_size must be positive"):
+        head(ok, h, w, y, temperature=1.0, chunk_size=0)
+    with pytest.raises(ValueError, match="temperature must be positive"):
+        head(ok, h, w, y, temperature=0.0, chunk_size=4)
+    with pytest.raises(_lib.ArealHipError):  # valid arguments reach the kernels, which need the GPU
+        head(ok, h, w, y, temperature=1.0, chunk_size=4)
+
