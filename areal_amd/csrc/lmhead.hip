@@ -1,15 +1,24 @@
 // Fused lm_head -> log-softmax -> label log-prob + entropy, forward and backward, for gfx950.
 //
-// One bf16 MFMA contraction D[i][j] = sum_k A[i][k] * B[j][k] (both operands k-contiguous)
-// serves all four matrix products of the path; only the epilogue differs:
-//   forward   : A = W [V,H],        B = hidden [T,H]      -> online softmax statistics
-//   recompute : A = W [V,H],        B = hidden [Tc,H]     -> dlogits (bf16, two layouts)
-//   dHidden   : A = W^T [H,V'],     B = dlogits [Tc,V']   -> bf16 store
-//   dWeight   : A = hidden^T [H,T'],B = dlogits^T [V,T']  -> fp32 accumulate
-// The vocabulary is put on the MFMA "A" side so that, in the accumulator layout of
-// v_mfma_f32_32x32x16_bf16 (lane -> column j, registers -> rows i), each lane owns one token
+// Every matrix product of the path is one bf16 MFMA contraction D[i][j] = sum_k A[.]*B[.] over
+// 256 x 256 x 64 tiles; three kernels differ in how the operands are stored, the epilogues in
+// what happens to the accumulators:
+//   gemm_nt_sweep  (A[i][k], B[j][k], both k-contiguous)
+//     forward   : A = W [V,H],       B = hidden [T,H]     -> online softmax statistics, and in
+//                                                            the saving variant the bf16
+//                                                            exponentials e [T,V]
+//     recompute : A = W [V,H],       B = hidden [Tc,H]    -> dlogits (bf16, one or two layouts)
+//   gemm_mix_sweep (A[k][i] k-major, B[j][k] k-contiguous)
+//     dHidden   : A = W [V,H] as stored, B = e or dlogits [T,V'] -> bf16 store, rows scaled
+//                 (gemm_nt_sweep on a zero-padded W^T when V is not a multiple of 64)
+//   gemm_tn_sweep  (A[k][i], B[k][j], both k-major)
+//     dWeight   : A = hidden [T,H] (scaled per row in the saved mode), B = e or dlogits [T,V']
+//                 -> bf16 store, or fp32 store / accumulate over token chunks
+//   gemm_nt_generic: any K (not a multiple of 64), register-staged loads.
+// The vocabulary is put on the MFMA "A" side of the forward so that, in the accumulator layout
+// of v_mfma_f32_32x32x16_bf16 (lane -> column j, registers -> rows i), each lane owns one token
 // and 16 vocabulary entries per 32x32 block: the softmax reductions over the vocabulary run
-// inside a lane and the [T,V] logits never leave registers.
+// inside a lane and the fp32 logits never leave registers.
 //
 // Follows the algorithm of the reference's chunked LM head
 // (areal/models/mcore/vocab_parallel_head.py:564-735 forward, :737-938 backward) and the
@@ -30,11 +39,11 @@ struct GemmArgs {
   const u16* A; int64_t lda; int M;   // A rows (index i)
   const u16* B; int64_t ldb; int N;   // B rows (index j)
   int K;                              // multiple of 8
-  int acols, bcols;                   // k-major (TN) form only: readable columns of A and B
-                                      // (both operands must have K readable rows)
-  // split-K (gemm_nt_sweep with a store epilogue only): the grid is ksplit copies of the tile
-  // schedule; copy z contracts k-tiles [z*kt_per_split, (z+1)*kt_per_split) and writes its
-  // partial result zstride bytes after the previous copy's. ksplit <= 1: off.
+  int acols, bcols;                   // k-major operands only: readable columns of A and B
+                                      // (a k-major operand must have K readable rows)
+  // split-K (gemm_nt_sweep / gemm_mix_sweep with a store epilogue only): the grid is ksplit
+  // copies of the tile schedule; copy z contracts k-tiles [z*kt_per_split, (z+1)*kt_per_split)
+  // and writes its partial result zstride bytes after the previous copy's. ksplit <= 1: off.
   int ksplit, kt_per_split;
   int64_t zstride;
 };
