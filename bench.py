@@ -162,6 +162,12 @@ def hbm_rooflines(dev):
     norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
     add("norm_stats1+norm_stats2+norm_apply", "config 3: [1024, 1600] advantages, groups of 16 rows, 20 B/token",
         20 * x.numel(), timed(lambda: norm(x, mk)))
+    # the same normalisation at the padded size, where launch latency no longer dominates
+    xl_ = torch.randn(1024, 8192, device=dev)
+    ml_ = (torch.rand(1024, 8192, device=dev) > 0.25).float()
+    add("norm_stats1+norm_stats2+norm_apply", "[1024, 8192] advantages, groups of 16 rows, 20 B/token",
+        20 * xl_.numel(), timed(lambda: norm(xl_, ml_)))
+    del xl_, ml_
     Tl = 4 << 20
     lp = (torch.randn(Tl, device=dev) * 0.5 - 1).requires_grad_(True)
     prox = lp.detach() + torch.randn(Tl, device=dev) * 0.1
