@@ -94,6 +94,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_masked_norm_workspace_bytes": (SZ, [I64]),
     "areal_masked_norm": (I, [P, P, I64, I, D, P, P, SZ, P]),
     "areal_masked_norm_rows": (I, [P, P, I64, I64, I, D, P, P]),
+    "areal_advantage_prep": (I, [P, P, P, P, P, I64, I64, I, I, I, I, I, F, P, P, P, P, P, P, P, P, P]),
 }
 
 

@@ -734,6 +734,86 @@ __global__ __launch_bounds__(NORM_THREADS) void masked_norm_rows_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// Reward shaping in front of GAE (PPOActor.compute_advantages, areal/trainer/ppo/actor.py:224-283):
+// one pass over a padded [bs, L] batch instead of some twenty elementwise tensor ops. One block
+// per row; the row's sequence length (sum of the attention mask) first, then per token t:
+//   lm[t]   = float(loss_mask[(t + 1) % L])                       (torch.roll(..., -1))
+//   old[t]  = logp[(t + 1) % L] * lm[t]   (logp[t] * lm[t] when the log-probs are not rolled)
+//   ref[t]  = ref_logp[t] * lm[t]         (0 when there is no reference policy)
+//   kl[t]   = -kl_ctl * estimator(old[t] - ref[t])                (data.py:1662-1698)
+//   gkl[t]  = kl[t], zero at t = seqlen - 1
+//   out[t]  = reward_score at t = max(seqlen - 2, 0), else 0 (0 everywhere for a truncated
+//             row when mask_no_eos_with_zero)
+//   tot[t]  = gkl[t] + out[t]
+// The arithmetic follows the reference's tensor ops in their order (this file is compiled
+// without floating-point contraction). Index -1 of an empty row addresses the last slot, as
+// Python indexing does.
+// ---------------------------------------------------------------------------------------
+struct PrepArgs {
+  const uint8_t* loss_mask;  // [bs, L] nonzero = 1
+  const uint8_t* attn_mask;  // [bs, L]
+  const float* logp;         // [bs, L]
+  float* ref_logp;           // [bs, L] or null; masked in place when ref_in_place
+  const float* reward_score; // [bs]
+  int64_t L;
+  int roll_logp;             // 1: old = roll(logp, -1); 0: old = logp
+  int estimator;             // 1, 2, 3
+  int apply_clamp;
+  int mask_no_eos_with_zero;
+  int ref_in_place;
+  float kl_ctl;
+  float* lm_out;             // [bs, L]
+  float* old_out;            // [bs, L]
+  float* kl_out;             // [bs, L]  kl rewards before the end-of-sequence zero
+  float* gkl_out;            // [bs, L] or null
+  float* outcome_out;        // [bs, L] or null
+  float* tot_out;            // [bs, L]
+  int64_t* seqlens_out;      // [bs]
+  uint8_t* no_eos_out;       // [bs]
+};
+
+__global__ __launch_bounds__(NORM_THREADS) void adv_prep_kernel(PrepArgs a) {
+  __shared__ double smem[4];
+  const int64_t b = blockIdx.x, L = a.L;
+  const uint8_t* am = a.attn_mask + b * L;
+  const uint8_t* lmk = a.loss_mask + b * L;
+  const float* lp = a.logp + b * L;
+  float* rf = a.ref_logp ? a.ref_logp + b * L : nullptr;
+  double cnt = 0.0;
+  for (int64_t t = threadIdx.x; t < L; t += blockDim.x) cnt += am[t] ? 1.0 : 0.0;
+  const int64_t seqlen = (int64_t)block_sum_d(cnt, smem);
+  const bool no_eos = seqlen == L;
+  if (threadIdx.x == 0) { a.seqlens_out[b] = seqlen; a.no_eos_out[b] = no_eos ? 1 : 0; }
+  const int64_t t_end = seqlen - 1 >= 0 ? seqlen - 1 : seqlen - 1 + L;  // rewards[b, seqlen - 1] = 0
+  const int64_t t_out = seqlen - 2 > 0 ? seqlen - 2 : 0;                 // clip(seqlen - 2, min = 0)
+  float score = a.reward_score[b];
+  if (a.mask_no_eos_with_zero && no_eos) score = 0.f;
+  const float neg_ctl = -a.kl_ctl;
+  for (int64_t t = threadIdx.x; t < L; t += blockDim.x) {
+    const int64_t tn = t + 1 < L ? t + 1 : 0;
+    const float lm = lmk[tn] ? 1.f : 0.f;
+    const float old = (a.roll_logp ? lp[tn] : lp[t]) * lm;
+    const float ref = rf ? rf[t] * lm : 0.f * lm;
+    if (rf && a.ref_in_place) rf[t] = ref;
+    const float diff = old - ref;
+    float est;
+    if (a.estimator == 1) est = diff;
+    else if (a.estimator == 2) est = diff * diff / 2.0f;
+    else { const float neg = -diff; est = expf(neg) - 1.f - neg; }
+    if (a.apply_clamp) est = fminf(fmaxf(est, -10.f), 10.f);
+    const float kl = neg_ctl * est;
+    const float gkl = t == t_end ? 0.f : kl;
+    const float oc = t == t_out ? score : 0.f;
+    a.lm_out[b * L + t] = lm;
+    a.old_out[b * L + t] = old;
+    a.kl_out[b * L + t] = kl;
+    if (a.gkl_out) a.gkl_out[b * L + t] = gkl;
+    if (a.outcome_out) a.outcome_out[b * L + t] = oc;
+    a.tot_out[b * L + t] = gkl + oc;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Turn-level GAE (areal/trainer/ppo/gae.py:82-163): every generated turn is one timestep.
 // One block per padded row. Active tokens carry non-decreasing turn ids (checked; a violation
 // sets *status), so a turn starts at the first active token whose id exceeds every active id on
@@ -1184,6 +1264,31 @@ int areal_masked_norm_rows(const float* x, const float* mask, int64_t rows, int6
   if (!x || !out) return AREAL_ERR_BAD_ARG;
   hipLaunchKernelGGL(masked_norm_rows_kernel, dim3((unsigned)rows), dim3(NORM_THREADS), 0, stream, x,
                      mask, cols, unbiased, eps, out);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// Reward shaping in front of GAE on a padded [bs, L] batch; see adv_prep_kernel. loss_mask and
+// attn_mask are bytes (nonzero = set); ref_logp, gkl_out and outcome_out may be null. With
+// ref_in_place the masked reference log-probs are written back (the reference's `ref_logp *=
+// loss_mask`); old_out may be logp itself when roll_logp is 0 (its `old_logp *= loss_mask`).
+int areal_advantage_prep(const uint8_t* loss_mask, const uint8_t* attn_mask, const float* logp,
+                         float* ref_logp, const float* reward_score, int64_t bs, int64_t L,
+                         int roll_logp, int estimator, int apply_clamp, int mask_no_eos_with_zero,
+                         int ref_in_place, float kl_ctl, float* lm_out, float* old_out,
+                         float* kl_out, float* gkl_out, float* outcome_out, float* tot_out,
+                         int64_t* seqlens_out, uint8_t* no_eos_out, hipStream_t stream) {
+  if (bs < 0 || L < 0 || bs > 0x7fffffffLL) return AREAL_ERR_BAD_ARG;
+  if (estimator < 1 || estimator > 3) return AREAL_ERR_BAD_ARG;
+  if (bs == 0) return AREAL_OK;
+  if (L == 0) return AREAL_ERR_BAD_ARG;
+  if (!loss_mask || !attn_mask || !logp || !reward_score || !lm_out || !old_out || !kl_out ||
+      !tot_out || !seqlens_out || !no_eos_out)
+    return AREAL_ERR_BAD_ARG;
+  PrepArgs a{loss_mask, attn_mask, logp, ref_logp, reward_score, L, roll_logp, estimator,
+             apply_clamp, mask_no_eos_with_zero, ref_in_place, kl_ctl, lm_out, old_out, kl_out,
+             gkl_out, outcome_out, tot_out, seqlens_out, no_eos_out};
+  hipLaunchKernelGGL(adv_prep_kernel, dim3((unsigned)bs), dim3(NORM_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

@@ -465,7 +465,6 @@ def compute_advantages(
         kl_estimator = KLEstimator("k1")
     bs = data["input_ids"].shape[0]
     dev = data["input_ids"].device
-    batch_indices = torch.arange(bs, device=dev, dtype=torch.long)
 
     if overlong_reward_penalty:
         assert overlong_tokens is not None
@@ -482,8 +481,6 @@ def compute_advantages(
     if reward_norm is not None:
         reward_score = reward_norm(reward_score, group_sizes=group_sizes)
 
-    loss_mask = torch.roll(data["loss_mask"].float(), shifts=-1, dims=-1)
-
     # structural turn ids follow the same next-token convention as the mask and the log-probs
     turn_ids = data.get("turn_ids")
     if turn_ids is not None:
@@ -495,41 +492,78 @@ def compute_advantages(
             "include 'turn_ids'."
         )
 
-    if not use_decoupled_loss and recompute_logprob:
-        prox = data["prox_logp"]
-        if prox is None:
+    recompute = not use_decoupled_loss and recompute_logprob
+    if recompute:
+        logp_src = data["prox_logp"]
+        if logp_src is None:
             raise ValueError(
                 "prox_logp is None but recompute_logprob=True. "
                 "This indicates compute_logp() was skipped incorrectly."
             )
-        old_logp = data["logprobs"] = prox
     else:
-        old_logp = torch.roll(data["logprobs"], shifts=-1, dims=-1)
-        if not use_decoupled_loss:
-            data["prox_logp"] = old_logp
-    ref_logp = data.get("ref_logp")
-    if ref_logp is None:
-        ref_logp = torch.zeros_like(old_logp)
-    ref_logp = ref_logp * loss_mask
-    old_logp = old_logp * loss_mask
+        logp_src = data["logprobs"]
+    # One pass (areal_advantage_prep) instead of the reference's chain of tensor ops
+    # (actor.py:215-283): rolled float mask, masked old / reference log-probs, KL rewards, their
+    # copy zeroed after EOS, the outcome reward at the second-to-last token, and their sum. The
+    # reference's in-place updates are kept: `old_logp *= loss_mask` also masks the tensor that
+    # prox_logp names (and, in the recompute branch, the caller's prox_logp itself), and
+    # `ref_logp *= loss_mask` masks the caller's ref_logp.
+    lib = _lib.load()
+    _lib.require_gpu(logp_src, data["loss_mask"], data["attention_mask"])
+    L = logp_src.shape[-1]
 
-    attn_mask = data["attention_mask"]
-    seqlens = attn_mask.sum(-1).long()
-    seq_no_eos_mask = seqlens == attn_mask.shape[1]
-    rewards = -kl_ctl * kl_estimator(old_logp, ref_logp)
-    kl_rewards = rewards.clone()
-    rewards[batch_indices, seqlens - 1] = 0
-    gae_kl_rewards = rewards.clone()
-    indices = torch.clip(seqlens - 2, min=0)
-    gae_outcome_rewards = torch.zeros_like(rewards)
-    if mask_no_eos_with_zero:
-        gae_outcome_rewards[batch_indices, indices] = torch.where(
-            seq_no_eos_mask, torch.zeros_like(reward_score), reward_score
-        )
-    else:
-        gae_outcome_rewards[batch_indices, indices] = reward_score
+    def as_bytes(t):
+        t = t.reshape(bs, L)
+        t = t if t.dtype == torch.bool else t != 0
+        return t.contiguous().view(torch.uint8)
+
+    def in_place_ok(t):
+        return t.dtype == torch.float32 and t.is_contiguous() and not t.requires_grad
+
+    f32 = dict(dtype=torch.float32, device=dev)
+    logp_in = logp_src.detach().reshape(bs, L)
+    if not in_place_ok(logp_in):
+        logp_in = logp_in.float().contiguous()
+    old_logp = logp_in if (recompute and in_place_ok(logp_src)) else torch.empty((bs, L), **f32)
+    ref_src = data.get("ref_logp")
+    ref_in = None
+    ref_in_place = False
+    if ref_src is not None:
+        ref_in_place = in_place_ok(ref_src)
+        ref_in = ref_src.reshape(bs, L) if ref_in_place else ref_src.detach().float().contiguous().reshape(bs, L)
+    turn_mode = gae_timestep_unit == "turn"
+    loss_mask = torch.empty((bs, L), **f32)
+    kl_rewards = torch.empty((bs, L), **f32)
+    tot_rewards = torch.empty((bs, L), **f32)
+    gae_kl_rewards = torch.empty((bs, L), **f32) if turn_mode else None
+    gae_outcome_rewards = torch.empty((bs, L), **f32) if turn_mode else None
+    seqlens = torch.empty(bs, dtype=torch.int64, device=dev)
+    seq_no_eos_mask = torch.empty(bs, dtype=torch.bool, device=dev)
+    if getattr(kl_estimator, "kl_estimator", None) not in ("k1", "k2", "k3"):
+        raise TypeError("kl_estimator must be a KLEstimator (k1, k2 or k3)")
+    est = {"k1": 1, "k2": 2, "k3": 3}[kl_estimator.kl_estimator]
+    # temporaries are named so that they outlive the launch (a freed block is handed to the next
+    # allocation at once)
+    lm_bytes, am_bytes = as_bytes(data["loss_mask"]), as_bytes(data["attention_mask"])
+    score_f = reward_score.float().contiguous()
+    rc = lib.areal_advantage_prep(
+        _lib.ptr(lm_bytes), _lib.ptr(am_bytes),
+        _lib.ptr(logp_in), _lib.ptr(ref_in), _lib.ptr(score_f), bs, L,
+        0 if recompute else 1, est, int(bool(kl_estimator.apply_clamp)), int(bool(mask_no_eos_with_zero)),
+        int(ref_in_place), float(kl_ctl), _lib.ptr(loss_mask), _lib.ptr(old_logp), _lib.ptr(kl_rewards),
+        _lib.ptr(gae_kl_rewards), _lib.ptr(gae_outcome_rewards), _lib.ptr(tot_rewards),
+        _lib.ptr(seqlens), _lib.ptr(seq_no_eos_mask), _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_advantage_prep")
+    old_logp = old_logp.view(logp_src.shape)
+    if recompute:
+        data["logprobs"] = old_logp
+        if old_logp.data_ptr() == logp_src.data_ptr():
+            data["prox_logp"] = old_logp
+    elif not use_decoupled_loss:
+        data["prox_logp"] = old_logp
     # turn mode keeps the token KL as a local actor penalty instead of summing it into turns
-    rewards = gae_outcome_rewards if gae_timestep_unit == "turn" else gae_kl_rewards + gae_outcome_rewards
+    rewards = gae_outcome_rewards if turn_mode else tot_rewards
 
     values = data["values"] if "values" in data else torch.zeros_like(rewards)
     if gae_lambda_fn is not None:
@@ -564,7 +598,7 @@ def compute_advantages(
 
     data["advantages"] = advantages
     data["kl_rewards"] = kl_rewards
-    data["tot_rewards"] = gae_kl_rewards + gae_outcome_rewards
+    data["tot_rewards"] = tot_rewards
     data["loss_mask"] = loss_mask
     data["logprobs"] = old_logp
     return data

@@ -156,7 +156,25 @@ def hbm_rooflines(dev):
     no_eos = torch.zeros(1024, dtype=torch.bool, device=dev)
     add("gae_owned_kernel", "config 3 padded form: [1024, 8192] slots, 20 B/slot",
         20 * rp.numel(), timed(lambda: _compute_token_level_gae(rp, vp, mp, no_eos, 1.0, 0.95)))
-    del rp, vp, mp
+    # the whole advantage step on that padded batch: reward shaping (one pass), GAE, group
+    # normalisation of rewards and advantages
+    from areal_amd.data import KLEstimator
+    from areal_amd.ppo.actor import compute_advantages
+
+    attn = pos < lens.to(dev)[:, None]
+    adv_data = dict(input_ids=torch.zeros(1024, 8192, dtype=torch.long, device=dev), attention_mask=attn,
+                    loss_mask=(pos >= (lens.to(dev) // 4)[:, None]) & attn,
+                    logprobs=torch.randn(1024, 8192, device=dev) * 0.1 - 1,
+                    ref_logp=torch.randn(1024, 8192, device=dev) * 0.1 - 1, values=vp,
+                    rewards=(torch.rand(1024, device=dev) > 0.5).float())
+    gnorm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
+    add("adv_prep_kernel + gae_owned_kernel + norm kernels (compute_advantages, API level)",
+        "config 3 padded form: [1024, 8192], KL-shaped rewards, GAE, group normalisation; "
+        "26 + 20 + 20 B/slot",
+        66 * rp.numel(),
+        timed(lambda: compute_advantages(dict(adv_data), kl_ctl=0.01, kl_estimator=KLEstimator("k1"),
+                                         reward_norm=gnorm, adv_norm=gnorm, discount=1.0, gae_lambda=0.95)))
+    del rp, vp, mp, adv_data
     x = torch.randn(1024, 1600, device=dev)
     mk = (torch.rand(1024, 1600, device=dev) > 0.25).float()
     norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))

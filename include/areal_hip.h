@@ -293,6 +293,22 @@ size_t areal_masked_norm_workspace_bytes(int64_t n);
 int areal_masked_norm(const float* x, const float* mask, int64_t n, int unbiased, double eps,
                       float* out, void* workspace, size_t workspace_bytes, areal_stream_t stream);
 
+/* Reward shaping in front of GAE (PPOActor.compute_advantages, areal/trainer/ppo/actor.py:224-283)
+ * on a padded [bs, L] batch, one pass instead of the reference's elementwise tensor ops: rolled
+ * float loss mask, masked old log-probs, KL rewards by the k1/k2/k3 estimator
+ * (areal/utils/data.py:1662-1698; estimator = 1, 2, 3), their copy zeroed at the last token, the
+ * outcome reward placed at max(seqlen - 2, 0), and their sum; per row the sequence length (sum of
+ * attn_mask) and whether the row is full (no EOS). loss_mask / attn_mask are bytes; ref_logp,
+ * gkl_out, outcome_out may be NULL. roll_logp = 0 takes logp as already aligned (the
+ * recompute_logprob branch, actor.py:246-253) and then old_out may be logp itself; ref_in_place
+ * writes the masked ref_logp back, as the reference's in-place `ref_logp *= loss_mask` does. */
+int areal_advantage_prep(const uint8_t* loss_mask, const uint8_t* attn_mask, const float* logp,
+                         float* ref_logp, const float* reward_score, int64_t bs, int64_t L,
+                         int roll_logp, int estimator, int apply_clamp, int mask_no_eos_with_zero,
+                         int ref_in_place, float kl_ctl, float* lm_out, float* old_out,
+                         float* kl_out, float* gkl_out, float* outcome_out, float* tot_out,
+                         int64_t* seqlens_out, uint8_t* no_eos_out, areal_stream_t stream);
+
 /* masked_normalization with dim = the trailing dimensions (areal/utils/functional/functional.py:16-53,
  * the `dim` argument): x, mask (NULL allowed) and out are [rows, cols]; every row is whitened with
  * its own masked mean and variance. */

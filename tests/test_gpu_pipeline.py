@@ -66,6 +66,60 @@ def test_compute_advantages_matches_oracle_composition(dev):
     assert torch.equal(out["logprobs"].cpu(), old)
 
 
+@pytest.mark.parametrize("est", ["k1", "k2", "k3"])
+@pytest.mark.parametrize("recompute,with_ref,no_eos_zero", [(False, True, False), (True, True, True), (False, False, True)])
+def test_reward_shaping_kernel_matches_oracle(dev, est, recompute, with_ref, no_eos_zero):
+    """compute_advantages' single-pass reward shaping (areal_advantage_prep) against the oracle's
+    restatement of the reference's tensor ops: same operations in the same order, so everything
+    but the k3 exponential is bit-identical; the reference's in-place updates of prox_logp and
+    ref_logp are reproduced."""
+    from oracle import advantages as ADV
+
+    g = torch.Generator().manual_seed(11)
+    bs, Lw = 9, 130
+    lens = torch.randint(1, Lw + 1, (bs,), generator=g)
+    lens[0], lens[1], lens[2] = Lw, 0, 1  # full row (no EOS), empty row, one token
+    attn = torch.arange(Lw)[None] < lens[:, None]
+    loss_mask = (torch.arange(Lw)[None] >= (lens // 3)[:, None]) & attn
+    logp = -torch.rand(bs, Lw, generator=g) * 3
+    ref = -torch.rand(bs, Lw, generator=g) * 3 if with_ref else None
+    rewards = torch.randn(bs, generator=g)
+    kl_ctl = 0.2
+    want = ADV.shape_rewards(loss_mask, attn, logp, ref, rewards, kl_ctl, est, True, no_eos_zero,
+                             roll_logp=not recompute)
+    data = dict(input_ids=torch.zeros(bs, Lw, dtype=torch.long, device=dev), attention_mask=attn.to(dev),
+                loss_mask=loss_mask.to(dev), rewards=rewards.to(dev))
+    if recompute:
+        data["prox_logp"] = logp.to(dev)
+        data["logprobs"] = torch.zeros(bs, Lw, device=dev)  # the inference engine's, overwritten
+    else:
+        data["logprobs"] = logp.to(dev)
+    if with_ref:
+        data["ref_logp"] = ref.to(dev)
+    ref_given = data.get("ref_logp")
+    prox_given = data.get("prox_logp")
+    out = compute_advantages(data, kl_ctl=kl_ctl, kl_estimator=KLEstimator(est), discount=1.0, gae_lambda=1.0,
+                             mask_no_eos_with_zero=no_eos_zero, recompute_logprob=recompute, reward_clip=100.0)
+    assert torch.equal(out["loss_mask"].cpu(), want["loss_mask"])
+    assert torch.equal(out["logprobs"].cpu(), want["old_logp"])
+    if est == "k3":
+        torch.testing.assert_close(out["kl_rewards"].cpu(), want["kl_rewards"], rtol=1e-6, atol=1e-7)
+        torch.testing.assert_close(out["tot_rewards"].cpu(), want["tot_rewards"], rtol=1e-6, atol=1e-7)
+    else:
+        assert torch.equal(out["kl_rewards"].cpu(), want["kl_rewards"])
+        assert torch.equal(out["tot_rewards"].cpu(), want["tot_rewards"])
+    # in-place semantics of the reference (actor.py:236-246): prox_logp names the masked log-probs
+    assert out["prox_logp"] is out["logprobs"]
+    if recompute:
+        assert out["logprobs"].data_ptr() == prox_given.data_ptr()
+    if with_ref:
+        assert torch.equal(ref_given.cpu(), want["ref_logp"])  # masked in place
+    # GAE with lambda = discount = 1 and zero values: advantage = suffix sum of the shaped rewards
+    adv_want, _ = G.gae_padded(want["tot_rewards"], torch.zeros(bs, Lw), want["loss_mask"],
+                               want["seq_no_eos_mask"], 1.0, 1.0)
+    torch.testing.assert_close(out["advantages"].cpu(), adv_want, rtol=1e-5, atol=1e-5)
+
+
 def test_engine_loss_step_matches_oracle(dev):
     """Label roll, pad trim, loss scaling and the fused kernels together (config-1-like shape)."""
     g = torch.Generator().manual_seed(1)

@@ -248,3 +248,50 @@ def test_turn_level_gae_with_one_token_turns_is_token_level_gae():
     a, _ = G.gae_turn_level(r, v, m, ids, ne, 0.9, 0.8)
     want, _ = G.gae_padded(r, v, m, ne, 0.9, 0.8)
     torch.testing.assert_close(a, want * m, rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- reward shaping before GAE
+def test_kl_estimators_closed_forms():
+    from oracle import advantages as ADV
+
+    a = torch.tensor([-1.0, -2.0, -0.5, -30.0])
+    b = torch.tensor([-1.5, -1.0, -0.5, -1.0])
+    d = a - b  # 0.5, -1.0, 0.0, -29.0
+    assert torch.equal(ADV.approx_kl(a, b, "k1"), torch.tensor([0.5, -1.0, 0.0, -10.0]))
+    assert torch.equal(ADV.approx_kl(a, b, "k1", apply_clamp=False), d)
+    assert torch.equal(ADV.approx_kl(a, b, "k2"), torch.tensor([0.125, 0.5, 0.0, 10.0]))
+    k3 = ADV.approx_kl(a, b, "k3", apply_clamp=False)
+    want = torch.tensor([math.exp(-0.5) - 1 + 0.5, math.e - 2.0, 0.0, math.exp(29.0) - 1 - 29.0])
+    torch.testing.assert_close(k3, want, rtol=1e-6, atol=1e-7)
+    with pytest.raises(ValueError, match="Invalid KL estimator"):
+        ADV.approx_kl(a, b, "k4")
+
+
+def test_shape_rewards_hand_computed():
+    from oracle import advantages as ADV
+
+    # row 0: 4 tokens then padding; row 1: full (no EOS); row 2: empty
+    attn = torch.tensor([[1, 1, 1, 1, 0], [1, 1, 1, 1, 1], [0, 0, 0, 0, 0]])
+    loss_mask = torch.tensor([[0, 1, 1, 1, 0], [0, 0, 1, 1, 1], [0, 0, 0, 0, 0]])
+    logp = torch.tensor([[-1.0, -2.0, -3.0, -4.0, -5.0]] * 3)
+    ref = torch.tensor([[-1.0, -1.0, -1.0, -1.0, -1.0]] * 3)
+    score = torch.tensor([2.0, 3.0, 4.0])
+    out = ADV.shape_rewards(loss_mask, attn, logp, ref, score, kl_ctl=0.5)
+    # rolled mask: row 0 -> [1,1,1,0,0]; row 1 -> [0,1,1,1,0]
+    assert out["loss_mask"].tolist() == [[1, 1, 1, 0, 0], [0, 1, 1, 1, 0], [0, 0, 0, 0, 0]]
+    # old = roll(logp) * mask = [-2,-3,-4,0,0]; ref * mask = [-1,-1,-1,0,0]; kl = -0.5 * (old - ref)
+    assert out["old_logp"][0].tolist() == [-2.0, -3.0, -4.0, 0.0, 0.0]
+    assert out["kl_rewards"][0].tolist() == [0.5, 1.0, 1.5, 0.0, 0.0]
+    # zero at seqlen - 1 = 3 (already 0), outcome at seqlen - 2 = 2
+    assert out["tot_rewards"][0].tolist() == [0.5, 1.0, 3.5, 0.0, 0.0]
+    # row 1: kl = [0, 1.0, 1.5, 2.0, 0]; zero at 4; outcome 3.0 at 3
+    assert out["tot_rewards"][1].tolist() == [0.0, 1.0, 1.5, 5.0, 0.0]
+    assert out["seq_no_eos_mask"].tolist() == [False, True, False]
+    # empty row: index -1 zeroes the last slot, the outcome lands at 0
+    assert out["tot_rewards"][2].tolist() == [4.0, 0.0, 0.0, 0.0, 0.0]
+    out = ADV.shape_rewards(loss_mask, attn, logp, ref, score, kl_ctl=0.5, mask_no_eos_with_zero=True)
+    assert out["tot_rewards"][1].tolist() == [0.0, 1.0, 1.5, 2.0, 0.0]  # truncated row: no outcome
+    out = ADV.shape_rewards(loss_mask, attn, logp, None, score, kl_ctl=0.5, roll_logp=False)
+    assert out["old_logp"][0].tolist() == [-1.0, -2.0, -3.0, 0.0, 0.0]  # not rolled, no reference
+    assert out["kl_rewards"][0].tolist() == [0.5, 1.0, 1.5, 0.0, 0.0]
+
