@@ -772,6 +772,25 @@ struct PrepArgs {
   uint8_t* no_eos_out;       // [bs]
 };
 
+DEVI void adv_prep_token(const PrepArgs& a, float lm, float lp, float rf_in, bool has_ref, bool at_end,
+                         bool at_out, float score, float neg_ctl, float& old, float& ref, float& kl,
+                         float& gkl, float& oc) {
+  old = lp * lm;
+  ref = has_ref ? rf_in * lm : 0.f * lm;
+  const float diff = old - ref;
+  float est;
+  if (a.estimator == 1) est = diff;
+  else if (a.estimator == 2) est = diff * diff / 2.0f;
+  else { const float neg = -diff; est = expf(neg) - 1.f - neg; }
+  if (a.apply_clamp) est = fminf(fmaxf(est, -10.f), 10.f);
+  kl = neg_ctl * est;
+  gkl = at_end ? 0.f : kl;
+  oc = at_out ? score : 0.f;
+}
+
+// VEC: L % 16 == 0 and every array 16-byte aligned: four tokens per thread and step, 16-byte
+// loads and stores (the rolled neighbour of a group's last token is one extra scalar load).
+template <bool VEC>
 __global__ __launch_bounds__(NORM_THREADS) void adv_prep_kernel(PrepArgs a) {
   __shared__ double smem[4];
   const int64_t b = blockIdx.x, L = a.L;
@@ -780,7 +799,19 @@ __global__ __launch_bounds__(NORM_THREADS) void adv_prep_kernel(PrepArgs a) {
   const float* lp = a.logp + b * L;
   float* rf = a.ref_logp ? a.ref_logp + b * L : nullptr;
   double cnt = 0.0;
-  for (int64_t t = threadIdx.x; t < L; t += blockDim.x) cnt += am[t] ? 1.0 : 0.0;
+  if (VEC) {
+    for (int64_t t = (int64_t)threadIdx.x * 16; t < L; t += (int64_t)blockDim.x * 16) {
+      const u32x4 w = *(const u32x4*)(am + t);
+      int c = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) c += ((w[i] >> (8 * k)) & 0xffu) ? 1 : 0;
+      cnt += (double)c;
+    }
+  } else {
+    for (int64_t t = threadIdx.x; t < L; t += blockDim.x) cnt += am[t] ? 1.0 : 0.0;
+  }
   const int64_t seqlen = (int64_t)block_sum_d(cnt, smem);
   const bool no_eos = seqlen == L;
   if (threadIdx.x == 0) { a.seqlens_out[b] = seqlen; a.no_eos_out[b] = no_eos ? 1 : 0; }
@@ -789,21 +820,44 @@ __global__ __launch_bounds__(NORM_THREADS) void adv_prep_kernel(PrepArgs a) {
   float score = a.reward_score[b];
   if (a.mask_no_eos_with_zero && no_eos) score = 0.f;
   const float neg_ctl = -a.kl_ctl;
+  const bool has_ref = rf != nullptr;
+  if (VEC) {
+    for (int64_t t = (int64_t)threadIdx.x * 4; t < L; t += (int64_t)blockDim.x * 4) {
+      const int64_t tn = t + 4 < L ? t + 4 : 0;  // the roll's neighbour of the group's last token
+      const uint32_t mw = *(const uint32_t*)(lmk + t);
+      const float lmv[4] = {((mw >> 8) & 0xffu) ? 1.f : 0.f, ((mw >> 16) & 0xffu) ? 1.f : 0.f,
+                            (mw >> 24) ? 1.f : 0.f, lmk[tn] ? 1.f : 0.f};
+      const f32x4 lv = *(const f32x4*)(lp + t);
+      const float lpv[4] = {a.roll_logp ? lv[1] : lv[0], a.roll_logp ? lv[2] : lv[1],
+                            a.roll_logp ? lv[3] : lv[2], a.roll_logp ? lp[tn] : lv[3]};
+      f32x4 rv = {0.f, 0.f, 0.f, 0.f};
+      if (has_ref) rv = *(const f32x4*)(rf + t);
+      f32x4 o_lm, o_old, o_ref, o_kl, o_gkl, o_oc, o_tot;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float old, ref, kl, gkl, oc;
+        adv_prep_token(a, lmv[i], lpv[i], rv[i], has_ref, t + i == t_end, t + i == t_out, score, neg_ctl,
+                       old, ref, kl, gkl, oc);
+        o_lm[i] = lmv[i]; o_old[i] = old; o_ref[i] = ref; o_kl[i] = kl; o_gkl[i] = gkl; o_oc[i] = oc;
+        o_tot[i] = gkl + oc;
+      }
+      if (has_ref && a.ref_in_place) *(f32x4*)(rf + t) = o_ref;
+      *(f32x4*)(a.lm_out + b * L + t) = o_lm;
+      *(f32x4*)(a.old_out + b * L + t) = o_old;
+      *(f32x4*)(a.kl_out + b * L + t) = o_kl;
+      if (a.gkl_out) *(f32x4*)(a.gkl_out + b * L + t) = o_gkl;
+      if (a.outcome_out) *(f32x4*)(a.outcome_out + b * L + t) = o_oc;
+      *(f32x4*)(a.tot_out + b * L + t) = o_tot;
+    }
+    return;
+  }
   for (int64_t t = threadIdx.x; t < L; t += blockDim.x) {
     const int64_t tn = t + 1 < L ? t + 1 : 0;
     const float lm = lmk[tn] ? 1.f : 0.f;
-    const float old = (a.roll_logp ? lp[tn] : lp[t]) * lm;
-    const float ref = rf ? rf[t] * lm : 0.f * lm;
-    if (rf && a.ref_in_place) rf[t] = ref;
-    const float diff = old - ref;
-    float est;
-    if (a.estimator == 1) est = diff;
-    else if (a.estimator == 2) est = diff * diff / 2.0f;
-    else { const float neg = -diff; est = expf(neg) - 1.f - neg; }
-    if (a.apply_clamp) est = fminf(fmaxf(est, -10.f), 10.f);
-    const float kl = neg_ctl * est;
-    const float gkl = t == t_end ? 0.f : kl;
-    const float oc = t == t_out ? score : 0.f;
+    float old, ref, kl, gkl, oc;
+    adv_prep_token(a, lm, a.roll_logp ? lp[tn] : lp[t], has_ref ? rf[t] : 0.f, has_ref, t == t_end,
+                   t == t_out, score, neg_ctl, old, ref, kl, gkl, oc);
+    if (has_ref && a.ref_in_place) rf[t] = ref;
     a.lm_out[b * L + t] = lm;
     a.old_out[b * L + t] = old;
     a.kl_out[b * L + t] = kl;
@@ -1288,7 +1342,12 @@ int areal_advantage_prep(const uint8_t* loss_mask, const uint8_t* attn_mask, con
   PrepArgs a{loss_mask, attn_mask, logp, ref_logp, reward_score, L, roll_logp, estimator,
              apply_clamp, mask_no_eos_with_zero, ref_in_place, kl_ctl, lm_out, old_out, kl_out,
              gkl_out, outcome_out, tot_out, seqlens_out, no_eos_out};
-  hipLaunchKernelGGL(adv_prep_kernel, dim3((unsigned)bs), dim3(NORM_THREADS), 0, stream, a);
+  auto al16 = [](const void* q) { return q == nullptr || ((uintptr_t)q & 15) == 0; };
+  const bool vec = L % 16 == 0 && al16(loss_mask) && al16(attn_mask) && al16(logp) && al16(ref_logp) &&
+                   al16(lm_out) && al16(old_out) && al16(kl_out) && al16(gkl_out) && al16(outcome_out) &&
+                   al16(tot_out);
+  if (vec) hipLaunchKernelGGL(adv_prep_kernel<true>, dim3((unsigned)bs), dim3(NORM_THREADS), 0, stream, a);
+  else hipLaunchKernelGGL(adv_prep_kernel<false>, dim3((unsigned)bs), dim3(NORM_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

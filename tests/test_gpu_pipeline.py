@@ -68,7 +68,8 @@ def test_compute_advantages_matches_oracle_composition(dev):
 
 @pytest.mark.parametrize("est", ["k1", "k2", "k3"])
 @pytest.mark.parametrize("recompute,with_ref,no_eos_zero", [(False, True, False), (True, True, True), (False, False, True)])
-def test_reward_shaping_kernel_matches_oracle(dev, est, recompute, with_ref, no_eos_zero):
+@pytest.mark.parametrize("Lw", [130, 144])  # scalar path, and the 16-byte path (L a multiple of 16)
+def test_reward_shaping_kernel_matches_oracle(dev, est, recompute, with_ref, no_eos_zero, Lw):
     """compute_advantages' single-pass reward shaping (areal_advantage_prep) against the oracle's
     restatement of the reference's tensor ops: same operations in the same order, so everything
     but the k3 exponential is bit-identical; the reference's in-place updates of prox_logp and
@@ -76,7 +77,7 @@ def test_reward_shaping_kernel_matches_oracle(dev, est, recompute, with_ref, no_
     from oracle import advantages as ADV
 
     g = torch.Generator().manual_seed(11)
-    bs, Lw = 9, 130
+    bs = 9
     lens = torch.randint(1, Lw + 1, (bs,), generator=g)
     lens[0], lens[1], lens[2] = Lw, 0, 1  # full row (no EOS), empty row, one token
     attn = torch.arange(Lw)[None] < lens[:, None]
