@@ -296,6 +296,7 @@ __global__ __launch_bounds__(AUX_THREADS) void dpo_seq_grad_kernel(const double*
 // order. Ties at the cut value are kept in index order.
 // ---------------------------------------------------------------------------------------
 constexpr int M2_BLOCKS = 512;
+constexpr int M2_FOLD = 32;  // partial histograms summed per block of m2_fold_kernel
 struct M2State {
   unsigned int prefix;          // decided high bits of the cut value
   int all_kept;                 // every token kept: nothing to cut
@@ -336,17 +337,50 @@ __global__ __launch_bounds__(AUX_THREADS) void m2_hist_kernel(const float* old, 
   part_cnt[(int64_t)blockIdx.x * 256 + threadIdx.x] = h_cnt[threadIdx.x];
   part_sum[(int64_t)blockIdx.x * 256 + threadIdx.x] = h_sum[threadIdx.x];
 }
-__global__ __launch_bounds__(AUX_THREADS) void m2_select_kernel(const unsigned int* part_cnt,
-                                                                const double* part_sum, int nparts,
-                                                                int shift, double thr, M2State* st) {
-  __shared__ unsigned long long cnt[256];
-  __shared__ double sum[256];
+// Sums M2_FOLD consecutive partial histograms into one (fixed order), so that the single block of
+// m2_select_kernel reads nparts / M2_FOLD of them: one CU cannot stream all the partials fast.
+__global__ __launch_bounds__(256) void m2_fold_kernel(const unsigned int* part_cnt, const double* part_sum,
+                                                       int nparts, unsigned long long* fold_cnt,
+                                                       double* fold_sum) {
+  const int i0 = blockIdx.x * M2_FOLD;
+  const int i1 = i0 + M2_FOLD < nparts ? i0 + M2_FOLD : nparts;
   unsigned long long c = 0; double s = 0.0;
-  for (int i = 0; i < nparts; ++i) {
+#pragma unroll 8
+  for (int i = i0; i < i1; ++i) {
     c += part_cnt[(int64_t)i * 256 + threadIdx.x];
     s += part_sum[(int64_t)i * 256 + threadIdx.x];
   }
-  cnt[threadIdx.x] = c; sum[threadIdx.x] = s;
+  fold_cnt[(int64_t)blockIdx.x * 256 + threadIdx.x] = c;
+  fold_sum[(int64_t)blockIdx.x * 256 + threadIdx.x] = s;
+}
+// One block of M2_SELECT_THREADS: bin = thread % 256, and the partial histograms are split over
+// the thread / 256 lanes of a bin, whose sums meet in LDS in a fixed order.
+constexpr int M2_SELECT_THREADS = 1024;
+__global__ __launch_bounds__(M2_SELECT_THREADS) void m2_select_kernel(const unsigned long long* part_cnt,
+                                                                      const double* part_sum, int nparts,
+                                                                      int shift, double thr, M2State* st) {
+  constexpr int LANES = M2_SELECT_THREADS / 256;
+  __shared__ unsigned long long cnt_l[LANES][256];
+  __shared__ double sum_l[LANES][256];
+  __shared__ unsigned long long cnt[256];
+  __shared__ double sum[256];
+  {
+    const int bin = threadIdx.x & 255, q = threadIdx.x >> 8;
+    unsigned long long c = 0; double s = 0.0;
+#pragma unroll 8
+    for (int i = q; i < nparts; i += LANES) {
+      c += part_cnt[(int64_t)i * 256 + bin];
+      s += part_sum[(int64_t)i * 256 + bin];
+    }
+    cnt_l[q][bin] = c; sum_l[q][bin] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < 256) {
+    unsigned long long c = 0; double s = 0.0;
+#pragma unroll
+    for (int q = 0; q < LANES; ++q) { c += cnt_l[q][threadIdx.x]; s += sum_l[q][threadIdx.x]; }
+    cnt[threadIdx.x] = c; sum[threadIdx.x] = s;
+  }
   __syncthreads();
   if (threadIdx.x != 0 || st->all_kept) return;
   unsigned long long C = st->kept; double S = st->kept_sum;
@@ -606,6 +640,7 @@ int areal_dpo_seq_logps_grad(const double* grad_seq, const uint8_t* shifted_mask
 size_t areal_m2po_mask_workspace_bytes(int64_t n_tokens) {
   (void)n_tokens;
   return sizeof(M2State) + (size_t)M2_BLOCKS * 256 * (sizeof(unsigned int) + sizeof(double)) +
+         (size_t)(M2_BLOCKS / M2_FOLD) * 256 * (sizeof(unsigned long long) + sizeof(double)) +
          (size_t)M2_BLOCKS * sizeof(unsigned long long) + 1024;
 }
 
@@ -626,6 +661,8 @@ int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
   double* part_sum = (double*)(wp + 256);
   unsigned int* part_cnt = (unsigned int*)(part_sum + (size_t)M2_BLOCKS * 256);
   unsigned long long* block_eq = (unsigned long long*)(part_cnt + (size_t)M2_BLOCKS * 256);
+  double* fold_sum = (double*)(block_eq + M2_BLOCKS);
+  unsigned long long* fold_cnt = (unsigned long long*)(fold_sum + (size_t)(M2_BLOCKS / M2_FOLD) * 256);
   int blocks = (int)ceil_div_i64(n_tokens, AUX_THREADS * 4);
   if (blocks > M2_BLOCKS) blocks = M2_BLOCKS;
   if (blocks < 1) blocks = 1;
@@ -635,8 +672,12 @@ int areal_m2po_mask(const float* old_logprobs, const float* proximal_logprobs,
     hipLaunchKernelGGL(m2_hist_kernel, dim3(blocks), dim3(AUX_THREADS), 0, stream, old_logprobs,
                        proximal_logprobs, loss_mask, n_tokens, shift, st, part_cnt, part_sum);
     AREAL_CHECK_LAUNCH();
-    hipLaunchKernelGGL(m2_select_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, part_cnt, part_sum,
-                       blocks, shift, (double)m2_threshold, st);
+    const int nfold = (blocks + M2_FOLD - 1) / M2_FOLD;
+    hipLaunchKernelGGL(m2_fold_kernel, dim3(nfold), dim3(256), 0, stream, part_cnt, part_sum, blocks,
+                       fold_cnt, fold_sum);
+    AREAL_CHECK_LAUNCH();
+    hipLaunchKernelGGL(m2_select_kernel, dim3(1), dim3(M2_SELECT_THREADS), 0, stream, fold_cnt, fold_sum,
+                       nfold, shift, (double)m2_threshold, st);
     AREAL_CHECK_LAUNCH();
   }
   const int64_t per_block = ceil_div_i64(n_tokens, blocks);

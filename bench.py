@@ -225,6 +225,57 @@ def hbm_rooflines(dev):
 
     add("loss_token+loss_finalize+loss_grad_scale", "PPO + IcePop, 4 Mi tokens, fwd+bwd kernels through the C ABI, "
         "47 B/token + 8 B/token grad scale", 55 * Tl, timed(loss_kernels, iters=50))
+    # kernels of the steps either side of the loss (API level: each call includes its own host work)
+    from areal_amd.functional import ppo_critic_loss_fn, sapo_loss_fn
+    from areal_amd.packing import pack_tensor_dict
+    from areal_amd.ppo.actor import _apply_m2po_masking
+    from areal_amd.ppo.gae import _compute_turn_level_gae
+    from areal_amd.stats import masked_stats
+
+    def sapo_step():
+        lp.grad = None
+        loss, _ = sapo_loss_fn(lp, old, adv, 1.0, 1.05, mask)
+        loss.backward()
+
+    add("sapo_token_kernel + backward (API level)", "SAPO, 4 Mi tokens, 7 output tensors, 41 B/token + 8 B/token grad scale",
+        49 * Tl, timed(sapo_step))
+    val = torch.randn(Tl, device=dev).requires_grad_(True)
+    oldv, tgt = val.detach() + 0.1 * torch.randn(Tl, device=dev), torch.randn(Tl, device=dev)
+
+    def critic_step():
+        val.grad = None
+        loss, _ = ppo_critic_loss_fn(val, oldv, tgt, 0.2, mask)
+        loss.backward()
+
+    add("critic_token_kernel + backward (API level)", "clipped value loss, 4 Mi tokens, 22 B/token + 8 B/token grad scale",
+        30 * Tl, timed(critic_step))
+    add("m2_hist x4 + m2_select x4 + m2_tie_count + m2_apply (API level)",
+        "M2PO mask by radix select, 4 Mi tokens, 6 passes x 9 B/token",
+        54 * Tl, timed(lambda: _apply_m2po_masking(old, prox, mask, 0.04)))
+    stat_vals = {f"s{i}": (adv if i % 2 else prox) for i in range(24)}
+    stat_den = {f"s{i}": mask for i in range(24)}
+    add("stats_partial_kernel + stats_final_kernel (API level)",
+        "24 masked statistics (sum, count, min, max) over 4 Mi tokens, 5 B/token each",
+        24 * 5 * Tl, timed(lambda: masked_stats(stat_vals, stat_den)))
+    bsz, Lp = 1024, 8192
+    plens = torch.clamp((torch.randn(bsz, generator=g) + 7.0).exp().long(), 16, Lp).to(dev)
+    ppos = torch.arange(Lp, device=dev)[None, :]
+    pattn = ppos < plens[:, None]
+    pdata = dict(attention_mask=pattn, input_ids=torch.randint(0, 1000, (bsz, Lp), device=dev),
+                 loss_mask=pattn & (ppos >= (plens // 4)[:, None]), logprobs=torch.randn(bsz, Lp, device=dev),
+                 advantages=torch.randn(bsz, Lp, device=dev))
+    n_packed = int(plens.sum())
+    add("rowlens + cu_scan + pack_kernel (API level)",
+        f"pack_tensor_dict: [1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write",
+        2 * 25 * n_packed + bsz * Lp, timed(lambda: pack_tensor_dict(dict(pdata))))
+    turn_ids = (torch.cumsum((torch.rand(bsz, Lp, device=dev) < 0.002).int(), dim=1)).to(torch.int32)
+    tr = torch.zeros(bsz, Lp, device=dev)
+    tr[torch.arange(bsz, device=dev), (plens - 2).clamp(min=0)] = 1.0
+    tv, tm = torch.randn(bsz, Lp, device=dev), pdata["loss_mask"].float()
+    tne = torch.zeros(bsz, dtype=torch.bool, device=dev)
+    add("turn_gae_kernel (API level, with validation)", "turn-level GAE, [1024, 8192] slots, 2 x 16 B/slot read + 8 B/slot written",
+        40 * bsz * Lp, timed(lambda: _compute_turn_level_gae(tr, tv, tm, turn_ids, tne, 1.0, 0.95)))
+    del pdata, turn_ids, tr, tv, tm
     lg = torch.randn(4096, V_QWEN, device=dev).bfloat16()
     lab = torch.randint(0, V_QWEN, (4096,), device=dev)
     add("rows_fwd_kernel", "config 1: [4096, 151936] bf16 logits, logprob + entropy forward",
