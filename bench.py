@@ -102,6 +102,32 @@ def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int):
     return n / dt, dt
 
 
+def cpu_baseline_advantages(threads: int):
+    """The CPU oracle on BASELINE config 3 in full: the reference's padded GAE loop over
+    [1024, 8192] slots and the group normalisation of the advantages (groups of 16 rows)."""
+    import torch
+
+    from oracle import gae as ogae
+    from oracle import norm as onorm
+
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(2)
+    lens = torch.clamp((torch.randn(1024, generator=g) + 7.0).exp().long(), 16, 8192)
+    pos = torch.arange(8192)[None, :]
+    r = torch.zeros(1024, 8192)
+    r[torch.arange(1024), (lens - 2).clamp(min=0)] = 1.0
+    v = torch.randn(1024, 8192, generator=g)
+    m = ((pos >= (lens // 4)[:, None]) & (pos < (lens - 1)[:, None])).float()
+    no_eos = torch.zeros(1024, dtype=torch.bool)
+    t0 = time.perf_counter()
+    adv, _ = ogae.gae_padded(r, v, m, no_eos, 1.0, 0.95)
+    t1 = time.perf_counter()
+    onorm.normalization(adv, m, mean_level="group", std_level="group", group_size=16)
+    t2 = time.perf_counter()
+    return {"workload": "config 3 padded form in full: [1024, 8192] slots, PyTorch oracle",
+            "gae_ms": (t1 - t0) * 1e3, "group_norm_ms": (t2 - t1) * 1e3, "cores": threads, "kind": "port"}
+
+
 def hbm_rooflines(dev):
     """HBM-bound kernels of the path on their own workloads: algorithmic bytes / HIP-event time.
     GAE + group normalisation on BASELINE config 3 (1024 packed sequences, lognormal lengths),
@@ -358,11 +384,13 @@ def main() -> None:
     for _ in range(args.warmup):
         step(False)
     torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = step(True)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    peak_hbm_gb = torch.cuda.max_memory_allocated() / 1e9
     ms_per_step = wall * 1e3 / args.steps
     tokens_per_s = T * args.steps / wall
 
@@ -411,6 +439,7 @@ def main() -> None:
             "loss": "PPO clip eps=0.2, rejection sampling ratio in [0.5, 2.0] (token, mask)",
             "final_loss": float(loss.detach().item()),
             "backward": "saved bf16 exponentials" if saved else "recompute logits",
+            "peak_hbm_gb": peak_hbm_gb,
         },
         "pct_bf16_mfma_peak": 100.0 * (algo_flops / (ms_per_step * 1e-3) / 1e12) / PEAK_BF16_TFLOPS,
         "roofline": {
@@ -441,6 +470,8 @@ def main() -> None:
             "sample": f"{args.cpu_sample_tokens}-token slice at full vocabulary, fwd+bwd with the "
                       f"PyTorch oracle, {dt:.1f} s (rate is per token, so it scales linearly in T)",
         }
+        if not args.no_hbm_kernels:
+            result["cpu_baseline_advantages"] = cpu_baseline_advantages(threads)
     print(json.dumps(result))
 
 
