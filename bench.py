@@ -318,6 +318,8 @@ def main() -> None:
     ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true")
+    ap.add_argument("--no-library-gemm", action="store_true",
+                    help="skip timing torch.mm (the vendor library's bf16 GEMM) at the forward's shape")
     ap.add_argument("--recompute", action="store_true",
                     help="backward recomputes the logits (save_probs=False) instead of using the "
                          "bf16 exponentials kept by the forward")
@@ -405,6 +407,25 @@ def main() -> None:
     achieved = algo_flops / (gemm_ms * 1e-3) / 1e12
     fwd_tflops = 2.0 * T * H * V / (t_fwd / args.steps * 1e-3) / 1e12
 
+    # The vendor library's plain bf16 GEMM of the forward's shape on this same box, right after
+    # the timed steps: what a contraction without the softmax epilogue sustains here (boards are
+    # power-limited under this load, so the figure moves from box to box with the kernels').
+    lib_tflops = None
+    if not args.no_library_gemm:
+        with torch.no_grad():
+            hd, wt = hidden.detach(), weight.detach().t()
+            logits = torch.empty(T, V, dtype=torch.bfloat16, device=dev)
+            for _ in range(2):
+                torch.mm(hd, wt, out=logits)
+            a, c = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(5):
+                torch.mm(hd, wt, out=logits)
+            c.record()
+            torch.cuda.synchronize()
+            lib_tflops = 2.0 * T * H * V / (a.elapsed_time(c) / 5 * 1e-3) / 1e12
+            del logits
+
     # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
     # command (KiB per dispatch, scaled by the factors the same counters show for copy-like
     # kernels of known size, the operand-prep and the bf16 transpose: fetch x2.0, write x1.0). Only measured for the default
@@ -454,6 +475,7 @@ def main() -> None:
             "traffic": traffic,
             "traffic_bytes_per_launch": traffic_detail,
             "forward_only_tflops": fwd_tflops,
+            "library_gemm_same_box_tflops": lib_tflops,
             "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},
         },
