@@ -387,15 +387,24 @@ def test_config2_full_size_decoupled_ppo(dev):
     _check_lm_gradients(hidden, weight, labels, lp_cpu.grad.to(dev), h.grad, w.grad)
 
 
+def _config5_loss_inputs(T, g, dev):
+    """BASELINE config 5's packing (4 sequences of 32768 tokens) and loss inputs; sequence 1 is
+    far off-policy so that a sequence-level filter rejects exactly it."""
+    cu = torch.tensor([0, 32768, 65536, 98304, 131072], dtype=torch.int32)
+    seq_shift = torch.tensor([0.0, 2.0, 0.0, 0.0])
+    return cu, seq_shift
+
+
 def test_config5_full_size_cispo_sequence_rejection(dev):
-    """T=131072, H=5120: CISPO (eps 1.0 / 4.0) with sequence-level mean-ratio rejection (upper
-    5.0) over 128 packed sequences. The bf16 [T, V] buffer of the saved-exponentials mode is
-    39.8 GB, within the default limit; peak memory of the step stays under 64 GB."""
+    """T=131072, H=5120, 4 packed sequences of 32768 tokens: CISPO (eps 1.0 / 4.0) with
+    sequence-level mean-ratio rejection (upper 5.0). The bf16 [T, V] buffer of the
+    saved-exponentials mode is 39.8 GB, within the default limit; peak memory of the step stays
+    under 64 GB."""
     from areal_amd.functional import cispo_loss_fn
 
     T, H, V = 131072, 5120, 151936
     g, hidden, weight, labels = _make_lm_inputs(T, H, V, 4, dev)
-    cu = _segments(T, 128, g)
+    cu, seq_shift = _config5_loss_inputs(T, g, dev)
     h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
@@ -404,8 +413,6 @@ def test_config5_full_size_cispo_sequence_rejection(dev):
     assert out.logprobs.grad_fn.probs is not None  # saved mode fits the default limit
     lp = out.logprobs.detach()
     prox = lp + 0.2 * torch.randn(T, generator=g).to(dev)
-    # a few sequences far off-policy so that the sequence filter rejects some
-    seq_shift = (torch.rand(128, generator=g) < 0.1).float() * 2.0
     lens = (cu[1:] - cu[:-1]).long()
     old = prox - torch.repeat_interleave(seq_shift, lens).to(dev) + 0.05 * torch.randn(T, generator=g).to(dev)
     adv = torch.randn(T, generator=g).to(dev)
@@ -423,5 +430,196 @@ def test_config5_full_size_cispo_sequence_rejection(dev):
     lo.backward()
     torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-8)
     assert torch.equal(stat["behave_mask"].cpu(), so["behave_mask"])
-    assert 0.0 < stat["filtered_fraction"] < 0.5
+    # exactly the shifted sequence is rejected: a quarter of the valid tokens, up to mask noise
+    bm = stat["behave_mask"].cpu()
+    assert not bm[32768:65536].any() and bm[:32768].any() and bm[65536:].any()
+    assert 0.2 < stat["filtered_fraction"] < 0.3
     _check_lm_gradients(hidden, weight, labels, lp_cpu.grad.to(dev), h.grad, w.grad)
+
+
+@pytest.mark.parametrize("variant", ["cispo_seq_rejection", "gspo", "gspo_seq_rejection_max"])
+def test_config5_packing_loss_stage_on_32k_token_sequences(dev, variant):
+    """The loss stage alone on config 5's packing (4 x 32768 tokens): the block-per-sequence
+    reductions (sequence-level rejection aggregate, GSPO sequence ratio and mean advantage) run
+    over 32768-token sequences and are compared with the oracle."""
+    from areal_amd.functional import cispo_loss_fn
+
+    T = 131072
+    g = torch.Generator().manual_seed(4)
+    cu, seq_shift = _config5_loss_inputs(T, g, dev)
+    lens = (cu[1:] - cu[:-1]).long()
+    lp = -torch.rand(T, generator=g) * 3
+    prox = lp + 0.02 * torch.randn(T, generator=g)
+    old = prox - torch.repeat_interleave(seq_shift, lens) + 0.05 * torch.randn(T, generator=g)
+    adv = torch.randn(T, generator=g)
+    mask = torch.rand(T, generator=g) > 0.2
+    d = lambda t: t.to(dev)  # noqa: E731
+    lp_g = d(lp).requires_grad_(True)
+    lp_o = lp.clone().requires_grad_(True)
+    if variant == "cispo_seq_rejection":
+        rs = dict(level="sequence", action="mask", metric="ratio", agg="mean", upper=5.0)
+        lg, sg = cispo_loss_fn(lp_g, d(prox), d(adv), 1.0, d(mask), eps_clip_higher=4.0, old_logprobs=d(old),
+                               rejection_sampling=RejectionSamplingConfig(**rs), cu_seqlens=d(cu))
+        lo, so = O.cispo_loss(lp_o, prox, adv, 1.0, mask, eps_clip_higher=4.0, old_logprobs=old,
+                              rejection_sampling_cfg=rs, cu_seqlens=cu)
+    else:
+        rs = None
+        if variant == "gspo_seq_rejection_max":
+            rs = dict(level="sequence", action="mask", metric="kl_k2", agg="max", upper=1.5)
+        lg, sg = ppo_actor_loss_fn(lp_g, d(prox), d(old), d(adv), 0.2, d(mask), eps_clip_higher=0.28,
+                                   rejection_sampling=RejectionSamplingConfig(**rs) if rs else None,
+                                   importance_sampling_level="sequence", cu_seqlens=d(cu))
+        lo, so = O.ppo_actor_loss(lp_o, prox, old, adv, 0.2, mask, eps_clip_higher=0.28,
+                                  rejection_sampling_cfg=rs, importance_sampling_level="sequence", cu_seqlens=cu)
+    lg.backward()
+    lo.backward()
+    torch.testing.assert_close(lg.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-7)
+    assert torch.equal(sg["clip_mask"].cpu(), so["clip_mask"])
+    torch.testing.assert_close(sg["importance_weight"].cpu(), so["importance_weight"], rtol=1e-4, atol=1e-6)
+    if rs is not None:
+        assert torch.equal(sg["behave_mask"].cpu(), so["behave_mask"])
+        assert sg["filtered_fraction"] == pytest.approx(so["filtered_fraction"], abs=1e-12)
+        assert 0.0 < sg["filtered_fraction"] < 1.0
+    rel = (lp_g.grad.cpu() - lp_o.grad).norm() / lp_o.grad.norm()
+    assert rel < 1e-2, rel
+
+
+def test_config1_full_pipeline(dev):
+    """BASELINE config 1, every stage at its full size, against the oracle run in full on the CPU
+    (2.5 GB of fp32 logits): seed 0, hidden [4096, 896], 16 sequences of 64-512 tokens plus the
+    trailing pad segment, Bernoulli rewards normalised in 4 groups of 4, values 0 and
+    gamma = lambda = 1 (so every response token carries its sequence's normalised reward),
+    behaviour log-probs = policy log-probs + N(0, 0.05) (not decoupled: proximal = behaviour),
+    GRPO loss with eps_clip 0.2.  GPU route: compute_advantages -> pack_tensor_dict ->
+    pad_packed_tensor_dict -> compute_logprobs_and_loss -> backward."""
+    from areal_amd.packing import pack_tensor_dict, pad_packed_tensor_dict
+    from oracle import advantages as ADV
+    from oracle import packing as P
+
+    T, H, V, B = 4096, 896, 151936, 16
+    g = torch.Generator().manual_seed(0)
+    hidden = torch.randn(T, H, generator=g).bfloat16()
+    weight = torch.empty(V, H, dtype=torch.bfloat16)
+    for i in range(0, V, 32768):
+        n = min(32768, V - i)
+        weight[i:i + n] = (torch.randn(n, H, generator=g) * 0.02).bfloat16()
+    lens = torch.randint(64, 513, (B,), generator=g)
+    if int(lens.sum()) > T:
+        lens = torch.clamp((lens.double() * T / lens.sum()).floor().long(), min=64)
+    total = int(lens.sum())
+    pad = T - total
+    assert 0 < pad < T
+    Lmax = int(lens.max())
+    pos = torch.arange(Lmax)[None]
+    attn = pos < lens[:, None]
+    ids_padded = torch.randint(0, V, (B, Lmax), generator=g) * attn
+    loss_mask_padded = (pos >= (lens // 4)[:, None]) & attn
+    rewards = (torch.rand(B, generator=g) > 0.5).float()
+    rewards[0], rewards[1] = 1.0, 0.0  # no group is constant by accident in its first pair
+
+    # ---- the policy's log-probs of the packed, padded micro-batch: oracle in full on the CPU
+    packed_ids = torch.cat([ids_padded[b, : lens[b]] for b in range(B)] + [torch.zeros(pad, dtype=torch.long)])
+    labels = torch.roll(packed_ids, -1)
+    lp_o, ent_o, vmin_o, vmax_o, _, _ = L.lm_head_logprobs_entropy(hidden, weight, labels)
+
+    # rollout-convention log-probs of the padded batch: position i + 1 holds the log-prob of
+    # token i + 1, i.e. the label-aligned value of position i; compute_advantages rolls it back
+    old_packed = lp_o[:total] + 0.05 * torch.randn(total, generator=g)
+    cu_cpu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)])
+    logprobs_padded = torch.zeros(B, Lmax)
+    for b in range(B):
+        s0, e0 = int(cu_cpu[b]), int(cu_cpu[b + 1])
+        logprobs_padded[b, 1:e0 - s0] = old_packed[s0:e0 - 1]
+
+    # ---- advantages: GPU vs oracle composition (actor.py:178-323)
+    gnorm = dict(mean_level="group", std_level="group", group_size=4)
+    data = dict(input_ids=ids_padded.to(dev), attention_mask=attn.to(dev), loss_mask=loss_mask_padded.to(dev),
+                logprobs=logprobs_padded.to(dev), rewards=rewards.to(dev))
+    out = compute_advantages(data, kl_ctl=0.0, kl_estimator=KLEstimator("k1"), discount=1.0, gae_lambda=1.0,
+                             reward_norm=Normalization(NormConfig(**gnorm)))
+    score = N.normalization(rewards.clone(), None, **gnorm)
+    shaped = ADV.shape_rewards(loss_mask_padded, attn, logprobs_padded, None, score, 0.0, "k1", True, False)
+    adv_want, ret_want = G.gae_padded(shaped["tot_rewards"], torch.zeros(B, Lmax), shaped["loss_mask"],
+                                      shaped["seq_no_eos_mask"], 1.0, 1.0)
+    torch.testing.assert_close(out["advantages"].cpu(), adv_want, rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(out["returns"].cpu(), ret_want, rtol=1e-4, atol=1e-6)
+    assert torch.equal(out["loss_mask"].cpu(), shaped["loss_mask"])
+    assert torch.equal(out["logprobs"].cpu(), shaped["old_logp"])
+    # every response position of a sequence carries that sequence's normalised reward
+    m = shaped["loss_mask"].bool()
+    for b in (0, 5, 15):
+        torch.testing.assert_close(adv_want[b][m[b]], score[b].expand(int(m[b].sum())), rtol=1e-6, atol=1e-7)
+
+    # ---- pack and pad to 4096 tokens: GPU vs oracle
+    keys = ("input_ids", "attention_mask", "loss_mask", "logprobs", "advantages", "prox_logp")
+    packed_g = pack_tensor_dict({k: out[k] for k in keys})
+    cpu_batch = dict(input_ids=ids_padded, attention_mask=attn, loss_mask=shaped["loss_mask"],
+                     logprobs=shaped["old_logp"], advantages=adv_want, prox_logp=shaped["old_logp"])
+    packed_o = P.pack_tensor_dict(cpu_batch)
+    padded_g, pad_g, _, _ = pad_packed_tensor_dict(packed_g, T)
+    padded_o, pad_o, _, _ = P.pad_packed_tensor_dict(packed_o, T)
+    assert pad_g == pad_o == pad
+    assert padded_g["cu_seqlens"].tolist() == padded_o["cu_seqlens"].tolist() == cu_cpu.tolist() + [T]
+    for k in ("input_ids", "loss_mask", "logprobs", "advantages"):
+        torch.testing.assert_close(padded_g[k].cpu(), padded_o[k], rtol=1e-4, atol=1e-6)
+    assert torch.equal(padded_g["input_ids"].cpu(), packed_ids)
+
+    # ---- engine step: forward-only log-probs, then loss + backward
+    h = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    model_inputs = dict(input_ids=padded_g["input_ids"].unsqueeze(0))
+    lp_g0 = compute_logprobs(h, w, model_inputs, pad_length=pad)
+    assert (lp_g0.cpu() - lp_o[:total]).abs().max() < 2e-3
+    mb = dict(logprobs=packed_g["logprobs"], advantages=packed_g["advantages"], loss_mask=packed_g["loss_mask"],
+              prox_logp=packed_g["prox_logp"], cu_seqlens=packed_g["cu_seqlens"])
+    stats = {}
+    loss_fn = functools.partial(grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None, stats=stats)
+    weight_fn = lambda d: d["loss_mask"].count_nonzero()  # noqa: E731
+    loss = compute_logprobs_and_loss(h, w, model_inputs, mb, loss_fn, weight_fn,
+                                     total_loss_weight=weight_fn(mb).float(), pad_length=pad)
+    loss.backward()
+    lp_g = stats["new_logp"].cpu()
+    assert (lp_g - lp_o[:total]).abs().max() < 2e-3
+    assert (stats["entropy"].cpu() - ent_o[:total]).abs().max() < 2e-3
+    assert (stats["vocab_max_logits"].cpu() - vmax_o[:total]).abs().max() < 2e-3
+    assert (stats["vocab_min_logits"].cpu() - vmin_o[:total]).abs().max() < 2e-3
+
+    # the loss stage of the oracle on the GPU's log-probs: masks and counts bit-exact, loss 1e-4
+    mask_o = packed_o["loss_mask"].bool()
+    old_o, adv_o = packed_o["logprobs"], packed_o["advantages"]
+    lp_in = lp_g.clone().requires_grad_(True)
+    lo, so = O.ppo_actor_loss(lp_in, old_o, old_o, adv_o, 0.2, mask_o)
+    lo.backward()
+    ratio = torch.exp(lp_g - old_o)
+    guard = sum(int(((ratio - b).abs() <= 2 * (torch.nextafter(torch.tensor(b), torch.tensor(2.0)) - b)).sum())
+                for b in (torch.tensor(0.8).item(), torch.tensor(1.2).item()))
+    assert guard == 0, f"{guard} tokens within 2 ulp of a clip bound; pick another seed"
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-7)
+    assert torch.equal(stats["clipped_tokens"].cpu(), so["clip_mask"])
+    assert torch.equal(stats["n_valid_tokens"].cpu(), mask_o)
+    assert stats["scalar/n_valid_tokens"] == so["n_valid_tokens"] == float(mask_o.sum())
+    # N(0, 0.05) noise against eps_clip 0.2 is a 4-sigma event: (almost) nothing clips in the
+    # configuration as stated, so the clip decisions are also compared at eps_clip 0.05
+    lg5, sg5 = ppo_actor_loss_fn(stats["new_logp"], mb["prox_logp"], mb["logprobs"], mb["advantages"], 0.05,
+                                 mb["loss_mask"].bool())
+    lo5, so5 = O.ppo_actor_loss(lp_g.clone(), old_o, old_o, adv_o, 0.05, mask_o)
+    assert torch.equal(sg5["clip_mask"].cpu(), so5["clip_mask"]) and int(so5["clip_mask"].sum()) > 100
+    torch.testing.assert_close(lg5.cpu(), lo5, rtol=1e-4, atol=1e-7)
+
+    # the whole oracle chain on its own log-probs: the loss agrees to 1e-4 of the advantage scale
+    lp_full = lp_o[:total].clone().requires_grad_(True)
+    lo_full, so_full = O.ppo_actor_loss(lp_full, old_o, old_o, adv_o, 0.2, mask_o)
+    lo_full.backward()
+    assert abs(loss.item() - lo_full.item()) < 1e-4 * float(adv_o.abs().max())
+    flips = int((stats["clipped_tokens"].cpu() != so_full["clip_mask"]).sum())
+    near = int((((ratio - 0.8).abs() < 1e-4) | ((ratio - 1.2).abs() < 1e-4)).sum())
+    assert flips <= near  # clip decisions differ only where the ratio sits on a bound
+
+    # gradients: oracle closed form from its own chain, padded back to 4096 tokens
+    g_full = torch.zeros(T)
+    g_full[:total] = lp_full.grad
+    dh_want, dw_want = L.lm_head_backward(hidden, weight, labels, g_full)
+    rel_h = (h.grad.cpu().float() - dh_want).norm() / dh_want.norm()
+    rel_w = (w.grad.cpu().float() - dw_want).norm() / dw_want.norm()
+    assert rel_h < 1e-2 and rel_w < 1e-2, (rel_h, rel_w)
+    assert not h.grad[total:].any()  # pad tokens receive no gradient
