@@ -457,8 +457,10 @@ def compute_advantages(
     """Reward shaping, KL-regularised rewards, token- or turn-level GAE and advantage
     normalisation on a padded ``[bs, L]`` batch; writes ``returns, advantages, kl_rewards,
     tot_rewards, loss_mask, logprobs`` back into ``data`` exactly as ``actor.py:178-323`` does.
-    ``gae_lambda_fn`` (with ``gae_lambda_kwargs``) is a per-sample lambda function as resolved by
-    ``areal_amd.ppo.lambda_fn.resolve_gae_lambda_fn``; without it ``gae_lambda`` is used."""
+    ``gae_lambda_fn`` (with ``gae_lambda_kwargs``) is a per-sample lambda function
+    ``fn(context, **kwargs) -> [bs] tensor`` such as those of the reference's
+    ``areal/trainer/ppo/lambda_fn.py`` (plain torch on the length context, usable unchanged);
+    without it ``gae_lambda`` is used."""
     if gae_timestep_unit not in ("token", "turn"):
         raise ValueError(f"gae_timestep_unit must be 'token' or 'turn', got {gae_timestep_unit!r}")
     if kl_estimator is None:

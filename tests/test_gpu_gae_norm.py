@@ -298,7 +298,8 @@ def test_turn_level_gae_matches_oracle(dev, bs, L, max_turn_len):
 def test_gae_lambda_context_reference_literals(dev):
     # reference tests/test_ppo_gae.py:279-341, :436-480
     from areal_amd.ppo.gae import _build_gae_lambda_context, compute_gae_lambda
-    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda, vapo_length_adaptive_gae
+    from tests.lambda_formulas import relative_position as relative_position_gae_lambda
+    from tests.lambda_formulas import vapo as vapo_length_adaptive_gae
 
     mask = _t([[1, 1, 1, 1, 0], [1, 1, 0, 0, 0], [0, 0, 0, 0, 0]], dev)
     ids = torch.tensor([[0, 0, 1, 1, -1], [0, 1, -1, -1, -1], [-1, -1, -1, -1, -1]], dtype=torch.int32, device=dev)
@@ -333,7 +334,7 @@ def test_gae_lambda_context_reference_literals(dev):
 def test_compute_advantages_relative_position_lambda_main_path(dev):
     # reference tests/test_ppo_gae.py:406-433: a terminal reward decays as q^((L-k)/(L-1))
     from areal_amd.ppo.actor import compute_advantages
-    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda
+    from tests.lambda_formulas import relative_position as relative_position_gae_lambda
 
     q, L = 0.3, 10
     batch = {
