@@ -46,6 +46,28 @@ def test_binary_kl_matches_float64_closed_form():
     assert torch.equal(a, b)
 
 
+def test_binary_kl_matches_scipy_rel_entr_on_a_grid():
+    """An independent routine for the same quantity: the Bernoulli KL is
+    rel_entr(p, q) + rel_entr(1 - p, 1 - q) (scipy.special.rel_entr(x, y) = x log(x / y)).
+    A dropped term, swapped arguments or a wrong sign fail here; the fp32 clamp quirk
+    (p rounding to 1 -> NaN -> token rejected) is pinned by BINARY_KL_CASES above."""
+    import numpy as np
+    from scipy.special import rel_entr
+
+    ps = np.concatenate([np.linspace(0.001, 0.999, 41), [1e-6, 0.5, 1 - 1e-4]])
+    p, q = np.meshgrid(ps, ps, indexing="ij")
+    want = rel_entr(p, q) + rel_entr(1.0 - p, 1.0 - q)
+    got = O.binary_kl(torch.from_numpy(np.log(p)).float(), torch.from_numpy(np.log(q)).float())
+    # fp32 evaluation of exp(log p): relative 1e-6 on p, amplified by 1/q and 1/(1-q) near the edges
+    np.testing.assert_allclose(got.double().numpy(), want, rtol=5e-4, atol=2e-5)
+    assert np.all(np.diag(got.numpy()) == 0.0)  # KL(p || p) = 0 exactly
+    # asymmetry: the two directions differ, and the metric takes the larger
+    i, j = 3, 30
+    assert abs(want[i, j] - want[j, i]) > 1e-3
+    both = torch.maximum(got, got.T)
+    np.testing.assert_allclose(both.double().numpy(), np.maximum(want, want.T), rtol=5e-4, atol=2e-5)
+
+
 def test_kl_estimators_closed_forms():
     d = _t([-1.0, -0.3, 0.0, 0.5, 2.0])
     z = torch.zeros_like(d)
