@@ -79,7 +79,8 @@ def default_token_chunk(T: int, H: int, V: int, budget: int = DEFAULT_BWD_WORKSP
 class _FusedLMHead(torch.autograd.Function):
     @staticmethod
     def forward(
-        ctx, hidden, weight, bias, labels, temperature, logit_scale, token_chunk, save_probs
+        ctx, hidden, weight, bias, labels, temperature, logit_scale, token_chunk, save_probs,
+        with_moments, weight_grad_accum,
     ):
         lib = _lib.load()
         dev = _lib.require_gpu(hidden, weight, labels, bias)
@@ -91,10 +92,17 @@ class _FusedLMHead(torch.autograd.Function):
         T = hidden_2d.size(0)
         bias_f = bias.detach().float().contiguous() if bias is not None else None
 
-        outs = [torch.empty(labels.shape, dtype=torch.float32, device=dev) for _ in range(6)]
+        # vocabulary mean / norm cost two more operations per logit in the sweep's epilogue: they
+        # are computed only on request
+        outs = [torch.empty(labels.shape, dtype=torch.float32, device=dev) for _ in range(4)]
+        outs += [
+            torch.empty(labels.shape, dtype=torch.float32, device=dev) if with_moments else None
+            for _ in range(2)
+        ]
         outs += [torch.empty(T, dtype=torch.float32, device=dev) for _ in range(2)]
         logprobs, entropy, vmin, vmax, vmean, vnorm, row_max, sum_exp = outs
-        needs_grad = any(ctx.needs_input_grad[:2])  # the caller has ruled out no_grad mode
+        # the caller has ruled out no_grad mode
+        needs_grad = any(ctx.needs_input_grad[:2]) or weight_grad_accum is not None
         if save_probs is None:
             need = 2 * _round_up(T, 64) * _round_up(V, 64)
             save_probs = need <= SAVE_PROBS_BYTES_LIMIT and need <= 0.6 * _available_bytes(dev)
@@ -105,6 +113,7 @@ class _FusedLMHead(torch.autograd.Function):
             )
             probs_ref = torch.empty(T, dtype=torch.float32, device=dev)
             probs_status = torch.empty(1, dtype=torch.int32, device=dev)
+        ctx.status_host = ctx.status_event = None
         if T > 0:
             nbytes = lib.areal_lmhead_fwd_workspace_bytes(T, H, V)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
@@ -116,6 +125,14 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_fwd")
+            if probs_status is not None:
+                # Whether every row's saved exponentials are in range travels to pinned host
+                # memory behind the forward, so the backward reads it without a device-to-host
+                # copy of its own between the loss and its first launch.
+                ctx.status_host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+                ctx.status_host.copy_(probs_status, non_blocking=True)
+                ctx.status_event = torch.cuda.Event()
+                ctx.status_event.record(torch.cuda.current_stream(dev))
 
         ctx.save_for_backward(hidden_2d, weight_c, labels_1d, row_max, sum_exp)
         # Plain attributes, not saved tensors: the backward rewrites entries of probs in place.
@@ -130,8 +147,9 @@ class _FusedLMHead(torch.autograd.Function):
         ctx.hidden_shape = hidden.shape
         ctx.weight_dtype = weight.dtype
         ctx.bias_dtype = bias.dtype if bias is not None else None
+        ctx.weight_grad_accum = weight_grad_accum
         ctx.set_materialize_grads(False)
-        ctx.mark_non_differentiable(entropy, vmin, vmax, vmean, vnorm)
+        ctx.mark_non_differentiable(*[o for o in (entropy, vmin, vmax, vmean, vnorm) if o is not None])
         return tuple(outs[:6])
 
     @staticmethod
@@ -139,8 +157,14 @@ class _FusedLMHead(torch.autograd.Function):
         hidden_2d, weight_c, labels_1d, row_max, sum_exp = ctx.saved_tensors
         need_h, need_w, need_b = ctx.needs_input_grad[:3]
         want_h = need_h
+        # dWeight goes straight into the caller's fp32 accumulator when one was given (the master
+        # weight's .grad): the contraction's epilogue adds to it, nothing of size [V, H] is
+        # allocated and no gradient is returned for the weight
+        accum = ctx.weight_grad_accum
+        if accum is not None:
+            need_w = True
         if grad_logprobs is None or not (need_h or need_w or need_b):
-            return (None,) * 8
+            return (None,) * 10
         lib = _lib.load()
         dev = hidden_2d.device
         T, H = hidden_2d.shape
@@ -151,17 +175,23 @@ class _FusedLMHead(torch.autograd.Function):
         dh = torch.empty_like(hidden_2d) if need_h else None
         db32 = torch.empty(V, dtype=torch.float32, device=dev) if need_b else None
         probs, probs_ref = ctx.probs, ctx.probs_ref
-        # one small device-to-host copy: whether every row's saved exponentials are in range
-        if probs is not None and int(ctx.probs_status.item()) != 0:
-            probs = probs_ref = None
+        # whether every row's saved exponentials are in range: copied to pinned memory behind the
+        # forward; by now that copy has normally completed and the wait returns at once
+        if probs is not None:
+            ctx.status_event.synchronize()
+            if int(ctx.status_host[0]) != 0:
+                probs = probs_ref = None
         # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
         # the chunked recompute mode accumulates in fp32 and casts at the end
-        direct = probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
+        direct = accum is None and probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
         dw_direct = torch.empty((V, H), dtype=torch.bfloat16, device=dev) if (need_w and direct) else None
-        dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if (need_w and not direct) else None
+        if accum is not None:
+            dw32 = accum
+        else:
+            dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if (need_w and not direct) else None
         ctx.probs = ctx.probs_ref = ctx.probs_status = None  # consumed; a second backward recomputes
         if T == 0:
-            if dw32 is not None:
+            if dw32 is not None and accum is None:
                 dw32.zero_()
             if db32 is not None:
                 db32.zero_()
@@ -173,7 +203,8 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
                 _lib.ptr(probs), _lib.ptr(probs_ref),
-                _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32), 2 if direct else 0,
+                _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32),
+                2 if direct else (1 if accum is not None else 0),
                 _lib.ptr(db32), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd_saved")
@@ -186,12 +217,12 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(ctx.bias_f),
                 _lib.ptr(labels_1d), _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
-                _lib.ptr(dh), _lib.ptr(dw32), _lib.ptr(db32), 0, chunk,
+                _lib.ptr(dh), _lib.ptr(dw32), _lib.ptr(db32), 1 if accum is not None else 0, chunk,
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd")
         dw = dw_direct
-        if dw32 is not None:
+        if dw32 is not None and accum is None:
             if ctx.weight_dtype == torch.float32:
                 dw = dw32
             else:
@@ -202,7 +233,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.check(rc, "areal_cast_f32_to_bf16")
         dh = dh.view(ctx.hidden_shape) if (dh is not None and want_h) else None
         db = db32.to(ctx.bias_dtype) if db32 is not None else None
-        return dh, dw, db, None, None, None, None, None
+        return dh, dw, db, None, None, None, None, None, None, None
 
 
 def fused_lm_head_logprobs_entropy(
@@ -216,6 +247,8 @@ def fused_lm_head_logprobs_entropy(
     bias: torch.Tensor | None = None,
     token_chunk: int | None = None,
     save_probs: bool | None = None,
+    with_moments: bool = False,
+    weight_grad_accum: torch.Tensor | None = None,
 ) -> ChunkedLMHeadOutput:
     """Label log-probabilities, entropy and vocabulary statistics of ``hidden @ weight.T``.
 
@@ -232,6 +265,13 @@ def fused_lm_head_logprobs_entropy(
             ``None`` picks the largest chunk within ``DEFAULT_BWD_WORKSPACE_BYTES``.
         save_probs: keep the bf16 softmax exponentials for the backward instead of recomputing
             the logits; ``None`` decides by ``SAVE_PROBS_BYTES_LIMIT``.
+        with_moments: also return ``vocab_mean_logits`` and ``vocab_norm_logits`` (two more
+            operations per logit in the sweep); without it those two fields are ``None``.
+        weight_grad_accum: an fp32 ``[V, H]`` tensor (normally the ``.grad`` of an fp32 master
+            copy of ``weight``) that the weight gradient is ADDED to by the dWeight contraction
+            itself, as Megatron's fp32 ``main_grad`` accumulation does
+            (``vocab_parallel_head.py:873-879``); no gradient is then returned for ``weight``.
+            The bias gradient, if any, is added in the same way only through autograd.
 
     Gradient flows through ``logprobs`` only (to ``hidden`` and ``weight``), as in the
     reference (``vocab_parallel_head.py:732-734``).
@@ -264,11 +304,20 @@ def fused_lm_head_logprobs_entropy(
         raise ValueError(f"hidden size must be a multiple of 8, got {hidden.size(-1)}")
     if bias is not None and bias.shape != (weight.size(0),):
         raise ValueError(f"bias must have shape ({weight.size(0)},), got {tuple(bias.shape)}")
+    if weight_grad_accum is not None:
+        if weight_grad_accum.dtype != torch.float32 or weight_grad_accum.shape != weight.shape:
+            raise ValueError(
+                "weight_grad_accum must be an fp32 tensor of the weight's shape, got "
+                f"{weight_grad_accum.dtype} {tuple(weight_grad_accum.shape)}"
+            )
+        if not weight_grad_accum.is_contiguous():
+            raise ValueError("weight_grad_accum must be contiguous")
     if not torch.is_grad_enabled():
         save_probs = False  # no backward will come: keep nothing
+        weight_grad_accum = None
     values = _FusedLMHead.apply(
         hidden, weight, bias, labels, float(temperature), float(logit_scale), token_chunk,
-        save_probs,
+        save_probs, bool(with_moments), weight_grad_accum,
     )
     return ChunkedLMHeadOutput(*values)
 
@@ -315,5 +364,6 @@ def chunked_lm_head_logprobs_entropy(
         raise ValueError(f"chunk_size must be positive, got {chunk_size}")
     return fused_lm_head_logprobs_entropy(
         hidden_states, weight, labels, temperature=temperature, logit_scale=logit_scale, bias=bias,
+        with_moments=True,
     )
 
