@@ -71,10 +71,11 @@ def make_batch(name: str, device):
     )
 
 
-def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int):
+def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int, repeats: int = 3):
     """The CPU oracle (plain PyTorch port of the reference's op sequence) on a token slice at
     full vocabulary: fp32 logits from bf16 operands, log-softmax + entropy, PPO loss with
-    rejection sampling, autograd backward to hidden and weight."""
+    rejection sampling, autograd backward to hidden and weight. Returns (tokens/s of the median
+    repeat, the repeats' seconds)."""
     import torch
 
     from oracle import logprob as olp
@@ -88,18 +89,22 @@ def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int):
     labels = torch.randint(0, V_QWEN, (n,), generator=g)
     adv = torch.randn(n, generator=g)
     mask = torch.ones(n, dtype=torch.bool)
-    t0 = time.perf_counter()
-    h32 = hidden.float().requires_grad_(True)
-    w32 = weight.float().requires_grad_(True)
-    logits = h32 @ w32.T
-    lp, ent = olp.gather_logprobs_entropy(logits, labels, 1.0)
-    old = lp.detach() + 0.05
-    loss, _ = oloss.ppo_actor_loss(lp, lp.detach(), old, adv, 0.2, mask,
-                                   rejection_sampling_cfg=dict(level="token", action="mask", metric="ratio",
-                                                               upper=2.0, lower=0.5))
-    loss.backward()
-    dt = time.perf_counter() - t0
-    return n / dt, dt
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        h32 = hidden.float().requires_grad_(True)
+        w32 = weight.float().requires_grad_(True)
+        logits = h32 @ w32.T
+        lp, ent = olp.gather_logprobs_entropy(logits, labels, 1.0)
+        old = lp.detach() + 0.05
+        loss, _ = oloss.ppo_actor_loss(lp, lp.detach(), old, adv, 0.2, mask,
+                                       rejection_sampling_cfg=dict(level="token", action="mask", metric="ratio",
+                                                                   upper=2.0, lower=0.5))
+        loss.backward()
+        times.append(time.perf_counter() - t0)
+        del h32, w32, logits, lp, ent, loss
+    med = sorted(times)[len(times) // 2]
+    return n / med, times
 
 
 def cpu_baseline_advantages(threads: int):
@@ -315,11 +320,13 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="qwen3-8b", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-sample-tokens", type=int, default=4096)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true")
     ap.add_argument("--no-library-gemm", action="store_true",
                     help="skip timing torch.mm (the vendor library's bf16 GEMM) at the forward's shape")
+    ap.add_argument("--no-other-mode", action="store_true",
+                    help="skip the short second leg that times the other backward mode")
     ap.add_argument("--recompute", action="store_true",
                     help="backward recomputes the logits (save_probs=False) instead of using the "
                          "bf16 exponentials kept by the forward")
@@ -357,44 +364,72 @@ def main() -> None:
     )
 
     # None: keep the exponentials if the bf16 [T, V] buffer fits the library's default limit
-    save_probs = False if args.recompute else None
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-    t_fwd = t_loss = t_bwd = 0.0
     saved = False
 
-    def step(timed: bool):
-        nonlocal t_fwd, t_loss, t_bwd, saved
-        hidden.grad = None
-        weight.grad = None
-        ev[0].record()
-        out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0,
-                                             save_probs=save_probs)
-        saved = out.logprobs.grad_fn.probs is not None
-        ev[1].record()
-        loss = loss_fn(out.logprobs, out.entropy, input_data,
-                       vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
-        ev[2].record()
-        loss.backward()
-        ev[3].record()
-        if timed:
-            torch.cuda.synchronize()
-            t_fwd += ev[0].elapsed_time(ev[1])
-            t_loss += ev[1].elapsed_time(ev[2])
-            t_bwd += ev[2].elapsed_time(ev[3])
-        return loss
+    def run_steps(n_steps: int, n_warm: int, save_probs):
+        """n_warm untimed steps, then n_steps timed ones between two synchronisations. The
+        phase times come from HIP events recorded on the launch stream (read after the last
+        step, so nothing waits on the host inside the timed region)."""
+        nonlocal saved
+        evs = []
 
-    for _ in range(args.warmup):
-        step(False)
-    torch.cuda.synchronize()
-    torch.cuda.reset_peak_memory_stats()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step(True)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    peak_hbm_gb = torch.cuda.max_memory_allocated() / 1e9
+        def step(record: bool):
+            nonlocal saved
+            hidden.grad = None
+            weight.grad = None
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if record else None
+            if record:
+                ev[0].record()
+            out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0,
+                                                 save_probs=save_probs)
+            saved = out.logprobs.grad_fn.probs is not None
+            if record:
+                ev[1].record()
+            loss = loss_fn(out.logprobs, out.entropy, input_data,
+                           vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
+            if record:
+                ev[2].record()
+            loss.backward()
+            if record:
+                ev[3].record()
+                evs.append(ev)
+            return loss
+
+        for _ in range(n_warm):
+            step(False)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        t0 = time.perf_counter()
+        for _ in range(n_steps):
+            loss = step(True)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        phases = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) for i in range(3)]
+        return wall, phases, loss, torch.cuda.max_memory_allocated() / 1e9
+
+    wall, (t_fwd, t_loss, t_bwd), loss, peak_hbm_gb = run_steps(
+        args.steps, args.warmup, False if args.recompute else None)
+    main_saved = saved
     ms_per_step = wall * 1e3 / args.steps
     tokens_per_s = T * args.steps / wall
+
+    # The other memory mode, a short leg of its own: the backward recomputes the logits chunk by
+    # chunk and nothing of size [T, V] is kept between forward and backward (the reference's
+    # memory behaviour, vocab_parallel_head.py:704-713). Same algorithmic flops, one more
+    # contraction launch.
+    other = None
+    if not args.no_other_mode:
+        n_other = max(1, min(args.steps, 5))
+        o_wall, o_ph, _, o_peak = run_steps(n_other, 1, None if args.recompute else False)
+        other = {
+            "backward": "saved bf16 exponentials" if saved else "recompute logits",
+            "steps": n_other, "ms_per_step": o_wall * 1e3 / n_other,
+            "frac": 6.0 * T * H * V / (o_wall / n_other) / 1e12 / PEAK_BF16_TFLOPS,
+            "peak_hbm_gb": o_peak,
+            "ms": {"lmhead_fwd": o_ph[0] / n_other, "loss_fwd": o_ph[1] / n_other,
+                   "loss_bwd+lmhead_bwd": o_ph[2] / n_other},
+        }
+    saved = main_saved
 
     # Roofline of the MFMA contraction kernels (gemm_nt_sweep / gemm_tn_sweep): one step runs
     # 3 algorithmic GEMMs = 6*T*H*V flops (forward with the softmax epilogue, dHidden, dWeight);
@@ -478,6 +513,7 @@ def main() -> None:
             "library_gemm_same_box_tflops": lib_tflops,
             "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},
+            "other_backward_mode": other,
         },
     }
     if not args.no_hbm_kernels:
@@ -485,12 +521,16 @@ def main() -> None:
         torch.cuda.empty_cache()
         result["hbm_rooflines"] = hbm_rooflines(dev)
     if not args.no_cpu_baseline:
-        threads = min(16, os.cpu_count() or 1)
-        tps, dt = cpu_baseline(args.cpu_sample_tokens, H, WORKLOADS[args.workload]["seed"], threads)
+        # every core this process may run on (a GPU box grants a share of the host's cores)
+        threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+        threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)) or threads)
+        tps, times = cpu_baseline(args.cpu_sample_tokens, H, WORKLOADS[args.workload]["seed"], threads)
         result["cpu_baseline"] = {
             "value": tps, "unit": "tokens/s", "cores": threads, "kind": "port",
             "sample": f"{args.cpu_sample_tokens}-token slice at full vocabulary, fwd+bwd with the "
-                      f"PyTorch oracle, {dt:.1f} s (rate is per token, so it scales linearly in T)",
+                      f"PyTorch oracle, median of {len(times)} repeats ("
+                      + ", ".join(f"{t:.1f}" for t in times)
+                      + " s; the rate is per token, so it scales linearly in T)",
         }
         if not args.no_hbm_kernels:
             result["cpu_baseline_advantages"] = cpu_baseline_advantages(threads)
