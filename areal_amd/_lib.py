@@ -59,6 +59,10 @@ SIGNATURES: dict[str, tuple] = {
         I,
         [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
+    "areal_actor_loss_static": (
+        I,
+        [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P],
+    ),
     "areal_actor_loss_grad": (I, [P, P, P, P, I64, P]),
     "areal_aux_loss_workspace_bytes": (SZ, [I64, I64]),
     "areal_sapo_loss": (

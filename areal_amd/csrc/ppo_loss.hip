@@ -12,6 +12,8 @@
 // Sums use fp64 block partials reduced in a fixed order: results are run-to-run identical.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace {
 
 constexpr int LOSS_THREADS = 256;
@@ -410,8 +412,6 @@ int loss_grid(int64_t n) {
 
 }  // namespace
 
-extern "C" {
-
 // Plain-C mirror of LossCfg (see include/areal_hip.h).
 struct areal_loss_config {
   int loss_kind;
@@ -425,10 +425,57 @@ struct areal_loss_config {
   float rs_lower;
 };
 
-size_t areal_actor_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
-  (void)n_tokens;
+namespace {
+
+size_t loss_workspace_bytes(int64_t n_seqs) {
   if (n_seqs < 0) n_seqs = 0;
   return (size_t)MAX_LOSS_BLOCKS * sizeof(Partial) + (size_t)n_seqs * 6 * sizeof(float) + 256;
+}
+
+// Scratch of areal_actor_loss_static: the block partials and the per-sequence aggregates of
+// one call, for up to STATIC_MAX_SEQS sequences. Every GPU the library runs on holds its own
+// copy of this array for the life of the process (about 1.6 MB). Nothing in it has to start at
+// zero: a call writes every partial and every per-sequence slot it later reads.
+constexpr int64_t STATIC_MAX_SEQS = 65536;
+constexpr size_t STATIC_SCRATCH_BYTES =
+    (size_t)MAX_LOSS_BLOCKS * sizeof(Partial) + (size_t)STATIC_MAX_SEQS * 6 * sizeof(float) + 256;
+static_assert(STATIC_SCRATCH_BYTES < (2u << 20), "the static scratch is meant to stay small");
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on each GPU (the array's name is only a host-side handle).
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex scratch_lock;
+void* scratch_ptr[STATIC_MAX_DEVICES];
+
+int scratch_for_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return AREAL_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return AREAL_ERR_LAUNCH;
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return AREAL_OK;
+}
+
+int actor_loss_impl(const float* logprobs, const float* proximal, const float* old_logprobs,
+                    const float* advantages, const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                    int64_t n_tokens, int64_t n_seqs, int64_t uniform_len,
+                    const areal_loss_config* cfg, float* loss, float* dlogprobs, float* stat_loss,
+                    float* stat_ratio, float* stat_approx_kl, uint8_t* clip_mask,
+                    uint8_t* dual_clip_mask, uint8_t* new_mask, float* behave_imp_weight,
+                    float* behave_approx_kl, uint8_t* behave_mask, double* counters,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream);
+
+}  // namespace
+
+extern "C" {
+
+size_t areal_actor_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
+  (void)n_tokens;
+  return loss_workspace_bytes(n_seqs);
 }
 
 // Actor loss forward + backward in one pass over the tokens.
@@ -447,6 +494,48 @@ int areal_actor_loss(const float* logprobs, const float* proximal, const float* 
                      float* behave_imp_weight, float* behave_approx_kl, uint8_t* behave_mask,
                      double* counters, void* workspace, size_t workspace_bytes,
                      hipStream_t stream) {
+  return actor_loss_impl(logprobs, proximal, old_logprobs, advantages, loss_mask, cu_seqlens, n_tokens,
+                         n_seqs, uniform_len, cfg, loss, dlogprobs, stat_loss, stat_ratio,
+                         stat_approx_kl, clip_mask, dual_clip_mask, new_mask, behave_imp_weight,
+                         behave_approx_kl, behave_mask, counters, workspace, workspace_bytes, stream);
+}
+
+// The same computation with the scratch in a static device array instead of a caller's
+// workspace: no allocation anywhere on the call path. Must be called with the stream's device
+// current. Sequence-level options accept at most 65536 sequences (AREAL_ERR_UNSUPPORTED beyond).
+// Calls on one GPU share that GPU's array: two calls that overlap in time (different streams)
+// race; calls on one stream are ordered and safe.
+int areal_actor_loss_static(const float* logprobs, const float* proximal,
+                            const float* old_logprobs, const float* advantages,
+                            const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                            int64_t n_tokens, int64_t n_seqs, int64_t uniform_len,
+                            const areal_loss_config* cfg, float* loss, float* dlogprobs,
+                            float* stat_loss, float* stat_ratio, float* stat_approx_kl,
+                            uint8_t* clip_mask, uint8_t* dual_clip_mask, uint8_t* new_mask,
+                            float* behave_imp_weight, float* behave_approx_kl,
+                            uint8_t* behave_mask, double* counters, hipStream_t stream) {
+  if (n_seqs > STATIC_MAX_SEQS) return AREAL_ERR_UNSUPPORTED;
+  void* ws = nullptr;
+  const int rc = scratch_for_current_device(&ws);
+  if (rc != AREAL_OK) return rc;
+  return actor_loss_impl(logprobs, proximal, old_logprobs, advantages, loss_mask, cu_seqlens, n_tokens,
+                         n_seqs, uniform_len, cfg, loss, dlogprobs, stat_loss, stat_ratio,
+                         stat_approx_kl, clip_mask, dual_clip_mask, new_mask, behave_imp_weight,
+                         behave_approx_kl, behave_mask, counters, ws, STATIC_SCRATCH_BYTES, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int actor_loss_impl(const float* logprobs, const float* proximal, const float* old_logprobs,
+                    const float* advantages, const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                    int64_t n_tokens, int64_t n_seqs, int64_t uniform_len,
+                    const areal_loss_config* cfg, float* loss, float* dlogprobs, float* stat_loss,
+                    float* stat_ratio, float* stat_approx_kl, uint8_t* clip_mask,
+                    uint8_t* dual_clip_mask, uint8_t* new_mask, float* behave_imp_weight,
+                    float* behave_approx_kl, uint8_t* behave_mask, double* counters,
+                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (cfg == nullptr || n_tokens < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
   if (cfg->loss_kind < LOSS_NONE || cfg->loss_kind > LOSS_CISPO) return AREAL_ERR_BAD_ARG;
   if (n_tokens > 0 && (proximal == nullptr || loss_mask == nullptr)) return AREAL_ERR_BAD_ARG;
@@ -460,7 +549,7 @@ int areal_actor_loss(const float* logprobs, const float* proximal, const float* 
     if (cfg->rs_enabled && (new_mask == nullptr || behave_imp_weight == nullptr) && cfg->seq_is)
       return AREAL_ERR_BAD_ARG;
   }
-  if (workspace == nullptr || workspace_bytes < areal_actor_loss_workspace_bytes(n_tokens, n_seqs))
+  if (workspace == nullptr || workspace_bytes < loss_workspace_bytes(n_seqs))
     return AREAL_ERR_WORKSPACE;
 
   LossCfg c;
@@ -512,6 +601,10 @@ int areal_actor_loss(const float* logprobs, const float* proximal, const float* 
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
+
+}  // namespace
+
+extern "C" {
 
 // grad_logprobs[t] = dlogprobs[t] * upstream[0] / max(counters[1], 1)
 int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const double* counters,

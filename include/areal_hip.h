@@ -171,6 +171,24 @@ int areal_actor_loss(const float* logprobs, const float* proximal_logprobs,
                      uint8_t* behave_mask, double* counters, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
 
+/* areal_actor_loss without the workspace argument: the block partials and per-sequence
+ * aggregates live in a static device array inside the library (about 1.6 MB per GPU, held until
+ * the process ends), so nothing on the call path allocates. It has no counterpart in the
+ * reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. Call it with the stream's device current. At most
+ * 65536 sequences (n_seqs beyond that: AREAL_ERR_UNSUPPORTED). All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU race, calls on one stream do not. Outputs
+ * are bit-identical to areal_actor_loss. */
+int areal_actor_loss_static(const float* logprobs, const float* proximal_logprobs,
+                            const float* old_logprobs, const float* advantages,
+                            const uint8_t* loss_mask, const int32_t* cu_seqlens,
+                            int64_t n_tokens, int64_t n_seqs, int64_t uniform_len,
+                            const areal_loss_config* cfg, float* loss, float* dlogprobs,
+                            float* stat_loss, float* stat_ratio, float* stat_approx_kl,
+                            uint8_t* clip_mask, uint8_t* dual_clip_mask, uint8_t* new_mask,
+                            float* behave_imp_weight, float* behave_approx_kl,
+                            uint8_t* behave_mask, double* counters, areal_stream_t stream);
+
 /* grad_logprobs[t] = dlogprobs[t] * upstream[0] / max(counters[1], 1): the backward of
  * `loss = sum(where(mask, pg, 0)) / loss_mask_count` (functional.py:571). */
 int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const double* counters,
