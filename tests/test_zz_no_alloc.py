@@ -24,6 +24,9 @@ def _inputs(n, n_seqs, seed, dev):
     mask = torch.rand(n, generator=g) > 0.25
     cuts = torch.sort(torch.randperm(n - 1, generator=g)[: n_seqs - 1] + 1).values
     cu = torch.cat([torch.tensor([0]), cuts, torch.tensor([n])]).to(torch.int32)
+    longest = int((cu[1:] - cu[:-1]).argmax())
+    old[cu[longest]:cu[longest + 1]] -= 1.5  # one sequence far off-policy: rejected at either level
+    mask[cu[longest]] = True
     return [t.to(dev) for t in (lp, prox, old, adv, mask, cu)]
 
 
@@ -71,13 +74,13 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(dev, seq_level
     # two calls in a row on the shared scratch: a large batch, then a smaller one
     for n, n_seqs, seed in ((300_000, 700, 5), (4_099, 13, 6)):
         batch = _inputs(n, n_seqs, seed, dev)
-        free_before = torch.cuda.mem_get_info(dev)[0]
         got = _call(lib, True, cfg, *batch, dev)
         want = _call(lib, False, cfg, *batch, dev)
+        print("counters", n, want["counters"].tolist(), flush=True)
         for k in want:
             assert torch.equal(got[k], want[k]), (k, n)
-        assert float(want["counters"][1]) > 0 and float(want["counters"][3]) > 0
-        del free_before
+        n_valid, n_filtered = float(want["counters"][1]), float(want["counters"][3])
+        assert n_valid == float(batch[4].sum()) and 0 < n_filtered < n_valid
 
 
 def test_static_scratch_entry_point_rejects_too_many_sequences(dev):
