@@ -59,6 +59,11 @@ SIGNATURES: dict[str, tuple] = {
         I,
         [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
+    "areal_actor_loss_stats_workspace_bytes": (SZ, [I64, I64]),
+    "areal_actor_loss_stats": (
+        I,
+        [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
+    ),
     "areal_actor_loss_static": (
         I,
         [P, P, P, P, P, P, I64, I64, I64, P, P, P, P, P, P, P, P, P, P, P, P, P, P],

@@ -64,6 +64,26 @@ struct LossIO {
   float* behave_w;
   float* behave_kl;
   uint8_t* behave_mask;
+  // fused logging statistics (loss_token_kernel<true> only)
+  const float* entropy;   // optional per-token input
+  const float* extra0;    // optional per-token inputs reduced over all tokens
+  const float* extra1;
+};
+
+// Logged statistics reduced inside the token pass (the tensors grpo_loss_fn hands to the stats
+// tracker, areal/trainer/ppo/actor.py:662-733, each under its denominator mask).
+enum {
+  ST_IMPORTANCE_WEIGHT = 0, ST_APPROX_KL, ST_NEW_LOGP, ST_OLD_LOGP, ST_ENTROPY, ST_ACTOR_LOSS,
+  ST_CLIP_RATIO, ST_DUAL_CLIP_RATIO, ST_LOGP_DIFF, ST_LOGP_ABS_DIFF, ST_BEHAVE_FILTERED_RATIO,
+  ST_BEHAVE_IMP_WEIGHT, ST_BEHAVE_APPROX_KL, ST_CLIPPED_NEW_LOGP, ST_CLIPPED_OLD_LOGP,
+  ST_EXTRA0, ST_EXTRA1, N_LOSS_STATS
+};
+// denominators: 0 loss mask (before rejection), 1 clip mask, 2 behave mask, 3 every token
+__device__ const int STAT_DENOM[N_LOSS_STATS] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 2, 2, 1, 1, 3, 3};
+
+struct StatPartial {
+  double sum;
+  float mn, mx;
 };
 
 struct Partial {
@@ -257,12 +277,29 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_is_kernel(LossIO io, LossCfg
 // ---------------------------------------------------------------------------------------
 // Token kernel
 // ---------------------------------------------------------------------------------------
+// STATS: also reduce the logged statistics (sum, min, max per block) into stat_partials
+// [gridDim.x][N_LOSS_STATS]; min / max propagate NaN as torch.min / torch.max do.
+template <bool STATS>
 __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, LossCfg c,
-                                                                   Partial* partials) {
+                                                                   Partial* partials,
+                                                                   StatPartial* stat_partials) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
   double loss_sum = 0.0;
   long long n_valid = 0, n_kept = 0, n_filtered = 0, n_clip = 0, n_dual = 0, n_behave = 0;
+  double st_sum[STATS ? N_LOSS_STATS : 1];
+  float st_mn[STATS ? N_LOSS_STATS : 1], st_mx[STATS ? N_LOSS_STATS : 1];
+  if (STATS) {
+#pragma unroll
+    for (int k = 0; k < N_LOSS_STATS; ++k) { st_sum[k] = 0.0; st_mn[k] = pos_inf(); st_mx[k] = neg_inf(); }
+  }
+  auto stat = [&](int k, bool on, float v) {
+    if (STATS && on) {
+      st_sum[k] += (double)v;
+      st_mn[k] = torch_min(st_mn[k], v);
+      st_mx[k] = torch_max(st_mx[k], v);
+    }
+  };
 
   for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < io.n;
        t += (int64_t)gridDim.x * blockDim.x) {
@@ -279,6 +316,10 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
     }
     n_valid += m;
     n_kept += m2;
+    if (STATS) {
+      if (io.extra0) stat(ST_EXTRA0, true, io.extra0[t]);
+      if (io.extra1) stat(ST_EXTRA1, true, io.extra1[t]);
+    }
     if (c.loss_kind == LOSS_NONE) continue;
 
     const float lp = io.lp[t], prox = io.prox[t], adv = io.adv[t];
@@ -340,6 +381,28 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
       n_behave += bm;
       if (io.behave_mask) io.behave_mask[t] = bm;
       if (io.behave_kl) io.behave_kl[t] = bm ? (prox - io.old[t]) : 0.0f;
+      if (STATS) {
+        stat(ST_BEHAVE_IMP_WEIGHT, bm, w);
+        stat(ST_BEHAVE_APPROX_KL, bm, prox - io.old[t]);
+        stat(ST_BEHAVE_FILTERED_RATIO, m, (m && !bm) ? 1.0f : 0.0f);
+      }
+    }
+    if (STATS) {
+      stat(ST_IMPORTANCE_WEIGHT, m, ratio_out);
+      stat(ST_APPROX_KL, m, kl);
+      stat(ST_NEW_LOGP, m, lp);
+      stat(ST_ACTOR_LOSS, m, pg);
+      stat(ST_CLIP_RATIO, m, clip ? 1.0f : 0.0f);
+      stat(ST_DUAL_CLIP_RATIO, m, dual ? 1.0f : 0.0f);
+      stat(ST_CLIPPED_NEW_LOGP, clip, lp);
+      if (io.entropy) stat(ST_ENTROPY, m, io.entropy[t]);
+      if (io.old) {
+        const float o = io.old[t];
+        stat(ST_OLD_LOGP, m, o);
+        stat(ST_LOGP_DIFF, m, o - lp);
+        stat(ST_LOGP_ABS_DIFF, m, fabsf(o - lp));
+        stat(ST_CLIPPED_OLD_LOGP, clip, o);
+      }
     }
     if (m2) loss_sum += (double)pg;
     n_clip += clip;
@@ -361,6 +424,73 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
   if (threadIdx.x == 0) {
     Partial p{loss_sum, n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave};
     partials[blockIdx.x] = p;
+  }
+  if (STATS) {
+    // wave shuffles, then the four waves' values meet in LDS and are combined in wave order
+    __shared__ double sh_sum[LOSS_THREADS / 64][N_LOSS_STATS];
+    __shared__ float sh_mn[LOSS_THREADS / 64][N_LOSS_STATS], sh_mx[LOSS_THREADS / 64][N_LOSS_STATS];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < N_LOSS_STATS; ++k) {
+      const double sv = wave_sum(st_sum[k]);
+      float mn = st_mn[k], mx = st_mx[k];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        mn = torch_min(mn, __shfl_xor(mn, o, 64));
+        mx = torch_max(mx, __shfl_xor(mx, o, 64));
+      }
+      if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
+    }
+    __syncthreads();
+    if (threadIdx.x < N_LOSS_STATS) {
+      const int k = threadIdx.x;
+      StatPartial sp{sh_sum[0][k], sh_mn[0][k], sh_mx[0][k]};
+      for (int i = 1; i < LOSS_THREADS / 64; ++i) {
+        sp.sum += sh_sum[i][k];
+        sp.mn = torch_min(sp.mn, sh_mn[i][k]);
+        sp.mx = torch_max(sp.mx, sh_mx[i][k]);
+      }
+      stat_partials[(size_t)blockIdx.x * N_LOSS_STATS + k] = sp;
+    }
+  }
+}
+
+// stats [N_LOSS_STATS][4] = {sum, count, min, max}: block k folds statistic k over the token
+// kernel's blocks in a fixed order; the count is the statistic's denominator, taken from the
+// counters loss_finalize_kernel has written (this kernel is queued behind it).
+__global__ __launch_bounds__(LOSS_THREADS) void loss_stats_finalize_kernel(
+    const StatPartial* __restrict__ stat_partials, int nparts, const double* __restrict__ counters,
+    double n_tokens, double* __restrict__ stats) {
+  __shared__ double sm_d[8];
+  __shared__ float sm_f[8];
+  const int k = blockIdx.x;
+  double sum = 0.0;
+  float mn = pos_inf(), mx = neg_inf();
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    const StatPartial sp = stat_partials[(size_t)i * N_LOSS_STATS + k];
+    sum += sp.sum;
+    mn = torch_min(mn, sp.mn);
+    mx = torch_max(mx, sp.mx);
+  }
+  sum = block_sum(sum, sm_d);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = torch_min(mn, __shfl_xor(mn, o, 64));
+    mx = torch_max(mx, __shfl_xor(mx, o, 64));
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    mn = torch_min(torch_min(sm_f[0], sm_f[1]), torch_min(sm_f[2], sm_f[3]));
+    mx = torch_max(torch_max(sm_f[4], sm_f[5]), torch_max(sm_f[6], sm_f[7]));
+    const int d = STAT_DENOM[k];
+    const double count = d == 0 ? counters[1] : (d == 1 ? counters[4] : (d == 2 ? counters[6] : n_tokens));
+    stats[4 * k + 0] = sum;
+    stats[4 * k + 1] = count;
+    stats[4 * k + 2] = (double)mn;
+    stats[4 * k + 3] = (double)mx;
   }
 }
 
@@ -427,10 +557,21 @@ struct areal_loss_config {
 
 namespace {
 
-size_t loss_workspace_bytes(int64_t n_seqs) {
+constexpr size_t STAT_PARTIAL_BYTES = (size_t)MAX_LOSS_BLOCKS * N_LOSS_STATS * sizeof(StatPartial);
+
+size_t loss_workspace_bytes(int64_t n_seqs, bool with_stats) {
   if (n_seqs < 0) n_seqs = 0;
-  return (size_t)MAX_LOSS_BLOCKS * sizeof(Partial) + (size_t)n_seqs * 6 * sizeof(float) + 256;
+  return (size_t)MAX_LOSS_BLOCKS * sizeof(Partial) + (with_stats ? STAT_PARTIAL_BYTES : 0) +
+         (size_t)n_seqs * 6 * sizeof(float) + 256;
 }
+
+// Optional inputs and the output of the fused logging statistics.
+struct LossStatsArgs {
+  const float* entropy;
+  const float* extra0;
+  const float* extra1;
+  double* stats;  // [N_LOSS_STATS][4]
+};
 
 // Scratch of areal_actor_loss_static: the block partials and the per-sequence aggregates of
 // one call, for up to STATIC_MAX_SEQS sequences. Every GPU the library runs on holds its own
@@ -467,7 +608,8 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
                     float* stat_ratio, float* stat_approx_kl, uint8_t* clip_mask,
                     uint8_t* dual_clip_mask, uint8_t* new_mask, float* behave_imp_weight,
                     float* behave_approx_kl, uint8_t* behave_mask, double* counters,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream);
+                    const LossStatsArgs* sa, void* workspace, size_t workspace_bytes,
+                    hipStream_t stream);
 
 }  // namespace
 
@@ -475,7 +617,12 @@ extern "C" {
 
 size_t areal_actor_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
   (void)n_tokens;
-  return loss_workspace_bytes(n_seqs);
+  return loss_workspace_bytes(n_seqs, false);
+}
+
+size_t areal_actor_loss_stats_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
+  (void)n_tokens;
+  return loss_workspace_bytes(n_seqs, true);
 }
 
 // Actor loss forward + backward in one pass over the tokens.
@@ -497,7 +644,35 @@ int areal_actor_loss(const float* logprobs, const float* proximal, const float* 
   return actor_loss_impl(logprobs, proximal, old_logprobs, advantages, loss_mask, cu_seqlens, n_tokens,
                          n_seqs, uniform_len, cfg, loss, dlogprobs, stat_loss, stat_ratio,
                          stat_approx_kl, clip_mask, dual_clip_mask, new_mask, behave_imp_weight,
-                         behave_approx_kl, behave_mask, counters, workspace, workspace_bytes, stream);
+                         behave_approx_kl, behave_mask, counters, nullptr, workspace, workspace_bytes,
+                         stream);
+}
+
+// areal_actor_loss that also reduces the logged statistics in the token pass: stats
+// [17][4] double = {sum, count, min, max} of, in this order: importance_weight, approx_kl,
+// new_logp, old_logp, entropy, actor_loss, clip_ratio, dual_clip_ratio, logp_diff,
+// logp_abs_diff, behave_filtered_ratio (all under the loss mask before rejection),
+// behave_imp_weight, behave_approx_kl (under the behave mask), clipped_new_logp,
+// clipped_old_logp (under the clip mask), extra0, extra1 (every token). entropy / extra0 /
+// extra1 / old_logprobs may be null: their statistics then come out as sum 0, min +inf, max -inf.
+// Every per-token output may be null, so a caller that logs only reduced values moves
+// 17 bytes per token in and 4 out (dlogprobs).
+int areal_actor_loss_stats(const float* logprobs, const float* proximal, const float* old_logprobs,
+                           const float* advantages, const uint8_t* loss_mask,
+                           const int32_t* cu_seqlens, int64_t n_tokens, int64_t n_seqs,
+                           int64_t uniform_len, const areal_loss_config* cfg,
+                           const float* entropy, const float* extra0, const float* extra1,
+                           float* loss, float* dlogprobs, float* stat_loss, float* stat_ratio,
+                           float* stat_approx_kl, uint8_t* clip_mask, uint8_t* dual_clip_mask,
+                           uint8_t* new_mask, float* behave_imp_weight, float* behave_approx_kl,
+                           uint8_t* behave_mask, double* counters, double* stats, void* workspace,
+                           size_t workspace_bytes, hipStream_t stream) {
+  const LossStatsArgs sa{entropy, extra0, extra1, stats};
+  return actor_loss_impl(logprobs, proximal, old_logprobs, advantages, loss_mask, cu_seqlens, n_tokens,
+                         n_seqs, uniform_len, cfg, loss, dlogprobs, stat_loss, stat_ratio,
+                         stat_approx_kl, clip_mask, dual_clip_mask, new_mask, behave_imp_weight,
+                         behave_approx_kl, behave_mask, counters, &sa, workspace, workspace_bytes,
+                         stream);
 }
 
 // The same computation with the scratch in a static device array instead of a caller's
@@ -521,7 +696,8 @@ int areal_actor_loss_static(const float* logprobs, const float* proximal,
   return actor_loss_impl(logprobs, proximal, old_logprobs, advantages, loss_mask, cu_seqlens, n_tokens,
                          n_seqs, uniform_len, cfg, loss, dlogprobs, stat_loss, stat_ratio,
                          stat_approx_kl, clip_mask, dual_clip_mask, new_mask, behave_imp_weight,
-                         behave_approx_kl, behave_mask, counters, ws, STATIC_SCRATCH_BYTES, stream);
+                         behave_approx_kl, behave_mask, counters, nullptr, ws, STATIC_SCRATCH_BYTES,
+                         stream);
 }
 
 }  // extern "C"
@@ -535,8 +711,11 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
                     float* stat_ratio, float* stat_approx_kl, uint8_t* clip_mask,
                     uint8_t* dual_clip_mask, uint8_t* new_mask, float* behave_imp_weight,
                     float* behave_approx_kl, uint8_t* behave_mask, double* counters,
-                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                    const LossStatsArgs* sa, void* workspace, size_t workspace_bytes,
+                    hipStream_t stream) {
   if (cfg == nullptr || n_tokens < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
+  const bool with_stats = sa != nullptr;
+  if (with_stats && sa->stats == nullptr) return AREAL_ERR_BAD_ARG;
   if (cfg->loss_kind < LOSS_NONE || cfg->loss_kind > LOSS_CISPO) return AREAL_ERR_BAD_ARG;
   if (n_tokens > 0 && (proximal == nullptr || loss_mask == nullptr)) return AREAL_ERR_BAD_ARG;
   if (cfg->loss_kind != LOSS_NONE && n_tokens > 0 && (logprobs == nullptr || advantages == nullptr))
@@ -549,7 +728,7 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
     if (cfg->rs_enabled && (new_mask == nullptr || behave_imp_weight == nullptr) && cfg->seq_is)
       return AREAL_ERR_BAD_ARG;
   }
-  if (workspace == nullptr || workspace_bytes < loss_workspace_bytes(n_seqs))
+  if (workspace == nullptr || workspace_bytes < loss_workspace_bytes(n_seqs, with_stats))
     return AREAL_ERR_WORKSPACE;
 
   LossCfg c;
@@ -562,7 +741,10 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
 
   char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   Partial* partials = (Partial*)wp;
-  float* seq_rs = (float*)(wp + (size_t)MAX_LOSS_BLOCKS * sizeof(Partial));
+  wp += (size_t)MAX_LOSS_BLOCKS * sizeof(Partial);
+  StatPartial* stat_partials = with_stats ? (StatPartial*)wp : nullptr;
+  if (with_stats) wp += STAT_PARTIAL_BYTES;
+  float* seq_rs = (float*)wp;
   float* seq_is = seq_rs + 2 * (n_seqs > 0 ? n_seqs : 0);
 
   LossIO io;
@@ -573,6 +755,9 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
   io.stat_kl = stat_approx_kl; io.clip_mask = clip_mask; io.dual_mask = dual_clip_mask;
   io.new_mask = new_mask; io.behave_w = behave_imp_weight; io.behave_kl = behave_approx_kl;
   io.behave_mask = behave_mask;
+  io.entropy = with_stats ? sa->entropy : nullptr;
+  io.extra0 = with_stats ? sa->extra0 : nullptr;
+  io.extra1 = with_stats ? sa->extra1 : nullptr;
 
   const int grid = loss_grid(n_tokens);
   if (n_tokens > 0 && c.rs_enabled && c.rs_seq_level) {
@@ -586,19 +771,29 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
       LossCfg c0 = c;
       c0.loss_kind = LOSS_NONE;
       LossIO io0 = io;
-      hipLaunchKernelGGL(loss_token_kernel, dim3(grid), dim3(LOSS_THREADS), 0, stream, io0, c0,
-                         partials);
+      hipLaunchKernelGGL(loss_token_kernel<false>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io0, c0,
+                         partials, (StatPartial*)nullptr);
       AREAL_CHECK_LAUNCH();
     }
     hipLaunchKernelGGL(seq_is_kernel, dim3((unsigned)n_seqs), dim3(LOSS_THREADS), 0, stream, io, c,
                        seq_is);
     AREAL_CHECK_LAUNCH();
   }
-  hipLaunchKernelGGL(loss_token_kernel, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c, partials);
+  if (with_stats)
+    hipLaunchKernelGGL(loss_token_kernel<true>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c,
+                       partials, stat_partials);
+  else
+    hipLaunchKernelGGL(loss_token_kernel<false>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c,
+                       partials, (StatPartial*)nullptr);
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(LOSS_THREADS), 0, stream, partials, grid,
                      loss, counters);
   AREAL_CHECK_LAUNCH();
+  if (with_stats) {
+    hipLaunchKernelGGL(loss_stats_finalize_kernel, dim3(N_LOSS_STATS), dim3(LOSS_THREADS), 0, stream,
+                       stat_partials, grid, counters, (double)n_tokens, sa->stats);
+    AREAL_CHECK_LAUNCH();
+  }
   return AREAL_OK;
 }
 

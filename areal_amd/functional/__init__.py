@@ -2,6 +2,7 @@
 
 from areal_amd.functional.functional import (
     RejectionSamplingResult,
+    StatReduction,
     apply_rejection_sampling,
     cispo_loss_fn,
     masked_normalization,
@@ -26,6 +27,7 @@ from areal_amd.functional.vocab_parallel import (
 
 __all__ = [
     "RejectionSamplingResult",
+    "StatReduction",
     "apply_rejection_sampling",
     "cispo_loss_fn",
     "masked_normalization",

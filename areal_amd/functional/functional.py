@@ -37,6 +37,70 @@ def _f32(t: torch.Tensor) -> torch.Tensor:
     return t.detach().to(torch.float32).contiguous().view(-1)
 
 
+# Order of the statistics areal_actor_loss_stats reduces (include/areal_hip.h) and the
+# denominator each is taken under.
+REDUCED_STAT_KEYS = (
+    ("importance_weight", "n_valid_tokens"), ("approx_kl", "n_valid_tokens"),
+    ("new_logp", "n_valid_tokens"), ("old_logp", "n_valid_tokens"), ("entropy", "n_valid_tokens"),
+    ("actor_loss", "n_valid_tokens"), ("clip_ratio", "n_valid_tokens"),
+    ("dual_clip_ratio", "n_valid_tokens"), ("logp_diff", "n_valid_tokens"),
+    ("logp_abs_diff", "n_valid_tokens"), ("behave_filtered_ratio", "n_valid_tokens"),
+    ("behave_imp_weight", "unclipped_behave_tokens"), ("behave_approx_kl", "unclipped_behave_tokens"),
+    ("clipped_new_logp", "clipped_tokens"), ("clipped_old_logp", "clipped_tokens"),
+    ("extra0", "n_tokens"), ("extra1", "n_tokens"),
+)
+
+
+class StatReduction:
+    """Ask a loss call to reduce its logged statistics inside the kernel's token pass.
+
+    The reference logs about 25 per-token tensors per micro-batch through ``stats_tracker``
+    (each cloned, ``areal/utils/stats_tracker.py:133-171``) and reduces each under its
+    denominator mask at export (``:455-560``).  A loss call given a ``StatReduction`` writes none
+    of those ``[T]`` tensors: the token kernel accumulates sum, min and max of every statistic
+    in registers and ``results`` receives, after the call, ``{key: {"sum", "count", "avg",
+    "min", "max"}}`` (``avg`` / ``min`` / ``max`` are ``None`` under an empty denominator, as
+    the tracker's ``_avg_of`` / ``_min_of`` / ``_max_of`` return) and ``denominators``
+    ``{name: count}``.  The returned ``stat`` dict then holds the host scalars only.
+
+    ``entropy`` and up to two ``extras`` (``{name: tensor}``, reduced over every token, e.g. the
+    vocabulary min / max logits) are optional per-token inputs that ride along in the same pass.
+    """
+
+    def __init__(self, entropy: torch.Tensor | None = None, extras: dict[str, torch.Tensor] | None = None):
+        extras = dict(extras or {})
+        if len(extras) > 2:
+            raise ValueError(f"at most two extra statistics ride along, got {len(extras)}")
+        self.entropy = entropy
+        self.extras = extras
+        self.results: dict[str, dict[str, float | None]] = {}
+        self.denominators: dict[str, float] = {}
+
+    def _fill(self, host: torch.Tensor, counters, n_tokens: int, has_rs: bool, has_old: bool) -> None:
+        names = list(self.extras)
+        for i, (key, denom) in enumerate(REDUCED_STAT_KEYS):
+            if key == "entropy" and self.entropy is None:
+                continue
+            if key.startswith("behave_") and not has_rs:
+                continue
+            if key in ("old_logp", "logp_diff", "logp_abs_diff", "clipped_old_logp") and not has_old:
+                continue
+            if key.startswith("extra"):
+                j = int(key[-1])
+                if j >= len(names):
+                    continue
+                key = names[j]
+            s, c, mn, mx = host[i].tolist()
+            empty = c == 0
+            self.results[key] = dict(sum=s, count=c, avg=None if empty else s / c,
+                                     min=None if empty else mn, max=None if empty else mx,
+                                     denominator=denom)
+        self.denominators = dict(n_tokens=float(n_tokens), n_valid_tokens=float(counters[1]),
+                                 clipped_tokens=float(counters[4]), dual_clipped_tokens=float(counters[5]))
+        if has_rs:
+            self.denominators["unclipped_behave_tokens"] = float(counters[6])
+
+
 def _fill_rs(cfg: _lib.LossConfig, rs: RejectionSamplingConfig | None) -> None:
     if rs is None:
         cfg.rs_enabled = 0
@@ -73,8 +137,10 @@ def _run_loss_kernel(
     mask_bool,
     cu_seqlens,
     want_grad: bool,
+    reduction: "StatReduction | None" = None,
 ):
-    """Launch ``areal_actor_loss`` and return its outputs and the eight host counters."""
+    """Launch ``areal_actor_loss`` (or, with a ``reduction``, ``areal_actor_loss_stats`` without
+    the per-token statistic tensors) and return its outputs and the device counters."""
     lib = _lib.load()
     dev = _lib.require_gpu(proximal, mask_bool, logprobs, old, advantages)
     n = int(mask_bool.numel())
@@ -85,6 +151,9 @@ def _run_loss_kernel(
     has_loss = cfg.loss_kind != LOSS_NONE
     f32 = dict(dtype=torch.float32, device=dev)
     u8 = dict(dtype=torch.bool, device=dev)
+    if reduction is not None:
+        return _run_loss_kernel_reduced(lib, dev, cfg, n, n_seqs, uniform_len, cu, logprobs, proximal, old,
+                                        advantages, mask_bool, want_grad, reduction)
     out = {
         "loss": torch.empty((), **f32) if has_loss else None,
         "dlp": torch.empty(n, **f32) if (has_loss and want_grad) else None,
@@ -116,15 +185,58 @@ def _run_loss_kernel(
     return out
 
 
+def _run_loss_kernel_reduced(lib, dev, cfg, n, n_seqs, uniform_len, cu, logprobs, proximal, old,
+                             advantages, mask_bool, want_grad, reduction):
+    """The loss pass with the statistics reduced in the kernel: the only per-token outputs are
+    the gradient and, for the sequence-level importance ratio under rejection sampling, the
+    narrowed mask and behaviour weight that the per-sequence pass reads back."""
+    f32 = dict(dtype=torch.float32, device=dev)
+    need_seq_io = bool(cfg.rs_enabled and cfg.loss_kind == LOSS_PPO and cfg.seq_is)
+    out = {k: None for k in ("stat_loss", "ratio", "approx_kl", "clip_mask", "dual_clip_mask", "new_mask",
+                             "behave_imp_weight", "behave_approx_kl", "behave_mask")}
+    out["loss"] = torch.empty((), **f32)
+    out["dlp"] = torch.empty(n, **f32) if want_grad else None
+    if need_seq_io:
+        out["new_mask"] = torch.empty(n, dtype=torch.bool, device=dev)
+        out["behave_imp_weight"] = torch.empty(n, **f32)
+    # counters [8] and stats [17][4] share one buffer: one device-to-host copy serves both
+    n_stats = len(REDUCED_STAT_KEYS)
+    both = torch.empty(8 + 4 * n_stats, dtype=torch.float64, device=dev)
+    counters, stats = both[:8], both[8:]
+    extras = [_f32(t) for t in reduction.extras.values()]
+    for t in extras:
+        if t.numel() != n:
+            raise ValueError(f"extra statistic has {t.numel()} elements, expected {n}")
+    ent = _f32(reduction.entropy) if reduction.entropy is not None else None
+    if ent is not None and ent.numel() != n:
+        raise ValueError(f"entropy has {ent.numel()} elements, expected {n}")
+    nbytes = lib.areal_actor_loss_stats_workspace_bytes(n, n_seqs)
+    ws = _lib.workspace(nbytes, dev)
+    rc = lib.areal_actor_loss_stats(
+        _lib.ptr(logprobs), _lib.ptr(proximal), _lib.ptr(old), _lib.ptr(advantages),
+        _lib.ptr(mask_bool), _lib.ptr(cu), n, n_seqs, uniform_len, ctypes.byref(cfg),
+        _lib.ptr(ent), _lib.ptr(extras[0] if len(extras) > 0 else None),
+        _lib.ptr(extras[1] if len(extras) > 1 else None),
+        _lib.ptr(out["loss"]), _lib.ptr(out["dlp"]), None, None, None, None, None,
+        _lib.ptr(out["new_mask"]), _lib.ptr(out["behave_imp_weight"]), None, None,
+        _lib.ptr(counters), _lib.ptr(stats), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
+    )
+    _lib.check(rc, "areal_actor_loss_stats")
+    out["counters_dev"] = counters
+    out["counters_and_stats_dev"] = both
+    return out
+
+
 class _ActorLoss(torch.autograd.Function):
     """loss = sum(where(mask', pg, 0)) / N0 with the closed-form gradient w.r.t. logprobs."""
 
     @staticmethod
-    def forward(ctx, logprobs, cfg, shape, proximal, old, advantages, mask_bool, cu_seqlens, sink):
+    def forward(ctx, logprobs, cfg, shape, proximal, old, advantages, mask_bool, cu_seqlens, sink,
+                reduction=None):
         want_grad = logprobs.requires_grad
         lp = _f32(logprobs)
         out = _run_loss_kernel(cfg, shape, lp, proximal, old, advantages, mask_bool, cu_seqlens,
-                               want_grad)
+                               want_grad, reduction)
         sink.update(out)
         if want_grad:
             ctx.save_for_backward(out["dlp"], out["counters_dev"])
@@ -147,7 +259,7 @@ class _ActorLoss(torch.autograd.Function):
         grad = grad.view(ctx.shape)
         if ctx.in_dtype != torch.float32:
             grad = grad.to(ctx.in_dtype)
-        return (grad,) + (None,) * 8
+        return (grad,) + (None,) * 9
 
 
 def _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask):
@@ -212,7 +324,7 @@ def apply_rejection_sampling(
 
 
 def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-                 rejection_sampling, cu_seqlens):
+                 rejection_sampling, cu_seqlens, reduction=None):
     shape = logprobs.shape
     if rejection_sampling is not None:
         _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask)
@@ -220,13 +332,33 @@ def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, los
     _fill_rs(cfg, rejection_sampling)
     mask_bool = loss_mask.detach().bool().contiguous().view(-1)
     sink: dict = {}
+    # the behaviour log-probs enter the kernel for rejection sampling and, with a reduction,
+    # for the old_logp / logp_diff statistics
+    want_old = rejection_sampling is not None or (reduction is not None and old_logprobs is not None)
     loss = _ActorLoss.apply(
         logprobs, cfg, shape, _f32(proximal_logprobs),
-        _f32(old_logprobs) if (rejection_sampling is not None) else None,
-        _f32(advantages), mask_bool, cu_seqlens, sink,
+        _f32(old_logprobs) if want_old else None,
+        _f32(advantages), mask_bool, cu_seqlens, sink, reduction,
     )
-    c = sink["counters_dev"].cpu()  # the one host synchronisation of the call
+    if reduction is None:
+        c = sink["counters_dev"].cpu()  # the one host synchronisation of the call
+    else:
+        host = sink["counters_and_stats_dev"].cpu()  # counters and reduced statistics, one copy
+        c = host[:8]
+        reduction._fill(host[8:].view(-1, 4), c, int(mask_bool.numel()), rejection_sampling is not None,
+                        want_old)
     return loss, sink, c, shape
+
+
+def _scalar_stats(loss_mask, c):
+    n_total = float(loss_mask.numel())
+    n_valid = float(c[1])
+    return dict(
+        n_total_tokens=n_total,
+        n_valid_tokens=n_valid,
+        n_masked_tokens=n_total - n_valid,
+        masked_token_ratio=1.0 - n_valid / max(n_total, 1.0),
+    )
 
 
 def _rs_stats(stat, sink, c, shape, rejection_sampling):
@@ -252,10 +384,12 @@ def ppo_actor_loss_fn(
     rejection_sampling: RejectionSamplingConfig | None = None,
     importance_sampling_level: str = "token",
     cu_seqlens: torch.Tensor | None = None,
+    stat_reduction: StatReduction | None = None,
 ) -> tuple[torch.Tensor, dict]:
     """PPO/GRPO clipped surrogate with optional dual clip, GSPO sequence-level ratio and
     rejection sampling.  Signature, return structure and ``stat`` keys as in
-    ``functional.py:452-596``."""
+    ``functional.py:452-596``.  ``stat_reduction`` (not in the reference): reduce the logged
+    statistics in the kernel instead of returning per-token tensors, see ``StatReduction``."""
     if importance_sampling_level == "sequence":
         if logprobs.ndim == 1 and cu_seqlens is None:
             raise ValueError(
@@ -280,20 +414,20 @@ def ppo_actor_loss_fn(
     cfg.seq_is = int(importance_sampling_level == "sequence")
     loss, sink, c, shape = _loss_common(
         cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-        rejection_sampling, cu_seqlens,
+        rejection_sampling, cu_seqlens, stat_reduction,
     )
-    n_total = float(loss_mask.numel())
-    n_valid = float(c[1])
+    if stat_reduction is not None:
+        stat = _scalar_stats(loss_mask, c)
+        if rejection_sampling is not None:
+            stat["filtered_fraction"] = float(c[3]) / max(float(c[1]), 1.0)
+        return loss, stat
     stat = dict(
         loss=sink["stat_loss"].view(shape),
         importance_weight=sink["ratio"].view(shape),
         approx_kl=sink["approx_kl"].view(shape),
         clip_mask=sink["clip_mask"].view(shape),
         dual_clip_mask=sink["dual_clip_mask"].view(shape),
-        n_total_tokens=n_total,
-        n_valid_tokens=n_valid,
-        n_masked_tokens=n_total - n_valid,
-        masked_token_ratio=1.0 - n_valid / max(n_total, 1.0),
+        **_scalar_stats(loss_mask, c),
     )
     _rs_stats(stat, sink, c, shape, rejection_sampling)
     return loss, stat
@@ -309,9 +443,11 @@ def cispo_loss_fn(
     old_logprobs: torch.Tensor | None = None,
     rejection_sampling: RejectionSamplingConfig | None = None,
     cu_seqlens: torch.Tensor | None = None,
+    stat_reduction: StatReduction | None = None,
 ) -> tuple[torch.Tensor, dict]:
     """CISPO: clipped importance weight under stop-gradient times ``log pi`` (MiniMax-M1).
-    Signature, errors and ``stat`` keys as in ``functional.py:678-793``."""
+    Signature, errors and ``stat`` keys as in ``functional.py:678-793``; ``stat_reduction`` as in
+    ``ppo_actor_loss_fn``."""
     if eps_clip_higher is None or eps_clip_higher <= 0:
         raise ValueError(
             "CISPO requires a positive eps_clip_higher; the asymmetric upper "
@@ -323,8 +459,13 @@ def cispo_loss_fn(
     cfg.clip_hi = 1.0 + eps_clip_higher
     loss, sink, c, shape = _loss_common(
         cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-        rejection_sampling, cu_seqlens,
+        rejection_sampling, cu_seqlens, stat_reduction,
     )
+    if stat_reduction is not None:
+        stat = {}
+        if rejection_sampling is not None:
+            stat["filtered_fraction"] = float(c[3]) / max(float(c[1]), 1.0)
+        return loss, stat
     stat = dict(
         loss=sink["stat_loss"].view(shape),
         importance_weight=sink["ratio"].view(shape),

@@ -64,12 +64,30 @@ def grpo_loss_fn(
     vocab_mean_logits: torch.Tensor | None = None,
     vocab_norm_logits: torch.Tensor | None = None,
     stats: dict | None = None,
+    stats_mode: str = "tensors",
 ):
     """Actor loss of one packed micro-batch; returns the scalar loss.
 
-    ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``:
-    bool denominators and fp32 statistics, all of the micro-batch's token shape.
+    ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``.  With
+    ``stats_mode="tensors"`` these are the bool denominators and fp32 statistics of the
+    micro-batch's token shape, as in the reference.  With ``stats_mode="reduced"`` (PPO and CISPO
+    losses) no per-token statistic tensor is written at all: the loss kernel reduces every
+    logged statistic under its denominator in its own pass and ``stats[key]`` is
+    ``{"sum", "count", "avg", "min", "max", "denominator"}``, ``stats["denominator/<name>"]``
+    the token counts (what the tracker's export computes from the clones, ``actor.py:662-733``,
+    ``stats_tracker.py:455-560``); the proximal-approximation and staleness diagnostics, which
+    need per-token tensors, are not collected in that mode.
     """
+    if stats_mode not in ("tensors", "reduced"):
+        raise ValueError(f"stats_mode must be 'tensors' or 'reduced', got {stats_mode!r}")
+    reduction = None
+    if stats is not None and stats_mode == "reduced" and not use_sapo_loss:
+        from areal_amd.functional.functional import StatReduction
+
+        extras = {}
+        if vocab_min_logits is not None and vocab_max_logits is not None:
+            extras = dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits)
+        reduction = StatReduction(entropy=entropy, extras=extras)
     if prox_logp_method not in PROX_LOGP_METHODS_ALL:
         raise ValueError(f"'{prox_logp_method}' is not a valid ProxLogpMethod")
     old_logp = input_data["logprobs"]
@@ -121,6 +139,7 @@ def grpo_loss_fn(
             old_logprobs=old_logp,
             rejection_sampling=rejection_sampling,
             cu_seqlens=input_data.get("cu_seqlens"),
+            stat_reduction=reduction,
         )
     elif use_sapo_loss:
         if use_decoupled_loss:
@@ -151,6 +170,7 @@ def grpo_loss_fn(
             rejection_sampling=rejection_sampling,
             importance_sampling_level=importance_sampling_level,
             cu_seqlens=input_data.get("cu_seqlens"),
+            stat_reduction=reduction,
         )
 
     _raise_if_nonfinite(prox_nonfinite, prox_logp_method)
@@ -170,7 +190,18 @@ def grpo_loss_fn(
             loss = rl_loss_weight * loss + distill_loss_weight * value
             rkl_stat = term
 
-    if stats is not None:
+    if reduction is not None:
+        stats.update(reduction.results)
+        for name, count in reduction.denominators.items():
+            stats["denominator/" + name] = count
+        for key in ("n_total_tokens", "n_valid_tokens", "n_masked_tokens", "masked_token_ratio"):
+            if key in stat:
+                stats["scalar/" + key] = stat[key]
+        if "filtered_fraction" in stat:
+            stats["scalar/rs_filtered_fraction"] = stat["filtered_fraction"]
+        if rkl_stat is not None:
+            stats["rkl_loss"] = rkl_stat
+    elif stats is not None:
         lp = logprobs.detach()
         logp_diff = (old_logp - lp) * loss_mask
         stats.update(

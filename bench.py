@@ -256,6 +256,57 @@ def hbm_rooflines(dev):
 
     add("loss_token+loss_finalize+loss_grad_scale", "PPO + IcePop, 4 Mi tokens, fwd+bwd kernels through the C ABI, "
         "47 B/token + 8 B/token grad scale", 55 * Tl, timed(loss_kernels, iters=50))
+    # the same loss with every logged statistic reduced inside the token pass: no per-token
+    # statistic tensor is written (17 B/token of inputs + 4 B entropy read, 4 B gradient written)
+    ent = torch.rand(Tl, device=dev)
+    both = torch.empty(8 + 4 * len(F.REDUCED_STAT_KEYS), dtype=torch.float64, device=dev)
+    dlp = torch.empty(Tl, device=dev)
+    loss_out = torch.empty((), device=dev)
+    nb = lib.areal_actor_loss_stats_workspace_bytes(Tl, 0)
+    ws_r = torch.empty(nb, dtype=torch.uint8, device=dev)
+    import ctypes
+
+    def loss_kernels_reduced():
+        p = _lib.ptr
+        rc = lib.areal_actor_loss_stats(
+            p(lp32), p(prox), p(old), p(adv), p(mask_b), None, Tl, 0, 0, ctypes.byref(cfg), p(ent), None, None,
+            p(loss_out), p(dlp), None, None, None, None, None, None, None, None, None,
+            p(both[:8]), p(both[8:]), p(ws_r), nb, _lib.stream_ptr(dev))
+        _lib.check(rc, "areal_actor_loss_stats")
+        rc = lib.areal_actor_loss_grad(p(dlp), p(gout), p(both[:8]), p(grad), Tl, _lib.stream_ptr(dev))
+        _lib.check(rc, "areal_actor_loss_grad")
+
+    add("loss_token<stats>+loss_finalize+loss_stats_finalize+loss_grad_scale",
+        "PPO + IcePop, 4 Mi tokens, fwd+bwd kernels through the C ABI with the 13 logged statistics reduced in "
+        "the token pass instead of written as [T] tensors: 25 B/token + 8 B/token grad scale",
+        33 * Tl, timed(loss_kernels_reduced, iters=50))
+    from areal_amd.ppo.actor import grpo_loss_fn
+
+    gdata = dict(logprobs=old, advantages=adv, loss_mask=mask, prox_logp=prox)
+
+    def grpo_reduced():
+        lp.grad = None
+        st = {}
+        grpo_loss_fn(lp, ent, gdata, 0.2, None, None, rejection_sampling=rs, stats=st, stats_mode="reduced").backward()
+
+    def grpo_tensors():
+        lp.grad = None
+        st = {}
+        grpo_loss_fn(lp, ent, gdata, 0.2, None, None, rejection_sampling=rs, stats=st).backward()
+        masked_stats({k: st[k] for k in ("importance_weight", "approx_kl", "new_logp", "old_logp", "entropy",
+                                          "actor_loss", "clip_ratio", "dual_clip_ratio", "logp_diff",
+                                          "logp_abs_diff", "behave_filtered_ratio")},
+                     {k: st["n_valid_tokens"] for k in st})
+
+    from areal_amd.stats import masked_stats
+
+    add("grpo_loss_fn(stats_mode='reduced') + backward (API level)",
+        "PPO + IcePop with logging, 4 Mi tokens: statistics reduced in the loss pass, 25 + 8 B/token",
+        33 * Tl, timed(grpo_reduced))
+    add("grpo_loss_fn(stats_mode='tensors') + masked_stats + backward (API level)",
+        "the same logging through per-token tensors and a separate reduction launch: 47 + 8 B/token written and "
+        "read by the loss, 8 B of logp_diff tensors, then 11 x 5 B/token read by the reduction",
+        (47 + 8 + 8 + 55) * Tl, timed(grpo_tensors))
     # kernels of the steps either side of the loss (API level: each call includes its own host work)
     from areal_amd.functional import ppo_critic_loss_fn, sapo_loss_fn
     from areal_amd.packing import pack_tensor_dict

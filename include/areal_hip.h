@@ -171,6 +171,30 @@ int areal_actor_loss(const float* logprobs, const float* proximal_logprobs,
                      uint8_t* behave_mask, double* counters, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
 
+/* areal_actor_loss with the logging reductions folded into the token pass (replaces the clones
+ * and the masked sum / min / max per logged tensor of stats_tracker,
+ * areal/utils/stats_tracker.py:133-171, :455-560, as grpo_loss_fn uses them,
+ * areal/trainer/ppo/actor.py:662-733). stats [17][4] double = {sum, count, min, max} of, in this
+ * order: importance_weight, approx_kl, new_logp, old_logp, entropy, actor_loss, clip_ratio,
+ * dual_clip_ratio, logp_diff, logp_abs_diff, behave_filtered_ratio (under the loss mask before
+ * rejection), behave_imp_weight, behave_approx_kl (under the behave mask), clipped_new_logp,
+ * clipped_old_logp (under the clip mask), extra0, extra1 (over every token; e.g. the vocabulary
+ * min / max logits). min / max propagate NaN as torch.min / torch.max do; an empty denominator
+ * gives count 0, min +inf, max -inf. entropy, extra0, extra1 are optional per-token inputs. Every
+ * per-token output may be NULL: with only dlogprobs requested the call reads 17 (+4 entropy)
+ * bytes per token and writes 4. */
+size_t areal_actor_loss_stats_workspace_bytes(int64_t n_tokens, int64_t n_seqs);
+int areal_actor_loss_stats(const float* logprobs, const float* proximal_logprobs,
+                           const float* old_logprobs, const float* advantages,
+                           const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
+                           int64_t n_seqs, int64_t uniform_len, const areal_loss_config* cfg,
+                           const float* entropy, const float* extra0, const float* extra1,
+                           float* loss, float* dlogprobs, float* stat_loss, float* stat_ratio,
+                           float* stat_approx_kl, uint8_t* clip_mask, uint8_t* dual_clip_mask,
+                           uint8_t* new_mask, float* behave_imp_weight, float* behave_approx_kl,
+                           uint8_t* behave_mask, double* counters, double* stats, void* workspace,
+                           size_t workspace_bytes, areal_stream_t stream);
+
 /* areal_actor_loss without the workspace argument: the block partials and per-sequence
  * aggregates live in a static device array inside the library (about 1.6 MB per GPU, held until
  * the process ends), so nothing on the call path allocates. It has no counterpart in the

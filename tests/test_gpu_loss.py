@@ -230,3 +230,122 @@ def test_all_masked_and_determinism(dev):
     for l, s in outs[1:]:
         assert torch.equal(l, outs[0][0])  # bit-identical repeat runs
         assert torch.equal(s["loss"], outs[0][1]["loss"])
+
+
+# ---------------------------------------------------------------- statistics reduced in the loss pass
+REDUCED_VARIANTS = [
+    dict(),
+    dict(eps_clip_higher=0.28, c_clip=1.5, rs=RS_CONFIGS[0]),
+    dict(rs=RS_CONFIGS[5]),
+    dict(level="sequence", rs=RS_CONFIGS[6]),
+    dict(cispo=True, rs=RS_CONFIGS[0]),
+]
+
+
+@pytest.mark.parametrize("var", REDUCED_VARIANTS, ids=[str(i) for i in range(len(REDUCED_VARIANTS))])
+def test_reduced_stats_match_oracle_masked_stats(dev, var):
+    """grpo_loss_fn(stats_mode="reduced") writes no per-token statistic tensor; what it reports is
+    compared with the oracle's per-token stat tensors (assembled as actor.py:662-733 hands them to
+    the tracker) reduced by oracle.packing.masked_stats, the restatement of the tracker's masked
+    sum / min / max (stats_tracker.py:455-560)."""
+    from areal_amd.ppo.actor import grpo_loss_fn
+    from oracle.packing import masked_stats as oracle_masked_stats
+
+    n, n_seqs = 70_001, 24
+    lp, prox, old, adv, mask, cu = _random_batch(n, n_seqs, seed=31)
+    g = torch.Generator().manual_seed(32)
+    ent = torch.rand(n, generator=g) * 3
+    vmin, vmax = -torch.rand(n, generator=g) * 9 - 3, torch.rand(n, generator=g) * 20
+    rs = var.get("rs")
+    cispo = var.get("cispo", False)
+    hi = 4.0 if cispo else var.get("eps_clip_higher")
+    level = var.get("level", "token")
+
+    # oracle: per-token tensors, then the tracker's reductions
+    lp_o = lp.clone().requires_grad_(True)
+    if cispo:
+        lo, so = O.cispo_loss(lp_o, prox, adv, 0.2, mask, eps_clip_higher=hi, old_logprobs=old,
+                              rejection_sampling_cfg=rs, cu_seqlens=cu)
+        so["dual_clip_mask"] = torch.zeros(n, dtype=torch.bool)
+    else:
+        lo, so = O.ppo_actor_loss(lp_o, prox, old, adv, 0.2, mask, eps_clip_higher=hi, c_clip=var.get("c_clip"),
+                                  rejection_sampling_cfg=rs, importance_sampling_level=level, cu_seqlens=cu)
+    lo.backward()
+    lpd = lp_o.detach()
+    diff = (old - lpd) * mask
+    vals = dict(importance_weight=so["importance_weight"], approx_kl=so["approx_kl"], new_logp=lpd, old_logp=old,
+                entropy=ent, actor_loss=so["loss"], clip_ratio=so["clip_mask"].float(),
+                dual_clip_ratio=so["dual_clip_mask"].float(), logp_diff=diff, logp_abs_diff=diff.abs(),
+                clipped_new_logp=torch.where(so["clip_mask"], lpd, 0.0),
+                clipped_old_logp=torch.where(so["clip_mask"], old, 0.0),
+                vocab_min_logits=vmin, vocab_max_logits=vmax)
+    den = {k: mask for k in vals}
+    den["clipped_new_logp"] = den["clipped_old_logp"] = so["clip_mask"]
+    den["vocab_min_logits"] = den["vocab_max_logits"] = None
+    if rs is not None:
+        vals.update(behave_imp_weight=so["behave_imp_weight"], behave_approx_kl=so["behave_approx_kl"],
+                    behave_filtered_ratio=(mask & ~so["behave_mask"]).float())
+        den.update(behave_imp_weight=so["behave_mask"], behave_approx_kl=so["behave_mask"], behave_filtered_ratio=mask)
+    want = oracle_masked_stats(vals, den)
+
+    stats = {}
+    lp_g = lp.to(dev).requires_grad_(True)
+    data = dict(logprobs=old.to(dev), advantages=adv.to(dev), loss_mask=mask.to(dev), prox_logp=prox.to(dev),
+                cu_seqlens=cu.to(dev))
+    loss = grpo_loss_fn(lp_g, ent.to(dev), data, 0.2, hi, var.get("c_clip"),
+                        rejection_sampling=RejectionSamplingConfig(**rs) if rs else None,
+                        importance_sampling_level=level, use_cispo_loss=cispo,
+                        vocab_min_logits=vmin.to(dev), vocab_max_logits=vmax.to(dev),
+                        stats=stats, stats_mode="reduced")
+    loss.backward()
+    torch.testing.assert_close(loss.detach().cpu(), lo.detach(), rtol=1e-4, atol=1e-7)
+    rel = (lp_g.grad.cpu() - lp_o.grad).norm() / lp_o.grad.norm()
+    assert rel < 1e-2
+    assert not any(torch.is_tensor(v) for v in stats.values())  # nothing of token shape comes back
+    assert set(want) <= set(stats), sorted(set(want) - set(stats))
+    for k, w in want.items():
+        got = stats[k]
+        assert got["count"] == w["count"], k
+        if w["count"] == 0:
+            assert got["avg"] is None and got["min"] is None and got["max"] is None, k
+            continue
+        assert got["sum"] == pytest.approx(w["sum"], rel=2e-5, abs=1e-4 * max(1.0, w["count"]) * 1e-3), k
+        assert got["min"] == pytest.approx(w["min"], rel=2e-6, abs=1e-6), k
+        assert got["max"] == pytest.approx(w["max"], rel=2e-6, abs=1e-6), k
+    assert stats["denominator/n_valid_tokens"] == float(mask.sum())
+    assert stats["denominator/clipped_tokens"] == float(so["clip_mask"].sum())
+    assert stats["denominator/n_tokens"] == float(n)
+    if rs is not None:
+        assert stats["denominator/unclipped_behave_tokens"] == float(so["behave_mask"].sum())
+        assert stats["scalar/rs_filtered_fraction"] == pytest.approx(so["filtered_fraction"], abs=1e-12)
+
+
+def test_reduced_stats_agree_with_the_tensor_mode_on_the_gpu(dev):
+    """The same call in both modes: the reduced values equal masked_stats of the tensors the
+    default mode returns, and the loss and gradient are bit-identical."""
+    from areal_amd.ppo.actor import grpo_loss_fn
+    from areal_amd.stats import masked_stats
+
+    n = 200_000
+    lp, prox, old, adv, mask, cu = _random_batch(n, 50, seed=41)
+    rs = RejectionSamplingConfig(**RS_CONFIGS[1])
+    data = dict(logprobs=old.to(dev), advantages=adv.to(dev), loss_mask=mask.to(dev), prox_logp=prox.to(dev))
+    ent = torch.rand(n, device=dev)
+    out = {}
+    for mode in ("tensors", "reduced"):
+        st = {}
+        x = lp.to(dev).requires_grad_(True)
+        loss = grpo_loss_fn(x, ent, data, 0.2, 0.28, 3.0, rejection_sampling=rs, stats=st, stats_mode=mode)
+        loss.backward()
+        out[mode] = (loss.detach(), x.grad, st)
+    assert torch.equal(out["tensors"][0], out["reduced"][0]) and torch.equal(out["tensors"][1], out["reduced"][1])
+    t, r = out["tensors"][2], out["reduced"][2]
+    keys = ["importance_weight", "approx_kl", "new_logp", "old_logp", "entropy", "actor_loss", "clip_ratio",
+            "logp_abs_diff"]
+    want = masked_stats({k: t[k] for k in keys}, {k: t["n_valid_tokens"] for k in keys})
+    want.update(masked_stats({"behave_imp_weight": t["behave_imp_weight"]},
+                             {"behave_imp_weight": t["unclipped_behave_tokens"]}))
+    for k, w in want.items():
+        assert r[k]["count"] == w["count"]
+        assert r[k]["sum"] == pytest.approx(w["sum"], rel=1e-9, abs=1e-9), k
+        assert r[k]["min"] == w["min"] and r[k]["max"] == w["max"], k
