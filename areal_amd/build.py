@@ -6,7 +6,9 @@ sources.  ``python -m areal_amd.build`` rebuilds it.
 
 from __future__ import annotations
 
+import importlib.util
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -54,18 +56,70 @@ def _compile_one(src: Path, obj: Path) -> None:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{proc.stderr}")
 
 
+def generate_mainloop() -> Path:
+    """Write ``csrc/mainloop16.inc``, the hand-scheduled k-loop that ``lmhead.hip`` includes."""
+    spec = importlib.util.spec_from_file_location("gen_mainloop16", CSRC / "gen_mainloop16.py")
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    path = CSRC / "mainloop16.inc"
+    text = gen.emit()
+    if not path.exists() or path.read_text() != text:
+        path.write_text(text)
+    return path
+
+
+def check_accumulator_registers(asm_text: str) -> int:
+    """Verify what the hand-scheduled kernels rely on, on the compiler's own output.
+
+    ``gemm16_sweep`` keeps its 256 accumulators in ``a[0:255]`` between assembly blocks without
+    the compiler knowing (the main loop only lists them as clobbered, and the epilogues fetch
+    them with ``v_accvgpr_read`` blocks).  That is sound as long as no instruction the compiler
+    emits itself in those kernels touches an accumulator register, e.g. to park a spilled VGPR
+    there.  Returns the number of kernels checked; raises if one fails.
+    """
+    checked = 0
+    for m in re.finditer(r"^(\S*gemm16_sweep\S*):[^\n]*\n(.*?)^\.Lfunc_end", asm_text, re.S | re.M):
+        name, body = m.group(1), m.group(2)
+        in_block = False
+        for line in body.split("\n"):
+            if "#ASMSTART" in line:
+                in_block = True
+            elif "#ASMEND" in line:
+                in_block = False
+            elif not in_block:
+                code = line.split(";")[0]
+                if re.search(r"\ba(\d+|\[\d+:\d+\])(?![\w.])", code):
+                    raise RuntimeError(f"compiler-generated use of an accumulator register in {name}:\n{line}")
+        checked += 1
+    if checked == 0:
+        raise RuntimeError("no gemm16_sweep kernel found in the device assembly of lmhead.hip")
+    return checked
+
+
+def _check_lmhead(build_dir: Path) -> None:
+    asm = build_dir / "lmhead.gfx950.s"
+    cmd = [_hipcc(), *HIPCC_FLAGS, "--cuda-device-only", "-S", str(CSRC / "lmhead.hip"), "-o", str(asm)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed for lmhead.hip:\n{proc.stderr}")
+    check_accumulator_registers(asm.read_text())
+
+
 def build_all(verbose: bool = True) -> Path:
     """Compile every ``csrc/*.hip`` for gfx950 and link ``libareal_hip.so``."""
     build_dir = CSRC / "build"
     build_dir.mkdir(exist_ok=True)
+    generate_mainloop()
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC}")
     objs = [build_dir / (s.stem + ".o") for s in srcs]
     if verbose:
         print(f"[areal_amd.build] compiling {len(srcs)} HIP sources for gfx950", flush=True)
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs) + 1)) as pool:
+        check = pool.submit(_check_lmhead, build_dir)
         list(pool.map(_compile_one, srcs, objs))
+        check.result()
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -24,6 +24,7 @@
 // (areal/models/mcore/vocab_parallel_head.py:564-735 forward, :737-938 backward) and the
 // backward formula of areal/utils/functional/vocab_parallel_kernels.py:99-137.
 #include "common.hpp"
+#include "mainloop16.inc"
 
 namespace {
 
@@ -1342,6 +1343,515 @@ __global__ void cast_f32_to_bf16_kernel(const float* __restrict__ src, u16* __re
     for (int64_t j = n & ~(int64_t)3; j < n; ++j) dst[j] = f32_to_bf16_bits(src[j]);
 }
 
+
+// =======================================================================================
+// The contraction with the hand-scheduled main loop (mainloop16.inc, written by
+// gen_mainloop16.py): v_mfma_f32_16x16x32_bf16, accumulators in a[0:255], k-loop as one assembly
+// block per output tile. Same tile (256 x 256 x 64, four waves of 128 x 128), same operand
+// layouts as the three kernels above (nt / tn / mix), for K % 128 == 0.
+//
+// Accumulator layout of a wave: block (ia, jb) of 16 x 16, register r of a lane:
+//   i = ia*16 + 4*(lane/16) + r     (A row inside the wave's 128)
+//   j = jb*16 + (lane%16)           (B row inside the wave's 128)
+// and block (ia, jb) sits in tuple t[ia*2 + jb/4], elements (jb%4)*4 .. +3.
+// =======================================================================================
+//
+// The compiler does not know that values live in a[0:255] between the main loop's block (which
+// lists them as clobbered) and the blocks with which the epilogues fetch them, one block column
+// (fixed jb: 16 output rows j) at a time, x[ia * 4 + r]. The build checks on the generated
+// assembly that no compiler-emitted instruction of these kernels touches an accumulator register.
+template <int JB>
+DEVI void acc_col(float (&x)[32]) {
+  if constexpr (JB == 0) asm volatile(ML16_READ_COL0 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 1) asm volatile(ML16_READ_COL1 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 2) asm volatile(ML16_READ_COL2 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 3) asm volatile(ML16_READ_COL3 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 4) asm volatile(ML16_READ_COL4 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 5) asm volatile(ML16_READ_COL5 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else if constexpr (JB == 6) asm volatile(ML16_READ_COL6 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+  else asm volatile(ML16_READ_COL7 : ML16_COL_OUTPUTS(x) : : ML16_ACC_CLOBBERS);
+}
+// Nothing the compiler allocates may sit in an accumulator register across this point. Its
+// register allocator treats free accumulator registers as good homes for long-lived values, and
+// it believes them free after the main loop; with these fences (and the same clobber list on
+// every acc_col block) only a value defined and last used between two neighbouring fences could
+// still land there, which the build's check of the assembly would report.
+#define ML16_AGPR_FENCE() asm volatile("" ::: ML16_ACC_CLOBBERS)
+template <int N> struct IntC { static constexpr int value = N; };
+template <int JB = 0, class F>
+DEVI void for_each_col(F&& f) {
+  if constexpr (JB < 8) {
+    f(IntC<JB>{});
+    for_each_col<JB + 1>(f);
+  }
+}
+
+constexpr int RING16_BYTES = 2 * ML16_OPER_BYTES;  // [A stage 0][A stage 1][B stage 0][B stage 1]
+// Per-wave staging area behind the ring: one block column of the wave's sub-tile (16 output rows
+// j x 128 values i in bf16) is transposed through it so that global stores cover whole lines.
+constexpr int STAGE16_PITCH = 272;                 // bytes per j row: 256 + 16 (conflict-free)
+constexpr int STAGE16_BYTES = 16 * STAGE16_PITCH;  // per wave
+enum { VAR_NT = 0, VAR_TN = 1, VAR_MIX = 2 };
+
+// chunk swizzle of a k-contiguous stage row (measured: 0 LDS bank conflicts for the 16-row
+// fragment reads, lane l on row l % 16 at chunk ks * 4 + l / 16)
+DEVI int swz16(int r) { return r & 7; }
+
+// Per-lane byte offsets of the 8 direct loads of one operand half, and the LDS read addresses
+// (stage 0) of its fragments. KM: k-major operand (`tile` = its 256-column tile, nvalid = readable
+// columns); otherwise k-contiguous (nvalid = rows).
+template <bool KM>
+DEVI void setup_operand16(int64_t ld, int tile, int nvalid, int W, int oper, int wave, int lane,
+                          uint32_t lds_base, uint32_t (&off)[8], uint32_t (&rd)[8]) {
+  if (!KM) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = wave * 64 + i * 8 + (lane >> 3);
+      const int rr = tile * TILE + r < nvalid ? r : nvalid - 1 - tile * TILE;  // clamped rows are discarded later
+      off[i] = 2u * ((uint32_t)rr * (uint32_t)ld + (uint32_t)(((lane & 7) ^ swz16(r)) * 8));
+    }
+    const int rl = lane & 15, kg = lane >> 4, sw = swz16(rl);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+      rd[ks] = lds_base + oper * ML16_OPER_BYTES + (W * 128 + rl) * 128 + (((ks * 4 + kg) ^ sw) * 16);
+  } else {
+    // instruction i of a wave fills k-rows wave*16 + 2*i + (lane >> 5); the 64-byte chunks of a
+    // row are swizzled with k & 3 and the halves of a chunk swapped in rows with k & 8
+    const int hl = lane >> 5, piece = lane & 31;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int kr = wave * 16 + 2 * i + hl;
+      const int k3 = kr & 3, cf = ((kr >> 3) & 1) * 2;
+      int gp = tile * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + ((piece & 3) ^ cf);
+      const int last = nvalid / 8 - 1;
+      gp = gp < last ? gp : last;  // columns past the end are discarded later
+      off[i] = 2u * ((uint32_t)kr * (uint32_t)ld + (uint32_t)(gp * 8));
+    }
+    const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
+#pragma unroll
+    for (int x = 0; x < 8; ++x)
+      rd[x] = lds_base + oper * ML16_OPER_BYTES + (G * 8 + r4) * 512 + (((W * 4 + (x >> 1)) ^ r4) << 6) +
+              ((((x & 1) ^ G) & 1) << 5) + (q & 3) * 8;
+  }
+}
+
+// A workgroup sweeps the A tiles [ai_begin, ai_end) against one B tile. Requirements checked by
+// the host: K % 128 == 0; a sweep of more than one A tile has only full A tiles and a
+// k-contiguous A (the loader's lane offsets are those of the first tile); split-K ranges are an
+// even number of k-tiles.
+template <int VAR, class Epi>
+__global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, typename Epi::Params ep) {
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[RING16_BYTES + 4 * STAGE16_BYTES];
+  constexpr bool A_KM = VAR != VAR_NT, B_KM = VAR == VAR_TN;
+  int bj, split, ai_begin, ai_end;
+  int wg = blockIdx.x, nk = g.K / BK;
+  if (g.ksplit > 1) {
+    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
+    const int z = wg / per_copy;
+    wg -= z * per_copy;
+    wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);  // copies start on different XCDs
+    const int kt0 = z * g.kt_per_split;
+    nk -= kt0;
+    nk = nk < g.kt_per_split ? nk : g.kt_per_split;
+    g.A += A_KM ? (int64_t)kt0 * BK * g.lda : (int64_t)kt0 * BK;
+    g.B += B_KM ? (int64_t)kt0 * BK * g.ldb : (int64_t)kt0 * BK;
+    Epi::split_output(ep, (int64_t)z * g.zstride);
+    if (nk <= 0) return;
+  }
+  if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave >> 1, wb = wave & 1;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_AS(lds);
+
+  uint32_t oa[8], ob[8], ra[8], rb[8];
+  setup_operand16<A_KM>(g.lda, ai_begin, A_KM ? g.acols : g.M, wa, 0, wave, lane, lds_base, oa, ra);
+  setup_operand16<B_KM>(g.ldb, bj, B_KM ? g.bcols : g.N, wb, 1, wave, lane, lds_base, ob, rb);
+
+  // pointers to the next k-tile to fetch and their advance per k-tile in bytes. A k-major
+  // operand's tile column is part of the lane offsets, so its pointer only carries the k offset.
+  const uint32_t stride_a = A_KM ? (uint32_t)(BK * g.lda * 2) : 128u;
+  const uint32_t stride_b = B_KM ? (uint32_t)(BK * g.ldb * 2) : 128u;
+  auto a_tile_ptr = [&](int ai) -> const char* {
+    return (const char*)(A_KM ? g.A : g.A + (int64_t)ai * TILE * g.lda);
+  };
+  const char* pa = a_tile_ptr(ai_begin);
+  const char* pb = (const char*)(B_KM ? g.B : g.B + (int64_t)bj * TILE * g.ldb);
+  const char* pb_next = pb;
+  const uint32_t ldsw = lds_base + (uint32_t)wave * 8192u;
+  const int npairs = nk >> 1;
+  u16* stage = (u16*)(lds + RING16_BYTES + wave * STAGE16_BYTES);
+
+  if (VAR == VAR_NT)
+    asm volatile(ML16_NT_PROLOGUE
+                 : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb)
+                 : ML16_S_LDSW(ldsw), ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                   ML16_NT_VGPR_INPUTS(oa, ob, ra, rb)
+                 : "memory", "scc");
+  else if (VAR == VAR_TN)
+    asm volatile(ML16_TN_PROLOGUE
+                 : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb)
+                 : ML16_S_LDSW(ldsw), ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                   ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
+                 : "memory", "scc");
+  else
+    asm volatile(ML16_MIX_PROLOGUE
+                 : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb)
+                 : ML16_S_LDSW(ldsw), ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                   ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
+                 : "memory", "scc");
+
+  // Epilogue state does not stay in registers over the main loop, which leaves the compiler only
+  // v[0:ML16_*_FIRST_VGPR): an epilogue that carries values from tile to tile of a sweep keeps
+  // them in memory between its close() and the next open().
+  for (int ai = ai_begin; ai < ai_end; ++ai) {
+    // where the loader goes when this tile's k range is exhausted: the next A tile of the
+    // sweep, or (after the last tile) this tile again, whose first k-tiles are loaded and never used
+    const char* pa_next = a_tile_ptr(ai + 1 < ai_end ? ai + 1 : ai);
+    int cnt = npairs;
+    if (npairs == 1) { pa = pa_next; pb = pb_next; }
+    if (VAR == VAR_NT)
+      asm volatile(ML16_NT_TILE
+                   : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
+                   : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                     ML16_NT_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_NT_CLOBBERS, ML16_ACC_CLOBBERS);
+    else if (VAR == VAR_TN)
+      asm volatile(ML16_TN_TILE
+                   : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
+                   : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                     ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_TN_CLOBBERS, ML16_ACC_CLOBBERS);
+    else
+      asm volatile(ML16_MIX_TILE
+                   : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
+                   : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
+                     ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_MIX_CLOBBERS, ML16_ACC_CLOBBERS);
+    // The lane number goes through an empty block so that nothing of the epilogue's per-lane
+    // address arithmetic is computed ahead of the main loop, which leaves the compiler only
+    // v[0:ML16_*_FIRST_VGPR) for values that live across it.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    typename Epi::State st;
+    Epi::open(st, ep, bj * TILE + wb * 128, split, wa, lane_e, ai == ai_begin);
+    Epi::tile(st, ep, ai * TILE + wa * 128, bj * TILE + wb * 128, lane_e, stage);
+    Epi::close(st, ep, bj * TILE + wb * 128, split, wa, lane_e);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
+}
+
+// One block column of the wave's sub-tile (16 rows j x 128 bf16 values i) from the staging area
+// to global memory: lane -> (row 4*p + lane/16, 16-byte piece lane%16), so 16 lanes write the
+// 256 contiguous bytes of a row. out_row0 points at element (j0, i0) of the output.
+template <bool EDGE>
+DEVI void flush_stage16(const u16* stage, u16* out_row0, int64_t ld, int rows_valid, int cols_valid, int lane) {
+  const int piece = lane & 15;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int row = p * 4 + (lane >> 4);
+    const u32x4 v = *(const u32x4*)((const char*)stage + row * STAGE16_PITCH + piece * 16);
+    if (!EDGE || (row < rows_valid && piece * 8 < cols_valid))
+      *(u32x4*)(out_row0 + (int64_t)row * ld + piece * 8) = v;
+  }
+}
+DEVI void stage16_put(u16* stage, int lane, int ia, u32x2 v) {
+  *(u32x2*)((char*)stage + (lane & 15) * STAGE16_PITCH + (ia * 16 + 4 * (lane >> 4)) * 2) = v;
+}
+
+// ---- plain store (dHidden, dWeight, stand-alone GEMM): out[j * ldo + i]
+template <bool EDGE, int MODE>
+struct Store16 {
+  typedef StoreParams Params;
+  struct State {};
+  static DEVI void open(State&, const Params&, int, int, int, int, bool) {}
+  static DEVI void close(State&, const Params&, int, int, int, int) {}
+  static DEVI void split_output(Params& p, int64_t bytes) { p.out = (char*)p.out + bytes; }
+  static DEVI void tile(State&, const Params& p, int i0, int j0, int lane, u16* stage) {
+    for_each_col([&](auto bc) {
+      constexpr int b = decltype(bc)::value;
+      float x[32];
+      acc_col<b>(x);
+      const int j = j0 + b * 16 + (lane & 15);
+      if (MODE == 0 || MODE == 3) {
+        // bf16: through the staging area, whole lines out (needs 16-byte aligned rows: the host
+        // only takes this path when ldo % 8 == 0 and the output is 16-byte aligned)
+        float js = 1.f;
+        if (MODE == 3) js = (!EDGE || j < p.N) ? p.jscale[j] : 0.f;
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+          float x0 = x[a * 4], x1 = x[a * 4 + 1], x2 = x[a * 4 + 2], x3 = x[a * 4 + 3];
+          if (MODE == 3) { x0 *= js; x1 *= js; x2 *= js; x3 *= js; }
+          u32x2 v;
+          v[0] = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
+          v[1] = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
+          stage16_put(stage, lane, a, v);
+        }
+        flush_stage16<EDGE>(stage, (u16*)p.out + (int64_t)(j0 + b * 16) * p.ldo + i0, p.ldo,
+                            p.N - (j0 + b * 16), p.M - i0, lane);
+      } else {
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+          const int i = i0 + a * 16 + 4 * (lane >> 4);
+          if (!EDGE || (j < p.N && i < p.M)) {
+            f32x4* dst = (f32x4*)((float*)p.out + (int64_t)j * p.ldo + i);
+            f32x4 v = {x[a * 4], x[a * 4 + 1], x[a * 4 + 2], x[a * 4 + 3]};
+            if (MODE == 2) v += *dst;
+            *dst = v;
+          }
+        }
+      }
+    });
+  }
+};
+template <bool E> using Store16Bf16 = Store16<E, 0>;
+template <bool E> using Store16F32 = Store16<E, 1>;
+template <bool E> using Accum16F32 = Store16<E, 2>;
+template <bool E> using Store16Bf16Scaled = Store16<E, 3>;
+
+
+// ---- forward: online softmax statistics (see FwdEpi); a lane owns one token per block column
+// and 4 vocabulary entries per block, so 8 tokens x 32 entries per tile. Partial statistics go
+// to slot split*8 + wa*4 + lane/16.
+template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
+struct Fwd16 {
+  typedef FwdParams Params;
+  struct State {
+    float m[8], s[8], q[8], xl[8], mn[8], sx[MOMENTS ? 8 : 1], sx2[MOMENTS ? 8 : 1];
+    int lab[8];
+  };
+  static DEVI void split_output(Params&, int64_t) {}
+  // The running statistics of a sweep live in the workspace slots that the merge kernel reads
+  // (written by close() after every tile, read back by the next open()).
+  static DEVI void open(State& st, const Params& p, int t0, int split, int wa, int lane, bool first) {
+    const int slot = p.slot_base + split * 8 + wa * 4 + (lane >> 4);
+    const int64_t PT = (int64_t)p.P * p.T;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int t = t0 + b * 16 + (lane & 15);
+      const bool live = !EDGE || t < p.T;
+      int64_t l = live ? p.labels[t] : -1;
+      st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+      if (first || !live) {
+        st.m[b] = neg_inf(); st.s[b] = 0.f; st.q[b] = 0.f; st.xl[b] = 0.f;
+        st.mn[b] = pos_inf();
+        if (MOMENTS) { st.sx[b] = 0.f; st.sx2[b] = 0.f; }
+      } else {
+        const float* w = p.ws + (int64_t)slot * p.T + t;
+        st.m[b] = w[0 * PT]; st.s[b] = w[1 * PT]; st.q[b] = w[2 * PT]; st.xl[b] = w[3 * PT];
+        st.mn[b] = w[4 * PT];
+        if (MOMENTS) { st.sx[b] = w[5 * PT]; st.sx2[b] = w[6 * PT]; }
+      }
+      ML16_AGPR_FENCE();
+    }
+  }
+
+  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
+    const int vl = v0 + 4 * (lane >> 4);
+    auto vidx = [&](int a, int r) { return vl + a * 16 + r; };
+    for_each_col([&](auto bc) {
+      constexpr int b = decltype(bc)::value;
+      float x[32];
+      acc_col<b>(x);
+      if (AFFINE) {
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float bv = 0.f;
+            if (p.bias != nullptr && (!EDGE || vidx(a, r) < p.V)) bv = p.bias[vidx(a, r)];
+            x[a * 4 + r] = (x[a * 4 + r] + bv) * p.scale;
+          }
+      }
+      const int tok = t0 + b * 16 + (lane & 15);
+      float rr = 0.f;  // SAVE: the token's row reference
+      if (SAVE && (!EDGE || tok < p.T)) rr = p.probs_ref[tok];
+      float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
+#pragma unroll
+      for (int a = 0; a < 8; ++a) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float xv = x[a * 4 + r];
+          if (!EDGE || vidx(a, r) < p.V) {
+            tmax = fmaxf(tmax, xv);
+            tmin = fminf(tmin, xv);
+            if (MOMENTS) { sx += xv; sx2 = fmaf(xv, xv, sx2); }
+          }
+        }
+      }
+      ML16_AGPR_FENCE();
+      st.mn[b] = fminf(st.mn[b], tmin);
+      if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
+      const float m_old = st.m[b];
+      const float m_new = fmaxf(m_old, tmax);
+      // rescale the running sums to the new reference (see ref_of); on the first tile
+      // m_old = -inf and s = q = 0, so the factor is taken as 2^0 instead of evaluating -inf - x
+      float s = st.s[b], q = st.q[b];
+      const float mc = (!EDGE || m_new > neg_inf()) ? ref_of(m_new, p.c2) : 0.f;
+      const float dl = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
+      const float alpha = fast_exp2(dl);
+      q = alpha * fmaf(dl, s, q);
+      s = alpha * s;
+      if (!SAVE) {
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float t = fmaf(x[a * 4 + r], p.c2, -mc);
+            const float e = fast_exp2(t);
+            if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          ML16_AGPR_FENCE();
+        }
+      } else {
+        // The sums take the exponentials relative to the running maximum (in (0, 1] whatever
+        // the row reference is); what is stored is the same exponential moved to the row
+        // reference by one factor per (token, tile). That factor over- or underflows only where
+        // the stored value is not used: rows outside the reference window, and tiles whose
+        // maximum lies 126 binades below the row's. The 16 tokens x 128 entries of this block
+        // column go through the staging area and leave as whole lines.
+        const float gamma = fast_exp2(mc - rr);
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+          const int vq = vl + a * 16;
+          u16 d[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const float t = fmaf(x[a * 4 + k], p.c2, -mc);
+            const float e = fast_exp2(t);
+            float es = e * gamma;
+            if (EDGE && vq + k >= p.V) es = 0.f;
+            else { s += e; q = fmaf(t, e, q); }
+            d[k] = f32_to_bf16_bits(es);
+          }
+          u32x2 pk;
+          pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
+          pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+          stage16_put(stage, lane, a, pk);
+          // keeps the exponentials of one block next to the sums that consume them (left alone,
+          // the scheduler computes all 32 first and spills them)
+          __builtin_amdgcn_sched_barrier(0);
+          ML16_AGPR_FENCE();
+        }
+        flush_stage16<EDGE>(stage, p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv,
+                            p.T - (t0 + b * 16), (int)p.ldv - v0, lane);
+      }
+      // The sums pass through an empty block here: their only readers come after the last
+      // column, and the compiler otherwise moves the two summation chains of every column down
+      // there, keeping all the exponentials alive (in scratch memory) until then.
+      asm volatile("" : "+v"(s), "+v"(q) : : ML16_ACC_CLOBBERS);
+      st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
+      const int lab = st.lab[b];
+      const bool hit = (lab >= v0) && (lab < v0 + 128);
+      if (__builtin_amdgcn_ballot_w64(hit) != 0) {
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (vidx(a, r) == lab) st.xl[b] = x[a * 4 + r];
+      }
+      // everything this column updated is final here (see the note on the sums above)
+      asm volatile("" : "+v"(st.m[b]), "+v"(st.xl[b]), "+v"(st.mn[b]) : : ML16_ACC_CLOBBERS);
+      if (MOMENTS) asm volatile("" : "+v"(st.sx[b]), "+v"(st.sx2[b]));
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+
+  static DEVI void close(State& st, const Params& p, int t0, int split, int wa, int lane) {
+    const int slot = p.slot_base + split * 8 + wa * 4 + (lane >> 4);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int t = t0 + b * 16 + (lane & 15);
+      if (EDGE && t >= p.T) continue;
+      const int64_t PT = (int64_t)p.P * p.T;
+      float* w = p.ws + (int64_t)slot * p.T + t;
+      w[0 * PT] = st.m[b]; w[1 * PT] = st.s[b]; w[2 * PT] = st.q[b]; w[3 * PT] = st.xl[b];
+      w[4 * PT] = st.mn[b];
+      if (MOMENTS) { w[5 * PT] = st.sx[b]; w[6 * PT] = st.sx2[b]; }
+      ML16_AGPR_FENCE();
+    }
+  }
+};
+template <bool E> using Fwd16Plain = Fwd16<E, false, false, false>;
+template <bool E> using Fwd16PlainMom = Fwd16<E, false, true, false>;
+template <bool E> using Fwd16Affine = Fwd16<E, true, false, false>;
+template <bool E> using Fwd16AffineMom = Fwd16<E, true, true, false>;
+template <bool E> using Fwd16PlainSave = Fwd16<E, false, false, true>;
+template <bool E> using Fwd16PlainMomSave = Fwd16<E, false, true, true>;
+template <bool E> using Fwd16AffineSave = Fwd16<E, true, false, true>;
+template <bool E> using Fwd16AffineMomSave = Fwd16<E, true, true, true>;
+
+// ---- recompute: dlogits = (onehot - p) * g * invT * scale in bf16, [Tc, ldv] (see BwdEpi)
+template <bool EDGE, bool AFFINE>
+struct Bwd16 {
+  typedef BwdParams Params;
+  struct State {
+    float nb[8], gs[8];
+    int lab[8];
+  };
+  static DEVI void open(State& st, const Params& p, int t0, int, int, int lane, bool) {
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const int t = t0 + b * 16 + (lane & 15);
+      if (!EDGE || t < p.T) {
+        const int64_t l = p.labels[t];
+        st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+        st.nb[b] = -ref_plus(p.row_max[t], p.c2, fast_log2(p.sum_exp[t]));
+        st.gs[b] = p.grad[t] * p.inv_temp * p.scale;
+      } else {
+        st.lab[b] = -1; st.nb[b] = 0.f; st.gs[b] = 0.f;
+      }
+    }
+  }
+  static DEVI void close(State&, const Params&, int, int, int, int) {}
+  static DEVI void split_output(Params&, int64_t) {}
+
+  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
+    const int vl = v0 + 4 * (lane >> 4);
+    for_each_col([&](auto bc) {
+      constexpr int b = decltype(bc)::value;
+      float x[32];
+      acc_col<b>(x);
+      const int t = t0 + b * 16 + (lane & 15);
+      const float nb = st.nb[b], gs = st.gs[b];
+      const int lab = st.lab[b];
+#pragma unroll
+      for (int a = 0; a < 8; ++a) {
+        const int vq = vl + a * 16;
+        u16 d[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = vq + e;
+          float xv = x[a * 4 + e];
+          if (AFFINE) {
+            float bv = 0.f;
+            if (p.bias != nullptr && (!EDGE || v < p.V)) bv = p.bias[v];
+            xv = (xv + bv) * p.scale;
+          }
+          const float pr = fast_exp2(fmaf(xv, p.c2, nb));
+          float dv = -pr * gs;
+          if (v == lab) dv += gs;
+          if (EDGE && (v >= p.V || t >= p.T)) dv = 0.f;
+          d[e] = f32_to_bf16_bits(dv);
+        }
+        u32x2 pk;
+        pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
+        pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+        stage16_put(stage, lane, a, pk);
+      }
+      flush_stage16<EDGE>(stage, p.dl + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv, p.T - (t0 + b * 16),
+                          (int)p.ldv - v0, lane);
+    });
+  }
+};
+template <bool E> using Bwd16Plain = Bwd16<E, false>;
+template <bool E> using Bwd16Affine = Bwd16<E, true>;
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // Splits of the A range per B tile: enough workgroups to fill the chip, and at least 4 so that
@@ -1354,7 +1864,11 @@ int pick_splits(int nbj, int nai, int target_wgs) {
   return S;
 }
 
-enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2, KERNEL_MIX = 3 };
+enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2, KERNEL_MIX = 3,
+       KERNEL16_NT = 4, KERNEL16_TN = 5, KERNEL16_MIX = 6 };
+
+// K ranges the hand-scheduled main loop takes: whole pairs of k-tiles.
+bool k16_ok(int64_t K) { return K >= 2 * BK && K % (2 * BK) == 0; }
 
 template <class Epi, int KERNEL>
 int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
@@ -1379,6 +1893,16 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
     hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
   }
+  else if constexpr (KERNEL >= KERNEL16_NT) {
+    constexpr int VAR = KERNEL == KERNEL16_NT ? VAR_NT : KERNEL == KERNEL16_TN ? VAR_TN : VAR_MIX;
+    if (g.lda > (VAR == VAR_NT ? (1 << 22) : (1 << 24)) || g.ldb > (VAR == VAR_TN ? (1 << 24) : (1 << 22)))
+      return AREAL_ERR_UNSUPPORTED;
+    if (!k16_ok(g.K) || (g.ksplit > 1 && (g.kt_per_split & 1))) return AREAL_ERR_UNSUPPORTED;
+    // a k-major A operand carries its tile column in the lane offsets: one A tile per workgroup
+    if (VAR != VAR_NT && S != nai) return AREAL_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((gemm16_sweep<VAR, Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
+                       dim3(NTHREADS), 0, stream, g, sc, ep);
+  }
   else
     hipLaunchKernelGGL((gemm_nt_generic<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
@@ -1394,10 +1918,12 @@ struct Regions {
   int nai_full, nbj_full;  // tiles entirely inside M and N
   bool ragged_a, ragged_b;
   int S;                   // splits used for the interior and the ragged-B launch
+  bool k16;                // K suits the hand-scheduled main loop (callers may still clear it)
 };
 Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixed) {
   Regions r;
   r.fast = (K > 0 && K % BK == 0);
+  r.k16 = k16_ok(K);
   if (r.fast) {
     r.nai_full = (int)(M / TILE); r.nbj_full = (int)(N / TILE);
     r.ragged_a = (M % TILE) != 0; r.ragged_b = (N % TILE) != 0;
@@ -1420,8 +1946,11 @@ template <template <bool> class EpiT, class P, int FAST_KERNEL = KERNEL_NT, bool
 int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_edge_a,
                 hipStream_t stream) {
   int rc;
-  if (!r.fast)
+  if constexpr (FAST_KERNEL >= KERNEL16_NT) {
+    if (!r.fast || !r.k16) return AREAL_ERR_UNSUPPORTED;  // these epilogues have no generic kernel
+  } else if (!r.fast) {
     return launch_region<EpiT<true>, KERNEL_GENERIC>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
+  }
   if (MERGE_EDGES && (r.ragged_a || r.ragged_b)) {
     const int nai = r.nai_full + (r.ragged_a ? 1 : 0);
     return launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), 0, nai,
@@ -1445,8 +1974,34 @@ int check_operand(const void* p, int64_t ld) {
   return AREAL_OK;
 }
 
-// Slots of partial softmax statistics per token written by the forward launches.
-int fwd_slots(const Regions& r) { return 4 * r.S + (r.ragged_a ? 4 : 0); }
+// Slots of partial softmax statistics per token written by the forward launches: per split of
+// the vocabulary range, 2 wave rows x the lane groups that share a token (2 of 32 lanes in the
+// 32x32 kernels, 4 of 16 lanes in the hand-scheduled one).
+int fwd_slots_per_split(const Regions& r) { return r.k16 ? 8 : 4; }
+int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + (r.ragged_a ? 1 : 0)); }
+
+// The four plain-store epilogues over either family of kernels. mode: 0 bf16, 1 fp32,
+// 2 fp32 accumulate, 3 bf16 with a factor per output row. The hand-scheduled kernels write bf16
+// as 16-byte pieces of whole rows.
+template <int KERNEL, int KERNEL16>
+int launch_store(const GemmArgs& g, const Regions& r, const StoreParams& ep, int mode, hipStream_t stream) {
+  bool use16 = r.k16;
+  if (mode == 0 || mode == 3) use16 = use16 && ep.ldo % 8 == 0 && aligned16(ep.out) && ep.M % 8 == 0;
+  if (use16) {
+    switch (mode) {
+      case 0: return launch_gemm<Store16Bf16, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+      case 1: return launch_gemm<Store16F32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+      case 2: return launch_gemm<Accum16F32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+      default: return launch_gemm<Store16Bf16Scaled, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+    }
+  }
+  switch (mode) {
+    case 0: return launch_gemm<StoreBf16, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    case 1: return launch_gemm<StoreF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    case 2: return launch_gemm<AccumF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    default: return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+  }
+}
 
 // dHidden [T, H] has few output tiles when the model is small (H / 256 x T / 256). When the
 // tile count does not fill whole rounds of 256 workgroups, the vocabulary (K) range is split
@@ -1495,25 +2050,24 @@ bool dh_weight_in_place(int64_t V) { return V % BK == 0; }
 // dHidden[t, h] = tscale[t] * sum_v dl[t, v] * W[v, h] (tscale = 1 when null), bf16 out;
 // split-K through `partial` when it pays. w is the weight itself [V, H] when
 // dh_weight_in_place(V), else its transposed copy W^T [H, ldv].
-template <int KERNEL>
+template <int KERNEL, int KERNEL16>
 int launch_dhidden_k(const GemmArgs& g0, int64_t H, int64_t T, int64_t ldv, void* dhidden,
                      float* partial, const float* tscale, hipStream_t stream) {
   GemmArgs g = g0;
   const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
   int z = dh_ksplit(H, T, ldv);
-  const int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
+  int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
+  if (r.k16) kps += kps & 1;  // the hand-scheduled loop walks pairs of k-tiles
   if (z > 1) z = (int)ceil_div_i64(ldv / BK, kps);  // no empty split
   if (z <= 1 || partial == nullptr) {
     const StoreParams ep{dhidden, H, (int)H, (int)T, tscale};
-    if (tscale != nullptr)
-      return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
-    return launch_gemm<StoreBf16, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    return launch_store<KERNEL, KERNEL16>(g, r, ep, tscale != nullptr ? 3 : 0, stream);
   }
   g.ksplit = z;
   g.kt_per_split = kps;
   g.zstride = T * H * (int64_t)sizeof(float);
   const StoreParams ep{partial, H, (int)H, (int)T, nullptr};
-  int rc = launch_gemm<StoreF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+  int rc = launch_store<KERNEL, KERNEL16>(g, r, ep, 1, stream);
   if (rc != AREAL_OK) return rc;
   int64_t blocks = ceil_div_i64(T * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
@@ -1526,10 +2080,10 @@ int launch_dhidden(const u16* w, int64_t V, const u16* dl, int64_t ldv, int64_t 
                    void* dhidden, float* partial, const float* tscale, hipStream_t stream) {
   if (dh_weight_in_place(V)) {
     const GemmArgs g{w, H, (int)H, dl, ldv, (int)T, (int)ldv, (int)H, 0};
-    return launch_dhidden_k<KERNEL_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
+    return launch_dhidden_k<KERNEL_MIX, KERNEL16_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
   }
   const GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
-  return launch_dhidden_k<KERNEL_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
+  return launch_dhidden_k<KERNEL_NT, KERNEL16_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
 }
 
 }  // namespace
@@ -1556,9 +2110,7 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0};
   const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
   const StoreParams ep{out, ldo, (int)M, (int)N};
-  if (out_mode == 0) return launch_gemm<StoreBf16, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
-  if (out_mode == 1) return launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
-  return launch_gemm<AccumF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+  return launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, out_mode, stream);
 }
 
 static Regions fwd_regions(int64_t T, int64_t H, int64_t V) { return plan_regions(V, T, H, 512, 0); }
@@ -1604,7 +2156,7 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   FwdParams ep{labels, (int)T, (int)V, logit_scale, inv_temperature * LOG2E, bias,
                (float*)workspace, P, 0, (u16*)probs, round_up_i64(V, BK), probs_ref};
   FwdParams ep_a = ep;
-  ep_a.slot_base = 4 * r.S;
+  ep_a.slot_base = fwd_slots_per_split(r) * r.S;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
   const bool moments = (vocab_mean != nullptr) || (vocab_norm != nullptr);
   if (probs != nullptr) {
@@ -1613,7 +2165,17 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                        logit_scale, inv_temperature * LOG2E, probs_ref, probs_status);
     AREAL_CHECK_LAUNCH();
   }
-  if (probs == nullptr) {
+  if (r.k16 && probs == nullptr) {
+    if (!affine && !moments) rc = launch_gemm<Fwd16Plain, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else if (!affine) rc = launch_gemm<Fwd16PlainMom, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else if (!moments) rc = launch_gemm<Fwd16Affine, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else rc = launch_gemm<Fwd16AffineMom, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+  } else if (r.k16) {
+    if (!affine && !moments) rc = launch_gemm<Fwd16PlainSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else if (!affine) rc = launch_gemm<Fwd16PlainMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else if (!moments) rc = launch_gemm<Fwd16AffineSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    else rc = launch_gemm<Fwd16AffineMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+  } else if (probs == nullptr) {
     if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
     else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
     else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
@@ -1712,6 +2274,9 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       if (need_dlT)
         rc = affine ? launch_gemm<BwdAffineT>(g, r, ep, ep, stream)
                     : launch_gemm<BwdPlainT>(g, r, ep, ep, stream);
+      else if (r.k16)
+        rc = affine ? launch_gemm<Bwd16Affine, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream)
+                    : launch_gemm<Bwd16Plain, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream);
       else
         rc = affine ? launch_gemm<BwdAffine>(g, r, ep, ep, stream)
                     : launch_gemm<BwdPlain>(g, r, ep, ep, stream);
@@ -1734,8 +2299,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
-      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
-                                  : launch_gemm<StoreF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream);
+      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, (accumulate || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -1745,8 +2309,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
-      rc = (accumulate || t0 > 0) ? launch_gemm<AccumF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream)
-                                  : launch_gemm<StoreF32, StoreParams, KERNEL_NT, true>(g, r, ep, ep, stream);
+      rc = launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, (accumulate || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     }
   }
@@ -1829,9 +2392,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv};
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
-    rc = dweight_mode == 1   ? launch_gemm<AccumF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
-         : dweight_mode == 0 ? launch_gemm<StoreF32, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream)
-                             : launch_gemm<StoreBf16, StoreParams, KERNEL_TN, true>(g, r, ep, ep, stream);
+    rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : dweight_mode == 0 ? 1 : 0, stream);
     if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;

@@ -19,7 +19,11 @@ def _rel(a, b):
 
 
 @pytest.mark.parametrize("M,N,K", [(32, 32, 16), (256, 256, 64), (300, 200, 72), (1000, 520, 8), (96, 13, 32),
-                                   (260, 513, 200)])
+                                   (260, 513, 200),
+                                   # K a multiple of 128: the hand-scheduled main loop (one pair of
+                                   # k-tiles, several, ragged M and N, M not a multiple of 8)
+                                   (256, 256, 128), (512, 256, 1024), (300, 200, 256), (520, 1000, 384),
+                                   (96, 13, 128), (264, 513, 1280)])
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_gemm_nt(dev, M, N, K, mode):
     lib = _lib.load()
@@ -51,6 +55,11 @@ SHAPES = [
     # V a multiple of 64: dHidden reads the [V, H] weight in place (no transposed copy)
     (260, 200, 1088, 0.7, 1.0, True, 128),
     (700, 512, 4096, 1.0, 1.0, False, None),
+    # every contraction length (H, round_up(V, 64), the token chunk) a multiple of 128: all five
+    # contractions take the hand-scheduled main loop
+    (768, 256, 1536, 1.0, 1.0, False, None),
+    (384, 384, 2000, 0.8, 1.5, True, 128),
+    (1024, 128, 640, 1.0, 1.0, False, 256),
 ]
 
 
