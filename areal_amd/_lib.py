@@ -7,6 +7,10 @@ tensor is not on a HIP device the call raises.
 from __future__ import annotations
 
 import ctypes
+import functools
+import re
+import shutil
+import subprocess
 from ctypes import c_float, c_double, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
@@ -151,6 +155,42 @@ def load() -> ctypes.CDLL:
         fn.argtypes = argtypes
     _lib = lib
     return lib
+
+
+@functools.lru_cache(maxsize=1)
+def kernel_names() -> frozenset[str]:
+    """Names of the GPU kernels the built library launches, as a profiler prints them (demangled,
+    without the anonymous-namespace qualifier and the argument list), read from the launch stubs
+    in the shared object. Used to keep the kernel names quoted in benchmark output honest."""
+    symbols = sorted({m.decode() for m in re.findall(rb"_Z[A-Za-z0-9_]{4,600}", LIB_PATH.read_bytes())})
+    tool = shutil.which("c++filt") or shutil.which("llvm-cxxfilt") or "/opt/rocm/llvm/bin/llvm-cxxfilt"
+    out = subprocess.run([tool], input="\n".join(symbols), capture_output=True, text=True, check=True).stdout
+    names = set()
+    for line in out.splitlines():
+        line = line.replace("(anonymous namespace)::", "")
+        if line.startswith("void "):
+            line = line[5:]
+        depth, cut = 0, len(line)
+        for i, ch in enumerate(line):  # cut at the argument list: the first '(' outside <...>
+            if ch == "<":
+                depth += 1
+            elif ch == ">":
+                depth -= 1
+            elif ch == "(" and depth == 0:
+                cut = i
+                break
+        names.add(line[:cut].strip())
+    return frozenset(names)
+
+
+def has_kernel(name: str) -> bool:
+    """True for a kernel of the library; template arguments may be left out (``loss_token_kernel``
+    matches ``loss_token_kernel<false>``)."""
+    names = kernel_names()
+    for cand in (name, "__device_stub__" + name):
+        if cand in names or any(n.startswith(cand + "<") for n in names):
+            return True
+    return False
 
 
 def check(status: int, what: str) -> None:

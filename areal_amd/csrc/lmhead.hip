@@ -1502,9 +1502,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
                    ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
                  : "memory", "scc");
 
-  // Epilogue state does not stay in registers over the main loop, which leaves the compiler only
-  // v[0:ML16_*_FIRST_VGPR): an epilogue that carries values from tile to tile of a sweep keeps
-  // them in memory between its close() and the next open().
+  // What an epilogue carries from tile to tile of a sweep has to be small: over the main loop the
+  // compiler only has v[0:ML16_*_FIRST_VGPR) for it.
+  typename Epi::State st;
   for (int ai = ai_begin; ai < ai_end; ++ai) {
     // where the loader goes when this tile's k range is exhausted: the next A tile of the
     // sweep, or (after the last tile) this tile again, whose first k-tiles are loaded and never used
@@ -1537,12 +1537,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
     // v[0:ML16_*_FIRST_VGPR) for values that live across it.
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
-    typename Epi::State st;
     Epi::open(st, ep, bj * TILE + wb * 128, split, wa, lane_e, ai == ai_begin);
     Epi::tile(st, ep, ai * TILE + wa * 128, bj * TILE + wb * 128, lane_e, stage);
     Epi::close(st, ep, bj * TILE + wb * 128, split, wa, lane_e);
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
+  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
 }
 
 // One block column of the wave's sub-tile (16 rows j x 128 bf16 values i) from the staging area
@@ -1570,6 +1570,7 @@ struct Store16 {
   struct State {};
   static DEVI void open(State&, const Params&, int, int, int, int, bool) {}
   static DEVI void close(State&, const Params&, int, int, int, int) {}
+  static DEVI void end(State&, const Params&, int, int, int, int) {}
   static DEVI void split_output(Params& p, int64_t bytes) { p.out = (char*)p.out + bytes; }
   static DEVI void tile(State&, const Params& p, int i0, int j0, int lane, u16* stage) {
     for_each_col([&](auto bc) {
@@ -1614,47 +1615,56 @@ template <bool E> using Accum16F32 = Store16<E, 2>;
 template <bool E> using Store16Bf16Scaled = Store16<E, 3>;
 
 
-// ---- forward: online softmax statistics (see FwdEpi); a lane owns one token per block column
-// and 4 vocabulary entries per block, so 8 tokens x 32 entries per tile. Partial statistics go
-// to slot split*8 + wa*4 + lane/16.
+// ---- forward: online softmax statistics (see FwdEpi). In a block column the 16 lanes l % 16 own
+// the 16 tokens and the four lane groups l / 16 own 4 of every 16 vocabulary entries, so a token's
+// 128 entries of the wave's sub-tile sit in four lanes. Per column those four lanes agree on the
+// column's maximum, sum their exponentials relative to it, and lane group jb % 4 folds the result
+// into the running statistics of token column jb, of which it keeps two (jb and jb + 4): ten to
+// fourteen registers per lane live across the main loop. Partial statistics go to slot
+// split * 2 + wa at the end of the sweep.
+DEVI float xor_lanes16(float v) { return __shfl_xor(v, 16); }
+DEVI float xor_lanes32(float v) { return __shfl_xor(v, 32); }
+DEVI float group_max(float v) { v = fmaxf(v, xor_lanes16(v)); return fmaxf(v, xor_lanes32(v)); }
+DEVI float group_min(float v) { v = fminf(v, xor_lanes16(v)); return fminf(v, xor_lanes32(v)); }
+DEVI float group_sum(float v) { v += xor_lanes16(v); return v + xor_lanes32(v); }
+
 template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
 struct Fwd16 {
   typedef FwdParams Params;
   struct State {
-    float m[8], s[8], q[8], xl[8], mn[8], sx[MOMENTS ? 8 : 1], sx2[MOMENTS ? 8 : 1];
-    int lab[8];
+    float m[2], s[2], q[2], xl[2], mn[2], sx[MOMENTS ? 2 : 1], sx2[MOMENTS ? 2 : 1];
   };
   static DEVI void split_output(Params&, int64_t) {}
-  // The running statistics of a sweep live in the workspace slots that the merge kernel reads
-  // (written by close() after every tile, read back by the next open()).
-  static DEVI void open(State& st, const Params& p, int t0, int split, int wa, int lane, bool first) {
-    const int slot = p.slot_base + split * 8 + wa * 4 + (lane >> 4);
-    const int64_t PT = (int64_t)p.P * p.T;
+  static DEVI void open(State& st, const Params&, int, int, int, int, bool first) {
+    if (first) {
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        st.m[k] = neg_inf(); st.s[k] = 0.f; st.q[k] = 0.f; st.xl[k] = 0.f; st.mn[k] = pos_inf();
+        if (MOMENTS) { st.sx[k] = 0.f; st.sx2[k] = 0.f; }
+      }
+    }
+  }
+  static DEVI void close(State&, const Params&, int, int, int, int) {}
+
+  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
+    const int vl = v0 + 4 * (lane >> 4);
+    const int group = lane >> 4;
+    auto vidx = [&](int a, int r) { return vl + a * 16 + r; };
+    // labels and row references of the 8 tokens this lane sees, fetched ahead of the columns
+    int lab[8];
+    float rr[SAVE ? 8 : 1];
 #pragma unroll
     for (int b = 0; b < 8; ++b) {
       const int t = t0 + b * 16 + (lane & 15);
       const bool live = !EDGE || t < p.T;
-      int64_t l = live ? p.labels[t] : -1;
-      st.lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
-      if (first || !live) {
-        st.m[b] = neg_inf(); st.s[b] = 0.f; st.q[b] = 0.f; st.xl[b] = 0.f;
-        st.mn[b] = pos_inf();
-        if (MOMENTS) { st.sx[b] = 0.f; st.sx2[b] = 0.f; }
-      } else {
-        const float* w = p.ws + (int64_t)slot * p.T + t;
-        st.m[b] = w[0 * PT]; st.s[b] = w[1 * PT]; st.q[b] = w[2 * PT]; st.xl[b] = w[3 * PT];
-        st.mn[b] = w[4 * PT];
-        if (MOMENTS) { st.sx[b] = w[5 * PT]; st.sx2[b] = w[6 * PT]; }
-      }
-      ML16_AGPR_FENCE();
+      const int64_t l = live ? p.labels[t] : -1;
+      lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+      if (SAVE) rr[b] = live ? p.probs_ref[t] : 0.f;
     }
-  }
-
-  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
-    const int vl = v0 + 4 * (lane >> 4);
-    auto vidx = [&](int a, int r) { return vl + a * 16 + r; };
+    ML16_AGPR_FENCE();
     for_each_col([&](auto bc) {
       constexpr int b = decltype(bc)::value;
+      constexpr int k = b >> 2;
       float x[32];
       acc_col<b>(x);
       if (AFFINE) {
@@ -1667,9 +1677,6 @@ struct Fwd16 {
             x[a * 4 + r] = (x[a * 4 + r] + bv) * p.scale;
           }
       }
-      const int tok = t0 + b * 16 + (lane & 15);
-      float rr = 0.f;  // SAVE: the token's row reference
-      if (SAVE && (!EDGE || tok < p.T)) rr = p.probs_ref[tok];
       float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
 #pragma unroll
       for (int a = 0; a < 8; ++a) {
@@ -1683,19 +1690,12 @@ struct Fwd16 {
           }
         }
       }
+      // the column's reference: the maximum over the token's 128 entries in this sub-tile (see
+      // ref_of); -inf only if every entry lies past the vocabulary
+      tmax = group_max(tmax);
+      const float mc = (!EDGE || tmax > neg_inf()) ? ref_of(tmax, p.c2) : 0.f;
       ML16_AGPR_FENCE();
-      st.mn[b] = fminf(st.mn[b], tmin);
-      if (MOMENTS) { st.sx[b] += sx; st.sx2[b] += sx2; }
-      const float m_old = st.m[b];
-      const float m_new = fmaxf(m_old, tmax);
-      // rescale the running sums to the new reference (see ref_of); on the first tile
-      // m_old = -inf and s = q = 0, so the factor is taken as 2^0 instead of evaluating -inf - x
-      float s = st.s[b], q = st.q[b];
-      const float mc = (!EDGE || m_new > neg_inf()) ? ref_of(m_new, p.c2) : 0.f;
-      const float dl = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
-      const float alpha = fast_exp2(dl);
-      q = alpha * fmaf(dl, s, q);
-      s = alpha * s;
+      float s = 0.f, q = 0.f;
       if (!SAVE) {
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
@@ -1709,25 +1709,24 @@ struct Fwd16 {
           ML16_AGPR_FENCE();
         }
       } else {
-        // The sums take the exponentials relative to the running maximum (in (0, 1] whatever
-        // the row reference is); what is stored is the same exponential moved to the row
-        // reference by one factor per (token, tile). That factor over- or underflows only where
-        // the stored value is not used: rows outside the reference window, and tiles whose
-        // maximum lies 126 binades below the row's. The 16 tokens x 128 entries of this block
+        // What is stored is the exponential relative to the column's maximum (in (0, 1]) moved to
+        // the row reference by one factor per (token, column). That factor over- or underflows
+        // only where the stored value is not used: rows outside the reference window, and columns
+        // whose maximum lies 126 binades below the row's. The 16 tokens x 128 entries of the
         // column go through the staging area and leave as whole lines.
-        const float gamma = fast_exp2(mc - rr);
+        const float gamma = fast_exp2(mc - rr[b]);
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
           const int vq = vl + a * 16;
           u16 d[4];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const float t = fmaf(x[a * 4 + k], p.c2, -mc);
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const float t = fmaf(x[a * 4 + e4], p.c2, -mc);
             const float e = fast_exp2(t);
             float es = e * gamma;
-            if (EDGE && vq + k >= p.V) es = 0.f;
+            if (EDGE && vq + e4 >= p.V) es = 0.f;
             else { s += e; q = fmaf(t, e, q); }
-            d[k] = f32_to_bf16_bits(es);
+            d[e4] = f32_to_bf16_bits(es);
           }
           u32x2 pk;
           pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
@@ -1741,39 +1740,62 @@ struct Fwd16 {
         flush_stage16<EDGE>(stage, p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv,
                             p.T - (t0 + b * 16), (int)p.ldv - v0, lane);
       }
-      // The sums pass through an empty block here: their only readers come after the last
-      // column, and the compiler otherwise moves the two summation chains of every column down
-      // there, keeping all the exponentials alive (in scratch memory) until then.
-      asm volatile("" : "+v"(s), "+v"(q) : : ML16_ACC_CLOBBERS);
-      st.s[b] = s; st.q[b] = q; st.m[b] = m_new;
-      const int lab = st.lab[b];
-      const bool hit = (lab >= v0) && (lab < v0 + 128);
+      // the label's logit, if it is one of this lane's 32 entries
+      float xl = 0.f;
+      const bool hit = (lab[b] >= v0) && (lab[b] < v0 + 128);
       if (__builtin_amdgcn_ballot_w64(hit) != 0) {
 #pragma unroll
         for (int a = 0; a < 8; ++a)
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            if (vidx(a, r) == lab) st.xl[b] = x[a * 4 + r];
+            if (vidx(a, r) == lab[b]) xl = x[a * 4 + r];
       }
-      // everything this column updated is final here (see the note on the sums above)
-      asm volatile("" : "+v"(st.m[b]), "+v"(st.xl[b]), "+v"(st.mn[b]) : : ML16_ACC_CLOBBERS);
-      if (MOMENTS) asm volatile("" : "+v"(st.sx[b]), "+v"(st.sx2[b]));
+      // The partial results pass through an empty block here: their readers come later (the last
+      // one after the last column), and the compiler otherwise moves the summation chains of
+      // every column down there, keeping all the exponentials alive in scratch memory until then.
+      asm volatile("" : "+v"(s), "+v"(q), "+v"(tmin), "+v"(xl) : : ML16_ACC_CLOBBERS);
+      s = group_sum(s);
+      q = group_sum(q);
+      tmin = group_min(tmin);
+      xl = group_sum(xl);
+      if (MOMENTS) {
+        asm volatile("" : "+v"(sx), "+v"(sx2));
+        sx = group_sum(sx);
+        sx2 = group_sum(sx2);
+      }
+      // lane group b % 4 folds the column into the running statistics of token column b: both
+      // sets of sums move to the reference of the larger maximum
+      if (group == (b & 3)) {
+        const float m_old = st.m[k];
+        const float m_new = fmaxf(m_old, tmax);
+        const float d_old = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
+        const float d_col = (!EDGE || tmax > neg_inf()) ? ref_diff(tmax, m_new, p.c2) : 0.f;
+        const float a_old = fast_exp2(d_old), a_col = fast_exp2(d_col);
+        st.q[k] = a_old * fmaf(d_old, st.s[k], st.q[k]) + a_col * fmaf(d_col, s, q);
+        st.s[k] = a_old * st.s[k] + a_col * s;
+        st.m[k] = m_new;
+        st.mn[k] = fminf(st.mn[k], tmin);
+        st.xl[k] += xl;
+        if (MOMENTS) { st.sx[k] += sx; st.sx2[k] += sx2; }
+      }
+      asm volatile("" : "+v"(st.m[k]), "+v"(st.s[k]), "+v"(st.q[k]), "+v"(st.xl[k]), "+v"(st.mn[k])
+                   : : ML16_ACC_CLOBBERS);
+      if (MOMENTS) asm volatile("" : "+v"(st.sx[k]), "+v"(st.sx2[k]));
       __builtin_amdgcn_sched_barrier(0);
     });
   }
 
-  static DEVI void close(State& st, const Params& p, int t0, int split, int wa, int lane) {
-    const int slot = p.slot_base + split * 8 + wa * 4 + (lane >> 4);
+  static DEVI void end(State& st, const Params& p, int t0, int split, int wa, int lane) {
+    const int slot = p.slot_base + split * 2 + wa;
+    const int64_t PT = (int64_t)p.P * p.T;
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const int t = t0 + b * 16 + (lane & 15);
+    for (int k = 0; k < 2; ++k) {
+      const int t = t0 + ((lane >> 4) + 4 * k) * 16 + (lane & 15);
       if (EDGE && t >= p.T) continue;
-      const int64_t PT = (int64_t)p.P * p.T;
       float* w = p.ws + (int64_t)slot * p.T + t;
-      w[0 * PT] = st.m[b]; w[1 * PT] = st.s[b]; w[2 * PT] = st.q[b]; w[3 * PT] = st.xl[b];
-      w[4 * PT] = st.mn[b];
-      if (MOMENTS) { w[5 * PT] = st.sx[b]; w[6 * PT] = st.sx2[b]; }
-      ML16_AGPR_FENCE();
+      w[0 * PT] = st.m[k]; w[1 * PT] = st.s[k]; w[2 * PT] = st.q[k]; w[3 * PT] = st.xl[k];
+      w[4 * PT] = st.mn[k];
+      if (MOMENTS) { w[5 * PT] = st.sx[k]; w[6 * PT] = st.sx2[k]; }
     }
   }
 };
@@ -1809,6 +1831,7 @@ struct Bwd16 {
     }
   }
   static DEVI void close(State&, const Params&, int, int, int, int) {}
+  static DEVI void end(State&, const Params&, int, int, int, int) {}
   static DEVI void split_output(Params&, int64_t) {}
 
   static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
@@ -1975,9 +1998,9 @@ int check_operand(const void* p, int64_t ld) {
 }
 
 // Slots of partial softmax statistics per token written by the forward launches: per split of
-// the vocabulary range, 2 wave rows x the lane groups that share a token (2 of 32 lanes in the
-// 32x32 kernels, 4 of 16 lanes in the hand-scheduled one).
-int fwd_slots_per_split(const Regions& r) { return r.k16 ? 8 : 4; }
+// the vocabulary range, 2 wave rows x (in the 32x32 kernels) the 2 lane groups that share a
+// token; the hand-scheduled kernels combine their 4 lane groups in registers.
+int fwd_slots_per_split(const Regions& r) { return r.k16 ? 2 : 4; }
 int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + (r.ragged_a ? 1 : 0)); }
 
 // The four plain-store epilogues over either family of kernels. mode: 0 bf16, 1 fp32,

@@ -23,6 +23,16 @@ if ROOT not in sys.path:
 V_QWEN = 151936
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak used for the roofline fraction
 
+# The contraction kernels of the default workload as rocprofv3 names them (checked against the
+# loaded library before they are printed). gemm16_sweep<variant, epilogue>: variant 0 = both
+# operands k-contiguous, 1 = both k-major, 2 = A k-major; Fwd16<edge, affine, moments, save>,
+# Store16<edge, mode> with mode 0 = bf16, 3 = bf16 scaled per output row.
+KERNEL_FWD_SAVE = "gemm16_sweep<0, Fwd16<false, false, false, true> >"
+KERNEL_FWD = "gemm16_sweep<0, Fwd16<false, false, false, false> >"
+KERNEL_RECOMPUTE = "gemm16_sweep<0, Bwd16<false, false> >"
+KERNEL_DHIDDEN = "gemm16_sweep<2, Store16<false, 3> >"
+KERNEL_DWEIGHT = "gemm16_sweep<1, Store16<true, 0> >"
+
 WORKLOADS = {
     # name: (T, H, n_seqs, min_len, max_len, seed, description)
     "qwen3-8b": dict(T=32768, H=4096, n_seqs=32, lo=256, hi=2048, seed=3,
@@ -512,20 +522,30 @@ def main() -> None:
             lib_tflops = 2.0 * T * H * V / (a.elapsed_time(c) / 5 * 1e-3) / 1e12
             del logits
 
-    # L2<->fabric bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-    # command (KiB per dispatch, scaled by the factors the same counters show for copy-like
-    # kernels of known size, the operand-prep and the bf16 transpose: fetch x2.0, write x1.0). Only measured for the default
-    # workload; the forward's fetch count moves by +-20 % from run to run with L2 hit timing.
+    # L2<->fabric bytes per launch. Not measured by this run: constants from rocprofv3 --pmc
+    # FETCH_SIZE / WRITE_SIZE runs of this command on this workload (KiB per dispatch, scaled by
+    # the factors the same counters show for copy-like kernels of known size, the operand-prep
+    # and the bf16 transpose: fetch x2.0, write x1.0); profiles/lmhead_contraction_qwen3-8b.md
+    # has the commands and the table. The forward's fetch count moves by +-20 % from run to run
+    # with L2 hit timing.
     traffic = None
     traffic_detail = None
+    traffic_source = None
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            "gemm_nt_sweep<FwdEpi> forward": 3.38786e7 * kib * 2.0 + 1.29532e7 * kib,
-            "gemm_mix_sweep<StoreEpi> dHidden": 3.46954e7 * kib * 2.0 + 3.01056e5 * kib,
-            "gemm_tn_sweep<StoreEpi> dWeight": 3.05786e7 * kib * 2.0 + 1.26301e6 * kib,
+            KERNEL_FWD_SAVE + " forward": 3.80911e7 * kib * 2.0 + 1.27519e7 * kib,
+            KERNEL_DHIDDEN + " dHidden": 3.24272e7 * kib * 2.0 + 2.64192e5 * kib,
+            KERNEL_DWEIGHT + " dWeight": 2.93621e7 * kib * 2.0 + 1.21549e6 * kib,
         }
         traffic = sum(traffic_detail.values()) / 3.0
+        traffic_source = ("offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command "
+                          "(profiles/lmhead_contraction_qwen3-8b.md), mean of the three contraction "
+                          "launches; not re-measured by this run")
+    missing = [k for k in (KERNEL_FWD_SAVE, KERNEL_FWD, KERNEL_DHIDDEN, KERNEL_DWEIGHT, KERNEL_RECOMPUTE)
+               if not _lib.has_kernel(k)]
+    if missing:
+        sys.exit(f"bench.py names kernels that the loaded library does not contain: {missing}")
 
     result = {
         "metric": "packed tokens/sec, logprob+entropy+PPO loss fwd+bwd; % bf16 MFMA peak",
@@ -550,21 +570,23 @@ def main() -> None:
         },
         "pct_bf16_mfma_peak": 100.0 * (algo_flops / (ms_per_step * 1e-3) / 1e12) / PEAK_BF16_TFLOPS,
         "roofline": {
-            "kernel": ("gemm_nt_sweep<FwdEpi>, gemm_mix_sweep<StoreEpi> (dHidden), "
-                       "gemm_tn_sweep<StoreEpi> (dWeight)"
-                       + ("" if saved else ", gemm_nt_sweep<BwdEpi> (recompute)")),
+            "kernel": (f"{KERNEL_FWD_SAVE if saved else KERNEL_FWD} (forward), {KERNEL_DHIDDEN} (dHidden), "
+                       f"{KERNEL_DWEIGHT} (dWeight)"
+                       + ("" if saved else f", {KERNEL_RECOMPUTE} (recompute)")),
             "bound": "mfma",
             "achieved": achieved,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_BF16_TFLOPS,
             "traffic": traffic,
+            "traffic_source": traffic_source,
             "traffic_bytes_per_launch": traffic_detail,
             "forward_only_tflops": fwd_tflops,
             "library_gemm_same_box_tflops": lib_tflops,
             "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},
             "other_backward_mode": other,
+            "recompute_mode_ms": (ms_per_step if not saved else (other["ms_per_step"] if other else None)),
         },
     }
     if not args.no_hbm_kernels:

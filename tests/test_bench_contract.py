@@ -47,3 +47,18 @@ def test_json_line_has_the_contract_keys():
     c = d["cpu_baseline"]
     assert c["kind"] == "port" and c["unit"] == "tokens/s" and c["cores"] >= 1 and c["value"] > 0
     assert d["value"] > 0 and d["ms_per_step"] > 0
+
+
+def test_kernel_names_quoted_by_the_bench_exist_in_the_library():
+    # the roofline object names its kernels; a renamed kernel must not leave a stale label behind
+    sys.path.insert(0, ROOT)
+    import bench
+    from areal_amd import _lib
+
+    for name in (bench.KERNEL_FWD_SAVE, bench.KERNEL_FWD, bench.KERNEL_RECOMPUTE, bench.KERNEL_DHIDDEN,
+                 bench.KERNEL_DWEIGHT):
+        assert _lib.has_kernel(name), name
+    assert not _lib.has_kernel("gemm16_sweep<9, Store16<false, 0> >")
+    for name in ("gae_owned_kernel", "loss_token_kernel", "loss_finalize_kernel", "rows_fwd_kernel",
+                 "saved_prep_kernel", "lmhead_merge_kernel", "lmhead_rowref_kernel"):
+        assert _lib.has_kernel(name), name
