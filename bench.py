@@ -492,6 +492,30 @@ def main() -> None:
         }
     saved = main_saved
 
+    # The two backward contractions on their own (median of three): a backward that asks for one
+    # gradient launches one contraction, next to the loss backward and the operand preparation
+    # (in recompute mode also the recompute pass), so these are upper bounds of the kernels' times.
+    def backward_only(want_hidden):
+        ts = []
+        h_in = hidden.detach().requires_grad_(want_hidden)
+        w_in = weight.detach().requires_grad_(not want_hidden)
+        wrt = h_in if want_hidden else w_in
+        for _ in range(3):
+            out = fused_lm_head_logprobs_entropy(h_in, w_in, b["labels"], temperature=1.0,
+                                                 save_probs=False if args.recompute else None)
+            loss = loss_fn(out.logprobs, out.entropy, input_data,
+                           vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            torch.autograd.grad(loss, [wrt])
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        return sorted(ts)[1]
+
+    backward_split = {"dHidden launch sequence": backward_only(True),
+                      "dWeight launch sequence": backward_only(False)}
+
     # Roofline of the MFMA contraction kernels (gemm_nt_sweep / gemm_tn_sweep): one step runs
     # 3 algorithmic GEMMs = 6*T*H*V flops (forward with the softmax epilogue, dHidden, dWeight);
     # with --recompute a fourth launch recomputes the logits and carries no algorithmic flops.
@@ -507,6 +531,7 @@ def main() -> None:
     # the timed steps: what a contraction without the softmax epilogue sustains here (boards are
     # power-limited under this load, so the figure moves from box to box with the kernels').
     lib_tflops = None
+    lib_by_shape = None
     if not args.no_library_gemm:
         with torch.no_grad():
             hd, wt = hidden.detach(), weight.detach().t()
@@ -520,7 +545,21 @@ def main() -> None:
             c.record()
             torch.cuda.synchronize()
             lib_tflops = 2.0 * T * H * V / (a.elapsed_time(c) / 5 * 1e-3) / 1e12
-            del logits
+            # the same library at the two backward contractions' shapes and layouts
+            lib_by_shape = {"forward [T,H] x [V,H]^T": lib_tflops}
+            dh_out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+            dw_out = torch.empty(V, H, dtype=torch.bfloat16, device=dev)
+            for name, fn in (("dHidden [T,V] x [V,H]", lambda: torch.mm(logits, weight.detach(), out=dh_out)),
+                             ("dWeight [T,V]^T x [T,H]", lambda: torch.mm(logits.t(), hd, out=dw_out))):
+                for _ in range(2):
+                    fn()
+                a.record()
+                for _ in range(5):
+                    fn()
+                c.record()
+                torch.cuda.synchronize()
+                lib_by_shape[name] = 2.0 * T * H * V / (a.elapsed_time(c) / 5 * 1e-3) / 1e12
+            del logits, dh_out, dw_out
 
     # L2<->fabric bytes per launch. Not measured by this run: constants from rocprofv3 --pmc
     # FETCH_SIZE / WRITE_SIZE runs of this command on this workload (KiB per dispatch, scaled by
@@ -583,8 +622,10 @@ def main() -> None:
             "traffic_bytes_per_launch": traffic_detail,
             "forward_only_tflops": fwd_tflops,
             "library_gemm_same_box_tflops": lib_tflops,
+            "library_gemm_by_shape_tflops": lib_by_shape,
             "ms": {"lmhead_fwd": t_fwd / args.steps, "loss_fwd": t_loss / args.steps,
                    "loss_bwd+lmhead_bwd": t_bwd / args.steps},
+            "backward_split_ms": backward_split,
             "other_backward_mode": other,
             "recompute_mode_ms": (ms_per_step if not saved else (other["ms_per_step"] if other else None)),
         },
