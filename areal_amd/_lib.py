@@ -50,7 +50,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_lmhead_bwd_saved_workspace_bytes": (SZ, [I64, I64, I64]),
     "areal_lmhead_bwd_saved": (
         I,
-        [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, P, I, P, P, SZ, P],
+        [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, I, P, P, SZ, P],
     ),
     "areal_cast_f32_to_bf16": (I, [P, P, I64, P]),
     "areal_logits_logprobs_entropy_fwd": (I, [P, I, I64, P, I64, I64, F, P, P, P, P]),

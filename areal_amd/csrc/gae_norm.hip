@@ -21,15 +21,25 @@ constexpr int GAE_THREADS = 256;
 constexpr int GAE_ITEMS = 8;
 constexpr int GAE_TILE = GAE_THREADS * GAE_ITEMS;
 
-struct Map {
-  double a11, a12, a22, b1, b2;
+// R = double in the three-launch scan (maps composed over the whole array); R = float in the
+// single-pass kernel, where a map spans at most one tile and the state carried from tile to
+// tile stays in fp64 (each output then sees ~20 fp32 roundings, like the reference's fp32 loop
+// over as many tokens).
+template <class R>
+struct MapT {
+  R a11, a12, a22, b1, b2;
 };
-DEVI Map map_identity() { return Map{1.0, 0.0, 1.0, 0.0, 0.0}; }
+using Map = MapT<double>;
+using MapF = MapT<float>;
+template <class R>
+DEVI MapT<R> map_identity_t() { return MapT<R>{R(1), R(0), R(1), R(0), R(0)}; }
+DEVI Map map_identity() { return map_identity_t<double>(); }
 // (f o g): apply g first, then f.
-DEVI Map compose(const Map& f, const Map& g) {
+template <class R>
+DEVI MapT<R> compose(const MapT<R>& f, const MapT<R>& g) {
   // explicit fma: this file is compiled without contraction (the normalisation kernels follow
-  // the reference's fp32 rounding), but the fp64 maps are more exact with it and cost half
-  Map r;
+  // the reference's fp32 rounding), but the maps are more exact with it and cost half
+  MapT<R> r;
   r.a11 = f.a11 * g.a11;
   r.a12 = fma(f.a11, g.a12, f.a12 * g.a22);
   r.a22 = f.a22 * g.a22;
@@ -37,8 +47,9 @@ DEVI Map compose(const Map& f, const Map& g) {
   r.b2 = fma(f.a22, g.b2, f.b2);
   return r;
 }
-DEVI Map shfl_down_map(const Map& m, int d) {
-  Map r;
+template <class R>
+DEVI MapT<R> shfl_down_map(const MapT<R>& m, int d) {
+  MapT<R> r;
   r.a11 = __shfl_down(m.a11, d, 64); r.a12 = __shfl_down(m.a12, d, 64);
   r.a22 = __shfl_down(m.a22, d, 64); r.b1 = __shfl_down(m.b1, d, 64);
   r.b2 = __shfl_down(m.b2, d, 64);
@@ -136,22 +147,23 @@ DEVI Map thread_total(const Map (&mp)[GAE_ITEMS]) {
 }
 
 // Inclusive suffix scan over the block: returns for each thread the composition of the maps
-// of threads tid..blockDim-1 (thread tid applied last). smem: [4] wave totals.
-DEVI Map block_suffix_scan(Map mine, Map* smem, Map& block_total) {
+// of threads tid..blockDim-1 (thread tid applied last). smem: one slot per wave.
+template <class R>
+DEVI MapT<R> block_suffix_scan(MapT<R> mine, MapT<R>* smem, MapT<R>& block_total) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  Map acc = mine;
+  MapT<R> acc = mine;
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
-    const Map other = shfl_down_map(acc, d);
+    const MapT<R> other = shfl_down_map(acc, d);
     if (lane + d < 64) acc = compose(acc, other);
   }
   __syncthreads();
   if (lane == 0) smem[w] = acc;  // wave total (lanes 0..63)
   __syncthreads();
   const int nw = blockDim.x >> 6;
-  Map right = map_identity();
+  MapT<R> right = map_identity_t<R>();
   for (int i = nw - 1; i > w; --i) right = compose(smem[i], right);
-  Map tot = right;
+  MapT<R> tot = right;
   for (int i = w; i >= 0; --i) tot = compose(smem[i], tot);
   block_total = tot;
   return compose(acc, right);
@@ -265,9 +277,12 @@ DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
   return base;
 }
 
+// (Blocks of 1024 threads, one 8192-token tile per padded row instead of four serial tiles of
+// 2048, measured slower: 46.7 against 30.8 us on [1024, 8192]; one such block fills a CU's
+// registers and the latency of its single pass is not covered by anything.)
 __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
-  __shared__ Map smem[4];
-  __shared__ Map all[GAE_THREADS];
+  __shared__ MapF smem[GAE_THREADS / 64];
+  __shared__ MapF all[GAE_THREADS];
   __shared__ int32_t s_cu[GAE_TILE + 2];
   __shared__ int s_own[2];
   const int tid = threadIdx.x;
@@ -299,10 +314,10 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
     s_first = (int)(lo / g.uniform_len);
     s_last = (int)(hi / g.uniform_len) - 1;
   } else {
-    if (tid < 64) {
-      const int a = wave_count_le(g.cu + 1, g.n_seqs, lo, tid);
-      const int b = wave_count_le(g.cu + 1, g.n_seqs, hi, tid);
-      if (tid == 0) { s_own[0] = a; s_own[1] = b - 1; }
+    if (tid < 128) {  // the two searches are independent chains of global loads: one wave each
+      const int which = tid >> 6;
+      const int r = wave_count_le(g.cu + 1, g.n_seqs, which ? hi : lo, tid & 63);
+      if ((tid & 63) == 0) s_own[which] = which ? r - 1 : r;
     }
     __syncthreads();
     s_first = s_own[0];
@@ -400,49 +415,43 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
         }
       }
     }
-    const double gam = (double)g.discount;
-    auto token_map = [&](int i) -> Map {
-      const double val = (double)v[i];
+    const float gam = g.discount;
+    auto token_map = [&](int i) -> MapF {
+      const float val = v[i];
       // not owned: identity (m = 0 with no offsets); last token of a sequence: constant map
-      const double m = ((valid >> i) & 1u) ? (double)ms[i] : 0.0;
-      const double c = gam * (double)lm[i];
-      Map f;
-      f.a11 = fma(c, m, 1.0 - m);
+      const float m = ((valid >> i) & 1u) ? ms[i] : 0.f;
+      const float c = gam * lm[i];
+      MapF f;
+      f.a11 = fmaf(c, m, 1.f - m);
       f.a12 = gam * m;
-      f.a22 = 1.0 - m;
-      f.b1 = ((double)rw[i] - val) * m;
+      f.a22 = 1.f - m;
+      f.b1 = (rw[i] - val) * m;
       f.b2 = val * m;
-      if ((ends >> i) & 1u) f = Map{0.0, 0.0, 0.0, 0.0, ((boot >> i) & 1u) ? val : 0.0};
+      if ((ends >> i) & 1u) f = MapF{0.f, 0.f, 0.f, 0.f, ((boot >> i) & 1u) ? val : 0.f};
       return f;
     };
-    Map mine = token_map(GAE_ITEMS - 1);
+    MapF mine = token_map(GAE_ITEMS - 1);
 #pragma unroll
-    for (int i = GAE_ITEMS - 2; i >= 0; --i) {
-      mine = compose(token_map(i), mine);
-      if (i & 1) __builtin_amdgcn_sched_barrier(0);  // two maps in flight, not eight
-    }
-    Map total;
-    const Map incl = block_suffix_scan(mine, smem, total);
+    for (int i = GAE_ITEMS - 2; i >= 0; --i) mine = compose(token_map(i), mine);
+    MapF total;
+    const MapF incl = block_suffix_scan(mine, smem, total);
     all[tid] = incl;
     __syncthreads();
-    const Map excl = tid + 1 < GAE_THREADS ? all[tid + 1] : map_identity();
-    double A = fma(excl.a11, A0, fma(excl.a12, nv0, excl.b1));
-    double nv = fma(excl.a22, nv0, excl.b2);
+    const MapF excl = tid + 1 < GAE_THREADS ? all[tid + 1] : map_identity_t<float>();
+    // the state entering this thread's tokens: the fp32 map of everything to its right in the
+    // tile applied to the fp64 state entering the tile
+    float A = (float)fma((double)excl.a11, A0, fma((double)excl.a12, nv0, (double)excl.b1));
+    float nv = (float)fma((double)excl.a22, nv0, (double)excl.b2);
     if (any) {
-      // opaque to the optimiser: otherwise it keeps the 8 maps of the first use alive
-#pragma unroll
-      for (int i = 0; i < GAE_ITEMS; ++i)
-        asm volatile("" : "+v"(rw[i]), "+v"(v[i]), "+v"(ms[i]), "+v"(lm[i]));
       float oa[GAE_ITEMS], orr[GAE_ITEMS];
 #pragma unroll
       for (int i = GAE_ITEMS - 1; i >= 0; --i) {
-        const Map f = token_map(i);
-        const double A2 = fma(f.a11, A, fma(f.a12, nv, f.b1));
-        const double nv2 = fma(f.a22, nv, f.b2);
+        const MapF f = token_map(i);
+        const float A2 = fmaf(f.a11, A, fmaf(f.a12, nv, f.b1));
+        const float nv2 = fmaf(f.a22, nv, f.b2);
         A = A2; nv = nv2;
-        oa[i] = (float)A;
+        oa[i] = A;
         orr[i] = oa[i] + v[i];
-        if (i & 1) __builtin_amdgcn_sched_barrier(0);
       }
       if (valid == (1u << GAE_ITEMS) - 1u) {
 #pragma unroll
@@ -457,8 +466,8 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
       }
     }
     // state entering the next tile on the left
-    const double A1 = fma(total.a11, A0, fma(total.a12, nv0, total.b1));
-    const double nv1 = fma(total.a22, nv0, total.b2);
+    const double A1 = fma((double)total.a11, A0, fma((double)total.a12, nv0, (double)total.b1));
+    const double nv1 = fma((double)total.a22, nv0, (double)total.b2);
     A0 = A1; nv0 = nv1;
   }
 }
@@ -481,8 +490,10 @@ struct NormArgs {
   int mean_level, std_level;
   int leave1out, unbiased;
   double eps;
-  double* part;            // [3][G][nsplit]: count, sum, sum of squares
+  double* part;            // [3][G][nsplit]: count, sum, sum of squared deviations; or, with
+                           // closed_form, [5][G][nsplit]: sum m, sum x m, sum m^2, sum m^2 x, sum m^2 x^2
   float* out;
+  int closed_form;         // the squared deviations come from the five sums of one statistics pass
 };
 
 DEVI double block_sum_d(double v, double* smem) {
@@ -494,6 +505,26 @@ DEVI double block_sum_d(double v, double* smem) {
   double r = 0.0;
   for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i];
   return r;
+}
+
+// N sums at once: one pair of barriers instead of N.
+template <int N>
+DEVI void block_sum_n(double (&v)[N], double* smem /* [4][N] */) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < N; ++k) v[k] = wave_sum(v[k]);
+  __syncthreads();
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) smem[w * N + k] = v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    double r = 0.0;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i * N + k];
+    v[k] = r;
+  }
 }
 
 DEVI void split_range(const NormArgs& a, int g, int sp, int64_t& lo, int64_t& hi) {
@@ -592,6 +623,162 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_stats1_kernel(NormArgs a) {
     a.part[((int64_t)0 * a.G + g) * a.nsplit + sp] = cnt;
     a.part[((int64_t)1 * a.G + g) * a.nsplit + sp] = sum;
   }
+}
+
+// The only statistics pass of the two-launch form: five masked sums per (group, split). With a
+// mean that is the same for every element of a group (no leave-one-out), the sum of squared
+// deviations sum (x m - mean m)^2 is S(m^2 x^2) - 2 mean S(m^2 x) + mean^2 S(m^2), evaluated in
+// fp64 by the apply pass with the mean exactly as the elements see it (rounded to fp32 at group
+// level), so x and the mask are read once for the statistics instead of twice.
+__global__ __launch_bounds__(NORM_THREADS) void norm_stats5_kernel(NormArgs a) {
+  __shared__ double smem[4 * 5];
+  const int g = blockIdx.x, sp = blockIdx.y;
+  int64_t lo, hi;
+  split_range(a, g, sp, lo, hi);
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0, s4 = 0.0;
+  auto take = [&](float xf, float mf) {
+    const double x = (double)xf, m = (double)mf;
+    const double xm = x * m, mm = m * m;
+    s0 += m; s1 += xm; s2 += mm; s3 += xm * m; s4 += xm * xm;
+  };
+  const bool has_mask = a.mask != nullptr;
+  // scalar head up to a multiple of 4 elements, 16-byte loads in the middle, scalar tail
+  int64_t mid_lo = (lo + 3) & ~(int64_t)3, mid_hi = hi & ~(int64_t)3;
+  if (mid_lo > mid_hi) { mid_lo = hi; mid_hi = hi; }
+  for (int64_t i = lo + threadIdx.x; i < mid_lo; i += blockDim.x) take(a.x[i], has_mask ? a.mask[i] : 1.0f);
+  // four 16-byte loads of each array in flight per thread before the first sum needs them
+  const int64_t step = 4 * (int64_t)blockDim.x;
+  for (int64_t i = mid_lo + 4 * (int64_t)threadIdx.x; i < mid_hi; i += 4 * step) {
+    f32x4 xv[4], mv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t j = i + u * step;
+      xv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      mv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (j < mid_hi) {
+        xv[u] = *(const f32x4*)(a.x + j);
+        mv[u] = has_mask ? *(const f32x4*)(a.mask + j) : f32x4{1.f, 1.f, 1.f, 1.f};
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) take(xv[u][e], mv[u][e]);
+  }
+  for (int64_t i = mid_hi + threadIdx.x; i < hi; i += blockDim.x)
+    if (i >= mid_lo) take(a.x[i], has_mask ? a.mask[i] : 1.0f);
+  double v[5] = {s0, s1, s2, s3, s4};
+  block_sum_n<5>(v, smem);
+  if (threadIdx.x == 0) {
+    const int64_t o = (int64_t)g * a.nsplit + sp, st = (int64_t)a.G * a.nsplit;
+#pragma unroll
+    for (int k = 0; k < 5; ++k) a.part[k * st + o] = v[k];
+  }
+}
+
+// Apply pass of the two-launch form. Every block first sums what it needs of the five partial
+// arrays in one cooperative sweep (its group's five sums; the batch's count, or all five batch
+// sums when a level is "batch") and one fused block reduction, then derives the mean and the
+// deviation exactly as the three-launch kernels do, and streams its range with 16-byte accesses.
+__global__ __launch_bounds__(NORM_THREADS) void norm_apply_cf_kernel(NormArgs a) {
+  __shared__ double smem[4 * 10];
+  const int g = blockIdx.x, sp = blockIdx.y;
+  const bool has_mask = a.mask != nullptr;
+  int64_t lo, hi;
+  split_range(a, g, sp, lo, hi);
+  const bool any_batch = a.mean_level == LEVEL_BATCH || a.std_level == LEVEL_BATCH;
+  const int64_t st = (int64_t)a.G * a.nsplit;
+  double v[10];  // group sums 0..4, batch sums 5..9
+#pragma unroll
+  for (int k = 0; k < 10; ++k) v[k] = 0.0;
+  for (int i = threadIdx.x; i < a.nsplit; i += blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + (int64_t)g * a.nsplit + i];
+  }
+  if (any_batch) {
+    for (int64_t i = threadIdx.x; i < st; i += blockDim.x) {
+#pragma unroll
+      for (int k = 0; k < 5; ++k) v[5 + k] += a.part[k * st + i];
+    }
+  } else if (has_mask) {
+    for (int64_t i = threadIdx.x; i < st; i += blockDim.x) v[5] += a.part[i];
+  }
+  block_sum_n<10>(v, smem);
+  if (has_mask && v[5] == 0.0) {  // nothing active: the input is returned unchanged
+    for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) a.out[i] = a.x[i];
+    return;
+  }
+  // mean context (see make_mean_ctx; no leave-one-out here)
+  MeanCtx mc;
+  mc.level = a.mean_level; mc.identity = false; mc.zero = false; mc.loo = false; mc.cnt = 0.0; mc.sum = 0.0;
+  if (a.mean_level == LEVEL_BATCH) { mc.cnt = v[5]; mc.sum = v[6]; if (mc.cnt == 0.0) mc.zero = true; }
+  else if (a.mean_level == LEVEL_GROUP) {
+    if (g == a.tail_group) mc.zero = true;
+    else { mc.cnt = v[0]; mc.sum = v[1]; if (mc.cnt == 0.0) mc.zero = true; }
+  } else mc.zero = true;
+  const double mean = elem_mean(mc, 0.f, 1.f, false);  // one value for the whole group
+  auto ss_of = [&](int base) {
+    const double ss = v[base + 4] - 2.0 * mean * v[base + 3] + mean * mean * v[base + 2];
+    return ss > 0.0 ? ss : 0.0;
+  };
+  double std_d = 1.0;
+  double eps = a.eps;
+  if (a.std_level == LEVEL_BATCH) {
+    const double cnt = v[5], ss = ss_of(5);
+    if (a.unbiased) std_d = cnt <= 1.0 ? 1.0 : sqrt(ss / (cnt - 1.0));
+    else std_d = cnt == 0.0 ? 1.0 : sqrt(ss / cnt);
+  } else if (a.std_level == LEVEL_GROUP) {
+    if (g == a.tail_group) std_d = 0.0;
+    else if (a.grows[g] == 1 && a.unbiased) std_d = 1.0;
+    else {
+      const double cnt = v[0], ss = ss_of(0);
+      if (a.unbiased) std_d = cnt <= 1.0 ? 1.0 : sqrt(ss / (cnt - 1.0));
+      else std_d = cnt == 0.0 ? 1.0 : sqrt(ss / cnt);
+    }
+    std_d = (double)(float)std_d;
+  } else {
+    eps = 0.0;
+  }
+  const bool mean64 = a.mean_level == LEVEL_BATCH, std64 = a.std_level == LEVEL_BATCH;
+  auto one = [&](float x, float m) -> float {
+    if (mean64 || std64) {
+      double c = mean64 ? ((double)x - mean) : (double)(x - (float)mean);
+      if (has_mask) c = mean64 ? c * (double)m : (double)((float)c * m);
+      const double den = std64 ? (std_d + eps) : (double)((float)std_d + (float)eps);
+      return (float)(c / den);
+    }
+    float c = x - (float)mean;
+    if (has_mask) c = c * m;
+    return c / ((float)std_d + (float)eps);
+  };
+  int64_t mid_lo = (lo + 3) & ~(int64_t)3, mid_hi = hi & ~(int64_t)3;
+  if (mid_lo > mid_hi) { mid_lo = hi; mid_hi = hi; }
+  for (int64_t i = lo + threadIdx.x; i < mid_lo; i += blockDim.x) a.out[i] = one(a.x[i], has_mask ? a.mask[i] : 1.0f);
+  const int64_t step = 4 * (int64_t)blockDim.x;
+  for (int64_t i = mid_lo + 4 * (int64_t)threadIdx.x; i < mid_hi; i += 4 * step) {
+    f32x4 xv[4], mv[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t j = i + u * step;
+      xv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      mv[u] = f32x4{1.f, 1.f, 1.f, 1.f};
+      if (j < mid_hi) {
+        xv[u] = *(const f32x4*)(a.x + j);
+        if (has_mask) mv[u] = *(const f32x4*)(a.mask + j);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t j = i + u * step;
+      if (j >= mid_hi) break;
+      f32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = one(xv[u][e], mv[u][e]);
+      *(f32x4*)(a.out + j) = r;
+    }
+  }
+  for (int64_t i = mid_hi + threadIdx.x; i < hi; i += blockDim.x)
+    if (i >= mid_lo) a.out[i] = one(a.x[i], has_mask ? a.mask[i] : 1.0f);
 }
 
 // pass 2: sum of squared masked deviations per (group, split)
@@ -1248,7 +1435,7 @@ static int norm_nsplit(int64_t n_groups, int64_t max_group_len) {
 
 size_t areal_group_norm_workspace_bytes(int64_t n_groups, int64_t max_group_len) {
   if (n_groups <= 0) return 0;
-  return (size_t)3 * n_groups * norm_nsplit(n_groups, max_group_len) * sizeof(double) + 256;
+  return (size_t)5 * n_groups * norm_nsplit(n_groups, max_group_len) * sizeof(double) + 256;
 }
 
 // Normalization(x, mask, groups): levels 0 = none, 1 = batch, 2 = group.
@@ -1276,12 +1463,24 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
   a.unbiased = unbiased; a.eps = eps;
   a.part = (double*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   a.out = out;
+  // Two launches (one statistics pass) whenever every element of a group sees the same mean and a
+  // batch-level deviation does not sit on top of per-group means; otherwise the deviations need
+  // a pass of their own.
+  a.closed_form = (!leave_one_out && !(mean_level == LEVEL_GROUP && std_level == LEVEL_BATCH)) ? 1 : 0;
   const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
-  hipLaunchKernelGGL(norm_stats1_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
-  AREAL_CHECK_LAUNCH();
-  hipLaunchKernelGGL(norm_stats2_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
-  AREAL_CHECK_LAUNCH();
-  hipLaunchKernelGGL(norm_apply_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  if (a.closed_form) {
+    hipLaunchKernelGGL(norm_stats5_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+    AREAL_CHECK_LAUNCH();
+  } else {
+    hipLaunchKernelGGL(norm_stats1_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+    AREAL_CHECK_LAUNCH();
+    hipLaunchKernelGGL(norm_stats2_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+    AREAL_CHECK_LAUNCH();
+  }
+  if (a.closed_form)
+    hipLaunchKernelGGL(norm_apply_cf_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  else
+    hipLaunchKernelGGL(norm_apply_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

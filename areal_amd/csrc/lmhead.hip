@@ -47,7 +47,11 @@ struct GemmArgs {
   // and writes its partial result zstride bytes after the previous copy's. ksplit <= 1: off.
   int ksplit, kt_per_split;
   int64_t zstride;
+  // When set and the int it points to is non-zero, the launch does nothing (every workgroup
+  // returns at once): lets the host queue a launch sequence before it knows a device-side status.
+  const int* skip_if_set;
 };
+DEVI bool gemm_skipped(const GemmArgs& g) { return g.skip_if_set != nullptr && *g.skip_if_set != 0; }
 
 // Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
 // the 8 XCDs, so the 32 workgroups resident on one XCD are id = xcd + 8*q for 32 consecutive
@@ -156,6 +160,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_generic(GemmArgs g, Sched sc
                                                             typename Epi::Params ep) {
   __shared__ __attribute__((aligned(16))) u16 lds[2 * 2 * OPER];
   int bj, split, ai_begin, ai_end;
+  if (gemm_skipped(g)) return;
   if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -259,6 +264,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
     Epi::split_output(ep, (int64_t)z * g.zstride);
     if (nk <= 0) return;
   }
+  if (gemm_skipped(g)) return;
   if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -432,6 +438,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
                                                           typename Epi::Params ep) {
   __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
   int bj, split, ai_begin, ai_end;
+  if (gemm_skipped(g)) return;
   if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -606,6 +613,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_mix_sweep(GemmArgs g, Sched sc,
     Epi::split_output(ep, (int64_t)z * g.zstride);
     if (nk <= 0) return;
   }
+  if (gemm_skipped(g)) return;
   if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1223,7 +1231,9 @@ __global__ __launch_bounds__(256) void saved_prep_kernel(
     const int64_t* __restrict__ labels, const float* __restrict__ row_max,
     const float* __restrict__ sum_exp, const float* __restrict__ grad,
     const float* __restrict__ logprobs, const u16* __restrict__ hidden, int T, int H, int V,
-    float c2, float gscale, float* __restrict__ rowfac, u16* __restrict__ hs) {
+    float c2, float gscale, float* __restrict__ rowfac, u16* __restrict__ hs,
+    const int* __restrict__ skip_if_set) {
+  if (skip_if_set != nullptr && *skip_if_set != 0) return;
   const int t = blockIdx.x;
   if (t >= T) {
     u16* row = probs + (int64_t)t * ldv;
@@ -1267,7 +1277,9 @@ __global__ __launch_bounds__(256) void saved_prep_kernel(
 __global__ __launch_bounds__(256) void colsum_bf16_kernel(const u16* __restrict__ dl, int64_t ld,
                                                           int64_t rows, int V, int accumulate,
                                                           const float* __restrict__ w,
-                                                          float* __restrict__ out) {
+                                                          float* __restrict__ out,
+                                                          const int* __restrict__ skip_if_set) {
+  if (skip_if_set != nullptr && *skip_if_set != 0) return;
   __shared__ float sm[4][64];
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int lane_row = threadIdx.x >> 6;
@@ -1308,7 +1320,9 @@ __global__ __launch_bounds__(256) void transpose_pad_bf16_kernel(const u16* __re
 // split-K partial results of dHidden. row_len % 4 == 0.
 __global__ void splitk_reduce_bf16_kernel(const float* __restrict__ part, int Z, int64_t zstride,
                                           int64_t n, const float* __restrict__ scale,
-                                          int64_t row_len, u16* __restrict__ out) {
+                                          int64_t row_len, u16* __restrict__ out,
+                                          const int* __restrict__ skip_if_set) {
+  if (skip_if_set != nullptr && *skip_if_set != 0) return;
   int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
   for (; i < n; i += stride) {  // n % 4 == 0
@@ -1458,6 +1472,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
     Epi::split_output(ep, (int64_t)z * g.zstride);
     if (nk <= 0) return;
   }
+  if (gemm_skipped(g)) return;
   if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -2095,17 +2110,20 @@ int launch_dhidden_k(const GemmArgs& g0, int64_t H, int64_t T, int64_t ldv, void
   int64_t blocks = ceil_div_i64(T * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
   hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, partial,
-                     z, T * H, T * H, tscale, H, (u16*)dhidden);
+                     z, T * H, T * H, tscale, H, (u16*)dhidden, g.skip_if_set);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
 int launch_dhidden(const u16* w, int64_t V, const u16* dl, int64_t ldv, int64_t H, int64_t T,
-                   void* dhidden, float* partial, const float* tscale, hipStream_t stream) {
+                   void* dhidden, float* partial, const float* tscale, const int* skip_if_set,
+                   hipStream_t stream) {
   if (dh_weight_in_place(V)) {
-    const GemmArgs g{w, H, (int)H, dl, ldv, (int)T, (int)ldv, (int)H, 0};
+    GemmArgs g{w, H, (int)H, dl, ldv, (int)T, (int)ldv, (int)H, 0};
+    g.skip_if_set = skip_if_set;
     return launch_dhidden_k<KERNEL_MIX, KERNEL16_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
   }
-  const GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
+  GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
+  g.skip_if_set = skip_if_set;
   return launch_dhidden_k<KERNEL_NT, KERNEL16_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
 }
 
@@ -2308,13 +2326,13 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
     if (dhidden != nullptr) {
       if ((rc = launch_dhidden(w_in_place ? (const u16*)weight : wT, V, dl, ldv, H, Tc,
-                               (u16*)dhidden + t0 * H, dh_part, nullptr, stream)) != AREAL_OK)
+                               (u16*)dhidden + t0 * H, dh_part, nullptr, nullptr, stream)) != AREAL_OK)
         return rc;
     }
     // dBias[v] += sum_t dl[t, v]
     if (dbias != nullptr) {
       hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
-                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, nullptr, dbias);
+                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, nullptr, dbias, nullptr);
       AREAL_CHECK_LAUNCH();
     }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
@@ -2356,12 +2374,15 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // (and rows [T, round_up(T, 64)) are cleared), so probs can be used once. logprobs (nullable)
 // are the label log-probabilities of the forward; with them the label's entry is evaluated in
 // fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store (the
-// whole batch is one contraction, so no fp32 staging is needed).
+// whole batch is one contraction, so no fp32 staging is needed). probs_status (nullable): the
+// device int areal_lmhead_fwd set; when it reads non-zero at execution time every kernel of this
+// call returns at once and no output is touched, so the call can be queued before the host has
+// seen the status (which it then checks, and runs areal_lmhead_bwd instead if it was set).
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
-                           const float* probs_ref, void* dhidden, void* dweight,
+                           const float* probs_ref, const int* probs_status, void* dhidden, void* dweight,
                            int dweight_mode, float* dbias, void* workspace,
                            size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0) return AREAL_ERR_BAD_ARG;
@@ -2391,7 +2412,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   hipLaunchKernelGGL(saved_prep_kernel, dim3((unsigned)Tpad), dim3(256), 0, stream, e, ldv, probs_ref,
                      labels, row_max, sum_exp, grad_logprobs, logprobs, (const u16*)hidden, (int)T,
                      (int)H, (int)V, inv_temperature * LOG2E, inv_temperature * logit_scale, rowfac,
-                     dweight != nullptr ? hs : nullptr);
+                     dweight != nullptr ? hs : nullptr, probs_status);
   AREAL_CHECK_LAUNCH();
   if (dhidden != nullptr) {
     if (!w_in_place) {
@@ -2401,18 +2422,19 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
       AREAL_CHECK_LAUNCH();
     }
     if ((rc = launch_dhidden(w_in_place ? (const u16*)weight : wT, V, e, ldv, H, T, dhidden, dh_part,
-                             rowfac, stream)) != AREAL_OK)
+                             rowfac, probs_status, stream)) != AREAL_OK)
       return rc;
   }
   if (dbias != nullptr) {
     hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
-                       e, ldv, T, (int)V, dweight_mode == 1 ? 1 : 0, (const float*)rowfac, dbias);
+                       e, ldv, T, (int)V, dweight_mode == 1 ? 1 : 0, (const float*)rowfac, dbias, probs_status);
     AREAL_CHECK_LAUNCH();
   }
   if (dweight != nullptr) {
     // dWeight[v, h] += sum_t e'[t, v] * hs[t, h], k-major over the Tpad rows of both (rows past
     // T are cleared)
     GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv};
+    g.skip_if_set = probs_status;
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
     rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : dweight_mode == 0 ? 1 : 0, stream);

@@ -2,6 +2,7 @@
 
 from areal_amd.functional.functional import (
     RejectionSamplingResult,
+    DeferredFloat,
     StatReduction,
     apply_rejection_sampling,
     cispo_loss_fn,
@@ -27,6 +28,7 @@ from areal_amd.functional.vocab_parallel import (
 
 __all__ = [
     "RejectionSamplingResult",
+    "DeferredFloat",
     "StatReduction",
     "apply_rejection_sampling",
     "cispo_loss_fn",

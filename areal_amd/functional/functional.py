@@ -51,6 +51,89 @@ REDUCED_STAT_KEYS = (
 )
 
 
+class _HostCopy:
+    """A small device tensor on its way to pinned host memory: queued behind the kernels that
+    write it, waited for when the host first looks at it."""
+
+    def __init__(self, dev_tensor: torch.Tensor):
+        self._host = torch.empty(dev_tensor.shape, dtype=dev_tensor.dtype, pin_memory=True)
+        self._host.copy_(dev_tensor, non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record(torch.cuda.current_stream(dev_tensor.device))
+
+    def host(self) -> torch.Tensor:
+        self._event.synchronize()
+        return self._host
+
+
+class DeferredFloat:
+    """A host scalar of a loss call made with ``defer_host_reads=True``: the device-to-host copy
+    it comes from is waited for when the value is first used as a number (``float(x)``,
+    arithmetic, comparison, formatting), not when the loss function returns."""
+
+    __slots__ = ("_source", "_fn", "_value")
+
+    def __init__(self, source: _HostCopy, fn):
+        self._source, self._fn, self._value = source, fn, None
+
+    def __float__(self) -> float:
+        if self._value is None:
+            self._value = float(self._fn(self._source.host()))
+        return self._value
+
+    def __repr__(self) -> str:
+        return repr(float(self))
+
+    def __format__(self, spec: str) -> str:
+        return format(float(self), spec)
+
+    def __bool__(self) -> bool:
+        return bool(float(self))
+
+    def __eq__(self, other) -> bool:
+        return float(self) == other
+
+    def __lt__(self, other) -> bool:
+        return float(self) < other
+
+    def __le__(self, other) -> bool:
+        return float(self) <= other
+
+    def __gt__(self, other) -> bool:
+        return float(self) > other
+
+    def __ge__(self, other) -> bool:
+        return float(self) >= other
+
+    def __add__(self, other):
+        return float(self) + other
+
+    __radd__ = __add__
+
+    def __sub__(self, other):
+        return float(self) - other
+
+    def __rsub__(self, other):
+        return other - float(self)
+
+    def __mul__(self, other):
+        return float(self) * other
+
+    __rmul__ = __mul__
+
+    def __truediv__(self, other):
+        return float(self) / other
+
+    def __rtruediv__(self, other):
+        return other / float(self)
+
+
+def _host_value(c, fn):
+    """``fn(counters)`` as a float now, or as a ``DeferredFloat`` when the counters are still on
+    their way to the host."""
+    return DeferredFloat(c, fn) if isinstance(c, _HostCopy) else float(fn(c))
+
+
 class StatReduction:
     """Ask a loss call to reduce its logged statistics inside the kernel's token pass.
 
@@ -73,8 +156,26 @@ class StatReduction:
             raise ValueError(f"at most two extra statistics ride along, got {len(extras)}")
         self.entropy = entropy
         self.extras = extras
-        self.results: dict[str, dict[str, float | None]] = {}
-        self.denominators: dict[str, float] = {}
+        self._results: dict[str, dict[str, float | None]] = {}
+        self._denominators: dict[str, float] = {}
+        self._pending = None  # (host copy, arguments of _fill) of a call with deferred host reads
+
+    def _resolve(self) -> None:
+        if self._pending is not None:
+            copy, n_tokens, has_rs, has_old = self._pending
+            self._pending = None
+            host = copy.host()
+            self._fill(host[8:].view(-1, 4), host[:8], n_tokens, has_rs, has_old)
+
+    @property
+    def results(self) -> dict[str, dict[str, float | None]]:
+        self._resolve()
+        return self._results
+
+    @property
+    def denominators(self) -> dict[str, float]:
+        self._resolve()
+        return self._denominators
 
     def _fill(self, host: torch.Tensor, counters, n_tokens: int, has_rs: bool, has_old: bool) -> None:
         names = list(self.extras)
@@ -92,13 +193,13 @@ class StatReduction:
                 key = names[j]
             s, c, mn, mx = host[i].tolist()
             empty = c == 0
-            self.results[key] = dict(sum=s, count=c, avg=None if empty else s / c,
+            self._results[key] = dict(sum=s, count=c, avg=None if empty else s / c,
                                      min=None if empty else mn, max=None if empty else mx,
                                      denominator=denom)
-        self.denominators = dict(n_tokens=float(n_tokens), n_valid_tokens=float(counters[1]),
-                                 clipped_tokens=float(counters[4]), dual_clipped_tokens=float(counters[5]))
+        self._denominators = dict(n_tokens=float(n_tokens), n_valid_tokens=float(counters[1]),
+                                  clipped_tokens=float(counters[4]), dual_clipped_tokens=float(counters[5]))
         if has_rs:
-            self.denominators["unclipped_behave_tokens"] = float(counters[6])
+            self._denominators["unclipped_behave_tokens"] = float(counters[6])
 
 
 def _fill_rs(cfg: _lib.LossConfig, rs: RejectionSamplingConfig | None) -> None:
@@ -324,7 +425,7 @@ def apply_rejection_sampling(
 
 
 def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-                 rejection_sampling, cu_seqlens, reduction=None):
+                 rejection_sampling, cu_seqlens, reduction=None, defer=False):
     shape = logprobs.shape
     if rejection_sampling is not None:
         _check_rs_shapes(proximal_logprobs, old_logprobs, loss_mask)
@@ -340,7 +441,15 @@ def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, los
         _f32(old_logprobs) if want_old else None,
         _f32(advantages), mask_bool, cu_seqlens, sink, reduction,
     )
-    if reduction is None:
+    if defer:
+        # no host synchronisation in this call: the copy is queued and whoever reads a host
+        # scalar (or the reduction's results) waits for it then
+        if reduction is None:
+            c = _HostCopy(sink["counters_dev"])
+        else:
+            c = _HostCopy(sink["counters_and_stats_dev"])
+            reduction._pending = (c, int(mask_bool.numel()), rejection_sampling is not None, want_old)
+    elif reduction is None:
         c = sink["counters_dev"].cpu()  # the one host synchronisation of the call
     else:
         host = sink["counters_and_stats_dev"].cpu()  # counters and reduced statistics, one copy
@@ -352,13 +461,16 @@ def _loss_common(cfg, logprobs, proximal_logprobs, old_logprobs, advantages, los
 
 def _scalar_stats(loss_mask, c):
     n_total = float(loss_mask.numel())
-    n_valid = float(c[1])
     return dict(
         n_total_tokens=n_total,
-        n_valid_tokens=n_valid,
-        n_masked_tokens=n_total - n_valid,
-        masked_token_ratio=1.0 - n_valid / max(n_total, 1.0),
+        n_valid_tokens=_host_value(c, lambda h: h[1]),
+        n_masked_tokens=_host_value(c, lambda h: n_total - float(h[1])),
+        masked_token_ratio=_host_value(c, lambda h: 1.0 - float(h[1]) / max(n_total, 1.0)),
     )
+
+
+def _filtered_fraction(c):
+    return _host_value(c, lambda h: float(h[3]) / max(float(h[1]), 1.0))
 
 
 def _rs_stats(stat, sink, c, shape, rejection_sampling):
@@ -368,7 +480,7 @@ def _rs_stats(stat, sink, c, shape, rejection_sampling):
         behave_approx_kl=sink["behave_approx_kl"].view(shape),
         behave_imp_weight=sink["behave_imp_weight"].view(shape),
         behave_mask=sink["behave_mask"].view(shape),
-        filtered_fraction=float(c[3]) / max(float(c[1]), 1.0),
+        filtered_fraction=_filtered_fraction(c),
     )
 
 
@@ -385,11 +497,14 @@ def ppo_actor_loss_fn(
     importance_sampling_level: str = "token",
     cu_seqlens: torch.Tensor | None = None,
     stat_reduction: StatReduction | None = None,
+    defer_host_reads: bool = False,
 ) -> tuple[torch.Tensor, dict]:
     """PPO/GRPO clipped surrogate with optional dual clip, GSPO sequence-level ratio and
     rejection sampling.  Signature, return structure and ``stat`` keys as in
     ``functional.py:452-596``.  ``stat_reduction`` (not in the reference): reduce the logged
-    statistics in the kernel instead of returning per-token tensors, see ``StatReduction``."""
+    statistics in the kernel instead of returning per-token tensors, see ``StatReduction``.
+    ``defer_host_reads`` (not in the reference): the call does not wait for the GPU; the host
+    scalars of ``stat`` are ``DeferredFloat`` objects that wait when they are first used."""
     if importance_sampling_level == "sequence":
         if logprobs.ndim == 1 and cu_seqlens is None:
             raise ValueError(
@@ -414,12 +529,12 @@ def ppo_actor_loss_fn(
     cfg.seq_is = int(importance_sampling_level == "sequence")
     loss, sink, c, shape = _loss_common(
         cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-        rejection_sampling, cu_seqlens, stat_reduction,
+        rejection_sampling, cu_seqlens, stat_reduction, defer_host_reads,
     )
     if stat_reduction is not None:
         stat = _scalar_stats(loss_mask, c)
         if rejection_sampling is not None:
-            stat["filtered_fraction"] = float(c[3]) / max(float(c[1]), 1.0)
+            stat["filtered_fraction"] = _filtered_fraction(c)
         return loss, stat
     stat = dict(
         loss=sink["stat_loss"].view(shape),
@@ -444,10 +559,11 @@ def cispo_loss_fn(
     rejection_sampling: RejectionSamplingConfig | None = None,
     cu_seqlens: torch.Tensor | None = None,
     stat_reduction: StatReduction | None = None,
+    defer_host_reads: bool = False,
 ) -> tuple[torch.Tensor, dict]:
     """CISPO: clipped importance weight under stop-gradient times ``log pi`` (MiniMax-M1).
-    Signature, errors and ``stat`` keys as in ``functional.py:678-793``; ``stat_reduction`` as in
-    ``ppo_actor_loss_fn``."""
+    Signature, errors and ``stat`` keys as in ``functional.py:678-793``; ``stat_reduction`` and
+    ``defer_host_reads`` as in ``ppo_actor_loss_fn``."""
     if eps_clip_higher is None or eps_clip_higher <= 0:
         raise ValueError(
             "CISPO requires a positive eps_clip_higher; the asymmetric upper "
@@ -459,12 +575,12 @@ def cispo_loss_fn(
     cfg.clip_hi = 1.0 + eps_clip_higher
     loss, sink, c, shape = _loss_common(
         cfg, logprobs, proximal_logprobs, old_logprobs, advantages, loss_mask,
-        rejection_sampling, cu_seqlens, stat_reduction,
+        rejection_sampling, cu_seqlens, stat_reduction, defer_host_reads,
     )
     if stat_reduction is not None:
         stat = {}
         if rejection_sampling is not None:
-            stat["filtered_fraction"] = float(c[3]) / max(float(c[1]), 1.0)
+            stat["filtered_fraction"] = _filtered_fraction(c)
         return loss, stat
     stat = dict(
         loss=sink["stat_loss"].view(shape),

@@ -173,43 +173,52 @@ class _FusedLMHead(torch.autograd.Function):
         # the kernels need one of dHidden / dWeight as an output; a bias-only request computes dHidden
         need_h = need_h or (need_b and not need_w)
         dh = torch.empty_like(hidden_2d) if need_h else None
-        db32 = torch.empty(V, dtype=torch.float32, device=dev) if need_b else None
-        probs, probs_ref = ctx.probs, ctx.probs_ref
-        # whether every row's saved exponentials are in range: copied to pinned memory behind the
-        # forward; by now that copy has normally completed and the wait returns at once
-        if probs is not None:
-            ctx.status_event.synchronize()
-            if int(ctx.status_host[0]) != 0:
-                probs = probs_ref = None
+        # (zeroed when the kernels add to it, which they do together with the weight accumulator)
+        db32 = None
+        if need_b:
+            db32 = (torch.zeros if accum is not None else torch.empty)(V, dtype=torch.float32, device=dev)
+        probs, probs_ref, probs_status = ctx.probs, ctx.probs_ref, ctx.probs_status
         # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
         # the chunked recompute mode accumulates in fp32 and casts at the end
         direct = accum is None and probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
         dw_direct = torch.empty((V, H), dtype=torch.bfloat16, device=dev) if (need_w and direct) else None
-        if accum is not None:
-            dw32 = accum
-        else:
-            dw32 = torch.empty((V, H), dtype=torch.float32, device=dev) if (need_w and not direct) else None
+        dw32 = accum
+        if accum is None and need_w and not direct:
+            dw32 = torch.empty((V, H), dtype=torch.float32, device=dev)
         ctx.probs = ctx.probs_ref = ctx.probs_status = None  # consumed; a second backward recomputes
+        recompute = probs is None
         if T == 0:
+            recompute = False
             if dw32 is not None and accum is None:
                 dw32.zero_()
             if db32 is not None:
                 db32.zero_()
         elif probs is not None:
+            # Queued before the host knows whether every row's saved exponentials were in range:
+            # the kernels read that status on the device and return at once if it is set.
             nbytes = lib.areal_lmhead_bwd_saved_workspace_bytes(T, H, V)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             rc = lib.areal_lmhead_bwd_saved(
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(labels_1d),
                 _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
-                _lib.ptr(probs), _lib.ptr(probs_ref),
+                _lib.ptr(probs), _lib.ptr(probs_ref), _lib.ptr(probs_status),
                 _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32),
                 2 if direct else (1 if accum is not None else 0),
                 _lib.ptr(db32), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd_saved")
+            # The status travelled to pinned memory behind the forward. Looking at it now, with
+            # the launches above already queued, idles nothing; if it was set (a row's maximum
+            # far above its estimate) those launches did nothing and the recompute mode runs.
+            ctx.status_event.synchronize()
+            if int(ctx.status_host[0]) != 0:
+                recompute = True
+                if need_w and direct:
+                    direct, dw_direct = False, None
+                    dw32 = torch.empty((V, H), dtype=torch.float32, device=dev)
             del probs, probs_ref
-        else:
+        if recompute:
             chunk = ctx.token_chunk or default_token_chunk(T, H, V)
             nbytes = lib.areal_lmhead_bwd_workspace_bytes(T, H, V, chunk)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)

@@ -65,8 +65,16 @@ def grpo_loss_fn(
     vocab_norm_logits: torch.Tensor | None = None,
     stats: dict | None = None,
     stats_mode: str = "tensors",
+    defer_host_reads: bool = False,
 ):
     """Actor loss of one packed micro-batch; returns the scalar loss.
+
+    ``defer_host_reads=True`` (PPO and CISPO losses; not in the reference): the call queues its
+    kernels and returns without waiting for the GPU, so that the backward can be queued while the
+    forward still runs.  Host scalars in ``stats`` are then ``DeferredFloat`` objects that wait
+    when first used, reduced statistics stay in ``stats["reduction"]`` (a ``StatReduction`` whose
+    ``results`` wait likewise), and a NaN or Inf in the proximal log-probs, which the reference
+    reports by raising here, makes the returned loss NaN instead.
 
     ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``.  With
     ``stats_mode="tensors"`` these are the bool denominators and fp32 statistics of the
@@ -140,6 +148,7 @@ def grpo_loss_fn(
             rejection_sampling=rejection_sampling,
             cu_seqlens=input_data.get("cu_seqlens"),
             stat_reduction=reduction,
+            defer_host_reads=defer_host_reads,
         )
     elif use_sapo_loss:
         if use_decoupled_loss:
@@ -171,9 +180,13 @@ def grpo_loss_fn(
             importance_sampling_level=importance_sampling_level,
             cu_seqlens=input_data.get("cu_seqlens"),
             stat_reduction=reduction,
+            defer_host_reads=defer_host_reads,
         )
 
-    _raise_if_nonfinite(prox_nonfinite, prox_logp_method)
+    if defer_host_reads and not use_sapo_loss:
+        loss = loss + torch.where(prox_nonfinite, float("nan"), 0.0).to(loss.dtype)
+    else:
+        _raise_if_nonfinite(prox_nonfinite, prox_logp_method)
 
     # joint distillation (actor.py:629-658)
     teacher_logp = input_data.get("teacher_logp")
@@ -191,9 +204,12 @@ def grpo_loss_fn(
             rkl_stat = term
 
     if reduction is not None:
-        stats.update(reduction.results)
-        for name, count in reduction.denominators.items():
-            stats["denominator/" + name] = count
+        if defer_host_reads:
+            stats["reduction"] = reduction
+        else:
+            stats.update(reduction.results)
+            for name, count in reduction.denominators.items():
+                stats["denominator/" + name] = count
         for key in ("n_total_tokens", "n_valid_tokens", "n_masked_tokens", "masked_token_ratio"):
             if key in stat:
                 stats["scalar/" + key] = stat[key]

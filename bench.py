@@ -186,6 +186,33 @@ def hbm_rooflines(dev):
     m = (torch.rand(T, device=dev) > 0.25).float()
     add("gae_owned_kernel", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
         20 * T, timed(lambda: compute_gae_packed(r, v, m, cu, None, 1.0, 0.95)))
+    # the same batch through the C ABI, launches back to back on the stream (no host work between
+    # them): packed GAE, then group normalisation (groups of 16 sequences, mean and deviation at
+    # group level) of the advantages under the same mask. 3 launches: gae_owned_kernel,
+    # norm_stats5_kernel, norm_apply_cf_kernel.
+    from areal_amd import _lib as L_
+
+    lib_ = L_.load()
+    adv_o, ret_o, nrm_o = torch.empty(T, device=dev), torch.empty(T, device=dev), torch.empty(T, device=dev)
+    goff = cu[::16].to(torch.int64).contiguous()
+    grow = torch.full((64,), 16, dtype=torch.int64, device=dev)
+    max_glen = int((goff[1:] - goff[:-1]).max())
+    gae_ws_n = lib_.areal_gae_workspace_bytes(T)
+    nrm_ws_n = lib_.areal_group_norm_workspace_bytes(64, max_glen)
+    gae_ws, nrm_ws = L_.workspace(gae_ws_n, dev), L_.workspace(nrm_ws_n, dev)
+    strm = L_.stream_ptr(dev)
+
+    def gae_then_norm():
+        rc = lib_.areal_gae_packed(L_.ptr(r), L_.ptr(v), L_.ptr(m), L_.ptr(cu), None, None, T, 1024, 0, 1.0, 0.95,
+                                   L_.ptr(adv_o), L_.ptr(ret_o), L_.ptr(gae_ws), gae_ws_n, strm)
+        rc |= lib_.areal_group_norm(L_.ptr(adv_o), L_.ptr(m), T, L_.ptr(goff), L_.ptr(grow), 64, max_glen, -1, 2, 2,
+                                    0, 1, 1e-5, L_.ptr(nrm_o), L_.ptr(nrm_ws), nrm_ws_n, strm)
+        assert rc == 0
+
+    add("gae_owned_kernel + norm_stats5_kernel + norm_apply_cf_kernel (C ABI)",
+        f"config 3: 1024 packed sequences, {T} tokens, GAE then group normalisation of the advantages, "
+        "launches back to back, 20 + 20 B/token", 40 * T, timed(gae_then_norm))
+    del adv_o, ret_o, nrm_o
     # the padded drop-in signature on the same batch: [1024, 8192] (8.39 M slots)
     from areal_amd.ppo.gae import _compute_token_level_gae
 
@@ -219,12 +246,12 @@ def hbm_rooflines(dev):
     x = torch.randn(1024, 1600, device=dev)
     mk = (torch.rand(1024, 1600, device=dev) > 0.25).float()
     norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
-    add("norm_stats1+norm_stats2+norm_apply", "config 3: [1024, 1600] advantages, groups of 16 rows, 20 B/token",
+    add("norm_stats5_kernel + norm_apply_cf_kernel", "config 3: [1024, 1600] advantages, groups of 16 rows, 20 B/token",
         20 * x.numel(), timed(lambda: norm(x, mk)))
     # the same normalisation at the padded size, where launch latency no longer dominates
     xl_ = torch.randn(1024, 8192, device=dev)
     ml_ = (torch.rand(1024, 8192, device=dev) > 0.25).float()
-    add("norm_stats1+norm_stats2+norm_apply", "[1024, 8192] advantages, groups of 16 rows, 20 B/token",
+    add("norm_stats5_kernel + norm_apply_cf_kernel", "[1024, 8192] advantages, groups of 16 rows, 20 B/token",
         20 * xl_.numel(), timed(lambda: norm(xl_, ml_)))
     del xl_, ml_
     Tl = 4 << 20

@@ -87,12 +87,15 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * log-probabilities: with them the label's dlogit is -expm1(logprob) in fp32. dweight [V,H]:
  * dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store; dbias [V] fp32 or NULL
  * (added to in mode 1). Other arguments as areal_lmhead_bwd; the bias itself does not enter (it
- * is part of the saved exponentials). */
+ * is part of the saved exponentials). probs_status (NULL allowed): the device int the forward
+ * set; when it reads non-zero at execution time every kernel of this call returns at once and
+ * no output is touched, so the call can be queued before the host has seen the status (the
+ * caller then checks it and runs areal_lmhead_bwd instead if it was set). */
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
                            float inv_temperature, float logit_scale, void* probs,
-                           const float* probs_ref, void* dhidden, void* dweight,
+                           const float* probs_ref, const int* probs_status, void* dhidden, void* dweight,
                            int dweight_mode, float* dbias, void* workspace,
                            size_t workspace_bytes, areal_stream_t stream);
 

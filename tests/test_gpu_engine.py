@@ -158,3 +158,60 @@ def test_adapter_bf16_parameters_get_bf16_gradients_and_bad_modules_are_refused(
     assert lm.lm_head.weight.grad.dtype == torch.bfloat16 and lm.lm_head.weight.grad.any()
     with pytest.raises(TypeError):
         FusedLMHeadAdapter(nn.Linear(4, 4))
+
+
+def test_step_is_queued_without_waiting_for_the_gpu(dev):
+    """Forward, loss and backward of one micro-batch with deferred host reads: no call of the
+    step may synchronise with the device before its last launch is queued (the saved-mode
+    backward is queued before the host looks at the forward's status; the loss's host scalars and
+    reduced statistics are read afterwards).  Results equal those of the synchronising calls."""
+    from areal_amd.functional import DeferredFloat, fused_lm_head_logprobs_entropy
+
+    T, H, V = 1536, 256, 4096
+    g = torch.Generator().manual_seed(11)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * 0.05).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    cu = torch.tensor([0, 500, 1100, 1536], dtype=torch.int32, device=dev)
+    with torch.no_grad():
+        logp0 = fused_lm_head_logprobs_entropy(hidden, weight, labels).logprobs
+    old = logp0 + (torch.randn(T, generator=g) * 0.3).to(dev)
+    data = dict(logprobs=old, advantages=torch.randn(T, generator=g).to(dev),
+                loss_mask=(torch.rand(T, generator=g) > 0.2).to(dev), prox_logp=logp0, cu_seqlens=cu)
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", lower=0.5, upper=2.0)
+    loss_fn = functools.partial(grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None,
+                                rejection_sampling=rs, stats_mode="reduced")
+
+    def step(defer):
+        h = hidden.clone().requires_grad_(True)
+        w = weight.clone().requires_grad_(True)
+        stats = {}
+        out = fused_lm_head_logprobs_entropy(h, w, labels, save_probs=True)
+        loss = loss_fn(out.logprobs, out.entropy, data, stats=stats, defer_host_reads=defer)
+        loss.backward()
+        return loss, h.grad, w.grad, stats
+
+    want_loss, want_dh, want_dw, want_stats = step(False)
+    step(True)  # warm-up: allocator and pinned-memory pools
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        loss, dh, dw, stats = step(True)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert isinstance(stats["scalar/n_valid_tokens"], DeferredFloat)
+    assert torch.equal(loss, want_loss) and torch.equal(dh, want_dh) and torch.equal(dw, want_dw)
+    assert float(stats["scalar/n_valid_tokens"]) == want_stats["scalar/n_valid_tokens"]
+    assert float(stats["scalar/rs_filtered_fraction"]) == want_stats["scalar/rs_filtered_fraction"]
+    red = stats["reduction"]
+    for key, val in red.results.items():
+        assert want_stats[key] == val, key
+    for name, count in red.denominators.items():
+        assert want_stats["denominator/" + name] == count
+
+    # a NaN in the proximal log-probs: the synchronising call raises, the deferred one poisons the loss
+    bad = dict(data, prox_logp=logp0.clone().index_fill_(0, torch.tensor([7], device=dev), float("nan")))
+    out = fused_lm_head_logprobs_entropy(hidden, weight, labels)
+    with pytest.raises(RuntimeError, match="prox_logp contains NaN or Inf"):
+        loss_fn(out.logprobs, out.entropy, bad)
+    assert torch.isnan(loss_fn(out.logprobs, out.entropy, bad, defer_host_reads=True))

@@ -195,10 +195,11 @@ def test_config3_gae_and_group_norm_full_size(dev):
     a = adv.cpu()
     assert torch.isfinite(a).all() and (a[cu[1:].long() - 1] == 0).all()
     torch.testing.assert_close(ret.cpu(), a + values, rtol=0, atol=0)
-    # prompt tokens repeat the advantage of the first response token (masked carry)
+    # prompt tokens repeat the advantage of the first response token (masked carry); threads of a
+    # tile reach it through different fp32 compositions of the same maps, hence a few ulps
     s = int(cu[5])
     p = int(lens[5]) // 4
-    assert (a[s:s + p] == a[s + p]).all()
+    torch.testing.assert_close(a[s:s + p], a[s + p].expand(p), rtol=2e-6, atol=2e-6 * scale)
 
     # group normalisation on the packed layout = padded [1024, L] semantics per group of 16 rows
     norm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
