@@ -449,6 +449,9 @@ def main() -> None:
         grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None,
         rejection_sampling=RejectionSamplingConfig(level="token", action="mask", metric="ratio",
                                                    lower=0.5, upper=2.0),
+        # the step is queued without waiting for the GPU: the loss's host scalars are read after
+        # the backward is queued (nothing is skipped on the device)
+        defer_host_reads=True,
     )
 
     # None: keep the exponentials if the bf16 [T, V] buffer fits the library's default limit
@@ -631,6 +634,7 @@ def main() -> None:
             "tokens": T, "hidden": H, "vocab": V,
             "loss": "PPO clip eps=0.2, rejection sampling ratio in [0.5, 2.0] (token, mask)",
             "final_loss": float(loss.detach().item()),
+            "host_reads": "deferred (grpo_loss_fn(defer_host_reads=True): no host wait between the launches of a step)",
             "backward": "saved bf16 exponentials" if saved else "recompute logits",
             "peak_hbm_gb": peak_hbm_gb,
         },
