@@ -90,6 +90,8 @@ SIGNATURES: dict[str, tuple] = {
         I,
         [P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, SZ, P],
     ),
+    "areal_gae_padded_row_stats": (I, [P, P, P, P, P, I64, I64, F, F, P, P, P, P]),
+    "areal_group_norm_from_row_stats": (I, [P, P, I64, I64, P, P, I64, I64, I, I, I, I, D, P, P, P]),
     "areal_seqlens_from_mask": (I, [P, I64, I64, P, P, P, P]),
     "areal_pack_padded": (I, [P, P, P, I64, I64, I64, I64, P]),
     "areal_unpack_to_padded": (I, [P, P, P, P, I64, I64, I64, P, I, P]),
@@ -132,6 +134,9 @@ class LossConfig(ctypes.Structure):
     ]
 
 _lib = None
+
+
+ERR_UNSUPPORTED = -5  # AREAL_ERR_UNSUPPORTED
 
 
 class ArealHipError(RuntimeError):

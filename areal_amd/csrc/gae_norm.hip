@@ -56,6 +56,26 @@ DEVI MapT<R> shfl_down_map(const MapT<R>& m, int d) {
   return r;
 }
 
+// N sums at once: one pair of barriers instead of N.
+template <int N>
+DEVI void block_sum_n(double (&v)[N], double* smem /* [4][N] */) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < N; ++k) v[k] = wave_sum(v[k]);
+  __syncthreads();
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) smem[w * N + k] = v[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    double r = 0.0;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i * N + k];
+    v[k] = r;
+  }
+}
+
 struct GaeArgs {
   const float* rewards;
   const float* values;
@@ -71,6 +91,9 @@ struct GaeArgs {
   float* adv;
   float* ret;
   int block_per_seq;         // single-pass kernel, padded rows of at least a tile: block = row
+  double* row_stats;         // nullable, with block_per_seq only: [5][n_seqs] sums over each row of
+                             // m, x m, m^2, m^2 x, m^2 x^2 (x = the advantage written, m = mask):
+                             // the statistics pass of the normalisation that follows, for free
 };
 
 DEVI int gae_seq_of(const GaeArgs& g, int64_t t) {
@@ -280,6 +303,8 @@ DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
 // (Blocks of 1024 threads, one 8192-token tile per padded row instead of four serial tiles of
 // 2048, measured slower: 46.7 against 30.8 us on [1024, 8192]; one such block fills a CU's
 // registers and the latency of its single pass is not covered by anything.)
+// STATS: also sum each row's advantages under the mask (block = row only), see GaeArgs::row_stats.
+template <bool STATS>
 __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
   __shared__ MapF smem[GAE_THREADS / 64];
   __shared__ MapF all[GAE_THREADS];
@@ -341,6 +366,7 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
   if (t_end <= t_begin) return;
 
   double A0 = 0.0, nv0 = 0.0;  // state entering the current tile from its right
+  double rs[STATS ? 5 : 1] = {0.0};
   for (int64_t tile = (t_end - 1) / GAE_TILE; tile >= t_begin / GAE_TILE; --tile) {
     const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
     // The thread keeps its 8 tokens as raw inputs plus two bit masks and rebuilds a token's map
@@ -453,6 +479,15 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
         oa[i] = A;
         orr[i] = oa[i] + v[i];
       }
+      if constexpr (STATS) {
+#pragma unroll
+        for (int i = 0; i < GAE_ITEMS; ++i) {
+          if (!((valid >> i) & 1u)) continue;
+          const double x = (double)oa[i], m = (double)ms[i];
+          const double xm = x * m, mm = m * m;
+          rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
+        }
+      }
       if (valid == (1u << GAE_ITEMS) - 1u) {
 #pragma unroll
         for (int q = 0; q < GAE_ITEMS / 4; ++q) {
@@ -469,6 +504,14 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
     const double A1 = fma((double)total.a11, A0, fma((double)total.a12, nv0, (double)total.b1));
     const double nv1 = fma((double)total.a22, nv0, (double)total.b2);
     A0 = A1; nv0 = nv1;
+  }
+  if constexpr (STATS) {  // block = row: uniform for the block
+    __shared__ double s_rs[4 * 5];
+    block_sum_n<5>(rs, s_rs);
+    if (tid == 0) {
+#pragma unroll
+      for (int k = 0; k < 5; ++k) g.row_stats[(int64_t)k * g.n_seqs + blockIdx.x] = rs[k];
+    }
   }
 }
 
@@ -494,6 +537,10 @@ struct NormArgs {
                            // closed_form, [5][G][nsplit]: sum m, sum x m, sum m^2, sum m^2 x, sum m^2 x^2
   float* out;
   int closed_form;         // the squared deviations come from the five sums of one statistics pass
+  // closed form only: where the five sums of a group are. part_rows == 0: [5][G][nsplit], written
+  // by norm_stats5_kernel. part_rows > 0: [5][part_rows], one entry per row of row_len elements
+  // (written by the GAE kernel); group g owns the rows from goff[g] / row_len on, grows[g] of them.
+  int64_t part_rows, row_len;
 };
 
 DEVI double block_sum_d(double v, double* smem) {
@@ -505,26 +552,6 @@ DEVI double block_sum_d(double v, double* smem) {
   double r = 0.0;
   for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i];
   return r;
-}
-
-// N sums at once: one pair of barriers instead of N.
-template <int N>
-DEVI void block_sum_n(double (&v)[N], double* smem /* [4][N] */) {
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-#pragma unroll
-  for (int k = 0; k < N; ++k) v[k] = wave_sum(v[k]);
-  __syncthreads();
-  if (lane == 0) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) smem[w * N + k] = v[k];
-  }
-  __syncthreads();
-#pragma unroll
-  for (int k = 0; k < N; ++k) {
-    double r = 0.0;
-    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) r += smem[i * N + k];
-    v[k] = r;
-  }
 }
 
 DEVI void split_range(const NormArgs& a, int g, int sp, int64_t& lo, int64_t& hi) {
@@ -687,13 +714,15 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_apply_cf_kernel(NormArgs a)
   int64_t lo, hi;
   split_range(a, g, sp, lo, hi);
   const bool any_batch = a.mean_level == LEVEL_BATCH || a.std_level == LEVEL_BATCH;
-  const int64_t st = (int64_t)a.G * a.nsplit;
+  const int64_t st = a.part_rows > 0 ? a.part_rows : (int64_t)a.G * a.nsplit;
+  const int64_t p0 = a.part_rows > 0 ? a.goff[g] / a.row_len : (int64_t)g * a.nsplit;
+  const int64_t pn = a.part_rows > 0 ? (g == a.tail_group ? a.part_rows - p0 : a.grows[g]) : a.nsplit;
   double v[10];  // group sums 0..4, batch sums 5..9
 #pragma unroll
   for (int k = 0; k < 10; ++k) v[k] = 0.0;
-  for (int i = threadIdx.x; i < a.nsplit; i += blockDim.x) {
+  for (int64_t i = threadIdx.x; i < pn; i += blockDim.x) {
 #pragma unroll
-    for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + (int64_t)g * a.nsplit + i];
+    for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + p0 + i];
   }
   if (any_batch) {
     for (int64_t i = threadIdx.x; i < st; i += blockDim.x) {
@@ -1352,13 +1381,13 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
   Map* totals = (Map*)wp;
   double* carry = (double*)(wp + (size_t)nb * sizeof(Map));
   GaeArgs g{rewards, values, loss_mask, cu_seqlens, no_eos, lambda_seq, n_tokens, (int)n_seqs,
-            uniform_len, discount, gae_lambda, advantages, returns, 0};
+            uniform_len, discount, gae_lambda, advantages, returns, 0, nullptr};
   // sequences of ordinary length: single pass, one launch. Very long sequences on average (few
   // blocks would own any work): reduce-then-scan over all tokens.
   if (n_tokens / n_seqs <= 64 * GAE_TILE) {
     g.block_per_seq = uniform_len >= GAE_TILE;
     const int64_t grid = g.block_per_seq ? n_seqs : ceil_div_i64(nb, 8) * 8;
-    hipLaunchKernelGGL(gae_owned_kernel, dim3((unsigned)grid), dim3(GAE_THREADS), 0, stream, g);
+    hipLaunchKernelGGL(gae_owned_kernel<false>, dim3((unsigned)grid), dim3(GAE_THREADS), 0, stream, g);
     AREAL_CHECK_LAUNCH();
     return AREAL_OK;
   }
@@ -1369,6 +1398,27 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
                      carry);
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(gae_apply_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g, carry);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// areal_gae_packed on a padded [n_seqs, uniform_len] batch whose rows are at least one tile (2048
+// tokens) long, which also leaves in row_stats [5][n_seqs] (fp64) the masked sums of each row's
+// advantages that areal_group_norm_from_row_stats turns into means and deviations: the
+// statistics pass of a normalisation of the advantages under the same mask, at no extra traffic.
+int areal_gae_padded_row_stats(const float* rewards, const float* values, const float* loss_mask,
+                               const uint8_t* no_eos, const float* lambda_seq, int64_t n_seqs,
+                               int64_t uniform_len, float discount, float gae_lambda,
+                               float* advantages, float* returns, double* row_stats,
+                               hipStream_t stream) {
+  if (n_seqs < 0 || uniform_len < 0) return AREAL_ERR_BAD_ARG;
+  if (n_seqs == 0 || uniform_len == 0) return AREAL_OK;
+  if (!rewards || !values || !loss_mask || !advantages || !returns || !row_stats) return AREAL_ERR_BAD_ARG;
+  if (uniform_len < GAE_TILE || uniform_len > 64 * (int64_t)GAE_TILE || n_seqs > (1 << 30))
+    return AREAL_ERR_UNSUPPORTED;
+  GaeArgs g{rewards, values, loss_mask, nullptr, no_eos, lambda_seq, n_seqs * uniform_len, (int)n_seqs,
+            uniform_len, discount, gae_lambda, advantages, returns, 1, row_stats};
+  hipLaunchKernelGGL(gae_owned_kernel<true>, dim3((unsigned)n_seqs), dim3(GAE_THREADS), 0, stream, g);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -1423,10 +1473,13 @@ int areal_gae_lambda_context(const float* loss_mask, const int32_t* turn_ids, in
   return AREAL_OK;
 }
 
-// Blocks per group: about 4096 elements per block, and at most 2048 partials per array in all
+// Blocks per group: 4096 to 8192 elements per block, and at most 2048 partials per array in all
 // (every block of the later passes sums them) unless there are more groups than that.
+// (5 blocks of these kernels fit a CU at a time: beyond 1280 blocks a second, partly empty round
+// starts, so larger inputs take 8192 elements per block.)
 static int norm_nsplit(int64_t n_groups, int64_t max_group_len) {
   int64_t s = ceil_div_i64(max_group_len, 4096);
+  if (s * n_groups > 1280) s = ceil_div_i64(max_group_len, 8192);
   const int64_t cap = n_groups >= 2048 ? 1 : 2048 / n_groups;
   if (s > cap) s = cap;
   if (s < 1) s = 1;
@@ -1467,6 +1520,7 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
   // batch-level deviation does not sit on top of per-group means; otherwise the deviations need
   // a pass of their own.
   a.closed_form = (!leave_one_out && !(mean_level == LEVEL_GROUP && std_level == LEVEL_BATCH)) ? 1 : 0;
+  a.part_rows = 0; a.row_len = 0;
   const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
   if (a.closed_form) {
     hipLaunchKernelGGL(norm_stats5_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
@@ -1481,6 +1535,37 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
     hipLaunchKernelGGL(norm_apply_cf_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
   else
     hipLaunchKernelGGL(norm_apply_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// The apply pass of areal_group_norm alone, on a [n_rows, row_len] array whose per-row sums
+// (row_stats [5][n_rows], as areal_gae_padded_row_stats leaves them) are already known: one
+// launch. Groups are runs of whole rows (group_offsets in elements, multiples of row_len).
+// Only for the level combinations that need no second statistics pass: no leave-one-out, and
+// not a group-level mean under a batch-level deviation (AREAL_ERR_UNSUPPORTED otherwise).
+int areal_group_norm_from_row_stats(const float* x, const float* mask, int64_t n_rows, int64_t row_len,
+                                    const int64_t* group_offsets, const int64_t* group_rows,
+                                    int64_t n_groups, int64_t max_group_len, int tail_group,
+                                    int mean_level, int std_level, int unbiased, double eps,
+                                    const double* row_stats, float* out, hipStream_t stream) {
+  if (n_rows < 0 || row_len < 0 || n_groups < 0) return AREAL_ERR_BAD_ARG;
+  if (n_rows == 0 || row_len == 0) return AREAL_OK;
+  if (!x || !out || !group_offsets || !group_rows || !row_stats || n_groups == 0) return AREAL_ERR_BAD_ARG;
+  if (mean_level < 0 || mean_level > 2 || std_level < 0 || std_level > 2) return AREAL_ERR_BAD_ARG;
+  if (mean_level == LEVEL_GROUP && std_level == LEVEL_BATCH) return AREAL_ERR_UNSUPPORTED;
+  if (n_groups > 65535 * 16) return AREAL_ERR_UNSUPPORTED;
+  NormArgs a;
+  a.x = x; a.mask = mask; a.n = n_rows * row_len; a.goff = group_offsets; a.grows = group_rows;
+  a.G = (int)n_groups; a.tail_group = tail_group; a.nsplit = norm_nsplit(n_groups, max_group_len);
+  a.mean_level = mean_level; a.std_level = std_level; a.leave1out = 0;
+  a.unbiased = unbiased; a.eps = eps;
+  a.part = const_cast<double*>(row_stats);
+  a.out = out;
+  a.closed_form = 1;
+  a.part_rows = n_rows; a.row_len = row_len;
+  const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
+  hipLaunchKernelGGL(norm_apply_cf_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

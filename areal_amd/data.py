@@ -112,6 +112,42 @@ class Normalization:
         return out
 
 
+    def needs_one_statistics_pass(self) -> bool:
+        """True when the sums of one pass over the data determine the result: no leave-one-out
+        mean, and not a group-level mean under a batch-level deviation."""
+        return not self.mean_leave1out and not (self.mean_level == "group" and self.std_level == "batch")
+
+    @torch.no_grad()
+    def from_row_stats(self, x: torch.Tensor, mask_f32: torch.Tensor, row_stats: torch.Tensor,
+                       group_sizes: list[int] | None = None) -> torch.Tensor | None:
+        """``self(x, mask)`` for a 2-D fp32 ``x`` whose per-row masked sums are already known
+        (``row_stats`` ``[5, bs]`` fp64 as the GAE kernel leaves them): one launch. Returns
+        ``None`` when this configuration needs a second statistics pass."""
+        if not self.needs_one_statistics_pass() or x.ndim != 2:
+            return None
+        lib = _lib.load()
+        dev = _lib.require_gpu(x, mask_f32, row_stats)
+        bs, row_len = x.shape
+        if self.mean_level == "group" or self.std_level == "group":
+            groups, tail = self._group_rows(bs, group_sizes)
+        else:
+            groups, tail = (bs,), 0
+        if not groups and tail == 0:
+            return x
+        offsets, rows, tail_group, max_len = _group_tables(groups, tail, row_len, str(dev))
+        out = torch.empty_like(x)
+        rc = lib.areal_group_norm_from_row_stats(
+            _lib.ptr(x), _lib.ptr(mask_f32), bs, row_len, _lib.ptr(offsets), _lib.ptr(rows), rows.numel(),
+            max_len, tail_group, _LEVEL_ID[self.mean_level], _LEVEL_ID[self.std_level],
+            int(bool(self.std_unbiased)), float(self.eps), _lib.ptr(row_stats), _lib.ptr(out),
+            _lib.stream_ptr(dev),
+        )
+        if rc == _lib.ERR_UNSUPPORTED:
+            return None
+        _lib.check(rc, "areal_group_norm_from_row_stats")
+        return out
+
+
 class KLEstimator:
     """k1 / k2 / k3 estimators of KL(new || base) from log-probabilities
     (``data.py:1640-1698``).  Elementwise tensor arithmetic on whatever device holds the

@@ -24,7 +24,12 @@ from areal_amd.functional.functional import (
     ppo_actor_loss_fn,
     reward_overlong_penalty,
 )
-from areal_amd.ppo.gae import _compute_token_level_gae, _compute_turn_level_gae, compute_gae_lambda
+from areal_amd.ppo.gae import (
+    _compute_token_level_gae,
+    _compute_turn_level_gae,
+    _token_level_gae_with_row_stats,
+    compute_gae_lambda,
+)
 
 # areal/utils/constants.py:36-92
 PROX_LOGP_METHOD_RECOMPUTE = "recompute"
@@ -633,14 +638,26 @@ def compute_advantages(
         )
         advantages = advantages + gae_kl_rewards
     else:
-        advantages, returns = _compute_token_level_gae(
-            rewards=rewards,
-            values=values,
-            loss_mask=loss_mask,
-            seq_no_eos_mask=seq_no_eos_mask,
-            discount=discount,
-            gae_lambda=gae_lambda,
-        )
+        # With long padded rows and a normalisation that needs one statistics pass, the GAE kernel
+        # sums each row's advantages under the mask while it writes them, and the normalisation
+        # is its apply pass alone: two launches for the two stages (same results).
+        fused = None
+        if isinstance(adv_norm, Normalization) and adv_norm.needs_one_statistics_pass() and rewards.ndim == 2:
+            fused = _token_level_gae_with_row_stats(rewards, values, loss_mask, seq_no_eos_mask, discount, gae_lambda)
+        if fused is not None:
+            advantages, returns, row_stats, mask_f32 = fused
+            normed = adv_norm.from_row_stats(advantages, mask_f32, row_stats, group_sizes=group_sizes)
+            if normed is not None:
+                advantages, adv_norm = normed, None
+        else:
+            advantages, returns = _compute_token_level_gae(
+                rewards=rewards,
+                values=values,
+                loss_mask=loss_mask,
+                seq_no_eos_mask=seq_no_eos_mask,
+                discount=discount,
+                gae_lambda=gae_lambda,
+            )
     data["returns"] = returns
     if adv_norm is not None:
         advantages = adv_norm(advantages, loss_mask, group_sizes=group_sizes)

@@ -69,6 +69,32 @@ def _compute_token_level_gae(
     )
 
 
+def _token_level_gae_with_row_stats(rewards, values, loss_mask, seq_no_eos_mask, discount, gae_lambda):
+    """``_compute_token_level_gae`` that also returns, per row, the masked sums of the advantages
+    which ``Normalization.from_row_stats`` needs (``[5, bs]`` fp64), or ``None`` when the layout
+    does not allow it (rows shorter than one 2048-token tile)."""
+    bs, max_seqlen = rewards.shape
+    if max_seqlen < 2048 or bs == 0:
+        return None
+    lib = _lib.load()
+    dev = _lib.require_gpu(rewards, values, loss_mask)
+    lam_seq, lam = _split_lambda(gae_lambda, bs, dev)
+    r = rewards.to(torch.float32).contiguous()
+    v = values.to(torch.float32).contiguous()
+    m = loss_mask.to(torch.float32).contiguous()
+    no_eos = seq_no_eos_mask.to(torch.bool).contiguous()
+    adv, ret = torch.empty_like(r), torch.empty_like(r)
+    row_stats = torch.empty((5, bs), dtype=torch.float64, device=dev)
+    rc = lib.areal_gae_padded_row_stats(
+        _lib.ptr(r), _lib.ptr(v), _lib.ptr(m), _lib.ptr(no_eos), _lib.ptr(lam_seq), bs, max_seqlen,
+        float(discount), float(lam), _lib.ptr(adv), _lib.ptr(ret), _lib.ptr(row_stats), _lib.stream_ptr(dev),
+    )
+    if rc == _lib.ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "areal_gae_padded_row_stats")
+    return adv, ret, row_stats, m
+
+
 def compute_gae_packed(
     rewards: torch.Tensor,
     values: torch.Tensor,

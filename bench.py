@@ -236,8 +236,9 @@ def hbm_rooflines(dev):
                     ref_logp=torch.randn(1024, 8192, device=dev) * 0.1 - 1, values=vp,
                     rewards=(torch.rand(1024, device=dev) > 0.5).float())
     gnorm = Normalization(NormConfig(mean_level="group", std_level="group", group_size=16))
-    add("adv_prep_kernel + gae_owned_kernel + norm kernels (compute_advantages, API level)",
-        "config 3 padded form: [1024, 8192], KL-shaped rewards, GAE, group normalisation; "
+    add("adv_prep_kernel + gae_owned_kernel<stats> + norm_apply_cf_kernel (compute_advantages, API level)",
+        "config 3 padded form: [1024, 8192], KL-shaped rewards, GAE that also sums each row's advantages, "
+        "group normalisation as its apply pass alone (plus the [1024] reward normalisation); "
         "26 + 20 + 20 B/slot",
         66 * rp.numel(),
         timed(lambda: compute_advantages(dict(adv_data), kl_ctl=0.01, kl_estimator=KLEstimator("k1"),

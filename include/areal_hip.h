@@ -300,6 +300,17 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
                      float gae_lambda, float* advantages, float* returns, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
 
+/* areal_gae_packed on a padded [n_seqs, uniform_len] batch with rows of at least 2048 tokens
+ * (AREAL_ERR_UNSUPPORTED otherwise), which also leaves per row, in row_stats [5][n_seqs] fp64, the
+ * sums of m, x m, m^2, m^2 x, m^2 x^2 (x = the advantage written, m = loss_mask): the statistics
+ * pass of the advantage normalisation that follows in compute_advantages
+ * (areal/trainer/ppo/actor.py:344-350: adv_norm(advantages, loss_mask)), at no extra traffic. */
+int areal_gae_padded_row_stats(const float* rewards, const float* values, const float* loss_mask,
+                               const uint8_t* no_eos, const float* lambda_seq, int64_t n_seqs,
+                               int64_t uniform_len, float discount, float gae_lambda,
+                               float* advantages, float* returns, double* row_stats,
+                               areal_stream_t stream);
+
 /* Turn-level GAE (areal/trainer/ppo/gae.py:82-163) on padded [bs, max_seqlen] tensors: every
  * generated turn is one timestep. turn_ids int32 (-1 in prompt / tool gaps; non-decreasing over
  * the active tokens of a row), loss_mask fp32 (nonzero = active). *status (device int, zeroed
@@ -332,6 +343,19 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
                      int tail_group, int mean_level, int std_level, int leave_one_out,
                      int unbiased, double eps, float* out, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
+
+/* The apply pass of areal_group_norm alone (one launch), for a [n_rows, row_len] array whose
+ * per-row sums are already known (row_stats as areal_gae_padded_row_stats leaves them). Groups
+ * are runs of whole rows. Only for level combinations that need no second statistics pass: no
+ * leave-one-out mean, and not a group-level mean under a batch-level deviation
+ * (AREAL_ERR_UNSUPPORTED). Same arithmetic as Normalization.__call__
+ * (areal/utils/data.py:1382-1637) with the sum of squared deviations evaluated in fp64 from the
+ * sums. */
+int areal_group_norm_from_row_stats(const float* x, const float* mask, int64_t n_rows, int64_t row_len,
+                                    const int64_t* group_offsets, const int64_t* group_rows,
+                                    int64_t n_groups, int64_t max_group_len, int tail_group,
+                                    int mean_level, int std_level, int unbiased, double eps,
+                                    const double* row_stats, float* out, areal_stream_t stream);
 
 size_t areal_masked_norm_workspace_bytes(int64_t n);
 

@@ -379,3 +379,52 @@ def test_compute_advantages_turn_mode_keeps_kl_token_local(dev):
         b2 = dict(batch)
         del b2["turn_ids"]
         compute_advantages(b2, gae_timestep_unit="turn")
+
+
+@pytest.mark.parametrize("mean_level,std_level", [("group", "group"), ("batch", "batch"), ("batch", "group"),
+                                                  ("group", None), (None, "batch")])
+def test_compute_advantages_fused_gae_and_normalisation_equal_the_two_stage_route(dev, monkeypatch, mean_level,
+                                                                                   std_level):
+    """Long padded rows: the GAE kernel leaves each row's masked sums and the advantage
+    normalisation is its apply pass alone. Same advantages as GAE followed by the full
+    normalisation (and as the oracle), tail rows outside any group included."""
+    import areal_amd.ppo.actor as A
+    from areal_amd.config import NormConfig
+    from areal_amd.data import KLEstimator, Normalization
+    from oracle import gae as G
+    from oracle import norm as N
+
+    bs, L = 68, 4096  # 8 groups of 8 rows + 4 tail rows
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(300, L, (bs,), generator=g)
+    pos = torch.arange(L)[None]
+    attn = pos < lens[:, None]
+    data = dict(input_ids=torch.zeros(bs, L, dtype=torch.long), attention_mask=attn,
+                loss_mask=(pos >= (lens // 4)[:, None]) & attn,
+                logprobs=torch.randn(bs, L, generator=g) * 0.1 - 1,
+                values=torch.randn(bs, L, generator=g), rewards=(torch.rand(bs, generator=g) > 0.5).float())
+    data = {k: v.to(dev) for k, v in data.items()}
+    norm = Normalization(NormConfig(mean_level=mean_level, std_level=std_level, group_size=8))
+    kw = dict(kl_ctl=0.0, kl_estimator=KLEstimator("k1"), adv_norm=norm, discount=1.0, gae_lambda=0.95)
+
+    calls = []
+    real = A._token_level_gae_with_row_stats
+
+    def spy(*a, **k):
+        calls.append(1)
+        return real(*a, **k)
+
+    monkeypatch.setattr(A, "_token_level_gae_with_row_stats", spy)
+    fused = A.compute_advantages(dict(data), **kw)
+    assert calls, "the fused route was not taken"
+    monkeypatch.setattr(A, "_token_level_gae_with_row_stats", lambda *a, **k: None)
+    staged = A.compute_advantages(dict(data), **kw)
+    assert torch.equal(fused["returns"], staged["returns"])
+    scale = staged["advantages"].abs().max().item()
+    torch.testing.assert_close(fused["advantages"], staged["advantages"], rtol=1e-5, atol=1e-6 * scale)
+    # and against the oracle: GAE of the shaped rewards, then the normalisation
+    want_a, _ = G.gae_padded(fused["tot_rewards"].cpu(), data["values"].cpu(), fused["loss_mask"].cpu().float(),
+                             torch.zeros(bs, dtype=torch.bool), 1.0, 0.95)
+    want = N.normalization(want_a, fused["loss_mask"].cpu().float(), mean_level=mean_level, std_level=std_level,
+                           group_size=8)
+    torch.testing.assert_close(fused["advantages"].cpu(), want, rtol=1e-4, atol=1e-5 * want.abs().max().item())
