@@ -482,10 +482,15 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
       if constexpr (STATS) {
 #pragma unroll
         for (int i = 0; i < GAE_ITEMS; ++i) {
-          if (!((valid >> i) & 1u)) continue;
-          const double x = (double)oa[i], m = (double)ms[i];
-          const double xm = x * m, mm = m * m;
-          rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
+          if (!((valid >> i) & 1u) || ms[i] == 0.f) continue;
+          const double x = (double)oa[i];
+          if (ms[i] == 1.f) {  // the usual 0/1 mask: one fp64 multiplication per token
+            rs[0] += 1.0; rs[1] += x; rs[2] += 1.0; rs[3] += x; rs[4] += x * x;
+          } else {
+            const double m = (double)ms[i];
+            const double xm = x * m, mm = m * m;
+            rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
+          }
         }
       }
       if (valid == (1u << GAE_ITEMS) - 1u) {
