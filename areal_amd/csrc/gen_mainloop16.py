@@ -164,46 +164,7 @@ class Variant:
         out += ["s_waitcnt lgkmcnt(0)"] + barrier
         return out
 
-    def ktile_late(self, parity, init, x_pos, y_pos):
-        """The same k-tile with both barriers moved into the k-steps: barrier X behind MFMA x_pos
-        of k-step 0 (every wave has fetched this stage's last fragments: both halves of the stage
-        are refilled from there on), barrier Y behind MFMA y_pos of k-step 1 (the loads issued a
-        k-tile ago have landed for every wave: the other stage is read from there on). A load has
-        (63 - x_pos) + 64 + y_pos MFMAs to land instead of 128."""
-        stage = parity
-        barrier = [] if "no_barrier" in FLAGS else ["s_barrier"]
-        out = [f"; ---- k-tile on stage {stage}: k-step 0"]
-        pre, post = {}, {}
-        self.spread(self.a_reads(1, stage, 1), 2, x_pos - 1, post)
-        post.setdefault(x_pos, []).extend(["s_waitcnt lgkmcnt(0)"] + barrier)
-        loads = [self.load(stage, 1, i) for i in range(8)] + [self.load(stage, 0, i) for i in range(8)]
-        used = set()
-        for k, (setm0, ld) in enumerate(loads):
-            m = x_pos + 1 + (k * (63 - x_pos)) // 16
-            if m in used:
-                post[m] += [setm0, "s_nop 0", ld]
-            else:
-                used.add(m)
-                pre.setdefault(m, []).append(setm0)
-                post.setdefault(m, []).append(ld)
-            if k == 7:
-                post[m] += self.advance(1)
-            if k == 15:
-                post[m] += self.advance(0)
-        out += self.kstep(self.fa[0], self.fb[parity][0], init, pre, post)
-        out += [f"; ---- k-tile on stage {stage}: k-step 1"]
-        pre, post = {}, {}
-        post[y_pos] = ["s_waitcnt vmcnt(16)"] + barrier
-        self.spread(self.a_reads(0, stage ^ 1, 0) + self.b_reads(parity ^ 1, stage ^ 1), y_pos + 1, 60, post)
-        out += self.kstep(self.fa[1], self.fb[parity][1], False, pre, post)
-        out += ["s_waitcnt lgkmcnt(0)"]
-        return out
-
     def pair(self, init):
-        late = [f for f in FLAGS if f.startswith("late=")]
-        if late:
-            x_pos, y_pos = (int(v) for v in late[0][5:].split(","))
-            return self.ktile_late(0, init, x_pos, y_pos) + self.ktile_late(1, False, x_pos, y_pos)
         return self.ktile(0, init) + self.ktile(1, False)
 
     def tile_loop(self):
