@@ -16,7 +16,8 @@ order is the one written here, whatever the compiler would have scheduled:
   half of a stage is refilled from the start of the k-tile that consumes the stage and the A
   half from its middle: two half-batches of loads are in flight at any time and each has a full
   k-tile (the B half one and a half) to land, so the load pipe never drains.  One barrier at the
-  start and one in the middle of a k-tile publish a landed half and retire a consumed one;
+  start and one in the middle of a k-tile publish a landed half and retire a consumed one.  The
+  8 loads of a half-batch are issued several MFMAs apart (``LOAD_SPACING``), not back to back;
 * two k-tiles (one per stage) form the loop body, and the LDS is laid out as
   ``[A stage 0][A stage 1][B stage 0][B stage 1]`` (32 KB each) so that the two stages of an
   operand differ by an immediate offset: every LDS address is one register plus an immediate
@@ -133,12 +134,19 @@ class Variant:
             post.setdefault(m, []).append(op)
         return post
 
-    def put_loads(self, stage, oper, pre, post, first=0):
+    # MFMAs between two direct loads of a half-batch. Issued back to back (one per MFMA) the 8
+    # loads of a wave congest the address path and the whole loop runs 6-8 % slower; spaced 3 to 8
+    # MFMAs apart it does not matter much by how many. The B half, which has a k-tile and a half
+    # to land, is spread wider than the A half, which has one k-tile.
+    LOAD_SPACING = {0: 4, 1: 6}
+
+    def put_loads(self, stage, oper, pre, post):
+        step = self.LOAD_SPACING[oper]
         for i in range(8):
             setm0, ld = self.load(stage, oper, i)
-            pre.setdefault(first + i, []).append(setm0)
-            post.setdefault(first + i, []).append(ld)
-        post.setdefault(first + 8, []).extend(self.advance(oper))
+            pre.setdefault(i * step, []).append(setm0)
+            post.setdefault(i * step, []).append(ld)
+        post.setdefault(7 * step + 1, []).extend(self.advance(oper))
 
     def ktile(self, parity, init):
         stage = parity
