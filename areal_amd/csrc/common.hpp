@@ -45,6 +45,14 @@ DEVI u16 f32_to_bf16_bits(float f) {
   __bf16 h = (__bf16)f;
   return __builtin_bit_cast(u16, h);
 }
+// Two floats to a pair of bf16 in one register (lo in bits 0-15): one v_cvt_pk_bf16_f32, the same
+// round-to-nearest-even as the scalar conversion.
+typedef float f32x2_cvt __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_cvt __attribute__((ext_vector_type(2)));
+DEVI uint32_t pack_bf16x2(float lo, float hi) {
+  const bf16x2_cvt h = __builtin_convertvector(f32x2_cvt{lo, hi}, bf16x2_cvt);
+  return __builtin_bit_cast(uint32_t, h);
+}
 DEVI float bf16_bits_to_f32(u16 b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }

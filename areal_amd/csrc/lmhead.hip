@@ -1603,8 +1603,8 @@ struct Store16 {
           float x0 = x[a * 4], x1 = x[a * 4 + 1], x2 = x[a * 4 + 2], x3 = x[a * 4 + 3];
           if (MODE == 3) { x0 *= js; x1 *= js; x2 *= js; x3 *= js; }
           u32x2 v;
-          v[0] = (uint32_t)f32_to_bf16_bits(x0) | ((uint32_t)f32_to_bf16_bits(x1) << 16);
-          v[1] = (uint32_t)f32_to_bf16_bits(x2) | ((uint32_t)f32_to_bf16_bits(x3) << 16);
+          v[0] = pack_bf16x2(x0, x1);
+          v[1] = pack_bf16x2(x2, x3);
           stage16_put(stage, lane, a, v);
         }
         flush_stage16<EDGE>(stage, (u16*)p.out + (int64_t)(j0 + b * 16) * p.ldo + i0, p.ldo,
@@ -1733,7 +1733,7 @@ struct Fwd16 {
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
           const int vq = vl + a * 16;
-          u16 d[4];
+          float d[4];
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
             const float t = fmaf(x[a * 4 + e4], p.c2, -mc);
@@ -1741,11 +1741,11 @@ struct Fwd16 {
             float es = e * gamma;
             if (EDGE && vq + e4 >= p.V) es = 0.f;
             else { s += e; q = fmaf(t, e, q); }
-            d[e4] = f32_to_bf16_bits(es);
+            d[e4] = es;
           }
           u32x2 pk;
-          pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
-          pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+          pk[0] = pack_bf16x2(d[0], d[1]);
+          pk[1] = pack_bf16x2(d[2], d[3]);
           stage16_put(stage, lane, a, pk);
           // keeps the exponentials of one block next to the sums that consume them (left alone,
           // the scheduler computes all 32 first and spills them)
@@ -1861,7 +1861,7 @@ struct Bwd16 {
 #pragma unroll
       for (int a = 0; a < 8; ++a) {
         const int vq = vl + a * 16;
-        u16 d[4];
+        float d[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int v = vq + e;
@@ -1875,11 +1875,11 @@ struct Bwd16 {
           float dv = -pr * gs;
           if (v == lab) dv += gs;
           if (EDGE && (v >= p.V || t >= p.T)) dv = 0.f;
-          d[e] = f32_to_bf16_bits(dv);
+          d[e] = dv;
         }
         u32x2 pk;
-        pk[0] = (uint32_t)d[0] | ((uint32_t)d[1] << 16);
-        pk[1] = (uint32_t)d[2] | ((uint32_t)d[3] << 16);
+        pk[0] = pack_bf16x2(d[0], d[1]);
+        pk[1] = pack_bf16x2(d[2], d[3]);
         stage16_put(stage, lane, a, pk);
       }
       flush_stage16<EDGE>(stage, p.dl + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv, p.T - (t0 + b * 16),
