@@ -271,14 +271,16 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_apply_kernel(GaeArgs g, const
 }
 
 // ---------------------------------------------------------------------------------------
-// Single-pass GAE. Sequences are independent, so a block that starts at the end of a sequence
-// needs no carry from its right. Block b owns the sequences whose END lies in the token range
-// (b*TILE, (b+1)*TILE] and walks from the end of its last owned sequence down to the start of
-// its first one, tile by tile (tiles are absolute multiples of TILE, so the vector loads stay
-// aligned), carrying (A, nv) across its tiles. Every token is read once and written once:
-// 20 B/token, one launch, no dependency between blocks. A sequence much longer than a tile is
-// walked by one block; the host picks the three-launch scan above when the average sequence
-// is very long.
+// Single-pass GAE: one launch, every token read once and written once (20 B/token), no block
+// waits for another. Sequences are independent, so nothing enters a sequence's last token from
+// its right. Two kernels:
+//  * padded rows (gae_owned_kernel): block b owns the rows whose END lies in the token range
+//    (b*TILE, (b+1)*TILE] (one block per row when rows are at least a tile long) and walks them
+//    right to left tile by tile, carrying (A, nv) across its tiles;
+//  * packed sequences (gae_tile_kernel): block = tile; the state entering the tile is recomputed
+//    from the crossing sequence's remaining tokens.
+// Tiles are absolute multiples of TILE, so the 16-byte loads stay aligned. The host picks the
+// three-launch scan above when sequences are long on average.
 // ---------------------------------------------------------------------------------------
 
 // #{i in [0, n) : ends[i] <= x} for a non-decreasing array, by one wave: every round probes 64
@@ -300,6 +302,177 @@ DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
   return base;
 }
 
+// One tile of the single-pass kernels: the block's 256 threads take 8 consecutive tokens each
+// of tile `tile` (tokens [tile * TILE, (tile + 1) * TILE)), of which [t_begin, t_end) are this
+// block's to write. cu_own[i] = cu[s_first + i] for i in [0, n_own] covers every sequence that
+// holds one of those tokens (cu_own[0] <= t_begin, cu_own[n_own] >= t_end); with uniform rows
+// cu_own is unused. (A0, nv0) is the fp64 state entering the tile from its right and is replaced
+// by the state leaving it on the left. rs: the row sums of GaeArgs::row_stats (STATS only).
+// The thread's 8 consecutive tokens from t0 (a multiple of 8) as raw inputs; zeros where `want`
+// is false and beyond the array.
+DEVI void gae_load_items(const GaeArgs& g, int64_t t0, bool want, float (&rw)[GAE_ITEMS],
+                         float (&v)[GAE_ITEMS], float (&ms)[GAE_ITEMS]) {
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) { rw[i] = 0.f; v[i] = 0.f; ms[i] = 0.f; }
+  if (!want) return;
+  if (t0 + GAE_ITEMS <= g.n) {
+#pragma unroll
+    for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+      const f32x4 a = *(const f32x4*)(g.rewards + t0 + 4 * q);
+      const f32x4 b = *(const f32x4*)(g.values + t0 + 4 * q);
+      const f32x4 c = *(const f32x4*)(g.mask + t0 + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { rw[4 * q + e] = a[e]; v[4 * q + e] = b[e]; ms[4 * q + e] = c[e]; }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < GAE_ITEMS; ++i) {
+      const bool in = t0 + i < g.n;
+      rw[i] = in ? g.rewards[t0 + i] : 0.f;
+      v[i] = in ? g.values[t0 + i] : 0.f;
+      ms[i] = in ? g.mask[t0 + i] : 0.f;
+    }
+  }
+}
+
+// local indices [i_lo, i_hi) of the thread's 8 tokens from t0 that lie in [t_begin, t_end)
+DEVI void gae_owned_items(int64_t t0, int64_t t_begin, int64_t t_end, int& i_lo, int& i_hi) {
+  const int64_t d_lo = t_begin - t0, d_hi = t_end - t0;
+  i_lo = d_lo > 0 ? (d_lo < GAE_ITEMS ? (int)d_lo : GAE_ITEMS) : 0;
+  i_hi = d_hi < GAE_ITEMS ? (d_hi > 0 ? (int)d_hi : 0) : GAE_ITEMS;
+}
+
+// (rw, v, ms): the tile's inputs as gae_load_items leaves them (at least the owned tokens).
+template <bool STATS>
+DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t t_end, int s_first,
+                       int n_own, const int32_t* cu_own, bool uniform, double& A0, double& nv0,
+                       double (&rs)[STATS ? 5 : 1], MapF* smem, MapF* all,
+                       const float (&rw)[GAE_ITEMS], const float (&v)[GAE_ITEMS],
+                       const float (&ms)[GAE_ITEMS]) {
+  const int tid = threadIdx.x;
+  const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
+  // The thread keeps its 8 tokens as raw inputs plus two bit masks and rebuilds a token's map
+  // where it is needed (twice): holding 8 fp64 maps would halve the occupancy.
+  float lm[GAE_ITEMS];
+  unsigned valid = 0, ends = 0, boot = 0;  // bit i: token owned / last of its sequence / no_eos
+  int i_lo, i_hi;  // owned tokens of this thread
+  gae_owned_items(t0, t_begin, t_end, i_lo, i_hi);
+  const bool any = i_lo < i_hi;
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) lm[i] = g.lam;
+  if (any) {
+    // sequence of the first owned token of this thread (index relative to s_first)
+    const int64_t tf = t0 + i_lo;
+    int sq;
+    int e_loc;  // local index one past the last token of sequence sq (clamped)
+    if (uniform) {
+      sq = (int)(tf / g.uniform_len) - s_first;
+      const int64_t e = (int64_t)(sq + s_first + 1) * g.uniform_len - t0;
+      e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+    } else {
+      int a = 0, b = n_own;  // cu_own[a] <= tf < cu_own[b]
+      while (b - a > 1) {
+        const int mid = (a + b) >> 1;
+        if ((int64_t)cu_own[mid] <= tf) a = mid; else b = mid;
+      }
+      sq = a;
+      const int64_t e = (int64_t)cu_own[sq + 1] - t0;
+      e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+    }
+    valid = ((1u << i_hi) - 1u) & ~((1u << i_lo) - 1u);
+    if (e_loc > i_hi && g.lam_seq == nullptr) {
+      // common case: all owned tokens inside one sequence, none of them its last
+    } else {
+      // a sequence ends among these tokens (or lambda is per sequence): walk them
+      for (int i = i_lo; i < i_hi; ++i) {
+        while (i >= e_loc && sq + 1 < n_own) {
+          ++sq;
+          const int64_t e = (uniform ? (int64_t)(sq + s_first + 1) * g.uniform_len
+                                     : (int64_t)cu_own[sq + 1]) - t0;
+          e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+        }
+        if (g.lam_seq != nullptr) {
+          const float l = g.lam_seq[s_first + sq];
+#pragma unroll
+          for (int k = 0; k < GAE_ITEMS; ++k) if (k == i) lm[k] = l;
+        }
+        if (i == e_loc - 1) {
+          ends |= 1u << i;
+          if (g.no_eos != nullptr && g.no_eos[s_first + sq] != 0) boot |= 1u << i;
+        }
+      }
+    }
+  }
+  const float gam = g.discount;
+  auto token_map = [&](int i) -> MapF {
+    const float val = v[i];
+    // not owned: identity (m = 0 with no offsets); last token of a sequence: constant map
+    const float m = ((valid >> i) & 1u) ? ms[i] : 0.f;
+    const float c = gam * lm[i];
+    MapF f;
+    f.a11 = fmaf(c, m, 1.f - m);
+    f.a12 = gam * m;
+    f.a22 = 1.f - m;
+    f.b1 = (rw[i] - val) * m;
+    f.b2 = val * m;
+    if ((ends >> i) & 1u) f = MapF{0.f, 0.f, 0.f, 0.f, ((boot >> i) & 1u) ? val : 0.f};
+    return f;
+  };
+  MapF mine = token_map(GAE_ITEMS - 1);
+#pragma unroll
+  for (int i = GAE_ITEMS - 2; i >= 0; --i) mine = compose(token_map(i), mine);
+  MapF total;
+  const MapF incl = block_suffix_scan(mine, smem, total);
+  all[tid] = incl;
+  __syncthreads();
+  const MapF excl = tid + 1 < GAE_THREADS ? all[tid + 1] : map_identity_t<float>();
+  // the state entering this thread's tokens: the fp32 map of everything to its right in the
+  // tile applied to the fp64 state entering the tile
+  float A = (float)fma((double)excl.a11, A0, fma((double)excl.a12, nv0, (double)excl.b1));
+  float nv = (float)fma((double)excl.a22, nv0, (double)excl.b2);
+  if (any) {
+    float oa[GAE_ITEMS], orr[GAE_ITEMS];
+#pragma unroll
+    for (int i = GAE_ITEMS - 1; i >= 0; --i) {
+      const MapF f = token_map(i);
+      const float A2 = fmaf(f.a11, A, fmaf(f.a12, nv, f.b1));
+      const float nv2 = fmaf(f.a22, nv, f.b2);
+      A = A2; nv = nv2;
+      oa[i] = A;
+      orr[i] = oa[i] + v[i];
+    }
+    if constexpr (STATS) {
+#pragma unroll
+      for (int i = 0; i < GAE_ITEMS; ++i) {
+        if (!((valid >> i) & 1u) || ms[i] == 0.f) continue;
+        const double x = (double)oa[i];
+        if (ms[i] == 1.f) {  // the usual 0/1 mask: one fp64 multiplication per token
+          rs[0] += 1.0; rs[1] += x; rs[2] += 1.0; rs[3] += x; rs[4] += x * x;
+        } else {
+          const double m = (double)ms[i];
+          const double xm = x * m, mm = m * m;
+          rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
+        }
+      }
+    }
+    if (valid == (1u << GAE_ITEMS) - 1u) {
+#pragma unroll
+      for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+        *(f32x4*)(g.adv + t0 + 4 * q) = f32x4{oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};
+        *(f32x4*)(g.ret + t0 + 4 * q) = f32x4{orr[4 * q], orr[4 * q + 1], orr[4 * q + 2], orr[4 * q + 3]};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < GAE_ITEMS; ++i)
+        if ((valid >> i) & 1u) { g.adv[t0 + i] = oa[i]; g.ret[t0 + i] = orr[i]; }
+    }
+  }
+  // state entering the next tile on the left
+  const double A1 = fma((double)total.a11, A0, fma((double)total.a12, nv0, (double)total.b1));
+  const double nv1 = fma((double)total.a22, nv0, (double)total.b2);
+  A0 = A1; nv0 = nv1;
+}
+
 // (Blocks of 1024 threads, one 8192-token tile per padded row instead of four serial tiles of
 // 2048, measured slower: 46.7 against 30.8 us on [1024, 8192]; one such block fills a CU's
 // registers and the latency of its single pass is not covered by anything.)
@@ -308,207 +481,35 @@ template <bool STATS>
 __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
   __shared__ MapF smem[GAE_THREADS / 64];
   __shared__ MapF all[GAE_THREADS];
-  __shared__ int32_t s_cu[GAE_TILE + 2];
-  __shared__ int s_own[2];
   const int tid = threadIdx.x;
   // Workgroups go to the 8 XCDs round-robin by id. Giving XCD x the x-th eighth of the token
-  // ranges keeps the work even when only every k-th range owns a sequence end (padded rows).
+  // ranges keeps neighbouring ranges on one XCD.
   const int64_t per_xcd = (gridDim.x + 7) >> 3;
   const int64_t range = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  // padded rows of at least a tile: only every (L / TILE)-th range would own a row, so the grid
-  // is one block per row instead (lo, hi] = the range holding the row's end
+  // rows of at least a tile: only every (L / TILE)-th range would own a row, so the grid is one
+  // block per row instead, (lo, hi] = the range holding the row's end
   const int64_t lo = g.block_per_seq ? ((int64_t)(blockIdx.x + 1) * g.uniform_len - 1)
                                      : range * GAE_TILE;
   if (!g.block_per_seq && (range >= per_xcd * 8 || lo >= g.n)) return;
   const int64_t hi = g.block_per_seq ? lo + 1 : (lo + GAE_TILE < g.n ? lo + GAE_TILE : g.n);
-  const bool uniform = g.uniform_len > 0;
-
-  // tokens outside every sequence (none in a well-formed batch) are written as zero
-  {
-    const int64_t cov_lo = uniform ? 0 : (int64_t)g.cu[0];
-    const int64_t cov_hi = uniform ? g.n : (int64_t)g.cu[g.n_seqs];
-    if (lo < cov_lo || hi > cov_hi) {
-      for (int64_t t = lo + tid; t < hi; t += GAE_THREADS)
-        if (t < cov_lo || t >= cov_hi) { g.adv[t] = 0.f; g.ret[t] = 0.f; }
-    }
-  }
-
-  // owned sequences [s_first, s_last]: lo < end(s) <= hi
-  int s_first, s_last;
-  if (uniform) {
-    s_first = (int)(lo / g.uniform_len);
-    s_last = (int)(hi / g.uniform_len) - 1;
-  } else {
-    if (tid < 128) {  // the two searches are independent chains of global loads: one wave each
-      const int which = tid >> 6;
-      const int r = wave_count_le(g.cu + 1, g.n_seqs, which ? hi : lo, tid & 63);
-      if ((tid & 63) == 0) s_own[which] = which ? r - 1 : r;
-    }
-    __syncthreads();
-    s_first = s_own[0];
-    s_last = s_own[1];
-  }
+  // owned rows [s_first, s_last]: lo < end(s) <= hi
+  const int s_first = (int)(lo / g.uniform_len);
+  const int s_last = (int)(hi / g.uniform_len) - 1;
   if (s_first > s_last) return;  // uniform for the block
-
   const int n_own = s_last - s_first + 1;
-  const int32_t* cu_own = nullptr;  // cu_own[i] = cu[s_first + i], i in [0, n_own]
-  if (!uniform) {
-    if (n_own <= GAE_TILE + 1) {
-      for (int i = tid; i <= n_own; i += GAE_THREADS) s_cu[i] = g.cu[s_first + i];
-      __syncthreads();
-      cu_own = s_cu;
-    } else {
-      cu_own = g.cu + s_first;  // only with many empty sequences
-    }
-  }
-  const int64_t t_begin = uniform ? (int64_t)s_first * g.uniform_len : (int64_t)cu_own[0];
-  const int64_t t_end = uniform ? (int64_t)(s_last + 1) * g.uniform_len : (int64_t)cu_own[n_own];
-  if (t_end <= t_begin) return;
+  const int64_t t_begin = (int64_t)s_first * g.uniform_len;
+  const int64_t t_end = (int64_t)(s_last + 1) * g.uniform_len;
 
   double A0 = 0.0, nv0 = 0.0;  // state entering the current tile from its right
   double rs[STATS ? 5 : 1] = {0.0};
   for (int64_t tile = (t_end - 1) / GAE_TILE; tile >= t_begin / GAE_TILE; --tile) {
     const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
-    // The thread keeps its 8 tokens as raw inputs plus two bit masks and rebuilds a token's map
-    // where it is needed (twice): holding 8 fp64 maps would halve the occupancy.
-    float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS], lm[GAE_ITEMS];
-    unsigned valid = 0, ends = 0, boot = 0;  // bit i: token owned / last of its sequence / no_eos
-    // owned tokens of this thread: local indices [i_lo, i_hi)
-    const int64_t d_lo = t_begin - t0, d_hi = t_end - t0;
-    const int i_lo = d_lo > 0 ? (d_lo < GAE_ITEMS ? (int)d_lo : GAE_ITEMS) : 0;
-    const int i_hi = d_hi < GAE_ITEMS ? (d_hi > 0 ? (int)d_hi : 0) : GAE_ITEMS;
-    const bool any = i_lo < i_hi;
-#pragma unroll
-    for (int i = 0; i < GAE_ITEMS; ++i) { rw[i] = 0.f; v[i] = 0.f; ms[i] = 0.f; lm[i] = g.lam; }
-    if (any) {
-      if (t0 + GAE_ITEMS <= g.n) {
-#pragma unroll
-        for (int q = 0; q < GAE_ITEMS / 4; ++q) {
-          const f32x4 a = *(const f32x4*)(g.rewards + t0 + 4 * q);
-          const f32x4 b = *(const f32x4*)(g.values + t0 + 4 * q);
-          const f32x4 c = *(const f32x4*)(g.mask + t0 + 4 * q);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { rw[4 * q + e] = a[e]; v[4 * q + e] = b[e]; ms[4 * q + e] = c[e]; }
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < GAE_ITEMS; ++i) {
-          const bool in = t0 + i < g.n;
-          rw[i] = in ? g.rewards[t0 + i] : 0.f;
-          v[i] = in ? g.values[t0 + i] : 0.f;
-          ms[i] = in ? g.mask[t0 + i] : 0.f;
-        }
-      }
-      // sequence of the first owned token of this thread (index relative to s_first)
-      const int64_t tf = t0 + i_lo;
-      int sq;
-      int e_loc;  // local index one past the last token of sequence sq (clamped)
-      if (uniform) {
-        sq = (int)(tf / g.uniform_len) - s_first;
-        const int64_t e = (int64_t)(sq + s_first + 1) * g.uniform_len - t0;
-        e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
-      } else {
-        int a = 0, b = n_own;  // cu_own[a] <= tf < cu_own[b]
-        while (b - a > 1) {
-          const int mid = (a + b) >> 1;
-          if ((int64_t)cu_own[mid] <= tf) a = mid; else b = mid;
-        }
-        sq = a;
-        const int64_t e = (int64_t)cu_own[sq + 1] - t0;
-        e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
-      }
-      valid = ((1u << i_hi) - 1u) & ~((1u << i_lo) - 1u);
-      if (e_loc > i_hi && g.lam_seq == nullptr) {
-        // common case: all owned tokens inside one sequence, none of them its last
-      } else {
-        // a sequence ends among these tokens (or lambda is per sequence): walk them
-        for (int i = i_lo; i < i_hi; ++i) {
-          while (i >= e_loc && sq + 1 < n_own) {
-            ++sq;
-            const int64_t e = (uniform ? (int64_t)(sq + s_first + 1) * g.uniform_len
-                                       : (int64_t)cu_own[sq + 1]) - t0;
-            e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
-          }
-          if (g.lam_seq != nullptr) {
-            const float l = g.lam_seq[s_first + sq];
-#pragma unroll
-            for (int k = 0; k < GAE_ITEMS; ++k) if (k == i) lm[k] = l;
-          }
-          if (i == e_loc - 1) {
-            ends |= 1u << i;
-            if (g.no_eos != nullptr && g.no_eos[s_first + sq] != 0) boot |= 1u << i;
-          }
-        }
-      }
-    }
-    const float gam = g.discount;
-    auto token_map = [&](int i) -> MapF {
-      const float val = v[i];
-      // not owned: identity (m = 0 with no offsets); last token of a sequence: constant map
-      const float m = ((valid >> i) & 1u) ? ms[i] : 0.f;
-      const float c = gam * lm[i];
-      MapF f;
-      f.a11 = fmaf(c, m, 1.f - m);
-      f.a12 = gam * m;
-      f.a22 = 1.f - m;
-      f.b1 = (rw[i] - val) * m;
-      f.b2 = val * m;
-      if ((ends >> i) & 1u) f = MapF{0.f, 0.f, 0.f, 0.f, ((boot >> i) & 1u) ? val : 0.f};
-      return f;
-    };
-    MapF mine = token_map(GAE_ITEMS - 1);
-#pragma unroll
-    for (int i = GAE_ITEMS - 2; i >= 0; --i) mine = compose(token_map(i), mine);
-    MapF total;
-    const MapF incl = block_suffix_scan(mine, smem, total);
-    all[tid] = incl;
-    __syncthreads();
-    const MapF excl = tid + 1 < GAE_THREADS ? all[tid + 1] : map_identity_t<float>();
-    // the state entering this thread's tokens: the fp32 map of everything to its right in the
-    // tile applied to the fp64 state entering the tile
-    float A = (float)fma((double)excl.a11, A0, fma((double)excl.a12, nv0, (double)excl.b1));
-    float nv = (float)fma((double)excl.a22, nv0, (double)excl.b2);
-    if (any) {
-      float oa[GAE_ITEMS], orr[GAE_ITEMS];
-#pragma unroll
-      for (int i = GAE_ITEMS - 1; i >= 0; --i) {
-        const MapF f = token_map(i);
-        const float A2 = fmaf(f.a11, A, fmaf(f.a12, nv, f.b1));
-        const float nv2 = fmaf(f.a22, nv, f.b2);
-        A = A2; nv = nv2;
-        oa[i] = A;
-        orr[i] = oa[i] + v[i];
-      }
-      if constexpr (STATS) {
-#pragma unroll
-        for (int i = 0; i < GAE_ITEMS; ++i) {
-          if (!((valid >> i) & 1u) || ms[i] == 0.f) continue;
-          const double x = (double)oa[i];
-          if (ms[i] == 1.f) {  // the usual 0/1 mask: one fp64 multiplication per token
-            rs[0] += 1.0; rs[1] += x; rs[2] += 1.0; rs[3] += x; rs[4] += x * x;
-          } else {
-            const double m = (double)ms[i];
-            const double xm = x * m, mm = m * m;
-            rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
-          }
-        }
-      }
-      if (valid == (1u << GAE_ITEMS) - 1u) {
-#pragma unroll
-        for (int q = 0; q < GAE_ITEMS / 4; ++q) {
-          *(f32x4*)(g.adv + t0 + 4 * q) = f32x4{oa[4 * q], oa[4 * q + 1], oa[4 * q + 2], oa[4 * q + 3]};
-          *(f32x4*)(g.ret + t0 + 4 * q) = f32x4{orr[4 * q], orr[4 * q + 1], orr[4 * q + 2], orr[4 * q + 3]};
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < GAE_ITEMS; ++i)
-          if ((valid >> i) & 1u) { g.adv[t0 + i] = oa[i]; g.ret[t0 + i] = orr[i]; }
-      }
-    }
-    // state entering the next tile on the left
-    const double A1 = fma((double)total.a11, A0, fma((double)total.a12, nv0, (double)total.b1));
-    const double nv1 = fma((double)total.a22, nv0, (double)total.b2);
-    A0 = A1; nv0 = nv1;
+    int i_lo, i_hi;
+    gae_owned_items(t0, t_begin, t_end, i_lo, i_hi);
+    float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS];
+    gae_load_items(g, t0, i_lo < i_hi, rw, v, ms);
+    gae_one_tile<STATS>(g, tile, t_begin, t_end, s_first, n_own, nullptr, true, A0, nv0, rs, smem, all,
+                        rw, v, ms);
   }
   if constexpr (STATS) {  // block = row: uniform for the block
     __shared__ double s_rs[4 * 5];
@@ -518,6 +519,187 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
       for (int k = 0; k < 5; ++k) g.row_stats[(int64_t)k * g.n_seqs + blockIdx.x] = rs[k];
     }
   }
+}
+
+// Single-pass GAE for packed sequences of ordinary length, one block per tile. What enters the
+// tile from its right is the state of the sequence that crosses the tile's right edge, and it
+// depends only on that sequence's tokens beyond the edge: the block reads them too (rewards,
+// values, mask; nothing written), two tiles' worth at a time with all loads in flight together,
+// and composes their maps onto the zero state. No block waits for another, and the remainder is
+// read once per tile of the sequence, from L2 mostly: the blocks of an XCD are neighbours in the
+// array. Against blocks that walk the sequences they own tile by tile, carrying the state (the
+// padded-row kernel above, which also took cu_seqlens once): equal on 1024 sequences of mean
+// length 1760 (18.7 / 18.3 us; of the tile kernel's time 6.5 us are the tile's loads and stores,
+// 1.3 us the sequence layout, 5.7 us the remainder and 5.2 us the scan), 19 against 24 us on
+// 64 x 16384 tokens and 24 against 38 us on 4 x 32768, where a walking block has 16 tiles in a
+// row. The kernel is bound by vector instruction issue (about 1400 per wave and tile), so it is
+// held to 128 registers: all blocks of a 1.8 M-token batch are then resident at once (186
+// registers with three tiles per round: two rounds of blocks, 25.6 us).
+constexpr int GAE_CARRY_BATCH = 2;
+constexpr int GAE_CU_LDS = 16 * GAE_THREADS;  // entries of cu_seqlens the block can hold (>= TILE + 2)
+
+__global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
+  __shared__ MapF smem[GAE_THREADS / 64];
+  __shared__ MapF all[GAE_THREADS];
+  __shared__ MapF s_part[GAE_THREADS / 64][GAE_CARRY_BATCH];
+  __shared__ int32_t s_cu[GAE_CU_LDS];
+  __shared__ int s_own[2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // XCD x (workgroup ids congruent to x modulo 8) takes the x-th eighth of the tiles
+  const int64_t per_xcd = (gridDim.x + 7) >> 3;
+  const int64_t tile = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int64_t lo = tile * GAE_TILE;
+  if (tile >= per_xcd * 8 || lo >= g.n) return;
+  const int64_t hi = lo + GAE_TILE < g.n ? lo + GAE_TILE : g.n;
+  // The tile's inputs do not depend on the sequence layout: their loads go out first, together
+  // with those of the layout.
+  float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS];
+  gae_load_items(g, lo + (int64_t)tid * GAE_ITEMS, true, rw, v, ms);
+  const bool cu_in_lds = g.n_seqs + 1 <= GAE_CU_LDS;
+  int64_t cov_lo, cov_hi;
+  if (cu_in_lds) {
+    // the whole of cu_seqlens into LDS, every load in flight at once
+    int32_t c[GAE_CU_LDS / GAE_THREADS];
+#pragma unroll
+    for (int k = 0; k < GAE_CU_LDS / GAE_THREADS; ++k) {
+      const int i = tid + k * GAE_THREADS;
+      c[k] = i <= g.n_seqs ? g.cu[i] : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < GAE_CU_LDS / GAE_THREADS; ++k) s_cu[tid + k * GAE_THREADS] = c[k];
+    if (tid < 2) s_own[tid] = 0;
+    __syncthreads();
+    cov_lo = (int64_t)s_cu[0];
+    cov_hi = (int64_t)s_cu[g.n_seqs];
+  } else {
+    cov_lo = (int64_t)g.cu[0];
+    cov_hi = (int64_t)g.cu[g.n_seqs];
+  }
+  // tokens outside every sequence (none in a well-formed batch) are written as zero
+  if (lo < cov_lo || hi > cov_hi) {
+    for (int64_t t = lo + tid; t < hi; t += GAE_THREADS)
+      if (t < cov_lo || t >= cov_hi) { g.adv[t] = 0.f; g.ret[t] = 0.f; }
+  }
+  const int64_t t_begin = lo > cov_lo ? lo : cov_lo;
+  const int64_t t_end = hi < cov_hi ? hi : cov_hi;
+  if (t_end <= t_begin) return;  // uniform for the block
+
+  // sequences holding the first and the last token of [t_begin, t_end): the number of sequence
+  // ends at or before each
+  const int32_t* cu_own;
+  int s_first, s_last;
+  if (cu_in_lds) {
+    int n_lo = 0, n_hi = 0;
+    for (int i = tid + 1; i <= g.n_seqs; i += GAE_THREADS) {
+      const int64_t end = (int64_t)s_cu[i];
+      n_lo += end <= t_begin;
+      n_hi += end <= t_end - 1;
+    }
+    n_lo = wave_sum(n_lo);
+    n_hi = wave_sum(n_hi);
+    if (lane == 0) { atomicAdd(&s_own[0], n_lo); atomicAdd(&s_own[1], n_hi); }
+    __syncthreads();
+    s_first = s_own[0];
+    s_last = s_own[1];
+    cu_own = s_cu + s_first;
+  } else {
+    if (tid < 128) {  // one wave each
+      const int r = wave_count_le(g.cu + 1, g.n_seqs, wave ? t_end - 1 : t_begin, lane);
+      if (lane == 0) s_own[wave] = r;
+    }
+    __syncthreads();
+    s_first = s_own[0];
+    s_last = s_own[1];
+    if (s_last - s_first + 2 <= GAE_CU_LDS) {
+      for (int i = tid; i <= s_last - s_first + 1; i += GAE_THREADS) s_cu[i] = g.cu[s_first + i];
+      __syncthreads();
+      cu_own = s_cu;
+    } else {
+      cu_own = g.cu + s_first;  // only with many empty sequences
+    }
+  }
+  const int n_own = s_last - s_first + 1;
+
+  // the crossing sequence's tokens [t_end, e): in whole tiles from t_end (a multiple of the tile
+  // when e > t_end), the rightmost batch first
+  double A0 = 0.0, nv0 = 0.0;
+  const int64_t e = (int64_t)cu_own[n_own];
+  if (e > t_end) {
+    const float gam = g.discount;
+    const float c = gam * (g.lam_seq != nullptr ? g.lam_seq[s_last] : g.lam);
+    const bool boot = g.no_eos != nullptr && g.no_eos[s_last] != 0;
+    const int64_t n_right = (e - t_end + GAE_TILE - 1) / GAE_TILE;
+    for (int64_t j = n_right; j > 0; j -= GAE_CARRY_BATCH) {
+      const int64_t j0 = j > GAE_CARRY_BATCH ? j - GAE_CARRY_BATCH : 0;
+      float rw[GAE_CARRY_BATCH][GAE_ITEMS], v[GAE_CARRY_BATCH][GAE_ITEMS], ms[GAE_CARRY_BATCH][GAE_ITEMS];
+#pragma unroll
+      for (int k = 0; k < GAE_CARRY_BATCH; ++k) {
+        const int64_t t0 = t_end + (j0 + k) * GAE_TILE + (int64_t)tid * GAE_ITEMS;
+        const bool live = j0 + k < j && t0 < e;
+        if (live && t0 + GAE_ITEMS <= g.n) {
+#pragma unroll
+          for (int q = 0; q < GAE_ITEMS / 4; ++q) {
+            const f32x4 a = *(const f32x4*)(g.rewards + t0 + 4 * q);
+            const f32x4 b = *(const f32x4*)(g.values + t0 + 4 * q);
+            const f32x4 m = *(const f32x4*)(g.mask + t0 + 4 * q);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) { rw[k][4 * q + x] = a[x]; v[k][4 * q + x] = b[x]; ms[k][4 * q + x] = m[x]; }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < GAE_ITEMS; ++i) {
+            const bool in = live && t0 + i < g.n;
+            rw[k][i] = in ? g.rewards[t0 + i] : 0.f;
+            v[k][i] = in ? g.values[t0 + i] : 0.f;
+            ms[k][i] = in ? g.mask[t0 + i] : 0.f;
+          }
+        }
+      }
+      MapF part[GAE_CARRY_BATCH];
+#pragma unroll
+      for (int k = 0; k < GAE_CARRY_BATCH; ++k) {
+        const int64_t t0 = t_end + (j0 + k) * GAE_TILE + (int64_t)tid * GAE_ITEMS;
+        MapF acc = map_identity_t<float>();
+#pragma unroll
+        for (int i = GAE_ITEMS - 1; i >= 0; --i) {
+          const int64_t t = t0 + i;
+          // beyond the sequence (or the batch): identity; its last token: the constant map
+          const float m = (j0 + k < j && t < e) ? ms[k][i] : 0.f;
+          MapF f;
+          f.a11 = fmaf(c, m, 1.f - m);
+          f.a12 = gam * m;
+          f.a22 = 1.f - m;
+          f.b1 = (rw[k][i] - v[k][i]) * m;
+          f.b2 = v[k][i] * m;
+          if (j0 + k < j && t == e - 1) f = MapF{0.f, 0.f, 0.f, 0.f, boot ? v[k][i] : 0.f};
+          acc = compose(f, acc);
+        }
+        // wave total in lane 0 (the upper lanes' values are not used)
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) acc = compose(acc, shfl_down_map(acc, d));
+        part[k] = acc;
+      }
+      __syncthreads();  // the previous batch's readers are done
+      if (lane == 0) {
+#pragma unroll
+        for (int k = 0; k < GAE_CARRY_BATCH; ++k) s_part[wave][k] = part[k];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int k = GAE_CARRY_BATCH - 1; k >= 0; --k) {
+        if (j0 + k >= j) continue;
+        MapF tot = s_part[GAE_THREADS / 64 - 1][k];
+#pragma unroll
+        for (int w = GAE_THREADS / 64 - 2; w >= 0; --w) tot = compose(s_part[w][k], tot);
+        const double A1 = fma((double)tot.a11, A0, fma((double)tot.a12, nv0, (double)tot.b1));
+        const double nv1 = fma((double)tot.a22, nv0, (double)tot.b2);
+        A0 = A1; nv0 = nv1;
+      }
+    }
+  }
+  double rs[1];
+  gae_one_tile<false>(g, tile, t_begin, t_end, s_first, n_own, cu_own, false, A0, nv0, rs, smem, all,
+                      rw, v, ms);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1387,15 +1569,27 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
   double* carry = (double*)(wp + (size_t)nb * sizeof(Map));
   GaeArgs g{rewards, values, loss_mask, cu_seqlens, no_eos, lambda_seq, n_tokens, (int)n_seqs,
             uniform_len, discount, gae_lambda, advantages, returns, 0, nullptr};
-  // sequences of ordinary length: single pass, one launch. Very long sequences on average (few
-  // blocks would own any work): reduce-then-scan over all tokens.
-  if (n_tokens / n_seqs <= 64 * GAE_TILE) {
+  // Measured on 1024 lognormal sequences (1.8 M tokens) / 64 x 16384 / 128 long-tailed up to
+  // 32768 / 4 x 32768: tile kernel 19 / 19 / 28 / 24 us, three launches 32 / 21 / 21 / 15 us.
+  const int64_t mean_len = n_tokens / n_seqs;
+  if (uniform_len <= 0 && mean_len <= 8 * GAE_TILE) {
+    // packed sequences: block = tile, the state entering from the right recomputed per tile
+    hipLaunchKernelGGL(gae_tile_kernel, dim3((unsigned)(ceil_div_i64(nb, 8) * 8)), dim3(GAE_THREADS), 0,
+                       stream, g);
+    AREAL_CHECK_LAUNCH();
+    return AREAL_OK;
+  }
+  // padded rows: blocks that own whole rows, as long as there are rows enough to fill the chip
+  // or the rows are short (a block walks its row's tiles one after the other)
+  if (uniform_len > 0 && uniform_len <= 64 * (int64_t)GAE_TILE &&
+      (n_seqs >= 256 || uniform_len <= 4 * GAE_TILE)) {
     g.block_per_seq = uniform_len >= GAE_TILE;
     const int64_t grid = g.block_per_seq ? n_seqs : ceil_div_i64(nb, 8) * 8;
     hipLaunchKernelGGL(gae_owned_kernel<false>, dim3((unsigned)grid), dim3(GAE_THREADS), 0, stream, g);
     AREAL_CHECK_LAUNCH();
     return AREAL_OK;
   }
+  // long sequences: reduce-then-scan over all tokens
   hipLaunchKernelGGL(gae_block_total_kernel, dim3((unsigned)nb), dim3(GAE_THREADS), 0, stream, g,
                      totals);
   AREAL_CHECK_LAUNCH();

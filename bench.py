@@ -184,11 +184,11 @@ def hbm_rooflines(dev):
     r[cu[1:].long() - 2] = 1.0
     v = torch.randn(T, device=dev)
     m = (torch.rand(T, device=dev) > 0.25).float()
-    add("gae_owned_kernel", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
+    add("gae_tile_kernel", f"config 3: 1024 packed sequences, {T} tokens, 20 B/token",
         20 * T, timed(lambda: compute_gae_packed(r, v, m, cu, None, 1.0, 0.95)))
     # the same batch through the C ABI, launches back to back on the stream (no host work between
     # them): packed GAE, then group normalisation (groups of 16 sequences, mean and deviation at
-    # group level) of the advantages under the same mask. 3 launches: gae_owned_kernel,
+    # group level) of the advantages under the same mask. 3 launches: gae_tile_kernel,
     # norm_stats5_kernel, norm_apply_cf_kernel.
     from areal_amd import _lib as L_
 
@@ -209,7 +209,7 @@ def hbm_rooflines(dev):
                                     0, 1, 1e-5, L_.ptr(nrm_o), L_.ptr(nrm_ws), nrm_ws_n, strm)
         assert rc == 0
 
-    add("gae_owned_kernel + norm_stats5_kernel + norm_apply_cf_kernel (C ABI)",
+    add("gae_tile_kernel + norm_stats5_kernel + norm_apply_cf_kernel (C ABI)",
         f"config 3: 1024 packed sequences, {T} tokens, GAE then group normalisation of the advantages, "
         "launches back to back, 20 + 20 B/token", 40 * T, timed(gae_then_norm))
     del adv_o, ret_o, nrm_o

@@ -59,6 +59,6 @@ def test_kernel_names_quoted_by_the_bench_exist_in_the_library():
                  bench.KERNEL_DWEIGHT):
         assert _lib.has_kernel(name), name
     assert not _lib.has_kernel("gemm16_sweep<9, Store16<false, 0> >")
-    for name in ("gae_owned_kernel", "loss_token_kernel", "loss_finalize_kernel", "rows_fwd_kernel",
+    for name in ("gae_owned_kernel", "gae_tile_kernel", "loss_token_kernel", "loss_finalize_kernel", "rows_fwd_kernel",
                  "saved_prep_kernel", "lmhead_merge_kernel", "lmhead_rowref_kernel"):
         assert _lib.has_kernel(name), name

@@ -86,9 +86,12 @@ def test_gae_packed_matches_oracle_and_edge_cases(dev):
     [140_000],                                   # one very long sequence: the reduce-then-scan launches
     [1] * 5000,                                  # one-token sequences: thousands of ends per tile
     [0, 3, 0, 0, 2500, 0, 7, 0],                 # empty sequences between real ones
-    [5, 70_000, 1, 2049, 2047, 4096, 1, 30_000], # ends on and around tile edges, long next to short
+    [5, 70_000, 1, 2049, 2047, 4096, 1, 30_000], # ends on and around tile edges, long next to short (34 tiles
+                                                 # of one sequence to the right of a tile)
     [2048] * 9,                                  # every end exactly on a tile edge
-], ids=["one-long", "unit", "empty", "mixed", "tile-aligned"])
+    [40_000, 3, 50_000],                         # long on average: the reduce-then-scan launches again
+    [0, 0, 9000, 0, 8192, 0],                    # empty sequences at both ends and on a tile edge
+], ids=["one-long", "unit", "empty", "mixed", "tile-aligned", "long-average", "empty-ends"])
 def test_gae_packed_sequence_layouts(dev, lens):
     g = torch.Generator().manual_seed(len(lens) * 13 + lens[0])
     lens = torch.tensor(lens)
@@ -110,7 +113,7 @@ def test_gae_packed_sequence_layouts(dev, lens):
 
 def test_gae_padded_long_rows(dev):
     # rows longer than a tile, and far longer (takes the reduce-then-scan launches)
-    for bs, L in ((7, 8192), (2, 140_000)):
+    for bs, L in ((7, 8192), (3, 20_000), (300, 10_000), (2, 140_000)):
         g = torch.Generator().manual_seed(L)
         r = torch.randn(bs, L, generator=g) * (torch.rand(bs, L, generator=g) > 0.95)
         v = torch.randn(bs, L, generator=g)
