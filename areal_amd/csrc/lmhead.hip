@@ -2045,33 +2045,35 @@ int launch_store(const GemmArgs& g, const Regions& r, const StoreParams& ep, int
 // tile count does not fill whole rounds of 256 workgroups, the vocabulary (K) range is split
 // over copies of the schedule, each writing an fp32 partial result that
 // splitk_reduce_bf16_kernel sums.
+// The launch is a schedule of super-blocks of up to 32 workgroups; super-block sb of copy c
+// runs on XCD (sb + c * n_sb) % 8, whose 32 CUs take its workgroups as they free up. Cost of
+// z copies in units of one workgroup's full K range = the busiest XCD's rounds of 32
+// workgroups, each K / z long, plus a small charge per split for the reduction of the partial
+// results.
+double sched_cost(const Sched& sc, int z) {
+  int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int c = 0; c < z; ++c)
+    for (int sb = 0; sb < sc.n_sb; ++sb) {
+      const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
+      const int nb = sc.nbj - sbj * sc.RB < sc.RB ? sc.nbj - sbj * sc.RB : sc.RB;
+      const int ns = sc.S - sbs * sc.RS < sc.RS ? sc.S - sbs * sc.RS : sc.RS;
+      load[(sb + c * sc.n_sb) & 7] += (int64_t)(nb > 0 ? nb : 0) * (ns > 0 ? ns : 0);
+    }
+  int64_t worst = 0;
+  for (int x = 0; x < 8; ++x) worst = load[x] > worst ? load[x] : worst;
+  return (double)ceil_div_i64(worst, 32) / z + 0.03 * (z - 1);
+}
+
 int dh_ksplit(int64_t H, int64_t T, int64_t K) {
   const int64_t tiles = ceil_div_i64(H, TILE) * ceil_div_i64(T, TILE);
   if (tiles >= 2048 || K % BK != 0) return 1;
   const int64_t nk = K / BK;
-  // The launch is a schedule of super-blocks of up to 32 workgroups; super-block sb of copy c
-  // runs on XCD (sb + c * n_sb) % 8, whose 32 CUs take its workgroups as they free up. Cost of
-  // z copies = the busiest XCD's rounds of 32 workgroups, each K / z long, plus a small charge
-  // per split for the reduction of the partial results.
   const int nai = (int)ceil_div_i64(H, TILE), nbj = (int)ceil_div_i64(T, TILE);
   const Sched sc = make_sched(0, nbj, 0, nai, nai);
-  auto cost_of = [&](int z) {
-    int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int c = 0; c < z; ++c)
-      for (int sb = 0; sb < sc.n_sb; ++sb) {
-        const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
-        const int nb = nbj - sbj * sc.RB < sc.RB ? nbj - sbj * sc.RB : sc.RB;
-        const int ns = sc.S - sbs * sc.RS < sc.RS ? sc.S - sbs * sc.RS : sc.RS;
-        load[(sb + c * sc.n_sb) & 7] += (int64_t)(nb > 0 ? nb : 0) * (ns > 0 ? ns : 0);
-      }
-    int64_t worst = 0;
-    for (int x = 0; x < 8; ++x) worst = load[x] > worst ? load[x] : worst;
-    return (double)ceil_div_i64(worst, 32) / z + 0.03 * (z - 1);
-  };
   int best = 1;
-  double best_cost = cost_of(1);
+  double best_cost = sched_cost(sc, 1);
   for (int z = 2; z <= 16 && z <= nk / 8; ++z) {
-    const double cost = cost_of(z);
+    const double cost = sched_cost(sc, z);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = z; }
   }
   return best;
@@ -2125,6 +2127,52 @@ int launch_dhidden(const u16* w, int64_t V, const u16* dl, int64_t ldv, int64_t 
   GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
   g.skip_if_set = skip_if_set;
   return launch_dhidden_k<KERNEL_NT, KERNEL16_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
+}
+
+// dWeight [V, H] in bf16 has ceil(V / 256) x ceil(H / 256) output tiles, one per workgroup, in
+// super-blocks of 32 that go round-robin to the XCDs. When their number is not a multiple of 8 the
+// last round occupies a few XCDs for a whole K range while the others idle (594 x 16 tiles: 298
+// super-blocks, 38 rounds on two XCDs against 37 on six). The B tiles of that last partial round
+// are then contracted by a second launch that splits the token (K) range over z copies of its
+// schedule, fp32 partial results summed by splitk_reduce_bf16_kernel.
+struct DwTail {
+  int nbj_main;  // B tiles of the first launch
+  int z, kps;    // copies and k-tiles per copy of the second (z <= 1: there is none)
+  int64_t rows;  // vocabulary rows of the second launch
+};
+DwTail plan_dw_tail(int64_t H, int64_t V, int64_t Tpad) {
+  const int nai = (int)ceil_div_i64(H, TILE), nbj = (int)ceil_div_i64(V, TILE);
+  DwTail t{nbj, 1, 0, 0};
+  if (!k16_ok(Tpad) || H % 8 != 0) return t;
+  const Sched sc = make_sched(0, nbj, 0, nai, nai);
+  if (sc.n_sb % 8 == 0) return t;
+  const int n_sb_s = sc.n_sb / sc.n_sb_j;
+  int nj = sc.n_sb_j;
+  while (nj > 0 && (nj * n_sb_s) % 8 != 0) --nj;
+  if (nj == 0) return t;
+  const Sched st = make_sched(nj * sc.RB, nbj - nj * sc.RB, 0, nai, nai);
+  const int64_t nk = Tpad / BK;
+  int best = 1;
+  double best_cost = sched_cost(st, 1);
+  for (int z = 2; z <= 8 && z <= nk / 8; ++z) {
+    const double cost = sched_cost(st, z);
+    if (cost < best_cost - 1e-9) { best_cost = cost; best = z; }
+  }
+  // rounds of a whole K range: before, and after with the first launch's even rounds. A k-tile
+  // takes about a microsecond; the two extra launches have to be paid for.
+  const double before = (double)ceil_div_i64(sc.n_sb, 8), after = (double)(nj * n_sb_s / 8) + best_cost;
+  if (best <= 1 || (before - after) * (double)nk < 16.0) return t;
+  t.nbj_main = nj * sc.RB;
+  t.kps = (int)ceil_div_i64(nk, best);
+  t.kps += t.kps & 1;  // the hand-scheduled loop walks pairs of k-tiles
+  t.z = (int)ceil_div_i64(nk, t.kps);
+  t.rows = V - (int64_t)t.nbj_main * TILE;
+  if (t.z <= 1) t = DwTail{nbj, 1, 0, 0};
+  return t;
+}
+size_t dw_tail_bytes(int64_t H, int64_t V, int64_t Tpad) {
+  const DwTail t = plan_dw_tail(H, V, Tpad);
+  return t.z > 1 ? (size_t)t.z * (size_t)(t.rows * H) * sizeof(float) + 256 : 0;
 }
 
 }  // namespace
@@ -2359,12 +2407,12 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 
 // Workspace of the backward from saved exponentials: row factors [T] fp32, scaled hidden states
 // [round_up(T, 64), H] bf16, W^T [H, round_up(V, 64)] bf16 (only when V is not a multiple of 64)
-// and the split-K partials of dHidden.
+// and the split-K partials of dHidden and of dWeight's last partial round.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
   const size_t wt = dh_weight_in_place(V) ? 0 : (size_t)(H * round_up_i64(V, BK)) * 2;
   return (size_t)T * 4 + (size_t)(round_up_i64(T, BK) * H) * 2 + wt +
-         dh_partial_bytes(H, T, round_up_i64(V, BK)) + 4 * 256;
+         dh_partial_bytes(H, T, round_up_i64(V, BK)) + dw_tail_bytes(H, V, round_up_i64(T, BK)) + 5 * 256;
 }
 
 // Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref, with *probs_status
@@ -2408,6 +2456,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   const bool w_in_place = dh_weight_in_place(V);
   u16* wT = (u16*)align256(hs + Tpad * H);
   float* dh_part = dh_partial_bytes(H, T, ldv) ? (float*)align256(wT + (w_in_place ? 0 : H * ldv)) : nullptr;
+  float* dw_part = (float*)align256((char*)align256(wT + (w_in_place ? 0 : H * ldv)) + dh_partial_bytes(H, T, ldv));
   u16* e = (u16*)probs;
   hipLaunchKernelGGL(saved_prep_kernel, dim3((unsigned)Tpad), dim3(256), 0, stream, e, ldv, probs_ref,
                      labels, row_max, sum_exp, grad_logprobs, logprobs, (const u16*)hidden, (int)T,
@@ -2435,6 +2484,30 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     // T are cleared)
     GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv};
     g.skip_if_set = probs_status;
+    const DwTail tail = dweight_mode == 2 ? plan_dw_tail(H, V, Tpad) : DwTail{0, 1, 0, 0};
+    if (tail.z > 1) {
+      // whole rounds of super-blocks, then the remaining vocabulary rows with the token range split
+      const int64_t v0 = (int64_t)tail.nbj_main * TILE;
+      g.N = (int)v0;
+      const StoreParams ep{dweight, H, (int)H, (int)v0, nullptr};
+      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, plan_regions(H, v0, Tpad, 0, 1 << 20), ep, 0, stream);
+      if (rc != AREAL_OK) return rc;
+      GemmArgs gt{hs, H, (int)H, e + v0, ldv, (int)tail.rows, (int)Tpad, (int)H, (int)(ldv - v0)};
+      gt.skip_if_set = probs_status;
+      gt.ksplit = tail.z;
+      gt.kt_per_split = tail.kps;
+      gt.zstride = tail.rows * H * (int64_t)sizeof(float);
+      const StoreParams ept{dw_part, H, (int)H, (int)tail.rows, nullptr};
+      rc = launch_store<KERNEL_TN, KERNEL16_TN>(gt, plan_regions(H, tail.rows, Tpad, 0, 1 << 20), ept, 1, stream);
+      if (rc != AREAL_OK) return rc;
+      int64_t blocks = ceil_div_i64(tail.rows * H, 256 * 4);
+      if (blocks > 65535) blocks = 65535;
+      hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dw_part,
+                         tail.z, tail.rows * H, tail.rows * H, (const float*)nullptr, H,
+                         (u16*)dweight + v0 * H, probs_status);
+      AREAL_CHECK_LAUNCH();
+      return AREAL_OK;
+    }
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
     rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : dweight_mode == 0 ? 1 : 0, stream);

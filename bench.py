@@ -31,7 +31,7 @@ KERNEL_FWD_SAVE = "gemm16_sweep<0, Fwd16<false, false, false, true> >"
 KERNEL_FWD = "gemm16_sweep<0, Fwd16<false, false, false, false> >"
 KERNEL_RECOMPUTE = "gemm16_sweep<0, Bwd16<false, false> >"
 KERNEL_DHIDDEN = "gemm16_sweep<2, Store16<false, 3> >"
-KERNEL_DWEIGHT = "gemm16_sweep<1, Store16<true, 0> >"
+KERNEL_DWEIGHT = "gemm16_sweep<1, Store16<false, 0> >"
 
 WORKLOADS = {
     # name: (T, H, n_seqs, min_len, max_len, seed, description)

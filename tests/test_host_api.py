@@ -50,6 +50,14 @@ def test_workspace_size_queries_run_without_gpu():
     assert lib.areal_lmhead_bwd_workspace_bytes(1024, 64, 1000, 256) >= 2 * (64 * 1024 + 256 * 1024)
     assert (lib.areal_lmhead_bwd_workspace_bytes(1000, 64, 1000, 256)
             > lib.areal_lmhead_bwd_workspace_bytes(1024, 64, 1000, 256) + 2 * 1000 * 256)
+    # backward from saved exponentials: 594 x 16 dWeight tiles are 298 super-blocks of 32 workgroups,
+    # 2 more than whole rounds of 8; those 384 vocabulary rows get fp32 partial results of 6 splits of
+    # the token range (12 half-filled super-blocks, at most 32 workgroups on an XCD). 592 x 16 tiles are
+    # whole rounds and need none.
+    saved = lib.areal_lmhead_bwd_saved_workspace_bytes
+    assert saved(32768, 4096, 151936) - saved(32768, 4096, 151552) == 6 * 384 * 4096 * 4 + 256
+    # 144 x 2 tiles = 9 super-blocks: the last 16 tile columns (the test shape of tests/test_gpu_lmhead.py)
+    assert saved(2048, 512, 36764) > 2 * (36764 - 128 * 256) * 512 * 4
     assert lib.areal_gae_workspace_bytes(0) == 0
     assert lib.areal_actor_loss_workspace_bytes(10, 3) > 0
 
