@@ -604,9 +604,9 @@ def main() -> None:
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            KERNEL_FWD_SAVE + " forward": 3.63869e7 * kib * 2.0 + 9.72237e6 * kib,
-            KERNEL_DHIDDEN + " dHidden": 2.91991e7 * kib * 2.0 + 2.64192e5 * kib,
-            KERNEL_DWEIGHT + " dWeight": 2.94247e7 * kib * 2.0 + 1.21549e6 * kib,
+            KERNEL_FWD_SAVE + " forward": 3.66677e7 * kib * 2.0 + 9.72237e6 * kib,
+            KERNEL_DHIDDEN + " dHidden": 2.92022e7 * kib * 2.0 + 2.64192e5 * kib,
+            KERNEL_DWEIGHT + " dWeight": 2.92275e7 * kib * 2.0 + 1.22189e6 * kib,
         }
         traffic = sum(traffic_detail.values()) / 3.0
         traffic_source = ("offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command "
