@@ -2215,7 +2215,7 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // only when one of them is requested.
 //
 // probs / probs_ref / probs_status (all null or all set) keep the exponentials of the softmax
-// for areal_lmhead_bwd_saved: probs bf16 [round_up(T, 64)][round_up(V, 64)] (rows >= T are not
+// for areal_lmhead_bwd_saved: probs bf16 [round_up(T, 128)][round_up(V, 64)] (rows >= T are not
 // written) holds e = 2^(c2 x - probs_ref[t]); probs_ref fp32 [T] is a per-row reference taken
 // from a few logits of the row before the sweep; *probs_status (one int) is set to 0 when every
 // row's exponentials are in range and to 1 when some row's maximum lies more than 150 binades
@@ -2406,20 +2406,21 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
 }
 
 // Workspace of the backward from saved exponentials: row factors [T] fp32, scaled hidden states
-// [round_up(T, 64), H] bf16, W^T [H, round_up(V, 64)] bf16 (only when V is not a multiple of 64)
+// [round_up(T, 128), H] bf16, W^T [H, round_up(V, 64)] bf16 (only when V is not a multiple of 64)
 // and the split-K partials of dHidden and of dWeight's last partial round.
 size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || H <= 0 || V <= 0) return 0;
   const size_t wt = dh_weight_in_place(V) ? 0 : (size_t)(H * round_up_i64(V, BK)) * 2;
-  return (size_t)T * 4 + (size_t)(round_up_i64(T, BK) * H) * 2 + wt +
-         dh_partial_bytes(H, T, round_up_i64(V, BK)) + dw_tail_bytes(H, V, round_up_i64(T, BK)) + 5 * 256;
+  return (size_t)T * 4 + (size_t)(round_up_i64(T, 2 * BK) * H) * 2 + wt +
+         dh_partial_bytes(H, T, round_up_i64(V, BK)) + dw_tail_bytes(H, V, round_up_i64(T, 2 * BK)) + 5 * 256;
 }
 
 // Backward from the exponentials areal_lmhead_fwd saved (probs, probs_ref, with *probs_status
 // read back as 0): no logits are recomputed and no pass rewrites the [T, V] buffer. Per row,
 // dlogits = f[t] * e' with a row factor f; dHidden scales its output rows by f and dWeight
 // contracts e' with f[t] * hidden[t]. Only the label's entry of each row of probs is rewritten
-// (and rows [T, round_up(T, 64)) are cleared), so probs can be used once. logprobs (nullable)
+// (and rows [T, round_up(T, 128)) are cleared: the token range of dWeight's contraction is whole
+// pairs of k-tiles, which the hand-scheduled main loop walks), so probs can be used once. logprobs (nullable)
 // are the label log-probabilities of the forward; with them the label's entry is evaluated in
 // fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store (the
 // whole batch is one contraction, so no fp32 staging is needed). probs_status (nullable): the
@@ -2449,7 +2450,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
   if (dweight != nullptr && !aligned16(dweight)) return AREAL_ERR_ALIGNMENT;
   if (workspace == nullptr || workspace_bytes < areal_lmhead_bwd_saved_workspace_bytes(T, H, V))
     return AREAL_ERR_WORKSPACE;
-  const int64_t ldv = round_up_i64(V, BK), Tpad = round_up_i64(T, BK);
+  const int64_t ldv = round_up_i64(V, BK), Tpad = round_up_i64(T, 2 * BK);
   auto align256 = [](void* q) { return (void*)(((uintptr_t)q + 255) & ~(uintptr_t)255); };
   float* rowfac = (float*)align256(workspace);
   u16* hs = (u16*)align256(rowfac + T);

@@ -104,12 +104,12 @@ class _FusedLMHead(torch.autograd.Function):
         # the caller has ruled out no_grad mode
         needs_grad = any(ctx.needs_input_grad[:2]) or weight_grad_accum is not None
         if save_probs is None:
-            need = 2 * _round_up(T, 64) * _round_up(V, 64)
+            need = 2 * _round_up(T, 128) * _round_up(V, 64)
             save_probs = need <= SAVE_PROBS_BYTES_LIMIT and need <= 0.6 * _available_bytes(dev)
         probs = probs_ref = probs_status = None
         if save_probs and needs_grad and T > 0:
             probs = torch.empty(
-                (_round_up(T, 64), _round_up(V, 64)), dtype=torch.bfloat16, device=dev
+                (_round_up(T, 128), _round_up(V, 64)), dtype=torch.bfloat16, device=dev
             )
             probs_ref = torch.empty(T, dtype=torch.float32, device=dev)
             probs_status = torch.empty(1, dtype=torch.int32, device=dev)

@@ -50,7 +50,7 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * exponentials for areal_lmhead_bwd_saved, the counterpart of autograd saving the logits in the
  * reference's logits-in path (_gather_logprobs_entropy,
  * areal/utils/functional/vocab_parallel.py:24-30): probs is bf16
- * [round_up(T,64)][round_up(V,64)] holding 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
+ * [round_up(T,128)][round_up(V,64)] holding 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
  * fp32 [T], a per-row reference estimated from a few logits of the row (its label's among
  * them) before the sweep; *probs_status (one int32 on the device) is written 0 when every
  * row's exponentials are in range, 1 when some row's maximum lies more than 150 binades above

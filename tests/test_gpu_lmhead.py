@@ -60,6 +60,9 @@ SHAPES = [
     (768, 256, 1536, 1.0, 1.0, False, None),
     (384, 384, 2000, 0.8, 1.5, True, 128),
     (1024, 128, 640, 1.0, 1.0, False, 256),
+    # T = 6.5 x 128: the saved buffer's rows are padded to 896 so that dWeight's token range is whole
+    # pairs of k-tiles
+    (832, 256, 1536, 1.0, 1.0, False, None),
     # 144 x 2 dWeight tiles = 9 super-blocks of 32 workgroups: the last one is contracted by a second
     # launch with the token range split over 8 copies (saved mode)
     (2048, 512, 36764, 1.0, 1.0, False, None),
