@@ -1637,11 +1637,41 @@ template <bool E> using Store16Bf16Scaled = Store16<E, 3>;
 // into the running statistics of token column jb, of which it keeps two (jb and jb + 4): ten to
 // fourteen registers per lane live across the main loop. Partial statistics go to slot
 // split * 2 + wa at the end of the sweep.
-DEVI float xor_lanes16(float v) { return __shfl_xor(v, 16); }
-DEVI float xor_lanes32(float v) { return __shfl_xor(v, 32); }
-DEVI float group_max(float v) { v = fmaxf(v, xor_lanes16(v)); return fmaxf(v, xor_lanes32(v)); }
-DEVI float group_min(float v) { v = fminf(v, xor_lanes16(v)); return fminf(v, xor_lanes32(v)); }
-DEVI float group_sum(float v) { v += xor_lanes16(v); return v + xor_lanes32(v); }
+// The four lanes that share a token are 16 and 32 lanes apart. v_permlane16_swap exchanges the
+// odd rows (of 16 lanes) of its first register with the even rows of its second, v_permlane32_swap
+// rows 2-3 of the first with rows 0-1 of the second: applied to two copies of a value they leave
+// (own, partner 16 / 32 lanes away) in every lane, as vector operations of a few cycles where a
+// shuffle goes through the LDS crossbar (about a hundred cycles that nothing overlaps here: the
+// wave is alone on its SIMD). The leading wait states are those a vector write needs before
+// these instructions read it. (The compiler's own builtin for them returns one register for
+// both results in this toolchain, hence the assembly.)
+DEVI void swap_rows16(float& a, float& b) {
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+DEVI void swap_rows32(float& a, float& b) {
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+DEVI float group_max(float v) {
+  float a = v, b = v;
+  swap_rows16(a, b);
+  a = b = fmaxf(a, b);
+  swap_rows32(a, b);
+  return fmaxf(a, b);
+}
+DEVI float group_min(float v) {
+  float a = v, b = v;
+  swap_rows16(a, b);
+  a = b = fminf(a, b);
+  swap_rows32(a, b);
+  return fminf(a, b);
+}
+DEVI float group_sum(float v) {
+  float a = v, b = v;
+  swap_rows16(a, b);
+  a = b = a + b;
+  swap_rows32(a, b);
+  return a + b;
+}
 
 template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
 struct Fwd16 {
