@@ -1,0 +1,79 @@
+"""Shape sweep of the fused lm_head kernels: ragged and aligned token counts, hidden sizes and
+vocabularies around every boundary the launch plan has (256-wide tiles, 64- and 128-deep
+contraction steps, split contraction ranges, the split of dWeight's last round), both backward
+modes, against a plain fp32 torch evaluation of the same operator on the GPU
+(areal/utils/functional/vocab_parallel.py:24-30 restated with torch ops; an implementation
+independent of the kernels under test: the library GEMM in fp32).
+
+Tolerances as in test_gpu_lmhead.py: logprobs / entropy 2e-3 absolute, gradients 1e-2 relative L2."""
+
+import pytest
+import torch
+
+from areal_amd.functional import fused_lm_head_logprobs_entropy
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
+
+
+def _reference(hidden, weight, labels, grad, temp, scale):
+    h = hidden.detach().float().requires_grad_(True)
+    w = weight.detach().float().requires_grad_(True)
+    logits = (h @ w.t()) * scale / temp
+    logp = torch.log_softmax(logits, dim=-1)
+    lp = logp.gather(-1, labels[:, None])[:, 0]
+    ent = -(logp.exp() * logp).sum(-1)
+    (lp * grad).sum().backward()
+    return lp.detach(), ent.detach(), logits.detach().min(-1).values * temp, logits.detach().max(-1).values * temp, h.grad, w.grad
+
+
+def _case_list():
+    g = torch.Generator().manual_seed(20240607)
+    tokens = [64, 128, 192, 200, 256, 257, 320, 448, 1000, 1088]
+    hiddens = [128, 256, 384, 640, 896, 1024]
+    vocabs = [640, 1000, 1536, 2176, 4160, 5000, 8192 + 128]
+    cases = []
+    for _ in range(28):
+        t = tokens[int(torch.randint(len(tokens), (1,), generator=g))]
+        h = hiddens[int(torch.randint(len(hiddens), (1,), generator=g))]
+        v = vocabs[int(torch.randint(len(vocabs), (1,), generator=g))]
+        cases.append((t, h, v))
+    # dWeight's last partial round of super-blocks with a ragged hidden size (2.5 tiles) and a
+    # ragged vocabulary: 80 x 3 tiles
+    cases.append((2048, 640, 20403))
+    # token count 64 short of a multiple of 128 with a contraction long enough to split
+    cases.append((1984, 256, 9000))
+    return sorted(set(cases))
+
+
+@pytest.mark.parametrize("save_probs", [True, False], ids=["saved", "recompute"])
+@pytest.mark.parametrize("T,H,V", _case_list())
+def test_shapes_against_fp32_torch(dev, T, H, V, save_probs):
+    g = torch.Generator(device="cpu").manual_seed(T * 31 + H * 7 + V)
+    temp, scale = (1.0, 1.0) if (T + V) % 3 else (0.7, 1.5)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * (2.0 / H ** 0.5)).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    grad = torch.randn(T, generator=g)
+    grad[::5] = 0
+    grad = grad.to(dev)
+    h = hidden.clone().requires_grad_(True)
+    w = weight.clone().requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels, temperature=temp, logit_scale=scale,
+                                         save_probs=save_probs)
+    (out.logprobs * grad).sum().backward()
+    lp, ent, vmin, vmax, dh, dw = _reference(hidden, weight, labels, grad, temp, scale)
+    assert (out.logprobs.detach() - lp).abs().max().item() < 2e-3
+    assert (out.entropy - ent).abs().max().item() < 2e-3
+    # the vocabulary extremes are those of the unscaled-by-temperature logits
+    # (areal/engine/fsdp_engine.py:2061-2105 takes them before the temperature division)
+    span = max(1.0, vmax.abs().max().item(), vmin.abs().max().item())
+    assert (out.vocab_max_logits - vmax).abs().max().item() < 2e-3 * span
+    assert (out.vocab_min_logits - vmin).abs().max().item() < 2e-3 * span
+    assert h.grad.dtype == torch.bfloat16 and w.grad.dtype == torch.bfloat16
+    assert _rel(h.grad.float(), dh) < 1e-2
+    assert _rel(w.grad.float(), dw) < 1e-2
+    assert (h.grad[::5] == 0).all()
