@@ -108,6 +108,10 @@ DEVI float torch_clamp(float x, float lo, float hi) {
 }
 DEVI float torch_max(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a > b ? a : b); }
 DEVI float torch_min(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a < b ? a : b); }
+// The same for the running extremes of the logged statistics, where the sign of a zero does not
+// matter: IEEE 754-2019 minimum / maximum, one instruction each (v_minimum3_f32 / v_maximum3_f32).
+DEVI float stat_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+DEVI float stat_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 
 // Bernoulli KL(P||Q) with p = clamp(exp(log_p), 1e-8, 1 - 1e-8): in fp32 the upper bound
 // rounds to 1.0f, which is what the reference's fp32 tensors see.
@@ -296,8 +300,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
   auto stat = [&](int k, bool on, float v) {
     if (STATS && on) {
       st_sum[k] += (double)v;
-      st_mn[k] = torch_min(st_mn[k], v);
-      st_mx[k] = torch_max(st_mx[k], v);
+      st_mn[k] = stat_min(st_mn[k], v);
+      st_mx[k] = stat_max(st_mx[k], v);
     }
   };
 
@@ -436,8 +440,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
       float mn = st_mn[k], mx = st_mx[k];
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) {
-        mn = torch_min(mn, __shfl_xor(mn, o, 64));
-        mx = torch_max(mx, __shfl_xor(mx, o, 64));
+        mn = stat_min(mn, __shfl_xor(mn, o, 64));
+        mx = stat_max(mx, __shfl_xor(mx, o, 64));
       }
       if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
     }
@@ -447,8 +451,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
       StatPartial sp{sh_sum[0][k], sh_mn[0][k], sh_mx[0][k]};
       for (int i = 1; i < LOSS_THREADS / 64; ++i) {
         sp.sum += sh_sum[i][k];
-        sp.mn = torch_min(sp.mn, sh_mn[i][k]);
-        sp.mx = torch_max(sp.mx, sh_mx[i][k]);
+        sp.mn = stat_min(sp.mn, sh_mn[i][k]);
+        sp.mx = stat_max(sp.mx, sh_mx[i][k]);
       }
       stat_partials[(size_t)blockIdx.x * N_LOSS_STATS + k] = sp;
     }
@@ -469,22 +473,22 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_stats_finalize_kernel(
   for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
     const StatPartial sp = stat_partials[(size_t)i * N_LOSS_STATS + k];
     sum += sp.sum;
-    mn = torch_min(mn, sp.mn);
-    mx = torch_max(mx, sp.mx);
+    mn = stat_min(mn, sp.mn);
+    mx = stat_max(mx, sp.mx);
   }
   sum = block_sum(sum, sm_d);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
-    mn = torch_min(mn, __shfl_xor(mn, o, 64));
-    mx = torch_max(mx, __shfl_xor(mx, o, 64));
+    mn = stat_min(mn, __shfl_xor(mn, o, 64));
+    mx = stat_max(mx, __shfl_xor(mx, o, 64));
   }
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   __syncthreads();
   if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    mn = torch_min(torch_min(sm_f[0], sm_f[1]), torch_min(sm_f[2], sm_f[3]));
-    mx = torch_max(torch_max(sm_f[4], sm_f[5]), torch_max(sm_f[6], sm_f[7]));
+    mn = stat_min(stat_min(sm_f[0], sm_f[1]), stat_min(sm_f[2], sm_f[3]));
+    mx = stat_max(stat_max(sm_f[4], sm_f[5]), stat_max(sm_f[6], sm_f[7]));
     const int d = STAT_DENOM[k];
     const double count = d == 0 ? counters[1] : (d == 1 ? counters[4] : (d == 2 ? counters[6] : n_tokens));
     stats[4 * k + 0] = sum;
