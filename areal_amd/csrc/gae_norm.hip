@@ -342,30 +342,42 @@ DEVI void gae_owned_items(int64_t t0, int64_t t_begin, int64_t t_end, int& i_lo,
   i_hi = d_hi < GAE_ITEMS ? (d_hi > 0 ? (int)d_hi : 0) : GAE_ITEMS;
 }
 
+// How a tile finds its sequences: in cu_seqlens, as rows of uniform length, or as part of the one
+// row the block walks.
+enum { GAE_LAYOUT_CU = 0, GAE_LAYOUT_ROWS = 1, GAE_LAYOUT_ONE_ROW = 2 };
+
 // (rw, v, ms): the tile's inputs as gae_load_items leaves them (at least the owned tokens).
-template <bool STATS>
+// LAMBDAS: a lambda per sequence (GaeArgs::lam_seq).
+template <bool STATS, int LAYOUT, bool LAMBDAS>
 DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t t_end, int s_first,
-                       int n_own, const int32_t* cu_own, bool uniform, double& A0, double& nv0,
+                       int n_own, const int32_t* cu_own, double& A0, double& nv0,
                        double (&rs)[STATS ? 5 : 1], MapF* smem, MapF* all,
                        const float (&rw)[GAE_ITEMS], const float (&v)[GAE_ITEMS],
                        const float (&ms)[GAE_ITEMS]) {
+  constexpr bool uniform = LAYOUT != GAE_LAYOUT_CU;
   const int tid = threadIdx.x;
   const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
   // The thread keeps its 8 tokens as raw inputs plus two bit masks and rebuilds a token's map
-  // where it is needed (twice): holding 8 fp64 maps would halve the occupancy.
-  float lm[GAE_ITEMS];
+  // where it is needed (twice): holding 8 maps would cost a wave of occupancy.
+  float lm[LAMBDAS ? GAE_ITEMS : 1], mm[GAE_ITEMS];
   unsigned valid = 0, ends = 0, boot = 0;  // bit i: token owned / last of its sequence / no_eos
   int i_lo, i_hi;  // owned tokens of this thread
   gae_owned_items(t0, t_begin, t_end, i_lo, i_hi);
   const bool any = i_lo < i_hi;
+  if (LAMBDAS) {
 #pragma unroll
-  for (int i = 0; i < GAE_ITEMS; ++i) lm[i] = g.lam;
+    for (int i = 0; i < (LAMBDAS ? GAE_ITEMS : 1); ++i) lm[i] = g.lam;
+  }
   if (any) {
     // sequence of the first owned token of this thread (index relative to s_first)
     const int64_t tf = t0 + i_lo;
     int sq;
     int e_loc;  // local index one past the last token of sequence sq (clamped)
-    if (uniform) {
+    if (LAYOUT == GAE_LAYOUT_ONE_ROW) {
+      sq = 0;
+      const int64_t e = t_end - t0;
+      e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
+    } else if (LAYOUT == GAE_LAYOUT_ROWS) {
       sq = (int)(tf / g.uniform_len) - s_first;
       const int64_t e = (int64_t)(sq + s_first + 1) * g.uniform_len - t0;
       e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
@@ -380,7 +392,7 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
       e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
     }
     valid = ((1u << i_hi) - 1u) & ~((1u << i_lo) - 1u);
-    if (e_loc > i_hi && g.lam_seq == nullptr) {
+    if (e_loc > i_hi && !LAMBDAS) {
       // common case: all owned tokens inside one sequence, none of them its last
     } else {
       // a sequence ends among these tokens (or lambda is per sequence): walk them
@@ -391,10 +403,10 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
                                      : (int64_t)cu_own[sq + 1]) - t0;
           e_loc = e < 2 * GAE_ITEMS ? (int)e : 2 * GAE_ITEMS;
         }
-        if (g.lam_seq != nullptr) {
+        if (LAMBDAS) {
           const float l = g.lam_seq[s_first + sq];
 #pragma unroll
-          for (int k = 0; k < GAE_ITEMS; ++k) if (k == i) lm[k] = l;
+          for (int k = 0; k < (LAMBDAS ? GAE_ITEMS : 1); ++k) if (k == i) lm[k] = l;
         }
         if (i == e_loc - 1) {
           ends |= 1u << i;
@@ -403,19 +415,26 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
       }
     }
   }
+  // not owned: identity (mask 0 with no offsets)
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) mm[i] = ((valid >> i) & 1u) ? ms[i] : 0.f;
   const float gam = g.discount;
+  const float c0 = gam * g.lam;
+  // few waves hold the last token of a sequence: the others skip its constant map by a scalar branch
+  const bool wave_has_end = __builtin_amdgcn_ballot_w64(ends != 0) != 0;
   auto token_map = [&](int i) -> MapF {
     const float val = v[i];
-    // not owned: identity (m = 0 with no offsets); last token of a sequence: constant map
-    const float m = ((valid >> i) & 1u) ? ms[i] : 0.f;
-    const float c = gam * lm[i];
+    const float m = mm[i];
+    const float c = LAMBDAS ? gam * lm[LAMBDAS ? i : 0] : c0;
     MapF f;
     f.a11 = fmaf(c, m, 1.f - m);
     f.a12 = gam * m;
     f.a22 = 1.f - m;
     f.b1 = (rw[i] - val) * m;
     f.b2 = val * m;
-    if ((ends >> i) & 1u) f = MapF{0.f, 0.f, 0.f, 0.f, ((boot >> i) & 1u) ? val : 0.f};
+    if (wave_has_end) {
+      if ((ends >> i) & 1u) f = MapF{0.f, 0.f, 0.f, 0.f, ((boot >> i) & 1u) ? val : 0.f};
+    }
     return f;
   };
   MapF mine = token_map(GAE_ITEMS - 1);
@@ -477,8 +496,9 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
 // 2048, measured slower: 46.7 against 30.8 us on [1024, 8192]; one such block fills a CU's
 // registers and the latency of its single pass is not covered by anything.)
 // STATS: also sum each row's advantages under the mask (block = row only), see GaeArgs::row_stats.
-template <bool STATS>
-__global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
+// ONE_ROW: block = row (GaeArgs::block_per_seq); LAMBDAS: a lambda per row.
+template <bool STATS, bool ONE_ROW, bool LAMBDAS>
+__global__ __launch_bounds__(GAE_THREADS, 4) void gae_owned_kernel(GaeArgs g) {
   __shared__ MapF smem[GAE_THREADS / 64];
   __shared__ MapF all[GAE_THREADS];
   const int tid = threadIdx.x;
@@ -488,10 +508,10 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
   const int64_t range = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   // rows of at least a tile: only every (L / TILE)-th range would own a row, so the grid is one
   // block per row instead, (lo, hi] = the range holding the row's end
-  const int64_t lo = g.block_per_seq ? ((int64_t)(blockIdx.x + 1) * g.uniform_len - 1)
+  const int64_t lo = ONE_ROW ? ((int64_t)(blockIdx.x + 1) * g.uniform_len - 1)
                                      : range * GAE_TILE;
-  if (!g.block_per_seq && (range >= per_xcd * 8 || lo >= g.n)) return;
-  const int64_t hi = g.block_per_seq ? lo + 1 : (lo + GAE_TILE < g.n ? lo + GAE_TILE : g.n);
+  if (!ONE_ROW && (range >= per_xcd * 8 || lo >= g.n)) return;
+  const int64_t hi = ONE_ROW ? lo + 1 : (lo + GAE_TILE < g.n ? lo + GAE_TILE : g.n);
   // owned rows [s_first, s_last]: lo < end(s) <= hi
   const int s_first = (int)(lo / g.uniform_len);
   const int s_last = (int)(hi / g.uniform_len) - 1;
@@ -508,8 +528,8 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
     gae_owned_items(t0, t_begin, t_end, i_lo, i_hi);
     float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS];
     gae_load_items(g, t0, i_lo < i_hi, rw, v, ms);
-    gae_one_tile<STATS>(g, tile, t_begin, t_end, s_first, n_own, nullptr, true, A0, nv0, rs, smem, all,
-                        rw, v, ms);
+    gae_one_tile<STATS, ONE_ROW ? GAE_LAYOUT_ONE_ROW : GAE_LAYOUT_ROWS, LAMBDAS>(
+        g, tile, t_begin, t_end, s_first, n_own, nullptr, A0, nv0, rs, smem, all, rw, v, ms);
   }
   if constexpr (STATS) {  // block = row: uniform for the block
     __shared__ double s_rs[4 * 5];
@@ -538,6 +558,7 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_owned_kernel(GaeArgs g) {
 constexpr int GAE_CARRY_BATCH = 2;
 constexpr int GAE_CU_LDS = 16 * GAE_THREADS;  // entries of cu_seqlens the block can hold (>= TILE + 2)
 
+template <bool LAMBDAS>
 __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
   __shared__ MapF smem[GAE_THREADS / 64];
   __shared__ MapF all[GAE_THREADS];
@@ -626,7 +647,7 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
   const int64_t e = (int64_t)cu_own[n_own];
   if (e > t_end) {
     const float gam = g.discount;
-    const float c = gam * (g.lam_seq != nullptr ? g.lam_seq[s_last] : g.lam);
+    const float c = gam * (LAMBDAS ? g.lam_seq[s_last] : g.lam);
     const bool boot = g.no_eos != nullptr && g.no_eos[s_last] != 0;
     const int64_t n_right = (e - t_end + GAE_TILE - 1) / GAE_TILE;
     for (int64_t j = n_right; j > 0; j -= GAE_CARRY_BATCH) {
@@ -698,8 +719,8 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
     }
   }
   double rs[1];
-  gae_one_tile<false>(g, tile, t_begin, t_end, s_first, n_own, cu_own, false, A0, nv0, rs, smem, all,
-                      rw, v, ms);
+  gae_one_tile<false, GAE_LAYOUT_CU, LAMBDAS>(g, tile, t_begin, t_end, s_first, n_own, cu_own, A0, nv0, rs, smem,
+                                              all, rw, v, ms);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1535,6 +1556,19 @@ __global__ __launch_bounds__(TURN_THREADS) void gae_context_kernel(const float* 
   if (bad) atomicOr(status, bad);
 }
 
+// gae_owned_kernel's instance for the batch (STATS needs block = row)
+template <bool STATS>
+void launch_gae_owned(const GaeArgs& g, int64_t grid, hipStream_t stream) {
+  const dim3 gr((unsigned)grid), bl(GAE_THREADS);
+  if (g.block_per_seq) {
+    if (g.lam_seq != nullptr) hipLaunchKernelGGL((gae_owned_kernel<STATS, true, true>), gr, bl, 0, stream, g);
+    else hipLaunchKernelGGL((gae_owned_kernel<STATS, true, false>), gr, bl, 0, stream, g);
+  } else if constexpr (!STATS) {
+    if (g.lam_seq != nullptr) hipLaunchKernelGGL((gae_owned_kernel<false, false, true>), gr, bl, 0, stream, g);
+    else hipLaunchKernelGGL((gae_owned_kernel<false, false, false>), gr, bl, 0, stream, g);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -1574,8 +1608,11 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
   const int64_t mean_len = n_tokens / n_seqs;
   if (uniform_len <= 0 && mean_len <= 8 * GAE_TILE) {
     // packed sequences: block = tile, the state entering from the right recomputed per tile
-    hipLaunchKernelGGL(gae_tile_kernel, dim3((unsigned)(ceil_div_i64(nb, 8) * 8)), dim3(GAE_THREADS), 0,
-                       stream, g);
+    const dim3 grid((unsigned)(ceil_div_i64(nb, 8) * 8));
+    if (lambda_seq != nullptr)
+      hipLaunchKernelGGL(gae_tile_kernel<true>, grid, dim3(GAE_THREADS), 0, stream, g);
+    else
+      hipLaunchKernelGGL(gae_tile_kernel<false>, grid, dim3(GAE_THREADS), 0, stream, g);
     AREAL_CHECK_LAUNCH();
     return AREAL_OK;
   }
@@ -1585,7 +1622,7 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
       (n_seqs >= 256 || uniform_len <= 4 * GAE_TILE)) {
     g.block_per_seq = uniform_len >= GAE_TILE;
     const int64_t grid = g.block_per_seq ? n_seqs : ceil_div_i64(nb, 8) * 8;
-    hipLaunchKernelGGL(gae_owned_kernel<false>, dim3((unsigned)grid), dim3(GAE_THREADS), 0, stream, g);
+    launch_gae_owned<false>(g, grid, stream);
     AREAL_CHECK_LAUNCH();
     return AREAL_OK;
   }
@@ -1617,7 +1654,7 @@ int areal_gae_padded_row_stats(const float* rewards, const float* values, const 
     return AREAL_ERR_UNSUPPORTED;
   GaeArgs g{rewards, values, loss_mask, nullptr, no_eos, lambda_seq, n_seqs * uniform_len, (int)n_seqs,
             uniform_len, discount, gae_lambda, advantages, returns, 1, row_stats};
-  hipLaunchKernelGGL(gae_owned_kernel<true>, dim3((unsigned)n_seqs), dim3(GAE_THREADS), 0, stream, g);
+  launch_gae_owned<true>(g, n_seqs, stream);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
