@@ -1563,15 +1563,21 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
 // One block column of the wave's sub-tile (16 rows j x 128 bf16 values i) from the staging area
 // to global memory: lane -> (row 4*p + lane/16, 16-byte piece lane%16), so 16 lanes write the
 // 256 contiguous bytes of a row. out_row0 points at element (j0, i0) of the output.
-template <bool EDGE>
+// STREAM: the output is a [T, V]-sized buffer that nothing reads before the kernel ends; its
+// stores carry the non-temporal hint so that they do not push the operand tiles the XCD's other
+// workgroups share out of L2.
+template <bool EDGE, bool STREAM = false>
 DEVI void flush_stage16(const u16* stage, u16* out_row0, int64_t ld, int rows_valid, int cols_valid, int lane) {
   const int piece = lane & 15;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = p * 4 + (lane >> 4);
     const u32x4 v = *(const u32x4*)((const char*)stage + row * STAGE16_PITCH + piece * 16);
-    if (!EDGE || (row < rows_valid && piece * 8 < cols_valid))
-      *(u32x4*)(out_row0 + (int64_t)row * ld + piece * 8) = v;
+    if (!EDGE || (row < rows_valid && piece * 8 < cols_valid)) {
+      u32x4* dst = (u32x4*)(out_row0 + (int64_t)row * ld + piece * 8);
+      if (STREAM) __builtin_nontemporal_store(v, dst);
+      else *dst = v;
+    }
   }
 }
 DEVI void stage16_put(u16* stage, int lane, int ia, u32x2 v) {
@@ -1782,7 +1788,7 @@ struct Fwd16 {
           __builtin_amdgcn_sched_barrier(0);
           ML16_AGPR_FENCE();
         }
-        flush_stage16<EDGE>(stage, p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv,
+        flush_stage16<EDGE, true>(stage, p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv,
                             p.T - (t0 + b * 16), (int)p.ldv - v0, lane);
       }
       // the label's logit, if it is one of this lane's 32 entries
@@ -1912,7 +1918,7 @@ struct Bwd16 {
         pk[1] = pack_bf16x2(d[2], d[3]);
         stage16_put(stage, lane, a, pk);
       }
-      flush_stage16<EDGE>(stage, p.dl + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv, p.T - (t0 + b * 16),
+      flush_stage16<EDGE, true>(stage, p.dl + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv, p.T - (t0 + b * 16),
                           (int)p.ldv - v0, lane);
     });
   }
