@@ -604,7 +604,7 @@ def main() -> None:
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            KERNEL_FWD_SAVE + " forward": 3.66677e7 * kib * 2.0 + 9.72237e6 * kib,
+            KERNEL_FWD_SAVE + " forward": 3.09126e7 * kib * 2.0 + 9.72083e6 * kib,
             KERNEL_DHIDDEN + " dHidden": 2.92022e7 * kib * 2.0 + 2.64192e5 * kib,
             KERNEL_DWEIGHT + " dWeight": 2.92275e7 * kib * 2.0 + 1.22189e6 * kib,
         }
