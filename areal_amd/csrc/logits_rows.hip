@@ -14,25 +14,28 @@ constexpr int ROW_THREADS = 256;
 constexpr float LOG2E_F = 1.4426950408889634f;
 constexpr float LN2_F = 0.6931471805599453f;
 
+// Vector loads and stores carry the non-temporal hint: every logit is read once per kernel (and every
+// dlogit written once), and a plain read of a [4096, 151936] bf16 array in this access pattern
+// measures 6.15 TB/s without the hint, 7.04 TB/s with it.
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int VEC = 4;
   static DEVI float load(const float* p) { return *p; }
   static DEVI void loadv(const float* p, float (&o)[4]) {
-    const f32x4 v = *(const f32x4*)p;
+    const f32x4 v = __builtin_nontemporal_load((const f32x4*)p);
     o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
   }
   static DEVI void store(float* p, float v) { *p = v; }
   static DEVI void storev(float* p, const float (&o)[4]) {
     f32x4 v = {o[0], o[1], o[2], o[3]};
-    *(f32x4*)p = v;
+    __builtin_nontemporal_store(v, (f32x4*)p);
   }
 };
 template <> struct Elem<u16> {  // bf16 bit patterns
   static constexpr int VEC = 8;
   static DEVI float load(const u16* p) { return bf16_bits_to_f32(*p); }
   static DEVI void loadv(const u16* p, float (&o)[8]) {
-    const u32x4 v = *(const u32x4*)p;
+    const u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       o[2 * i] = __builtin_bit_cast(float, v[i] << 16);
@@ -45,7 +48,7 @@ template <> struct Elem<u16> {  // bf16 bit patterns
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       v[i] = (uint32_t)f32_to_bf16_bits(o[2 * i]) | ((uint32_t)f32_to_bf16_bits(o[2 * i + 1]) << 16);
-    *(u32x4*)p = v;
+    __builtin_nontemporal_store(v, (u32x4*)p);
   }
 };
 
@@ -60,11 +63,15 @@ DEVI void online_merge(Online& a, const Online& b) {
   if (b.m > neg_inf()) { const float d = b.m - m, al = fast_exp2(d); s += al * b.s; q += al * fmaf(d, b.s, b.q); }
   a.m = m; a.s = s; a.q = q;
 }
+// x: raw logits; the exponents are z2 = x * c2 (c2 > 0). The running maximum is kept as the
+// rounded product of the largest logit and every exponent is taken relative to it with one fused
+// multiply-subtract, as the backward evaluates them against lse2.
 template <int N>
-DEVI void online_add(Online& st, const float (&z)[N]) {
-  float vm = z[0];
+DEVI void online_add(Online& st, const float (&x)[N], float c2) {
+  float xm = x[0];
 #pragma unroll
-  for (int i = 1; i < N; ++i) vm = fmaxf(vm, z[i]);
+  for (int i = 1; i < N; ++i) xm = fmaxf(xm, x[i]);
+  const float vm = xm * c2;
   if (vm > st.m) {
     if (st.m > neg_inf()) {
       const float d = st.m - vm, al = fast_exp2(d);
@@ -75,7 +82,7 @@ DEVI void online_add(Online& st, const float (&z)[N]) {
   }
 #pragma unroll
   for (int i = 0; i < N; ++i) {
-    const float t = z[i] - st.m;
+    const float t = fmaf(x[i], c2, -st.m);
     const float e = fast_exp2(t);
     st.s += e;
     st.q = fmaf(t, e, st.q);
@@ -117,14 +124,12 @@ __global__ __launch_bounds__(ROW_THREADS) void rows_fwd_kernel(const T* __restri
     for (int v0 = threadIdx.x * VEC; v0 < V; v0 += ROW_THREADS * VEC) {
       float z[VEC];
       Elem<T>::loadv(x + v0, z);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) z[i] *= c2;
-      online_add(st, z);
+      online_add(st, z, c2);
     }
   } else {
     for (int v = threadIdx.x; v < V; v += ROW_THREADS) {
-      float z[1] = {Elem<T>::load(x + v) * c2};
-      online_add(st, z);
+      float z[1] = {Elem<T>::load(x + v)};
+      online_add(st, z, c2);
     }
   }
   const Online r = block_merge(st, smem);
@@ -134,14 +139,10 @@ __global__ __launch_bounds__(ROW_THREADS) void rows_fwd_kernel(const T* __restri
     const int64_t lab = labels[row];
     float lp = 0.f;
     if (lab >= 0 && lab < V) {
-      // the label's exponent as the sums saw it: the rounded product, not fused into the
-      // subtraction (lse2 is built from such rounded products)
-      float zl;
-      {
-#pragma clang fp contract(off)
-        zl = Elem<T>::load(x + lab) * c2;
-      }
-      lp = fminf((zl - lse2) * LN2_F, 0.f);
+      // the label's exponent as the sums saw it: relative to the running maximum, by one fused
+      // multiply-subtract
+      const float tl = fmaf(Elem<T>::load(x + lab), c2, -r.m);
+      lp = fminf((tl - log2s) * LN2_F, 0.f);
     }
     if (logprobs) logprobs[row] = lp;
     if (entropy) entropy[row] = (log2s - r.q / r.s) * LN2_F;
