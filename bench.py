@@ -400,6 +400,19 @@ def hbm_rooflines(dev):
     lab = torch.randint(0, V_QWEN, (4096,), device=dev)
     add("rows_fwd_kernel", "config 1: [4096, 151936] bf16 logits, logprob + entropy forward",
         lg.numel() * 2 + 16 * 4096, timed(lambda: gather_logprobs_entropy(lg, lab), iters=10))
+    # its backward: logits read once more, dlogits written in the logits' dtype
+    lg.requires_grad_(True)
+    glp = torch.randn(4096, device=dev)
+
+    def rows_fwd_bwd():
+        lp, _ = gather_logprobs_entropy(lg, lab)
+        lp.backward(glp)
+        lg.grad = None
+
+    t_fb = timed(rows_fwd_bwd, iters=10)
+    add("rows_fwd_kernel + rows_bwd_kernel (API level)",
+        "config 1: [4096, 151936] bf16 logits, forward + backward of the label log-probabilities: "
+        "logits read twice, dlogits written once", lg.numel() * 6 + 32 * 4096, t_fb)
     return out
 
 
