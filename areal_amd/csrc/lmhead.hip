@@ -2334,15 +2334,22 @@ size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t
   return (size_t)elems * 2 + dh_partial_bytes(H, Tc, ldv) + 5 * 256;
 }
 
-// Backward. grad_logprobs [T] fp32 = dLoss/dlogprobs. Writes dhidden [T,H] bf16 and adds the
-// weight gradient into dweight_f32 [V,H] fp32 (overwrites it when accumulate == 0).
+// Backward. grad_logprobs [T] fp32 = dLoss/dlogprobs. Writes dhidden [T,H] bf16 and the weight
+// gradient into dweight [V,H]: fp32, overwritten (accumulate == 0) or added to (accumulate == 1),
+// or bf16 written by the contraction itself (accumulate == 2; one token chunk only, i.e.
+// token_chunk >= T: several chunks need the fp32 sum).
 int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, const float* row_max, const float* sum_exp,
                      const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
-                     float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
+                     float inv_temperature, float logit_scale, void* dhidden, void* dweight,
                      float* dbias, int accumulate, int64_t token_chunk, void* workspace,
                      size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0 || token_chunk <= 0) return AREAL_ERR_BAD_ARG;
+  if (accumulate < 0 || accumulate > 2) return AREAL_ERR_BAD_ARG;
+  // accumulate == 2: dweight is bf16 and written by the contraction itself, which a single chunk allows
+  const bool dw_bf16 = accumulate == 2;
+  if (dw_bf16 && token_chunk < T) return AREAL_ERR_UNSUPPORTED;
+  float* const dweight_f32 = (float*)dweight;
   if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr)
     return AREAL_ERR_BAD_ARG;
   if (dhidden == nullptr && dweight_f32 == nullptr) return AREAL_ERR_BAD_ARG;
@@ -2416,7 +2423,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     // dBias[v] += sum_t dl[t, v]
     if (dbias != nullptr) {
       hipLaunchKernelGGL(colsum_bf16_kernel, dim3((unsigned)ceil_div_i64(V, 64)), dim3(256), 0, stream,
-                         dl, ldv, Tc, (int)V, (accumulate || t0 > 0) ? 1 : 0, nullptr, dbias, nullptr);
+                         dl, ldv, Tc, (int)V, (accumulate == 1 || t0 > 0) ? 1 : 0, nullptr, dbias, nullptr);
       AREAL_CHECK_LAUNCH();
     }
     // 3. dWeight[v, h] += sum_t dl[t, v] * hidden[t, h]
@@ -2424,7 +2431,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
-      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, (accumulate || t0 > 0) ? 2 : 1, stream);
+      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dw_bf16 ? 0 : (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -2434,7 +2441,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
-      rc = launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, (accumulate || t0 > 0) ? 2 : 1, stream);
+      rc = launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, dw_bf16 ? 0 : (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     }
   }

@@ -178,9 +178,12 @@ class _FusedLMHead(torch.autograd.Function):
         if need_b:
             db32 = (torch.zeros if accum is not None else torch.empty)(V, dtype=torch.float32, device=dev)
         probs, probs_ref, probs_status = ctx.probs, ctx.probs_ref, ctx.probs_status
-        # saved mode contracts the whole batch at once and can store dWeight in bf16 directly;
-        # the chunked recompute mode accumulates in fp32 and casts at the end
-        direct = accum is None and probs is not None and T > 0 and ctx.weight_dtype == torch.bfloat16
+        # A contraction over the whole batch can store dWeight in bf16 itself: the saved mode always,
+        # the recompute mode when one token chunk covers the batch. Several chunks accumulate in
+        # fp32 and cast at the end.
+        chunk = (ctx.token_chunk or default_token_chunk(T, H, V)) if T > 0 else 1
+        bf16_out = accum is None and T > 0 and ctx.weight_dtype == torch.bfloat16
+        direct = bf16_out and (probs is not None or chunk >= T)
         dw_direct = torch.empty((V, H), dtype=torch.bfloat16, device=dev) if (need_w and direct) else None
         dw32 = accum
         if accum is None and need_w and not direct:
@@ -214,19 +217,19 @@ class _FusedLMHead(torch.autograd.Function):
             ctx.status_event.synchronize()
             if int(ctx.status_host[0]) != 0:
                 recompute = True
-                if need_w and direct:
+                if need_w and direct and chunk < T:
                     direct, dw_direct = False, None
                     dw32 = torch.empty((V, H), dtype=torch.float32, device=dev)
             del probs, probs_ref
         if recompute:
-            chunk = ctx.token_chunk or default_token_chunk(T, H, V)
             nbytes = lib.areal_lmhead_bwd_workspace_bytes(T, H, V, chunk)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             rc = lib.areal_lmhead_bwd(
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(ctx.bias_f),
                 _lib.ptr(labels_1d), _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
-                _lib.ptr(dh), _lib.ptr(dw32), _lib.ptr(db32), 1 if accum is not None else 0, chunk,
+                _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32), _lib.ptr(db32),
+                2 if direct else (1 if accum is not None else 0), chunk,
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_bwd")

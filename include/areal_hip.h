@@ -65,14 +65,17 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
 
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
 
-/* grad_logprobs [T] fp32. Writes dhidden [T,H] bf16 (NULL to skip) and dweight_f32 [V,H] fp32
- * (NULL to skip; added to when accumulate != 0); dbias [V] fp32 (NULL to skip) = column sums of
- * dlogits (vocab_parallel_head.py:862-863). dlogits are rounded to bf16 before the gradient
+/* grad_logprobs [T] fp32. Writes dhidden [T,H] bf16 (NULL to skip) and dweight [V,H] (NULL to
+ * skip): fp32 overwritten (accumulate 0) or added to (accumulate 1, Megatron's main_grad,
+ * vocab_parallel_head.py:873-879), or bf16 written by the contraction itself (accumulate 2;
+ * only with token_chunk >= T, else AREAL_ERR_UNSUPPORTED: several chunks need the fp32 sum);
+ * dbias [V] fp32 (NULL to skip; added to when accumulate is 1) = column sums of dlogits
+ * (vocab_parallel_head.py:862-863). dlogits are rounded to bf16 before the gradient
  * contractions, as in vocab_parallel_head.py:830-839. */
 int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, const float* row_max, const float* sum_exp,
                      const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
-                     float inv_temperature, float logit_scale, void* dhidden, float* dweight_f32,
+                     float inv_temperature, float logit_scale, void* dhidden, void* dweight,
                      float* dbias, int accumulate, int64_t token_chunk, void* workspace,
                      size_t workspace_bytes, areal_stream_t stream);
 

@@ -62,6 +62,16 @@ def test_workspace_size_queries_run_without_gpu():
     assert lib.areal_actor_loss_workspace_bytes(10, 3) > 0
 
 
+def test_bf16_weight_gradient_needs_a_single_token_chunk():
+    """areal_lmhead_bwd writes dWeight in bf16 itself (accumulate = 2) only when one token chunk
+    covers the batch; the request is refused before anything is launched or read."""
+    lib = _lib.load()
+    fake = 0x10000  # never dereferenced: the argument checks come first
+    args = [fake, fake, None, fake, fake, fake, fake, 512, 64, 1000, 1.0, 1.0, fake, fake, None]
+    assert lib.areal_lmhead_bwd(*args, 2, 256, fake, 1 << 30, None) == _lib.ERR_UNSUPPORTED
+    assert lib.areal_lmhead_bwd(*args, 3, 512, fake, 1 << 30, None) == -1  # bad argument
+
+
 def test_no_cpu_fallback():
     h = torch.randn(4, 8).bfloat16()
     w = torch.randn(16, 8).bfloat16()
