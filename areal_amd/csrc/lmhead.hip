@@ -2211,6 +2211,43 @@ size_t dw_tail_bytes(int64_t H, int64_t V, int64_t Tpad) {
   return t.z > 1 ? (size_t)t.z * (size_t)(t.rows * H) * sizeof(float) + 256 : 0;
 }
 
+// dWeight [V, H] in bf16 = B^T A over the K token rows of the k-major operands g.A [K, H] and
+// g.B [K, ldv]: whole rounds of super-blocks in one launch, then (plan_dw_tail) the remaining
+// vocabulary rows with the token range split, through dw_part (dw_tail_bytes(H, V, K) bytes).
+int launch_dweight_bf16(GemmArgs g, int64_t H, int64_t V, int64_t ldv, void* dweight, float* dw_part,
+                        hipStream_t stream) {
+  const int64_t K = g.K;
+  const DwTail tail = dw_part != nullptr ? plan_dw_tail(H, V, K) : DwTail{0, 1, 0, 0};
+  int rc;
+  if (tail.z <= 1) {
+    const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
+    return launch_store<KERNEL_TN, KERNEL16_TN>(g, plan_regions(H, V, K, 0, 1 << 20), ep, 0, stream);
+  }
+  const int64_t v0 = (int64_t)tail.nbj_main * TILE;
+  GemmArgs gm = g;
+  gm.N = (int)v0;
+  const StoreParams ep{dweight, H, (int)H, (int)v0, nullptr};
+  rc = launch_store<KERNEL_TN, KERNEL16_TN>(gm, plan_regions(H, v0, K, 0, 1 << 20), ep, 0, stream);
+  if (rc != AREAL_OK) return rc;
+  GemmArgs gt = g;
+  gt.B = g.B + v0;
+  gt.N = (int)tail.rows;
+  gt.bcols = (int)(ldv - v0);
+  gt.ksplit = tail.z;
+  gt.kt_per_split = tail.kps;
+  gt.zstride = tail.rows * H * (int64_t)sizeof(float);
+  const StoreParams ept{dw_part, H, (int)H, (int)tail.rows, nullptr};
+  rc = launch_store<KERNEL_TN, KERNEL16_TN>(gt, plan_regions(H, tail.rows, K, 0, 1 << 20), ept, 1, stream);
+  if (rc != AREAL_OK) return rc;
+  int64_t blocks = ceil_div_i64(tail.rows * H, 256 * 4);
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dw_part,
+                     tail.z, tail.rows * H, tail.rows * H, (const float*)nullptr, H,
+                     (u16*)dweight + v0 * H, g.skip_if_set);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
 }  // namespace
 
 // =======================================================================================
@@ -2331,7 +2368,8 @@ size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t
   const bool ragged = (Tc % BK != 0) || (T % Tc) % BK != 0;  // some chunk is not a multiple of 64
   if (ragged) elems += H * ldt + V * ldt;
   // slack for 256-byte sub-buffer alignment
-  return (size_t)elems * 2 + dh_partial_bytes(H, Tc, ldv) + 5 * 256;
+  // (the last term: partial results of the bf16 dWeight store, one chunk covering the batch)
+  return (size_t)elems * 2 + dh_partial_bytes(H, Tc, ldv) + (Tc >= T ? dw_tail_bytes(H, V, Tc) : 0) + 6 * 256;
 }
 
 // Backward. grad_logprobs [T] fp32 = dLoss/dlogprobs. Writes dhidden [T,H] bf16 and the weight
@@ -2379,6 +2417,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
   u16* hT = ragged ? carve(wp, H * ldt * 2) : nullptr;
   u16* dlT = ragged ? carve(wp, V * ldt * 2) : nullptr;
   float* dh_part = dh_partial_bytes(H, Tc_max, ldv) ? (float*)carve(wp, dh_partial_bytes(H, Tc_max, ldv)) : nullptr;
+  float* dw_part = (dw_bf16 && dw_tail_bytes(H, V, Tc_max)) ? (float*)carve(wp, dw_tail_bytes(H, V, Tc_max)) : nullptr;
 
   const float c2 = inv_temperature * LOG2E;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
@@ -2431,7 +2470,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
       const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
-      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dw_bf16 ? 0 : (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
+      rc = dw_bf16 ? launch_dweight_bf16(g, H, V, ldv, dweight, dw_part, stream)
+                   : launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -2528,33 +2568,10 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     // T are cleared)
     GemmArgs g{hs, H, (int)H, e, ldv, (int)V, (int)Tpad, (int)H, (int)ldv};
     g.skip_if_set = probs_status;
-    const DwTail tail = dweight_mode == 2 ? plan_dw_tail(H, V, Tpad) : DwTail{0, 1, 0, 0};
-    if (tail.z > 1) {
-      // whole rounds of super-blocks, then the remaining vocabulary rows with the token range split
-      const int64_t v0 = (int64_t)tail.nbj_main * TILE;
-      g.N = (int)v0;
-      const StoreParams ep{dweight, H, (int)H, (int)v0, nullptr};
-      rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, plan_regions(H, v0, Tpad, 0, 1 << 20), ep, 0, stream);
-      if (rc != AREAL_OK) return rc;
-      GemmArgs gt{hs, H, (int)H, e + v0, ldv, (int)tail.rows, (int)Tpad, (int)H, (int)(ldv - v0)};
-      gt.skip_if_set = probs_status;
-      gt.ksplit = tail.z;
-      gt.kt_per_split = tail.kps;
-      gt.zstride = tail.rows * H * (int64_t)sizeof(float);
-      const StoreParams ept{dw_part, H, (int)H, (int)tail.rows, nullptr};
-      rc = launch_store<KERNEL_TN, KERNEL16_TN>(gt, plan_regions(H, tail.rows, Tpad, 0, 1 << 20), ept, 1, stream);
-      if (rc != AREAL_OK) return rc;
-      int64_t blocks = ceil_div_i64(tail.rows * H, 256 * 4);
-      if (blocks > 65535) blocks = 65535;
-      hipLaunchKernelGGL(splitk_reduce_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, dw_part,
-                         tail.z, tail.rows * H, tail.rows * H, (const float*)nullptr, H,
-                         (u16*)dweight + v0 * H, probs_status);
-      AREAL_CHECK_LAUNCH();
-      return AREAL_OK;
-    }
+    if (dweight_mode == 2) return launch_dweight_bf16(g, H, V, ldv, dweight, dw_part, stream);
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
     const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
-    rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : dweight_mode == 0 ? 1 : 0, stream);
+    rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : 1, stream);
     if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;
