@@ -30,6 +30,7 @@ from areal_amd.ppo.gae import (
     _token_level_gae_with_row_stats,
     compute_gae_lambda,
 )
+from areal_amd.ppo.lambda_fn import resolve_gae_lambda_fn
 
 # areal/utils/constants.py:36-92
 PROX_LOGP_METHOD_RECOMPUTE = "recompute"
@@ -493,7 +494,7 @@ def compute_advantages(
     reward_norm: Normalization | None = None,
     adv_norm: Normalization | None = None,
     discount: float = 1.0,
-    gae_lambda: float | torch.Tensor = 1.0,
+    gae_lambda: float | str | torch.Tensor = 1.0,
     mask_no_eos_with_zero: bool = False,
     use_decoupled_loss: bool = False,
     recompute_logprob: bool = False,
@@ -509,10 +510,11 @@ def compute_advantages(
     """Reward shaping, KL-regularised rewards, token- or turn-level GAE and advantage
     normalisation on a padded ``[bs, L]`` batch; writes ``returns, advantages, kl_rewards,
     tot_rewards, loss_mask, logprobs`` back into ``data`` exactly as ``actor.py:178-323`` does.
-    ``gae_lambda_fn`` (with ``gae_lambda_kwargs``) is a per-sample lambda function
-    ``fn(context, **kwargs) -> [bs] tensor`` such as those of the reference's
-    ``areal/trainer/ppo/lambda_fn.py`` (plain torch on the length context, usable unchanged);
-    without it ``gae_lambda`` is used."""
+    ``gae_lambda`` is a number, a ``[bs]`` tensor, or (as in the reference's configuration,
+    ``actor.py:84-91``) the dotted path of a per-sample lambda function, which
+    ``areal_amd.ppo.lambda_fn.resolve_gae_lambda_fn`` imports; ``gae_lambda_fn`` passes such a
+    function ``fn(context, **kwargs) -> [bs] tensor`` directly.  Either way it is called with
+    ``gae_lambda_kwargs`` on the batch's length context."""
     if gae_timestep_unit not in ("token", "turn"):
         raise ValueError(f"gae_timestep_unit must be 'token' or 'turn', got {gae_timestep_unit!r}")
     if kl_estimator is None:
@@ -620,6 +622,8 @@ def compute_advantages(
     rewards = gae_outcome_rewards if turn_mode else tot_rewards
 
     values = data["values"] if "values" in data else torch.zeros_like(rewards)
+    if gae_lambda_fn is None and isinstance(gae_lambda, (str, bool)):
+        gae_lambda_fn, _ = resolve_gae_lambda_fn(gae_lambda)
     if gae_lambda_fn is not None:
         gae_lambda = compute_gae_lambda(gae_lambda_fn, gae_lambda_kwargs, loss_mask, turn_ids, gae_timestep_unit)
     elif not isinstance(gae_lambda, torch.Tensor):

@@ -301,8 +301,7 @@ def test_turn_level_gae_matches_oracle(dev, bs, L, max_turn_len):
 def test_gae_lambda_context_reference_literals(dev):
     # reference tests/test_ppo_gae.py:279-341, :436-480
     from areal_amd.ppo.gae import _build_gae_lambda_context, compute_gae_lambda
-    from tests.lambda_formulas import relative_position as relative_position_gae_lambda
-    from tests.lambda_formulas import vapo as vapo_length_adaptive_gae
+    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda, vapo_length_adaptive_gae
 
     mask = _t([[1, 1, 1, 1, 0], [1, 1, 0, 0, 0], [0, 0, 0, 0, 0]], dev)
     ids = torch.tensor([[0, 0, 1, 1, -1], [0, 1, -1, -1, -1], [-1, -1, -1, -1, -1]], dtype=torch.int32, device=dev)
@@ -337,7 +336,6 @@ def test_gae_lambda_context_reference_literals(dev):
 def test_compute_advantages_relative_position_lambda_main_path(dev):
     # reference tests/test_ppo_gae.py:406-433: a terminal reward decays as q^((L-k)/(L-1))
     from areal_amd.ppo.actor import compute_advantages
-    from tests.lambda_formulas import relative_position as relative_position_gae_lambda
 
     q, L = 0.3, 10
     batch = {
@@ -347,7 +345,9 @@ def test_compute_advantages_relative_position_lambda_main_path(dev):
         "attention_mask": torch.ones(1, L + 1, dtype=torch.bool, device=dev),
         "rewards": torch.tensor([1.0], device=dev),
     }
-    out = compute_advantages(batch, gae_lambda_fn=relative_position_gae_lambda, gae_lambda_kwargs={"q": q})
+    # the lambda function named by its dotted path, as the reference's configuration does
+    out = compute_advantages(batch, gae_lambda="areal_amd.ppo.lambda_fn.relative_position_gae_lambda",
+                             gae_lambda_kwargs={"q": q})
     want = torch.tensor([[q ** ((L - k) / (L - 1)) for k in range(1, L + 1)] + [0.0]])
     torch.testing.assert_close(out["advantages"].cpu(), want, rtol=1e-6, atol=1e-7)
     torch.testing.assert_close(out["returns"].cpu(), want, rtol=1e-6, atol=1e-7)

@@ -200,22 +200,82 @@ def test_grpo_loss_fn_rejects_out_of_scope_options():
         grpo_loss_fn(z, z, data, 0.2, None, None)
 
 
-def test_gae_lambda_schedules_reference_literals():
-    # the closed forms the reference's tests pin (tests/test_ppo_gae.py:344-403): host logic on
-    # [bs] tensors, here for the test helpers that stand in for areal/trainer/ppo/lambda_fn.py
-    from tests.lambda_formulas import relative_position, vapo
+def _length_context(lengths):
+    return {"effective_token_lengths": lengths, "turn_counts": lengths, "timestep_lengths": lengths}
 
-    def ctx(lengths):
-        return {"effective_token_lengths": lengths, "turn_counts": lengths, "timestep_lengths": lengths}
+
+def test_gae_lambda_schedules_reference_literals():
+    # the values the reference's tests pin for areal/trainer/ppo/lambda_fn.py
+    # (tests/test_ppo_gae.py:279-341 VAPO, :344-390 relative position), on the package's functions
+    from areal_amd.ppo.lambda_fn import (
+        constant_gae_lambda,
+        relative_position_gae_lambda,
+        vapo_length_adaptive_gae,
+    )
 
     q = 0.3
     lengths = torch.tensor([10, 19])
-    lam = relative_position(ctx(lengths), q=q)
+    lam = relative_position_gae_lambda(_length_context(lengths), q=q)
+    assert lam.dtype == torch.float32
     torch.testing.assert_close(lam.pow((lengths - 1).float()), torch.full((2,), q), rtol=1e-6, atol=1e-7)
+    # step 5 of 10 and step 9 of 19 are both at relative position 4 / 9
     torch.testing.assert_close(lam.pow(torch.tensor([5.0, 10.0])), torch.full((2,), q ** (5.0 / 9.0)), rtol=1e-6, atol=1e-7)
-    torch.testing.assert_close(relative_position(ctx(torch.tensor([0, 1, 2])), q=0.3),
+    torch.testing.assert_close(relative_position_gae_lambda(_length_context(torch.tensor([0, 1, 2])), q=0.3),
                                torch.tensor([0.0, 1.0, 0.3]), rtol=0.0, atol=1e-7)
-    assert torch.equal(vapo(ctx(torch.tensor([4, 2, 0])), alpha=1.0), torch.tensor([0.75, 0.5, 0.0]))
+    assert torch.equal(relative_position_gae_lambda(_length_context(torch.tensor([0, 1, 5])), q=1),
+                       torch.tensor([0.0, 1.0, 1.0]))
+    assert torch.equal(vapo_length_adaptive_gae(_length_context(torch.tensor([4, 2, 0])), alpha=1.0),
+                       torch.tensor([0.75, 0.5, 0.0]))
+    # short trajectories: 1 - 1 / (alpha L) < 0 is floored at 0
+    torch.testing.assert_close(vapo_length_adaptive_gae(_length_context(torch.tensor([1, 2, 3, 8])), alpha=0.5),
+                               torch.tensor([0.0, 0.0, 1.0 - 1.0 / 1.5, 0.75]), rtol=1e-6, atol=1e-7)
+    lam = constant_gae_lambda(_length_context(torch.tensor([3, 0, 7])), value=0.95)
+    assert lam.dtype == torch.float32 and torch.equal(lam, torch.full((3,), 0.95))
+
+
+@pytest.mark.parametrize("q", [True, -0.1, 0.0, 1.1, float("nan"), float("inf"), "0.5", None])
+def test_relative_position_gae_lambda_rejects_invalid_q(q):
+    # tests/test_ppo_gae.py:392-403
+    from areal_amd.ppo.lambda_fn import relative_position_gae_lambda
+
+    with pytest.raises(ValueError, match=r"q must be .* in \(0, 1\]"):
+        relative_position_gae_lambda(_length_context(torch.tensor([2])), q=q)
+
+
+@pytest.mark.parametrize("alpha", [0.0, -1.0, True, "1", None, float("nan")])
+def test_vapo_gae_lambda_rejects_non_positive_alpha(alpha):
+    # tests/test_ppo_gae.py:499-508: checked even when every trajectory is empty
+    from areal_amd.ppo.lambda_fn import vapo_length_adaptive_gae
+
+    with pytest.raises(ValueError, match="alpha must be a positive number"):
+        vapo_length_adaptive_gae(_length_context(torch.tensor([0])), alpha=alpha)
+
+
+def test_resolve_gae_lambda_fn():
+    # areal/trainer/ppo/lambda_fn.py:115-141: a number -> the constant schedule (not custom), a
+    # dotted path -> the imported callable (custom), anything else -> TypeError
+    from areal_amd.ppo import lambda_fn as LF
+
+    fn, custom = LF.resolve_gae_lambda_fn(0.9)
+    assert custom is False
+    assert torch.equal(fn(_length_context(torch.tensor([5, 0]))), torch.full((2,), 0.9))
+    fn, custom = LF.resolve_gae_lambda_fn(1)
+    assert custom is False and torch.equal(fn(_length_context(torch.tensor([2]))), torch.ones(1))
+    fn, custom = LF.resolve_gae_lambda_fn("areal_amd.ppo.lambda_fn.vapo_length_adaptive_gae")
+    assert custom is True and fn is LF.vapo_length_adaptive_gae
+    with pytest.raises(TypeError, match="not bool"):
+        LF.resolve_gae_lambda_fn(True)
+    for bad in ("", None, [0.9]):
+        with pytest.raises(TypeError, match="float or a non-empty dotted function path"):
+            LF.resolve_gae_lambda_fn(bad)
+    with pytest.raises(TypeError, match="not callable"):
+        LF.resolve_gae_lambda_fn("areal_amd.ppo.lambda_fn.__all__")
+    with pytest.raises(ValueError, match="Invalid module path"):
+        LF.resolve_gae_lambda_fn("no_dots")
+    with pytest.raises(ImportError, match="Failed to import module"):
+        LF.resolve_gae_lambda_fn("areal_amd.no_such_module.fn")
+    with pytest.raises(AttributeError, match="has no attribute"):
+        LF.resolve_gae_lambda_fn("areal_amd.ppo.lambda_fn.no_such_fn")
 
 
 def test_reward_overlong_penalty_matches_the_reference_loop():

@@ -20,6 +20,8 @@ CASES = [
     ("trainer/ppo/actor.py", "areal_amd.ppo.actor", ["grpo_loss_fn", "compute_prox_logp_approximations"]),
     ("trainer/ppo/gae.py", "areal_amd.ppo.gae",
      ["_compute_token_level_gae", "_compute_turn_level_gae", "_build_gae_lambda_context"]),
+    ("trainer/ppo/lambda_fn.py", "areal_amd.ppo.lambda_fn",
+     ["constant_gae_lambda", "vapo_length_adaptive_gae", "relative_position_gae_lambda", "resolve_gae_lambda_fn"]),
 ]
 
 
