@@ -105,8 +105,19 @@ def _check_lmhead(build_dir: Path) -> None:
     check_accumulator_registers(asm.read_text())
 
 
-def build_all(verbose: bool = True) -> Path:
-    """Compile every ``csrc/*.hip`` for gfx950 and link ``libareal_hip.so``."""
+def _up_to_date(src: Path, obj: Path) -> bool:
+    if not obj.exists():
+        return False
+    deps = [src, CSRC / "common.hpp", Path(__file__)]
+    if src.name == "lmhead.hip":
+        deps.append(CSRC / "mainloop16.inc")
+    return all(obj.stat().st_mtime > d.stat().st_mtime for d in deps)
+
+
+def build_all(verbose: bool = True, incremental: bool = False) -> Path:
+    """Compile every ``csrc/*.hip`` for gfx950 and link ``libareal_hip.so``.  ``incremental``
+    (``python -m areal_amd.build --incremental``, for work on one kernel file) leaves alone the
+    objects that are newer than their source, the shared header and this recipe."""
     build_dir = CSRC / "build"
     build_dir.mkdir(exist_ok=True)
     generate_mainloop()
@@ -114,12 +125,16 @@ def build_all(verbose: bool = True) -> Path:
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC}")
     objs = [build_dir / (s.stem + ".o") for s in srcs]
+    todo = [(s, o) for s, o in zip(srcs, objs) if not (incremental and _up_to_date(s, o))]
     if verbose:
-        print(f"[areal_amd.build] compiling {len(srcs)} HIP sources for gfx950", flush=True)
+        print(f"[areal_amd.build] compiling {len(todo)} of {len(srcs)} HIP sources for gfx950", flush=True)
     with ThreadPoolExecutor(max_workers=min(8, len(srcs) + 1)) as pool:
-        check = pool.submit(_check_lmhead, build_dir)
-        list(pool.map(_compile_one, srcs, objs))
-        check.result()
+        check = None
+        if any(s.name == "lmhead.hip" for s, _ in todo):
+            check = pool.submit(_check_lmhead, build_dir)
+        list(pool.map(lambda so: _compile_one(*so), todo))
+        if check is not None:
+            check.result()
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -132,5 +147,5 @@ def build_all(verbose: bool = True) -> Path:
 
 
 if __name__ == "__main__":
-    build_all()
+    build_all(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

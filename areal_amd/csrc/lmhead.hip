@@ -49,9 +49,19 @@ struct GemmArgs {
   int64_t zstride;
   // When set and the int it points to is non-zero, the launch does nothing (every workgroup
   // returns at once): lets the host queue a launch sequence before it knows a device-side status.
+  // With run_if_set != 0 the sense is inverted: the launch only does something when the int is
+  // non-zero (a fallback queued behind the launch that may raise the status).
   const int* skip_if_set;
+  int run_if_set;
+  // gemm16_sweep, both operands k-contiguous: when M is not a multiple of the tile, the last A tile
+  // is rows [M - 256, M) (it overlaps its predecessor) instead of a ragged tile; the epilogue is
+  // told which of its rows are new. Needs M >= 256.
+  int overlap_last_a;
 };
-DEVI bool gemm_skipped(const GemmArgs& g) { return g.skip_if_set != nullptr && *g.skip_if_set != 0; }
+DEVI bool gate_closed(const int* flag, int run_if_set) {
+  return flag != nullptr && ((*flag != 0) != (run_if_set != 0));
+}
+DEVI bool gemm_skipped(const GemmArgs& g) { return gate_closed(g.skip_if_set, g.run_if_set); }
 
 // Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
 // the 8 XCDs, so the 32 workgroups resident on one XCD are id = xcd + 8*q for 32 consecutive
@@ -821,52 +831,81 @@ template <bool E> using StoreBf16Scaled = StoreEpi<E, 3>;
 
 // Row reference of the saved exponentials e = 2^(c2 x - ref): ref[t] = c2 * (the largest of NREF
 // logits of token t: its label's and a fixed stride sample of the vocabulary) + REF_MARGIN. The
-// estimate never exceeds the row maximum, so the largest exponential of a row is at least
-// 2^-REF_MARGIN and everything within 2^-(126 - REF_MARGIN) of it is a normal bf16 number; the
-// exponentials stay usable while the row maximum is within REF_WINDOW binades above the estimate
-// (largest one 2^(REF_WINDOW - REF_MARGIN), small enough for fp32 accumulation over the
-// vocabulary). lmhead_merge_kernel checks that with the exact row maximum and raises *status
-// otherwise. One wave per token; also clears *status.
+// estimate does not exceed the row maximum (up to rounding), so the largest exponential of a row is
+// at least 2^-REF_MARGIN and everything within 2^-(126 - REF_MARGIN) of it is a normal bf16
+// number. The saving forward takes ALL its sums relative to this reference (no running maximum to
+// rescale by), so a row is only usable while its maximum is within REF_WINDOW binades above the
+// estimate: the largest exponential is then at most 2^(REF_WINDOW - REF_MARGIN), small enough for
+// fp32 accumulation over the vocabulary and for the row factor of the backward (its inverse times
+// the loss gradient) to stay a normal bf16 number. lmhead_merge_kernel checks that with the exact
+// row maximum and raises *status otherwise; the forward then runs again without saving.
+// One wave per REF_TOK tokens (the sampled weight rows are fetched once for all of them), bf16
+// pairs multiplied by v_dot2c_f32_bf16; also clears *status.
 constexpr int NREF = 8;
-constexpr float REF_MARGIN = 60.f;
-constexpr float REF_WINDOW = 150.f;
+constexpr int REF_TOK = 4;
+constexpr float REF_MARGIN = 16.f;
+constexpr float REF_WINDOW = 100.f;
+
+DEVI float dot8_bf16(u32x4 a, u32x4 b, float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // (the elements go through scalars: a bit cast applied to a vector element directly reads
+    // element 0 whatever the index in this toolchain)
+    const uint32_t x = a[i], y = b[i];
+    acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, x), __builtin_bit_cast(bf16x2, y), acc, false);
+  }
+  return acc;
+}
 
 __global__ __launch_bounds__(256) void lmhead_rowref_kernel(
     const u16* __restrict__ hidden, const u16* __restrict__ weight, const float* __restrict__ bias,
     const int64_t* __restrict__ labels, int T, int H, int V, float scale, float c2,
     float* __restrict__ row_ref, int* __restrict__ status) {
   if (blockIdx.x == 0 && threadIdx.x == 0) *status = 0;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int t0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * REF_TOK;
   const int lane = threadIdx.x & 63;
-  if (t >= T) return;
-  int ids[NREF];
+  if (t0 >= T) return;
+  int ids[NREF];  // ids[0]: replaced per token by its label
 #pragma unroll
   for (int k = 0; k < NREF; ++k) ids[k] = (int)(((int64_t)k * V) / NREF);
-  const int64_t lab = labels[t];
-  if (lab >= 0 && lab < V) ids[0] = (int)lab;
-  float acc[NREF];
+  int lab[REF_TOK];
+  const u16* hrow[REF_TOK];
 #pragma unroll
-  for (int k = 0; k < NREF; ++k) acc[k] = 0.f;
-  const u16* hrow = hidden + (int64_t)t * H;
+  for (int j = 0; j < REF_TOK; ++j) {
+    const int t = t0 + j < T ? t0 + j : T - 1;  // a short last group repeats the last token
+    const int64_t l = labels[t];
+    lab[j] = (l >= 0 && l < V) ? (int)l : ids[0];
+    hrow[j] = hidden + (int64_t)t * H;
+  }
+  float acc[REF_TOK][NREF];
+#pragma unroll
+  for (int j = 0; j < REF_TOK; ++j)
+#pragma unroll
+    for (int k = 0; k < NREF; ++k) acc[j][k] = 0.f;
   for (int h = lane * 8; h < H; h += 512) {  // H % 8 == 0
-    const u32x4 hv = *(const u32x4*)(hrow + h);
+    u32x4 wf[NREF];
 #pragma unroll
-    for (int k = 0; k < NREF; ++k) {
-      const u32x4 wv = *(const u32x4*)(weight + (int64_t)ids[k] * H + h);
+    for (int k = 1; k < NREF; ++k) wf[k] = *(const u32x4*)(weight + (int64_t)ids[k] * H + h);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[k] = fmaf(bf16_bits_to_f32((u16)(hv[i] & 0xffffu)), bf16_bits_to_f32((u16)(wv[i] & 0xffffu)), acc[k]);
-        acc[k] = fmaf(bf16_bits_to_f32((u16)(hv[i] >> 16)), bf16_bits_to_f32((u16)(wv[i] >> 16)), acc[k]);
-      }
+    for (int j = 0; j < REF_TOK; ++j) {
+      const u32x4 hv = *(const u32x4*)(hrow[j] + h);
+      const u32x4 lv = *(const u32x4*)(weight + (int64_t)lab[j] * H + h);
+      acc[j][0] = dot8_bf16(hv, lv, acc[j][0]);
+#pragma unroll
+      for (int k = 1; k < NREF; ++k) acc[j][k] = dot8_bf16(hv, wf[k], acc[j][k]);
     }
   }
-  float mx = neg_inf();
 #pragma unroll
-  for (int k = 0; k < NREF; ++k) {
-    const float x = (wave_sum(acc[k]) + (bias != nullptr ? bias[ids[k]] : 0.f)) * scale;
-    mx = fmaxf(mx, x);
+  for (int j = 0; j < REF_TOK; ++j) {
+    float mx = neg_inf();
+#pragma unroll
+    for (int k = 0; k < NREF; ++k) {
+      const int id = k == 0 ? lab[j] : ids[k];
+      const float x = (wave_sum(acc[j][k]) + (bias != nullptr ? bias[id] : 0.f)) * scale;
+      mx = fmaxf(mx, x);
+    }
+    if (lane == 0 && t0 + j < T) row_ref[t0 + j] = fmaf(mx, c2, REF_MARGIN);
   }
-  if (lane == 0) row_ref[t] = fmaf(mx, c2, REF_MARGIN);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1060,19 +1099,23 @@ template <bool E> using FwdAffineMomSave = FwdEpi<E, true, true, true>;
 // MERGE_WAVES waves; wave w takes slots w, w + MERGE_WAVES, ... (loads stay coalesced along the
 // tokens, and a launch with few tokens and many slots still has enough threads in flight), the
 // partial results meet in LDS and wave 0 adds them in a fixed order.
+// ref_sums: the slots' sums S, Q are relative to row_ref[t] (the saving forward of the
+// hand-scheduled kernels) instead of to each slot's own maximum; the final expressions are then
+// evaluated in fp64, where c2 x - ref and log S (each up to REF_WINDOW binades) cancel.
+// gate / gate_run_if_set: as GemmArgs::skip_if_set / run_if_set.
 constexpr int MERGE_WAVES = 8;
 __global__ __launch_bounds__(64 * MERGE_WAVES) void lmhead_merge_kernel(
-    const float* __restrict__ ws, int P, int T, int V, float inv_temp, float c2,
+    const float* __restrict__ ws, int P, int T, int V, int ref_sums, float c2,
     float* __restrict__ logprobs, float* __restrict__ entropy, float* __restrict__ vmin,
     float* __restrict__ vmax, float* __restrict__ vmean, float* __restrict__ vnorm,
     float* __restrict__ row_max, float* __restrict__ sum_exp, const float* __restrict__ row_ref,
-    int* __restrict__ status) {
+    int* __restrict__ status, const int* __restrict__ gate, int gate_run_if_set) {
+  if (gate_closed(gate, gate_run_if_set)) return;
   __shared__ float sh_f[5][MERGE_WAVES][64];   // max, S, Q, label logit, min
   __shared__ double sh_d[2][MERGE_WAVES][64];  // sum x, sum x^2
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 64 + lane;
   const int tt = t < T ? t : T - 1;  // lanes past the end repeat the last token and write nothing
-  (void)inv_temp;  // c2 = inv_temp * log2(e) carries it
   const int64_t PT = (int64_t)P * T;
   const bool moments = vmean != nullptr || vnorm != nullptr;
   float M = neg_inf();
@@ -1086,7 +1129,10 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void lmhead_merge_kernel(
   for (int p = wv; p < P; p += MERGE_WAVES) {
     const float* w = ws + (int64_t)p * T + tt;
     const float m = w[0];
-    if (m > neg_inf()) {
+    if (ref_sums) {
+      S += w[1 * PT];
+      Q += w[2 * PT];
+    } else if (m > neg_inf()) {
       const float dl = ref_diff(m, M, c2);  // as in the epilogue
       const float alpha = exp2f(dl);
       S += alpha * w[1 * PT];
@@ -1107,23 +1153,38 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void lmhead_merge_kernel(
     mn = fminf(mn, sh_f[4][i][lane]);
     sx += sh_d[0][i][lane]; sx2 += sh_d[1][i][lane];
   }
-  const float logS = logf(S);
-  // label exponent against the same rounded reference the sums use. For a label inside the
-  // vocabulary (xl <= M) the result is <= 0 in exact arithmetic; the last rounding may leave
-  // +1e-8 when p = 1 to fp32 precision.
-  if (logprobs) {
-    const float lp = fmaf(xl, c2, -ref_of(M, c2)) * LN2 - logS;
-    logprobs[t] = xl <= M ? fminf(lp, 0.f) : lp;
+  if (ref_sums) {
+    const double ln2 = 0.6931471805599453094;
+    const double rr = (double)row_ref[t];
+    const double lnS = log((double)S);
+    if (logprobs) {
+      const float lp = (float)(((double)xl * (double)c2 - rr) * ln2 - lnS);
+      logprobs[t] = xl <= M ? fminf(lp, 0.f) : lp;
+    }
+    if (entropy) entropy[t] = (float)(lnS - ln2 * (double)Q / (double)S);
+    // what the backward kernels expect: the sum relative to the rounded product fl(c2 * max)
+    if (sum_exp) sum_exp[t] = (float)((double)S * exp2(rr - (double)ref_of(M, c2)));
+    // usable only if the row maximum was inside the window (then no sum overflowed either)
+    if (!(fmaf(M, c2, -row_ref[t]) <= REF_WINDOW - REF_MARGIN) || !(S < pos_inf())) atomicMax(status, 1);
+  } else {
+    const float logS = logf(S);
+    // label exponent against the same rounded reference the sums use. For a label inside the
+    // vocabulary (xl <= M) the result is <= 0 in exact arithmetic; the last rounding may leave
+    // +1e-8 when p = 1 to fp32 precision.
+    if (logprobs) {
+      const float lp = fmaf(xl, c2, -ref_of(M, c2)) * LN2 - logS;
+      logprobs[t] = xl <= M ? fminf(lp, 0.f) : lp;
+    }
+    if (entropy) entropy[t] = logS - (Q * LN2) / S;
+    if (sum_exp) sum_exp[t] = S;
+    // the saved exponentials of this row are usable if its largest one is at most 2^(window - margin)
+    if (row_ref != nullptr && !(fmaf(M, c2, -row_ref[t]) <= REF_WINDOW - REF_MARGIN)) atomicMax(status, 1);
   }
-  if (entropy) entropy[t] = logS - (Q * LN2) / S;
   if (vmin) vmin[t] = mn;
   if (vmax) vmax[t] = M;
   if (vmean) vmean[t] = (float)(sx / (double)V);
   if (vnorm) vnorm[t] = (float)sqrt(sx2);
   if (row_max) row_max[t] = M;
-  if (sum_exp) sum_exp[t] = S;
-  // the saved exponentials of this row are usable if its largest one is at most 2^(window - margin)
-  if (row_ref != nullptr && !(fmaf(M, c2, -row_ref[t]) <= REF_WINDOW - REF_MARGIN)) atomicMax(status, 1);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1412,16 +1473,16 @@ enum { VAR_NT = 0, VAR_TN = 1, VAR_MIX = 2 };
 DEVI int swz16(int r) { return r & 7; }
 
 // Per-lane byte offsets of the 8 direct loads of one operand half, and the LDS read addresses
-// (stage 0) of its fragments. KM: k-major operand (`tile` = its 256-column tile, nvalid = readable
-// columns); otherwise k-contiguous (nvalid = rows).
+// (stage 0) of its fragments. KM: k-major operand (`first` = its 256-column tile, nvalid = readable
+// columns); otherwise k-contiguous (`first` = the tile's first row, nvalid = rows).
 template <bool KM>
-DEVI void setup_operand16(int64_t ld, int tile, int nvalid, int W, int oper, int wave, int lane,
+DEVI void setup_operand16(int64_t ld, int first, int nvalid, int W, int oper, int wave, int lane,
                           uint32_t lds_base, uint32_t (&off)[8], uint32_t (&rd)[8]) {
   if (!KM) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int r = wave * 64 + i * 8 + (lane >> 3);
-      const int rr = tile * TILE + r < nvalid ? r : nvalid - 1 - tile * TILE;  // clamped rows are discarded later
+      const int rr = first + r < nvalid ? r : nvalid - 1 - first;  // clamped rows are discarded later
       off[i] = 2u * ((uint32_t)rr * (uint32_t)ld + (uint32_t)(((lane & 7) ^ swz16(r)) * 8));
     }
     const int rl = lane & 15, kg = lane >> 4, sw = swz16(rl);
@@ -1436,7 +1497,7 @@ DEVI void setup_operand16(int64_t ld, int tile, int nvalid, int W, int oper, int
     for (int i = 0; i < 8; ++i) {
       const int kr = wave * 16 + 2 * i + hl;
       const int k3 = kr & 3, cf = ((kr >> 3) & 1) * 2;
-      int gp = tile * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + ((piece & 3) ^ cf);
+      int gp = first * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + ((piece & 3) ^ cf);
       const int last = nvalid / 8 - 1;
       gp = gp < last ? gp : last;  // columns past the end are discarded later
       off[i] = 2u * ((uint32_t)kr * (uint32_t)ld + (uint32_t)(gp * 8));
@@ -1450,9 +1511,11 @@ DEVI void setup_operand16(int64_t ld, int tile, int nvalid, int W, int oper, int
 }
 
 // A workgroup sweeps the A tiles [ai_begin, ai_end) against one B tile. Requirements checked by
-// the host: K % 128 == 0; a sweep of more than one A tile has only full A tiles and a
-// k-contiguous A (the loader's lane offsets are those of the first tile); split-K ranges are an
-// even number of k-tiles.
+// the host: K % 128 == 0; a sweep of more than one A tile has only full A tiles (a ragged last one
+// as rows [M - 256, M), see GemmArgs::overlap_last_a) and a k-contiguous A (the loader's lane
+// offsets are those of the first tile); split-K ranges are an even number of k-tiles.
+// Epi::tile gets the first row of the tile's sub-block of this wave and, last, the first row of the
+// tile that no earlier tile of the sweep covered.
 template <int VAR, class Epi>
 __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, typename Epi::Params ep) {
   __shared__ __attribute__((aligned(1024))) unsigned char lds[RING16_BYTES + 4 * STAGE16_BYTES];
@@ -1480,16 +1543,22 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
   const int wa = wave >> 1, wb = wave & 1;
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_AS(lds);
 
+  // first row of A tile ai (k-contiguous A): the last tile of a ragged M may overlap its predecessor
+  auto a_row0 = [&](int ai) -> int {
+    const int r = ai * TILE;
+    return (VAR == VAR_NT && g.overlap_last_a != 0 && r + TILE > g.M) ? g.M - TILE : r;
+  };
   uint32_t oa[8], ob[8], ra[8], rb[8];
-  setup_operand16<A_KM>(g.lda, ai_begin, A_KM ? g.acols : g.M, wa, 0, wave, lane, lds_base, oa, ra);
-  setup_operand16<B_KM>(g.ldb, bj, B_KM ? g.bcols : g.N, wb, 1, wave, lane, lds_base, ob, rb);
+  setup_operand16<A_KM>(g.lda, A_KM ? ai_begin : a_row0(ai_begin), A_KM ? g.acols : g.M, wa, 0, wave, lane,
+                        lds_base, oa, ra);
+  setup_operand16<B_KM>(g.ldb, B_KM ? bj : bj * TILE, B_KM ? g.bcols : g.N, wb, 1, wave, lane, lds_base, ob, rb);
 
   // pointers to the next k-tile to fetch and their advance per k-tile in bytes. A k-major
   // operand's tile column is part of the lane offsets, so its pointer only carries the k offset.
   const uint32_t stride_a = A_KM ? (uint32_t)(BK * g.lda * 2) : 128u;
   const uint32_t stride_b = B_KM ? (uint32_t)(BK * g.ldb * 2) : 128u;
   auto a_tile_ptr = [&](int ai) -> const char* {
-    return (const char*)(A_KM ? g.A : g.A + (int64_t)ai * TILE * g.lda);
+    return (const char*)(A_KM ? g.A : g.A + (int64_t)a_row0(ai) * g.lda);
   };
   const char* pa = a_tile_ptr(ai_begin);
   const char* pb = (const char*)(B_KM ? g.B : g.B + (int64_t)bj * TILE * g.ldb);
@@ -1553,7 +1622,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
     Epi::open(st, ep, bj * TILE + wb * 128, split, wa, lane_e, ai == ai_begin);
-    Epi::tile(st, ep, ai * TILE + wa * 128, bj * TILE + wb * 128, lane_e, stage);
+    Epi::tile(st, ep, a_row0(ai) + wa * 128, bj * TILE + wb * 128, lane_e, stage, ai * TILE);
     Epi::close(st, ep, bj * TILE + wb * 128, split, wa, lane_e);
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
@@ -1566,14 +1635,16 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
 // STREAM: the output is a [T, V]-sized buffer that nothing reads before the kernel ends; its
 // stores carry the non-temporal hint so that they do not push the operand tiles the XCD's other
 // workgroups share out of L2.
+// EDGE: only rows < rows_valid and columns [cols_from, cols_valid) are written (both multiples of 8).
 template <bool EDGE, bool STREAM = false>
-DEVI void flush_stage16(const u16* stage, u16* out_row0, int64_t ld, int rows_valid, int cols_valid, int lane) {
+DEVI void flush_stage16(const u16* stage, u16* out_row0, int64_t ld, int rows_valid, int cols_valid,
+                        int cols_from, int lane) {
   const int piece = lane & 15;
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = p * 4 + (lane >> 4);
     const u32x4 v = *(const u32x4*)((const char*)stage + row * STAGE16_PITCH + piece * 16);
-    if (!EDGE || (row < rows_valid && piece * 8 < cols_valid)) {
+    if (!EDGE || (row < rows_valid && piece * 8 < cols_valid && piece * 8 >= cols_from)) {
       u32x4* dst = (u32x4*)(out_row0 + (int64_t)row * ld + piece * 8);
       if (STREAM) __builtin_nontemporal_store(v, dst);
       else *dst = v;
@@ -1593,7 +1664,7 @@ struct Store16 {
   static DEVI void close(State&, const Params&, int, int, int, int) {}
   static DEVI void end(State&, const Params&, int, int, int, int) {}
   static DEVI void split_output(Params& p, int64_t bytes) { p.out = (char*)p.out + bytes; }
-  static DEVI void tile(State&, const Params& p, int i0, int j0, int lane, u16* stage) {
+  static DEVI void tile(State&, const Params& p, int i0, int j0, int lane, u16* stage, int) {
     for_each_col([&](auto bc) {
       constexpr int b = decltype(bc)::value;
       float x[32];
@@ -1614,7 +1685,7 @@ struct Store16 {
           stage16_put(stage, lane, a, v);
         }
         flush_stage16<EDGE>(stage, (u16*)p.out + (int64_t)(j0 + b * 16) * p.ldo + i0, p.ldo,
-                            p.N - (j0 + b * 16), p.M - i0, lane);
+                            p.N - (j0 + b * 16), p.M - i0, 0, lane);
       } else {
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
@@ -1679,9 +1750,15 @@ DEVI float group_sum(float v) {
   return a + b;
 }
 
+// A logit that takes no part (past the vocabulary, or a row that an earlier tile of the sweep
+// already covered): far below every real logit, finite so that 0 * it stays 0 in the entropy sum.
+constexpr float MASKED_LOGIT = -1e30f;
+
 template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
 struct Fwd16 {
   typedef FwdParams Params;
+  // SAVE: s and q are relative to the row reference of the saved exponentials (fixed for the whole
+  // sweep: nothing is rescaled); otherwise relative to the running maximum m.
   struct State {
     float m[2], s[2], q[2], xl[2], mn[2], sx[MOMENTS ? 2 : 1], sx2[MOMENTS ? 2 : 1];
   };
@@ -1697,7 +1774,11 @@ struct Fwd16 {
   }
   static DEVI void close(State&, const Params&, int, int, int, int) {}
 
-  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
+  // v_new: the first vocabulary entry of the tile that no earlier tile of the sweep covered (the
+  // last tile of a ragged vocabulary overlaps its predecessor); entries below it take no part.
+  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage, int v_new) {
+    if (v_new >= v0 + 128) return;    // every row of this wave's sub-tile is a repeat
+    const bool overlap = v_new > v0;  // wave-uniform
     const int vl = v0 + 4 * (lane >> 4);
     const int group = lane >> 4;
     auto vidx = [&](int a, int r) { return vl + a * 16 + r; };
@@ -1709,7 +1790,7 @@ struct Fwd16 {
       const int t = t0 + b * 16 + (lane & 15);
       const bool live = !EDGE || t < p.T;
       const int64_t l = live ? p.labels[t] : -1;
-      lab[b] = (l >= 0 && l < p.V) ? (int)l : -1;
+      lab[b] = (l >= v_new && l < p.V) ? (int)l : -1;
       if (SAVE) rr[b] = live ? p.probs_ref[t] : 0.f;
     }
     ML16_AGPR_FENCE();
@@ -1729,55 +1810,62 @@ struct Fwd16 {
           }
       }
       float tmax = neg_inf(), tmin = pos_inf(), sx = 0.f, sx2 = 0.f;
+      if (!EDGE && !overlap) {
 #pragma unroll
-      for (int a = 0; a < 8; ++a) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float xv = x[a * 4 + r];
-          if (!EDGE || vidx(a, r) < p.V) {
-            tmax = fmaxf(tmax, xv);
-            tmin = fminf(tmin, xv);
-            if (MOMENTS) { sx += xv; sx2 = fmaf(xv, xv, sx2); }
-          }
+        for (int i = 0; i < 32; ++i) {
+          tmax = fmaxf(tmax, x[i]);
+          tmin = fminf(tmin, x[i]);
+          if (MOMENTS) { sx += x[i]; sx2 = fmaf(x[i], x[i], sx2); }
         }
+      } else {
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float xv = x[a * 4 + r];
+            if ((!EDGE || vidx(a, r) < p.V) && vidx(a, r) >= v_new) {
+              tmax = fmaxf(tmax, xv);
+              tmin = fminf(tmin, xv);
+              if (MOMENTS) { sx += xv; sx2 = fmaf(xv, xv, sx2); }
+            } else {
+              x[a * 4 + r] = MASKED_LOGIT;
+            }
+          }
       }
-      // the column's reference: the maximum over the token's 128 entries in this sub-tile (see
-      // ref_of); -inf only if every entry lies past the vocabulary
-      tmax = group_max(tmax);
-      const float mc = (!EDGE || tmax > neg_inf()) ? ref_of(tmax, p.c2) : 0.f;
-      ML16_AGPR_FENCE();
       float s = 0.f, q = 0.f;
       if (!SAVE) {
+        // the column's reference: the maximum over the token's 128 entries in this sub-tile (see
+        // ref_of); -inf only if every entry lies past the vocabulary
+        tmax = group_max(tmax);
+        const float mc = (!EDGE || tmax > neg_inf()) ? ref_of(tmax, p.c2) : 0.f;
+        ML16_AGPR_FENCE();
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float t = fmaf(x[a * 4 + r], p.c2, -mc);
             const float e = fast_exp2(t);
-            if (!EDGE || vidx(a, r) < p.V) { s += e; q = fmaf(t, e, q); }
+            s += e;
+            q = fmaf(t, e, q);
           }
           __builtin_amdgcn_sched_barrier(0);
           ML16_AGPR_FENCE();
         }
       } else {
-        // What is stored is the exponential relative to the column's maximum (in (0, 1]) moved to
-        // the row reference by one factor per (token, column). That factor over- or underflows
-        // only where the stored value is not used: rows outside the reference window, and columns
-        // whose maximum lies 126 binades below the row's. The 16 tokens x 128 entries of the
-        // column go through the staging area and leave as whole lines.
-        const float gamma = fast_exp2(mc - rr[b]);
+        // Exponentials relative to the row reference, summed and stored as they are: one fma, one
+        // v_exp_f32, two sums and half a packed conversion per logit. The 16 tokens x 128 entries of
+        // the column go through the staging area and leave as whole lines.
+        const float nr = -rr[b];
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
-          const int vq = vl + a * 16;
           float d[4];
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
-            const float t = fmaf(x[a * 4 + e4], p.c2, -mc);
+            const float t = fmaf(x[a * 4 + e4], p.c2, nr);
             const float e = fast_exp2(t);
-            float es = e * gamma;
-            if (EDGE && vq + e4 >= p.V) es = 0.f;
-            else { s += e; q = fmaf(t, e, q); }
-            d[e4] = es;
+            s += e;
+            q = fmaf(t, e, q);
+            d[e4] = e;
           }
           u32x2 pk;
           pk[0] = pack_bf16x2(d[0], d[1]);
@@ -1788,8 +1876,12 @@ struct Fwd16 {
           __builtin_amdgcn_sched_barrier(0);
           ML16_AGPR_FENCE();
         }
-        flush_stage16<EDGE, true>(stage, p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv,
-                            p.T - (t0 + b * 16), (int)p.ldv - v0, lane);
+        u16* out = p.probs + (int64_t)(t0 + b * 16) * p.ldv + v0;
+        if (!EDGE && !overlap)
+          flush_stage16<false, true>(stage, out, p.ldv, 16, 128, 0, lane);
+        else
+          flush_stage16<true, true>(stage, out, p.ldv, EDGE ? p.T - (t0 + b * 16) : 16, (int)p.ldv - v0,
+                                    overlap ? v_new - v0 : 0, lane);
       }
       // the label's logit, if it is one of this lane's 32 entries
       float xl = 0.f;
@@ -1809,22 +1901,29 @@ struct Fwd16 {
       q = group_sum(q);
       tmin = group_min(tmin);
       xl = group_sum(xl);
+      if (SAVE) tmax = group_max(tmax);
       if (MOMENTS) {
         asm volatile("" : "+v"(sx), "+v"(sx2));
         sx = group_sum(sx);
         sx2 = group_sum(sx2);
       }
-      // lane group b % 4 folds the column into the running statistics of token column b: both
-      // sets of sums move to the reference of the larger maximum
+      // lane group b % 4 folds the column into the running statistics of token column b
       if (group == (b & 3)) {
-        const float m_old = st.m[k];
-        const float m_new = fmaxf(m_old, tmax);
-        const float d_old = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
-        const float d_col = (!EDGE || tmax > neg_inf()) ? ref_diff(tmax, m_new, p.c2) : 0.f;
-        const float a_old = fast_exp2(d_old), a_col = fast_exp2(d_col);
-        st.q[k] = a_old * fmaf(d_old, st.s[k], st.q[k]) + a_col * fmaf(d_col, s, q);
-        st.s[k] = a_old * st.s[k] + a_col * s;
-        st.m[k] = m_new;
+        if (SAVE) {
+          st.s[k] += s;
+          st.q[k] += q;
+          st.m[k] = fmaxf(st.m[k], tmax);
+        } else {
+          // both sets of sums move to the reference of the larger maximum
+          const float m_old = st.m[k];
+          const float m_new = fmaxf(m_old, tmax);
+          const float d_old = (m_old > neg_inf()) ? ref_diff(m_old, m_new, p.c2) : 0.f;
+          const float d_col = (!EDGE || tmax > neg_inf()) ? ref_diff(tmax, m_new, p.c2) : 0.f;
+          const float a_old = fast_exp2(d_old), a_col = fast_exp2(d_col);
+          st.q[k] = a_old * fmaf(d_old, st.s[k], st.q[k]) + a_col * fmaf(d_col, s, q);
+          st.s[k] = a_old * st.s[k] + a_col * s;
+          st.m[k] = m_new;
+        }
         st.mn[k] = fminf(st.mn[k], tmin);
         st.xl[k] += xl;
         if (MOMENTS) { st.sx[k] += sx; st.sx2[k] += sx2; }
@@ -1885,7 +1984,8 @@ struct Bwd16 {
   static DEVI void end(State&, const Params&, int, int, int, int) {}
   static DEVI void split_output(Params&, int64_t) {}
 
-  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage) {
+  // (a tile that overlaps its predecessor rewrites the shared rows with the same values)
+  static DEVI void tile(State& st, const Params& p, int v0, int t0, int lane, u16* stage, int) {
     const int vl = v0 + 4 * (lane >> 4);
     for_each_col([&](auto bc) {
       constexpr int b = decltype(bc)::value;
@@ -1919,7 +2019,7 @@ struct Bwd16 {
         stage16_put(stage, lane, a, pk);
       }
       flush_stage16<EDGE, true>(stage, p.dl + (int64_t)(t0 + b * 16) * p.ldv + v0, p.ldv, p.T - (t0 + b * 16),
-                          (int)p.ldv - v0, lane);
+                          (int)p.ldv - v0, 0, lane);
     });
   }
 };
@@ -1993,11 +2093,21 @@ struct Regions {
   bool ragged_a, ragged_b;
   int S;                   // splits used for the interior and the ragged-B launch
   bool k16;                // K suits the hand-scheduled main loop (callers may still clear it)
+  bool fold_a;             // the ragged last A tile runs as rows [M - 256, M) at the end of the last
+                           // split's sweep (GemmArgs::overlap_last_a) instead of a launch of its own;
+                           // set by fold_ragged_a() for the epilogues that support it
 };
+// The hand-scheduled forward and recompute launches take a ragged last vocabulary tile into the
+// main launch when there is a full tile for it to overlap and whole 64-column groups (the stores
+// of the saved buffers are 16-byte pieces, and columns [V, round_up(V, 64)) would stay unwritten).
+void fold_ragged_a(Regions& r, int64_t M) {
+  r.fold_a = r.fast && r.k16 && r.ragged_a && r.nai_full >= 1 && M % BK == 0;
+}
 Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixed) {
   Regions r;
   r.fast = (K > 0 && K % BK == 0);
   r.k16 = k16_ok(K);
+  r.fold_a = false;
   if (r.fast) {
     r.nai_full = (int)(M / TILE); r.nbj_full = (int)(N / TILE);
     r.ragged_a = (M % TILE) != 0; r.ragged_b = (N % TILE) != 0;
@@ -2030,12 +2140,17 @@ int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_ed
     return launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), 0, nai,
                                                   r.S == r.nai_full ? nai : r.S, ep, stream);
   }
-  if ((rc = launch_region<EpiT<false>, FAST_KERNEL>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+  GemmArgs gm = g;
+  int nai_main = r.nai_full;
+  if constexpr (FAST_KERNEL == KERNEL16_NT) {
+    if (r.fold_a) { gm.overlap_last_a = 1; ++nai_main; }
+  }
+  if ((rc = launch_region<EpiT<false>, FAST_KERNEL>(gm, 0, r.nbj_full, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_b &&
-      (rc = launch_region<EpiT<true>, FAST_KERNEL>(g, r.nbj_full, 1, 0, r.nai_full, r.S, ep, stream)) != AREAL_OK)
+      (rc = launch_region<EpiT<true>, FAST_KERNEL>(gm, r.nbj_full, 1, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
     return rc;
-  if (r.ragged_a &&
+  if (r.ragged_a && nai_main == r.nai_full &&
       (rc = launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
                                                    ep_edge_a, stream)) != AREAL_OK)
     return rc;
@@ -2052,7 +2167,7 @@ int check_operand(const void* p, int64_t ld) {
 // the vocabulary range, 2 wave rows x (in the 32x32 kernels) the 2 lane groups that share a
 // token; the hand-scheduled kernels combine their 4 lane groups in registers.
 int fwd_slots_per_split(const Regions& r) { return r.k16 ? 2 : 4; }
-int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + (r.ragged_a ? 1 : 0)); }
+int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + ((r.ragged_a && !r.fold_a) ? 1 : 0)); }
 
 // The four plain-store epilogues over either family of kernels. mode: 0 bf16, 1 fp32,
 // 2 fp32 accumulate, 3 bf16 with a factor per output row. The hand-scheduled kernels write bf16
@@ -2275,7 +2390,11 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   return launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, out_mode, stream);
 }
 
-static Regions fwd_regions(int64_t T, int64_t H, int64_t V) { return plan_regions(V, T, H, 512, 0); }
+static Regions fwd_regions(int64_t T, int64_t H, int64_t V) {
+  Regions r = plan_regions(V, T, H, 512, 0);
+  fold_ragged_a(r, V);
+  return r;
+}
 
 size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T <= 0 || V <= 0 || H <= 0) return 0;
@@ -2291,8 +2410,9 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // for areal_lmhead_bwd_saved: probs bf16 [round_up(T, 128)][round_up(V, 64)] (rows >= T are not
 // written) holds e = 2^(c2 x - probs_ref[t]); probs_ref fp32 [T] is a per-row reference taken
 // from a few logits of the row before the sweep; *probs_status (one int) is set to 0 when every
-// row's exponentials are in range and to 1 when some row's maximum lies more than 150 binades
-// above its estimate: then probs must not be used and the backward has to recompute.
+// row's exponentials are in range and to 1 when some row's maximum lies more than REF_WINDOW
+// binades above its estimate: then probs must not be used and the backward has to recompute
+// (the per-token outputs are right either way).
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
@@ -2321,38 +2441,61 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
   ep_a.slot_base = fwd_slots_per_split(r) * r.S;
   const bool affine = (logit_scale != 1.0f) || (bias != nullptr);
   const bool moments = (vocab_mean != nullptr) || (vocab_norm != nullptr);
+  const float c2 = inv_temperature * LOG2E;
   if (probs != nullptr) {
-    hipLaunchKernelGGL(lmhead_rowref_kernel, dim3((unsigned)ceil_div_i64(T, 4)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(lmhead_rowref_kernel, dim3((unsigned)ceil_div_i64(T, 4 * REF_TOK)), dim3(256), 0, stream,
                        (const u16*)hidden, (const u16*)weight, bias, labels, (int)T, (int)H, (int)V,
-                       logit_scale, inv_temperature * LOG2E, probs_ref, probs_status);
+                       logit_scale, c2, probs_ref, probs_status);
     AREAL_CHECK_LAUNCH();
   }
+  auto fwd16_plain = [&](const GemmArgs& gg) {
+    if (!affine && !moments) return launch_gemm<Fwd16Plain, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!affine) return launch_gemm<Fwd16PlainMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!moments) return launch_gemm<Fwd16Affine, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    return launch_gemm<Fwd16AffineMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+  };
+  auto merge = [&](int ref_sums, const float* ref, const int* gate, int gate_run_if_set) {
+    hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, 64)), dim3(64 * MERGE_WAVES),
+                       0, stream, (const float*)workspace, P, (int)T, (int)V, ref_sums, c2, logprobs,
+                       entropy, vocab_min, vocab_max, vocab_mean, vocab_norm, row_max, sum_exp, ref,
+                       probs_status, gate, gate_run_if_set);
+  };
   if (r.k16 && probs == nullptr) {
-    if (!affine && !moments) rc = launch_gemm<Fwd16Plain, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else if (!affine) rc = launch_gemm<Fwd16PlainMom, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else if (!moments) rc = launch_gemm<Fwd16Affine, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else rc = launch_gemm<Fwd16AffineMom, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
+    if ((rc = fwd16_plain(g)) != AREAL_OK) return rc;
+    merge(0, nullptr, nullptr, 0);
   } else if (r.k16) {
+    // The saving sweep takes its sums relative to the row references, which is only right for rows
+    // whose maximum is within the window above the estimate. The merge raises *probs_status if
+    // some row is outside; the plain sweep and its merge are queued behind it and do their work
+    // only in that case (otherwise every workgroup of them returns at once), so the outputs are
+    // right either way without the host looking at the status in between.
     if (!affine && !moments) rc = launch_gemm<Fwd16PlainSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
     else if (!affine) rc = launch_gemm<Fwd16PlainMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
     else if (!moments) rc = launch_gemm<Fwd16AffineSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
     else rc = launch_gemm<Fwd16AffineMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-  } else if (probs == nullptr) {
-    if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
-    else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
-    else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
-    else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
+    if (rc != AREAL_OK) return rc;
+    merge(1, probs_ref, nullptr, 0);
+    AREAL_CHECK_LAUNCH();
+    GemmArgs gf = g;
+    gf.skip_if_set = probs_status;
+    gf.run_if_set = 1;
+    if ((rc = fwd16_plain(gf)) != AREAL_OK) return rc;
+    merge(0, nullptr, probs_status, 1);
   } else {
-    if (!affine && !moments) rc = launch_gemm<FwdPlainSave>(g, r, ep, ep_a, stream);
-    else if (!affine) rc = launch_gemm<FwdPlainMomSave>(g, r, ep, ep_a, stream);
-    else if (!moments) rc = launch_gemm<FwdAffineSave>(g, r, ep, ep_a, stream);
-    else rc = launch_gemm<FwdAffineMomSave>(g, r, ep, ep_a, stream);
+    if (probs == nullptr) {
+      if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
+      else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
+      else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
+      else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
+    } else {
+      if (!affine && !moments) rc = launch_gemm<FwdPlainSave>(g, r, ep, ep_a, stream);
+      else if (!affine) rc = launch_gemm<FwdPlainMomSave>(g, r, ep, ep_a, stream);
+      else if (!moments) rc = launch_gemm<FwdAffineSave>(g, r, ep, ep_a, stream);
+      else rc = launch_gemm<FwdAffineMomSave>(g, r, ep, ep_a, stream);
+    }
+    if (rc != AREAL_OK) return rc;
+    merge(0, probs_ref, nullptr, 0);
   }
-  if (rc != AREAL_OK) return rc;
-  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, 64)), dim3(64 * MERGE_WAVES),
-                     0, stream, (const float*)workspace, P, (int)T, (int)V, inv_temperature,
-                     inv_temperature * LOG2E, logprobs, entropy, vocab_min, vocab_max, vocab_mean,
-                     vocab_norm, row_max, sum_exp, (const float*)probs_ref, probs_status);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -2441,7 +2584,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H, 0, 0};
       BwdParams ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
                    (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
-      const Regions r = plan_regions(V, Tc, H, 512, 0);
+      Regions r = plan_regions(V, Tc, H, 512, 0);
+      if (!need_dlT) fold_ragged_a(r, V);
       if (need_dlT)
         rc = affine ? launch_gemm<BwdAffineT>(g, r, ep, ep, stream)
                     : launch_gemm<BwdPlainT>(g, r, ep, ep, stream);

@@ -216,8 +216,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_rs_kernel(LossIO io, LossCfg
 
 // Rejection sampling for one token. Returns the narrowed mask; sets w (not yet zeroed outside
 // the mask) and whether the token counts as filtered / clamped.
-DEVI bool rs_token(const LossIO& io, const LossCfg& c, int64_t t, bool m, float& w, bool& counted) {
-  const float prox = io.prox[t], old = io.old[t];
+DEVI bool rs_token(const LossIO& io, const LossCfg& c, int64_t t, bool m, float prox, float old, float& w,
+                   bool& counted) {
   const float lr = sane_log_ratio(prox, old);
   w = expf(lr);
   bool keep = true;
@@ -281,150 +281,287 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_is_kernel(LossIO io, LossCfg
 // ---------------------------------------------------------------------------------------
 // Token kernel
 // ---------------------------------------------------------------------------------------
+// Per-token arrays are moved VEC elements per thread and access: VEC = 4 takes 16-byte loads and
+// stores for the fp32 arrays and 4-byte ones for the byte masks (every array 16-byte, resp.
+// 4-byte, aligned; the host checks), VEC = 1 is the element-wise form for anything else and for
+// the last n % 4 tokens. Each array is read and written once: the accesses carry the non-temporal
+// hint.
+template <int VEC>
+DEVI void load_f32(const float* p, int64_t t, float (&v)[VEC]) {
+  if (p == nullptr) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = 0.f;
+  } else if (VEC == 4) {
+    const f32x4 x = __builtin_nontemporal_load((const f32x4*)(p + t));
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = x[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = p[t + i];
+  }
+}
+template <int VEC>
+DEVI void load_mask(const uint8_t* p, int64_t t, bool (&v)[VEC]) {
+  if (VEC == 4) {
+    const uint32_t x = __builtin_nontemporal_load((const uint32_t*)(p + t));
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = ((x >> (8 * i)) & 0xffu) != 0;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = p[t + i] != 0;
+  }
+}
+template <int VEC>
+DEVI void store_f32(float* p, int64_t t, const float (&v)[VEC]) {
+  if (p == nullptr) return;
+  if (VEC == 4) {
+    const f32x4 x = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(x, (f32x4*)(p + t));
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
+  }
+}
+template <int VEC>
+DEVI void store_mask(uint8_t* p, int64_t t, const bool (&v)[VEC]) {
+  if (p == nullptr) return;
+  if (VEC == 4) {
+    uint32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) x |= (v[i] ? 1u : 0u) << (8 * i);
+    __builtin_nontemporal_store(x, (uint32_t*)(p + t));
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
+  }
+}
+
+// Running sums of one thread. Counts fit 32 bits per thread (a thread sees n / gridsize tokens).
+struct TokenAcc {
+  double loss_sum;
+  int n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave;
+};
+
+// The logged statistics a thread reduces itself. The three 0/1-valued ones (clip_ratio,
+// dual_clip_ratio, behave_filtered_ratio) are not among them: their sums are the integer counters
+// and their extremes follow from those (loss_stats_finalize_kernel). it_sum collects the tokens of
+// one iteration in fp32 and is added to the fp64 sum once per iteration.
+template <bool STATS>
+struct StatAcc {
+  double sum[STATS ? N_LOSS_STATS : 1];
+  float it_sum[STATS ? N_LOSS_STATS : 1], mn[STATS ? N_LOSS_STATS : 1], mx[STATS ? N_LOSS_STATS : 1];
+  DEVI void init() {
+    if (STATS) {
+#pragma unroll
+      for (int k = 0; k < N_LOSS_STATS; ++k) { sum[k] = 0.0; it_sum[k] = 0.f; mn[k] = pos_inf(); mx[k] = neg_inf(); }
+    }
+  }
+  DEVI void add(int k, float v) {
+    if (STATS) {
+      it_sum[k] += v;
+      mn[k] = stat_min(mn[k], v);
+      mx[k] = stat_max(mx[k], v);
+    }
+  }
+  DEVI void flush() {
+    if (STATS) {
+#pragma unroll
+      for (int k = 0; k < N_LOSS_STATS; ++k) { sum[k] += (double)it_sum[k]; it_sum[k] = 0.f; }
+    }
+  }
+};
+
+// One token: the loss term, its gradient and every per-token output, from values in registers.
+struct TokenIn {
+  float lp, prox, old, adv, entropy, extra0, extra1;
+  bool m;
+};
+struct TokenOut {
+  float dlp, loss, ratio, kl, behave_w, behave_kl;
+  bool clip, dual, m2, bm;
+};
+
+template <bool STATS>
+DEVI void token_body(const LossIO& io, const LossCfg& c, int64_t t, const TokenIn& in, TokenOut& out,
+                     TokenAcc& acc, StatAcc<STATS>& st) {
+  const bool m = in.m;
+  bool m2 = m;
+  float w = 1.0f;
+  if (c.rs_enabled) {
+    bool counted;
+    m2 = rs_token(io, c, t, m, in.prox, in.old, w, counted);
+    w = m2 ? w : 0.0f;
+    acc.n_filtered += counted;
+  }
+  out.m2 = m2;
+  out.behave_w = w;
+  acc.n_valid += m;
+  acc.n_kept += m2;
+  if (STATS) {
+    if (io.extra0) st.add(ST_EXTRA0, in.extra0);
+    if (io.extra1) st.add(ST_EXTRA1, in.extra1);
+  }
+  out.dlp = 0.f; out.loss = 0.f; out.ratio = 0.f; out.kl = 0.f; out.behave_kl = 0.f;
+  out.clip = false; out.dual = false; out.bm = false;
+  if (c.loss_kind == LOSS_NONE) return;
+
+  const float lp = in.lp, prox = in.prox, adv = in.adv;
+  const float kl = lp - prox;
+  float pg, dsel, ratio_out;
+  bool clip = false, dual = false;
+  if (c.loss_kind == LOSS_CISPO) {
+    const float ratio = expf(kl);
+    const float rc = torch_clamp(ratio, c.clip_lo, c.clip_hi);
+    const float coef = (-rc) * adv;
+    pg = coef * lp;
+    dsel = coef;  // d pg / d lp
+    clip = (rc != ratio) && m2;
+    ratio_out = ratio;
+  } else {
+    float ratio, a = adv, dratio;  // dratio = d ratio / d lp[t] factor handled below
+    if (c.seq_is) {
+      const int s = seq_of(io, t);
+      ratio = m2 ? io.seq_is[4 * s + 0] : 0.0f;
+      a = m2 ? io.seq_is[4 * s + 1] : 0.0f;
+      dratio = 0.f;  // gradient assembled per sequence below
+    } else {
+      ratio = m ? expf(kl) : 0.0f;
+      dratio = ratio;
+    }
+    const float clipped = torch_clamp(ratio, c.clip_lo, c.clip_hi);
+    const float pg1 = (-a) * ratio;
+    const float pg2 = (-a) * clipped;
+    clip = pg1 < pg2;
+    pg = torch_max(pg1, pg2);
+    // d pg / d ratio following torch.max (ties split evenly) and clamp (closed interval)
+    const float in_band = (ratio >= c.clip_lo && ratio <= c.clip_hi) ? 1.0f : 0.0f;
+    float g1 = pg1 > pg2 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
+    float g2 = pg2 > pg1 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
+    float dpg = (-a) * (g1 + g2 * in_band);
+    if (c.has_c_clip) {
+      const float sgn = a > 0.f ? 1.0f : (a < 0.f ? -1.0f : 0.0f);
+      const float pg3 = (sgn * c.c_clip) * a;
+      dual = pg3 < pg;
+      const float keep = pg < pg3 ? 1.0f : (pg == pg3 ? 0.5f : 0.0f);
+      pg = torch_min(pg, pg3);
+      dpg *= keep;
+    }
+    if (c.seq_is) {
+      // every kept token of the sequence receives ratio_s/count_s * sum_w_s * dpg_s
+      const int s = seq_of(io, t);
+      dsel = m2 ? dpg * ratio * io.seq_is[4 * s + 2] * io.seq_is[4 * s + 3] : 0.0f;
+    } else {
+      dsel = dpg * dratio;
+    }
+    clip = clip && m;
+    dual = dual && m;
+    ratio_out = ratio;
+  }
+  if (c.rs_enabled) {
+    pg = pg * w;
+    if (!(c.loss_kind == LOSS_PPO && c.seq_is)) dsel = dsel * w;
+    const bool bm = (w > 0.0f) && m2;
+    acc.n_behave += bm;
+    out.bm = bm;
+    out.behave_kl = bm ? (prox - in.old) : 0.0f;
+    if (STATS && bm) {
+      st.add(ST_BEHAVE_IMP_WEIGHT, w);
+      st.add(ST_BEHAVE_APPROX_KL, prox - in.old);
+    }
+  }
+  if (STATS) {
+    if (m) {
+      st.add(ST_IMPORTANCE_WEIGHT, ratio_out);
+      st.add(ST_APPROX_KL, kl);
+      st.add(ST_NEW_LOGP, lp);
+      st.add(ST_ACTOR_LOSS, pg);
+      if (io.entropy) st.add(ST_ENTROPY, in.entropy);
+      if (io.old) {
+        st.add(ST_OLD_LOGP, in.old);
+        st.add(ST_LOGP_DIFF, in.old - lp);
+        st.add(ST_LOGP_ABS_DIFF, fabsf(in.old - lp));
+      }
+    }
+    if (clip) {
+      st.add(ST_CLIPPED_NEW_LOGP, lp);
+      if (io.old) st.add(ST_CLIPPED_OLD_LOGP, in.old);
+    }
+  }
+  if (m2) acc.loss_sum += (double)pg;
+  acc.n_clip += clip;
+  acc.n_dual += dual;
+  out.dlp = m2 ? dsel : 0.0f;
+  out.loss = pg;
+  out.ratio = ratio_out;
+  out.kl = kl;
+  out.clip = clip;
+  out.dual = dual;
+}
+
+template <bool STATS, int VEC>
+DEVI void token_group(const LossIO& io, const LossCfg& c, int64_t t, TokenAcc& acc, StatAcc<STATS>& st) {
+  float lp[VEC], prox[VEC], old[VEC], adv[VEC], ent[VEC], x0[VEC], x1[VEC];
+  bool m[VEC];
+  load_mask<VEC>(io.mask, t, m);
+  load_f32<VEC>(io.prox, t, prox);
+  load_f32<VEC>(io.old, t, old);
+  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.lp, t, lp);
+  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.adv, t, adv);
+  load_f32<VEC>(STATS ? io.entropy : nullptr, t, ent);
+  load_f32<VEC>(STATS ? io.extra0 : nullptr, t, x0);
+  load_f32<VEC>(STATS ? io.extra1 : nullptr, t, x1);
+  float dlp[VEC], loss[VEC], ratio[VEC], kl[VEC], bw[VEC], bkl[VEC];
+  bool clip[VEC], dual[VEC], m2[VEC], bm[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    const TokenIn in{lp[i], prox[i], old[i], adv[i], ent[i], x0[i], x1[i], m[i]};
+    TokenOut o;
+    token_body<STATS>(io, c, t + i, in, o, acc, st);
+    dlp[i] = o.dlp; loss[i] = o.loss; ratio[i] = o.ratio; kl[i] = o.kl; bw[i] = o.behave_w; bkl[i] = o.behave_kl;
+    clip[i] = o.clip; dual[i] = o.dual; m2[i] = o.m2; bm[i] = o.bm;
+  }
+  st.flush();
+  if (c.rs_enabled) {
+    store_mask<VEC>(io.new_mask, t, m2);
+    store_f32<VEC>(io.behave_w, t, bw);
+  }
+  if (c.loss_kind == LOSS_NONE) return;
+  if (c.rs_enabled) {
+    store_mask<VEC>(io.behave_mask, t, bm);
+    store_f32<VEC>(io.behave_kl, t, bkl);
+  }
+  store_f32<VEC>(io.dlp, t, dlp);
+  store_f32<VEC>(io.stat_loss, t, loss);
+  store_f32<VEC>(io.stat_ratio, t, ratio);
+  store_f32<VEC>(io.stat_kl, t, kl);
+  store_mask<VEC>(io.clip_mask, t, clip);
+  store_mask<VEC>(io.dual_mask, t, dual);
+}
+
 // STATS: also reduce the logged statistics (sum, min, max per block) into stat_partials
 // [gridDim.x][N_LOSS_STATS]; min / max propagate NaN as torch.min / torch.max do.
-template <bool STATS>
+template <bool STATS, int VEC>
 __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, LossCfg c,
                                                                    Partial* partials,
                                                                    StatPartial* stat_partials) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
-  double loss_sum = 0.0;
-  long long n_valid = 0, n_kept = 0, n_filtered = 0, n_clip = 0, n_dual = 0, n_behave = 0;
-  double st_sum[STATS ? N_LOSS_STATS : 1];
-  float st_mn[STATS ? N_LOSS_STATS : 1], st_mx[STATS ? N_LOSS_STATS : 1];
-  if (STATS) {
-#pragma unroll
-    for (int k = 0; k < N_LOSS_STATS; ++k) { st_sum[k] = 0.0; st_mn[k] = pos_inf(); st_mx[k] = neg_inf(); }
-  }
-  auto stat = [&](int k, bool on, float v) {
-    if (STATS && on) {
-      st_sum[k] += (double)v;
-      st_mn[k] = stat_min(st_mn[k], v);
-      st_mx[k] = stat_max(st_mx[k], v);
-    }
-  };
+  TokenAcc acc{0.0, 0, 0, 0, 0, 0, 0};
+  StatAcc<STATS> st;
+  st.init();
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n_vec = io.n - io.n % VEC;
+  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) token_group<STATS, VEC>(io, c, t, acc, st);
+  if (VEC > 1 && n_vec + gid < io.n) token_group<STATS, 1>(io, c, n_vec + gid, acc, st);
 
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < io.n;
-       t += (int64_t)gridDim.x * blockDim.x) {
-    const bool m = io.mask[t] != 0;
-    bool m2 = m;
-    float w = 1.0f;
-    if (c.rs_enabled) {
-      bool counted;
-      m2 = rs_token(io, c, t, m, w, counted);
-      w = m2 ? w : 0.0f;
-      n_filtered += counted;
-      if (io.new_mask) io.new_mask[t] = m2;
-      if (io.behave_w) io.behave_w[t] = w;
-    }
-    n_valid += m;
-    n_kept += m2;
-    if (STATS) {
-      if (io.extra0) stat(ST_EXTRA0, true, io.extra0[t]);
-      if (io.extra1) stat(ST_EXTRA1, true, io.extra1[t]);
-    }
-    if (c.loss_kind == LOSS_NONE) continue;
-
-    const float lp = io.lp[t], prox = io.prox[t], adv = io.adv[t];
-    const float kl = lp - prox;
-    float pg, dsel, ratio_out;
-    bool clip = false, dual = false;
-    if (c.loss_kind == LOSS_CISPO) {
-      const float ratio = expf(kl);
-      const float rc = torch_clamp(ratio, c.clip_lo, c.clip_hi);
-      const float coef = (-rc) * adv;
-      pg = coef * lp;
-      dsel = coef;  // d pg / d lp
-      clip = (rc != ratio) && m2;
-      ratio_out = ratio;
-    } else {
-      float ratio, a = adv, dratio;  // dratio = d ratio / d lp[t] factor handled below
-      if (c.seq_is) {
-        const int s = seq_of(io, t);
-        ratio = m2 ? io.seq_is[4 * s + 0] : 0.0f;
-        a = m2 ? io.seq_is[4 * s + 1] : 0.0f;
-        dratio = 0.f;  // gradient assembled per sequence below
-      } else {
-        ratio = m ? expf(kl) : 0.0f;
-        dratio = ratio;
-      }
-      const float clipped = torch_clamp(ratio, c.clip_lo, c.clip_hi);
-      const float pg1 = (-a) * ratio;
-      const float pg2 = (-a) * clipped;
-      clip = pg1 < pg2;
-      pg = torch_max(pg1, pg2);
-      // d pg / d ratio following torch.max (ties split evenly) and clamp (closed interval)
-      const float in_band = (ratio >= c.clip_lo && ratio <= c.clip_hi) ? 1.0f : 0.0f;
-      float g1 = pg1 > pg2 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
-      float g2 = pg2 > pg1 ? 1.0f : (pg1 == pg2 ? 0.5f : 0.0f);
-      float dpg = (-a) * (g1 + g2 * in_band);
-      if (c.has_c_clip) {
-        const float sgn = a > 0.f ? 1.0f : (a < 0.f ? -1.0f : 0.0f);
-        const float pg3 = (sgn * c.c_clip) * a;
-        dual = pg3 < pg;
-        const float keep = pg < pg3 ? 1.0f : (pg == pg3 ? 0.5f : 0.0f);
-        pg = torch_min(pg, pg3);
-        dpg *= keep;
-      }
-      if (c.seq_is) {
-        // every kept token of the sequence receives ratio_s/count_s * sum_w_s * dpg_s
-        const int s = seq_of(io, t);
-        dsel = m2 ? dpg * ratio * io.seq_is[4 * s + 2] * io.seq_is[4 * s + 3] : 0.0f;
-      } else {
-        dsel = dpg * dratio;
-      }
-      clip = clip && m;
-      dual = dual && m;
-      ratio_out = ratio;
-    }
-    if (c.rs_enabled) {
-      pg = pg * w;
-      if (!(c.loss_kind == LOSS_PPO && c.seq_is)) dsel = dsel * w;
-      const bool bm = (w > 0.0f) && m2;
-      n_behave += bm;
-      if (io.behave_mask) io.behave_mask[t] = bm;
-      if (io.behave_kl) io.behave_kl[t] = bm ? (prox - io.old[t]) : 0.0f;
-      if (STATS) {
-        stat(ST_BEHAVE_IMP_WEIGHT, bm, w);
-        stat(ST_BEHAVE_APPROX_KL, bm, prox - io.old[t]);
-        stat(ST_BEHAVE_FILTERED_RATIO, m, (m && !bm) ? 1.0f : 0.0f);
-      }
-    }
-    if (STATS) {
-      stat(ST_IMPORTANCE_WEIGHT, m, ratio_out);
-      stat(ST_APPROX_KL, m, kl);
-      stat(ST_NEW_LOGP, m, lp);
-      stat(ST_ACTOR_LOSS, m, pg);
-      stat(ST_CLIP_RATIO, m, clip ? 1.0f : 0.0f);
-      stat(ST_DUAL_CLIP_RATIO, m, dual ? 1.0f : 0.0f);
-      stat(ST_CLIPPED_NEW_LOGP, clip, lp);
-      if (io.entropy) stat(ST_ENTROPY, m, io.entropy[t]);
-      if (io.old) {
-        const float o = io.old[t];
-        stat(ST_OLD_LOGP, m, o);
-        stat(ST_LOGP_DIFF, m, o - lp);
-        stat(ST_LOGP_ABS_DIFF, m, fabsf(o - lp));
-        stat(ST_CLIPPED_OLD_LOGP, clip, o);
-      }
-    }
-    if (m2) loss_sum += (double)pg;
-    n_clip += clip;
-    n_dual += dual;
-    if (io.dlp) io.dlp[t] = m2 ? dsel : 0.0f;
-    if (io.stat_loss) io.stat_loss[t] = pg;
-    if (io.stat_ratio) io.stat_ratio[t] = ratio_out;
-    if (io.stat_kl) io.stat_kl[t] = kl;
-    if (io.clip_mask) io.clip_mask[t] = clip;
-    if (io.dual_mask) io.dual_mask[t] = dual;
-  }
-  loss_sum = block_sum(loss_sum, sm_d);
-  n_valid = block_sum(n_valid, sm_l);
-  n_kept = block_sum(n_kept, sm_l);
-  n_filtered = block_sum(n_filtered, sm_l);
-  n_clip = block_sum(n_clip, sm_l);
-  n_dual = block_sum(n_dual, sm_l);
-  n_behave = block_sum(n_behave, sm_l);
+  const double loss_sum = block_sum(acc.loss_sum, sm_d);
+  const long long n_valid = block_sum((long long)acc.n_valid, sm_l);
+  const long long n_kept = block_sum((long long)acc.n_kept, sm_l);
+  const long long n_filtered = block_sum((long long)acc.n_filtered, sm_l);
+  const long long n_clip = block_sum((long long)acc.n_clip, sm_l);
+  const long long n_dual = block_sum((long long)acc.n_dual, sm_l);
+  const long long n_behave = block_sum((long long)acc.n_behave, sm_l);
   if (threadIdx.x == 0) {
     Partial p{loss_sum, n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave};
     partials[blockIdx.x] = p;
@@ -436,8 +573,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
     for (int k = 0; k < N_LOSS_STATS; ++k) {
-      const double sv = wave_sum(st_sum[k]);
-      float mn = st_mn[k], mx = st_mx[k];
+      const double sv = wave_sum(st.sum[k]);
+      float mn = st.mn[k], mx = st.mx[k];
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) {
         mn = stat_min(mn, __shfl_xor(mn, o, 64));
@@ -459,51 +596,21 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
   }
 }
 
-// stats [N_LOSS_STATS][4] = {sum, count, min, max}: block k folds statistic k over the token
-// kernel's blocks in a fixed order; the count is the statistic's denominator, taken from the
-// counters loss_finalize_kernel has written (this kernel is queued behind it).
-__global__ __launch_bounds__(LOSS_THREADS) void loss_stats_finalize_kernel(
-    const StatPartial* __restrict__ stat_partials, int nparts, const double* __restrict__ counters,
-    double n_tokens, double* __restrict__ stats) {
-  __shared__ double sm_d[8];
-  __shared__ float sm_f[8];
-  const int k = blockIdx.x;
-  double sum = 0.0;
-  float mn = pos_inf(), mx = neg_inf();
-  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
-    const StatPartial sp = stat_partials[(size_t)i * N_LOSS_STATS + k];
-    sum += sp.sum;
-    mn = stat_min(mn, sp.mn);
-    mx = stat_max(mx, sp.mx);
-  }
-  sum = block_sum(sum, sm_d);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    mn = stat_min(mn, __shfl_xor(mn, o, 64));
-    mx = stat_max(mx, __shfl_xor(mx, o, 64));
-  }
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  __syncthreads();
-  if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    mn = stat_min(stat_min(sm_f[0], sm_f[1]), stat_min(sm_f[2], sm_f[3]));
-    mx = stat_max(stat_max(sm_f[4], sm_f[5]), stat_max(sm_f[6], sm_f[7]));
-    const int d = STAT_DENOM[k];
-    const double count = d == 0 ? counters[1] : (d == 1 ? counters[4] : (d == 2 ? counters[6] : n_tokens));
-    stats[4 * k + 0] = sum;
-    stats[4 * k + 1] = count;
-    stats[4 * k + 2] = (double)mn;
-    stats[4 * k + 3] = (double)mx;
-  }
-}
-
 // counters: [0] loss_sum [1] n_valid [2] n_kept [3] n_filtered [4] n_clip [5] n_dual
 //           [6] n_behave [7] loss = loss_sum / max(n_valid, 1)
-__global__ void loss_finalize_kernel(const Partial* partials, int nparts, float* loss_out,
-                                     double* counters) {
+// Block 0 folds the token kernel's block partials into the counters and the loss, in a fixed order
+// (thread partials -> wave shuffles -> 4 wave slots). With statistics, block 1 + k folds statistic
+// k into stats [N_LOSS_STATS][4] = {sum, count, min, max}; the count is the statistic's denominator.
+// The three 0/1-valued statistics are not reduced per token: their sums are token counts and
+// their extremes follow from whether every / any counted token has the value 1. Each block sums
+// the counts it needs itself, so one launch does everything.
+__global__ __launch_bounds__(LOSS_THREADS) void loss_finalize_kernel(
+    const Partial* __restrict__ partials, const StatPartial* __restrict__ stat_partials, int nparts,
+    float* loss_out, double* __restrict__ counters, double n_tokens, double* __restrict__ stats,
+    int loss_active, int rs_enabled) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
+  __shared__ float sm_f[8];
   double ls = 0.0;
   long long a[6] = {0, 0, 0, 0, 0, 0};
   for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
@@ -512,33 +619,88 @@ __global__ void loss_finalize_kernel(const Partial* partials, int nparts, float*
     a[0] += p.n_valid; a[1] += p.n_kept; a[2] += p.n_filtered;
     a[3] += p.n_clip; a[4] += p.n_dual; a[5] += p.n_behave;
   }
-  // fixed-order reduction: thread partials -> wave shuffles -> 4 wave slots
   ls = block_sum(ls, sm_d);
   for (int k = 0; k < 6; ++k) a[k] = block_sum(a[k], sm_l);
+  if (blockIdx.x == 0) {
+    if (threadIdx.x == 0) {
+      counters[0] = ls;
+      for (int k = 0; k < 6; ++k) counters[1 + k] = (double)a[k];
+      const double denom = a[0] > 0 ? (double)a[0] : 1.0;
+      const float loss = (float)ls / (float)denom;
+      counters[7] = (double)loss;
+      if (loss_out) *loss_out = loss;
+    }
+    return;
+  }
+  const int k = blockIdx.x - 1;
+  const long long n_valid = a[0], n_clip = a[3], n_dual = a[4], n_behave = a[5];
+  const int d = STAT_DENOM[k];
+  const double count = d == 0 ? (double)n_valid : (d == 1 ? (double)n_clip : (d == 2 ? (double)n_behave : n_tokens));
+  double sum = 0.0;
+  float mn = pos_inf(), mx = neg_inf();
+  if (k == ST_CLIP_RATIO || k == ST_DUAL_CLIP_RATIO || k == ST_BEHAVE_FILTERED_RATIO) {
+    // ones among the n_valid tokens under the loss mask
+    const bool on = loss_active && (k != ST_BEHAVE_FILTERED_RATIO || rs_enabled);
+    const long long ones = k == ST_CLIP_RATIO ? n_clip : (k == ST_DUAL_CLIP_RATIO ? n_dual : n_valid - n_behave);
+    if (on && n_valid > 0) {
+      sum = (double)ones;
+      mn = ones == n_valid ? 1.0f : 0.0f;
+      mx = ones > 0 ? 1.0f : 0.0f;
+    }
+  } else {
+    for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+      const StatPartial sp = stat_partials[(size_t)i * N_LOSS_STATS + k];
+      sum += sp.sum;
+      mn = stat_min(mn, sp.mn);
+      mx = stat_max(mx, sp.mx);
+    }
+    sum = block_sum(sum, sm_d);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      mn = stat_min(mn, __shfl_xor(mn, o, 64));
+      mx = stat_max(mx, __shfl_xor(mx, o, 64));
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
+    __syncthreads();
+    mn = stat_min(stat_min(sm_f[0], sm_f[1]), stat_min(sm_f[2], sm_f[3]));
+    mx = stat_max(stat_max(sm_f[4], sm_f[5]), stat_max(sm_f[6], sm_f[7]));
+  }
   if (threadIdx.x == 0) {
-    counters[0] = ls;
-    for (int k = 0; k < 6; ++k) counters[1 + k] = (double)a[k];
-    const double denom = a[0] > 0 ? (double)a[0] : 1.0;
-    const float loss = (float)ls / (float)denom;
-    counters[7] = (double)loss;
-    if (loss_out) *loss_out = loss;
+    stats[4 * k + 0] = sum;
+    stats[4 * k + 1] = count;
+    stats[4 * k + 2] = (double)mn;
+    stats[4 * k + 3] = (double)mx;
   }
 }
 
-// out[t] = dlp[t] * upstream[0] / max(n_valid, 1)
+// out[t] = dlp[t] * upstream[0] / max(n_valid, 1); VEC as in the token kernel
+template <int VEC>
 __global__ void loss_grad_scale_kernel(const float* __restrict__ dlp,
                                        const float* __restrict__ upstream,
                                        const double* __restrict__ counters,
                                        float* __restrict__ out, int64_t n) {
   const float nv = (float)(counters[1] > 0.0 ? counters[1] : 1.0);
   const float g = upstream[0];
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
-       t += (int64_t)gridDim.x * blockDim.x)
-    out[t] = (dlp[t] * g) / nv;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n_vec = n - n % VEC;
+  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) {
+    float v[VEC];
+    load_f32<VEC>(dlp, t, v);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = (v[i] * g) / nv;
+    store_f32<VEC>(out, t, v);
+  }
+  if (VEC > 1 && n_vec + gid < n) out[n_vec + gid] = (dlp[n_vec + gid] * g) / nv;
 }
 
-int loss_grid(int64_t n) {
-  int64_t b = ceil_div_i64(n, LOSS_THREADS);
+// VEC = 4 needs every per-token fp32 array 16-byte aligned and every byte array 4-byte aligned.
+bool aligned_to(const void* p, uintptr_t a) { return p == nullptr || ((uintptr_t)p & (a - 1)) == 0; }
+
+int loss_grid(int64_t n, int vec = 1) {
+  int64_t b = ceil_div_i64(n, (int64_t)LOSS_THREADS * vec);
   if (b > MAX_LOSS_BLOCKS) b = MAX_LOSS_BLOCKS;
   if (b < 1) b = 1;
   return (int)b;
@@ -763,7 +925,24 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
   io.extra0 = with_stats ? sa->extra0 : nullptr;
   io.extra1 = with_stats ? sa->extra1 : nullptr;
 
-  const int grid = loss_grid(n_tokens);
+  const bool vec4 = aligned_to(logprobs, 16) && aligned_to(proximal, 16) && aligned_to(old_logprobs, 16) &&
+                    aligned_to(advantages, 16) && aligned_to(dlogprobs, 16) && aligned_to(stat_loss, 16) &&
+                    aligned_to(stat_ratio, 16) && aligned_to(stat_approx_kl, 16) &&
+                    aligned_to(behave_imp_weight, 16) && aligned_to(behave_approx_kl, 16) &&
+                    aligned_to(io.entropy, 16) && aligned_to(io.extra0, 16) && aligned_to(io.extra1, 16) &&
+                    aligned_to(loss_mask, 4) && aligned_to(clip_mask, 4) && aligned_to(dual_clip_mask, 4) &&
+                    aligned_to(new_mask, 4) && aligned_to(behave_mask, 4);
+  const int grid = loss_grid(n_tokens, vec4 ? 4 : 1);
+  auto token_pass = [&](const LossIO& i, const LossCfg& cc, bool stats) {
+    if (stats && vec4)
+      hipLaunchKernelGGL((loss_token_kernel<true, 4>), dim3(grid), dim3(LOSS_THREADS), 0, stream, i, cc, partials, stat_partials);
+    else if (stats)
+      hipLaunchKernelGGL((loss_token_kernel<true, 1>), dim3(grid), dim3(LOSS_THREADS), 0, stream, i, cc, partials, stat_partials);
+    else if (vec4)
+      hipLaunchKernelGGL((loss_token_kernel<false, 4>), dim3(grid), dim3(LOSS_THREADS), 0, stream, i, cc, partials, (StatPartial*)nullptr);
+    else
+      hipLaunchKernelGGL((loss_token_kernel<false, 1>), dim3(grid), dim3(LOSS_THREADS), 0, stream, i, cc, partials, (StatPartial*)nullptr);
+  };
   if (n_tokens > 0 && c.rs_enabled && c.rs_seq_level) {
     hipLaunchKernelGGL(seq_rs_kernel, dim3((unsigned)n_seqs), dim3(LOSS_THREADS), 0, stream, io, c,
                        seq_rs);
@@ -774,30 +953,19 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
       // first materialise the narrowed mask and the behaviour weight, then aggregate on them
       LossCfg c0 = c;
       c0.loss_kind = LOSS_NONE;
-      LossIO io0 = io;
-      hipLaunchKernelGGL(loss_token_kernel<false>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io0, c0,
-                         partials, (StatPartial*)nullptr);
+      token_pass(io, c0, false);
       AREAL_CHECK_LAUNCH();
     }
     hipLaunchKernelGGL(seq_is_kernel, dim3((unsigned)n_seqs), dim3(LOSS_THREADS), 0, stream, io, c,
                        seq_is);
     AREAL_CHECK_LAUNCH();
   }
-  if (with_stats)
-    hipLaunchKernelGGL(loss_token_kernel<true>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c,
-                       partials, stat_partials);
-  else
-    hipLaunchKernelGGL(loss_token_kernel<false>, dim3(grid), dim3(LOSS_THREADS), 0, stream, io, c,
-                       partials, (StatPartial*)nullptr);
+  token_pass(io, c, with_stats);
   AREAL_CHECK_LAUNCH();
-  hipLaunchKernelGGL(loss_finalize_kernel, dim3(1), dim3(LOSS_THREADS), 0, stream, partials, grid,
-                     loss, counters);
+  hipLaunchKernelGGL(loss_finalize_kernel, dim3(with_stats ? 1 + N_LOSS_STATS : 1), dim3(LOSS_THREADS), 0, stream,
+                     partials, stat_partials, grid, loss, counters, (double)n_tokens,
+                     with_stats ? sa->stats : nullptr, c.loss_kind != LOSS_NONE ? 1 : 0, c.rs_enabled);
   AREAL_CHECK_LAUNCH();
-  if (with_stats) {
-    hipLaunchKernelGGL(loss_stats_finalize_kernel, dim3(N_LOSS_STATS), dim3(LOSS_THREADS), 0, stream,
-                       stat_partials, grid, counters, (double)n_tokens, sa->stats);
-    AREAL_CHECK_LAUNCH();
-  }
   return AREAL_OK;
 }
 
@@ -811,8 +979,12 @@ int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const d
   if (n_tokens < 0) return AREAL_ERR_BAD_ARG;
   if (n_tokens == 0) return AREAL_OK;
   if (!dlogprobs || !upstream || !counters || !grad_logprobs) return AREAL_ERR_BAD_ARG;
-  hipLaunchKernelGGL(loss_grad_scale_kernel, dim3(loss_grid(n_tokens)), dim3(LOSS_THREADS), 0,
-                     stream, dlogprobs, upstream, counters, grad_logprobs, n_tokens);
+  if (aligned_to(dlogprobs, 16) && aligned_to(grad_logprobs, 16))
+    hipLaunchKernelGGL(loss_grad_scale_kernel<4>, dim3(loss_grid(n_tokens, 4)), dim3(LOSS_THREADS), 0,
+                       stream, dlogprobs, upstream, counters, grad_logprobs, n_tokens);
+  else
+    hipLaunchKernelGGL(loss_grad_scale_kernel<1>, dim3(loss_grid(n_tokens)), dim3(LOSS_THREADS), 0,
+                       stream, dlogprobs, upstream, counters, grad_logprobs, n_tokens);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

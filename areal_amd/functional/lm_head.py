@@ -17,8 +17,10 @@ Two ways of carrying state to the backward:
   rows of dHidden and to the hidden states for dWeight) and skips the recomputation, a quarter
   of the step's matrix work.  The reference's logits-in path saves the same amount through
   autograd; 288 GB of HBM make it the default while it fits ``SAVE_PROBS_BYTES_LIMIT`` and
-  60 % of the memory still available.  If some row's maximum logit lies more than 150 binades
-  above its estimate (the kernel reports it), the backward recomputes instead.
+  60 % of the memory still available.  If some row's maximum logit lies more than 100 binades
+  (69 nats at temperature 1) above its estimate, the kernel reports it, repeats the sweep
+  without saving on the device (so the outputs are right without a host round trip), and the
+  backward recomputes instead.
 """
 
 from __future__ import annotations

@@ -53,8 +53,11 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * [round_up(T,128)][round_up(V,64)] holding 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
  * fp32 [T], a per-row reference estimated from a few logits of the row (its label's among
  * them) before the sweep; *probs_status (one int32 on the device) is written 0 when every
- * row's exponentials are in range, 1 when some row's maximum lies more than 150 binades above
- * its estimate: probs must then not be used and the backward recomputes (areal_lmhead_bwd). */
+ * row's exponentials are in range, 1 when some row's maximum lies more than 100 binades (69 nats
+ * at temperature 1) above its estimate: probs must then not be used and the backward recomputes
+ * (areal_lmhead_bwd). The per-token outputs are right in both cases: when the status comes out
+ * 1 the sweep is repeated without saving inside this call (launches queued behind the first
+ * sweep that return at once otherwise), no host synchronisation involved. */
 int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
