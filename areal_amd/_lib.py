@@ -34,13 +34,17 @@ D = c_double
 I = c_int
 SZ = c_size_t
 
+ABI_VERSION = 3  # AREAL_HIP_ABI_VERSION of include/areal_hip.h
+
 # name -> (restype, argtypes).  Must list every symbol declared in include/areal_hip.h.
 SIGNATURES: dict[str, tuple] = {
     "areal_gemm_nt_bf16": (I, [P, I64, P, I64, P, I64, I64, I64, I64, I, P]),
     "areal_lmhead_fwd_workspace_bytes": (SZ, [I64, I64, I64]),
+    "areal_abi_version": (I, []),
+    "areal_lmhead_probs_bytes": (SZ, [I64, I64]),
     "areal_lmhead_fwd": (
         I,
-        [P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
+        [P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, P, P, P, P, SZ, P, P, P, SZ, P],
     ),
     "areal_lmhead_bwd_workspace_bytes": (SZ, [I64, I64, I64, I64]),
     "areal_lmhead_bwd": (
@@ -50,7 +54,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_lmhead_bwd_saved_workspace_bytes": (SZ, [I64, I64, I64]),
     "areal_lmhead_bwd_saved": (
         I,
-        [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, P, P, P, P, I, P, P, SZ, P],
+        [P, P, P, P, P, P, P, I64, I64, I64, F, F, P, SZ, P, P, P, P, I, P, P, SZ, P],
     ),
     "areal_cast_f32_to_bf16": (I, [P, P, I64, P]),
     "areal_logits_logprobs_entropy_fwd": (I, [P, I, I64, P, I64, I64, F, P, P, P, P]),
@@ -158,6 +162,13 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
+    # the argument lists above are those of one version of the interface (include/areal_hip.h)
+    built = lib.areal_abi_version()
+    if built != ABI_VERSION:
+        raise ArealHipError(
+            f"{LIB_PATH} was built with interface version {built}, this package binds version "
+            f"{ABI_VERSION}: rebuild it with `python -m areal_amd.build`"
+        )
     _lib = lib
     return lib
 

@@ -2390,6 +2390,13 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   return launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, out_mode, stream);
 }
 
+int areal_abi_version(void) { return 3; }  // AREAL_HIP_ABI_VERSION of include/areal_hip.h
+
+size_t areal_lmhead_probs_bytes(int64_t T, int64_t V) {
+  if (T <= 0 || V <= 0) return 0;
+  return (size_t)round_up_i64(T, 2 * BK) * (size_t)round_up_i64(V, BK) * 2;
+}
+
 static Regions fwd_regions(int64_t T, int64_t H, int64_t V) {
   Regions r = plan_regions(V, T, H, 512, 0);
   fold_ragged_a(r, V);
@@ -2417,12 +2424,13 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
-                     float* row_max, float* sum_exp, void* probs, float* probs_ref,
-                     int* probs_status, void* workspace, size_t workspace_bytes,
+                     float* row_max, float* sum_exp, void* probs, size_t probs_bytes,
+                     float* probs_ref, int* probs_status, void* workspace, size_t workspace_bytes,
                      hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0 || labels == nullptr) return AREAL_ERR_BAD_ARG;
   if ((probs == nullptr) != (probs_ref == nullptr) || (probs == nullptr) != (probs_status == nullptr))
     return AREAL_ERR_BAD_ARG;
+  if (probs != nullptr && probs_bytes < areal_lmhead_probs_bytes(T, V)) return AREAL_ERR_WORKSPACE;
   if (probs != nullptr && !aligned16(probs)) return AREAL_ERR_ALIGNMENT;
   if (!(inv_temperature > 0.f) || !(logit_scale > 0.f)) return AREAL_ERR_BAD_ARG;
   if (T == 0) return AREAL_OK;
@@ -2657,11 +2665,12 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
-                           float inv_temperature, float logit_scale, void* probs,
+                           float inv_temperature, float logit_scale, void* probs, size_t probs_bytes,
                            const float* probs_ref, const int* probs_status, void* dhidden, void* dweight,
                            int dweight_mode, float* dbias, void* workspace,
                            size_t workspace_bytes, hipStream_t stream) {
   if (T < 0 || H <= 0 || V <= 0) return AREAL_ERR_BAD_ARG;
+  if (probs != nullptr && probs_bytes < areal_lmhead_probs_bytes(T, V)) return AREAL_ERR_WORKSPACE;
   if (labels == nullptr || row_max == nullptr || sum_exp == nullptr || grad_logprobs == nullptr ||
       probs == nullptr || probs_ref == nullptr)
     return AREAL_ERR_BAD_ARG;

@@ -17,7 +17,8 @@
 namespace {
 
 constexpr int LOSS_THREADS = 256;
-constexpr int MAX_LOSS_BLOCKS = 1024;
+constexpr int MAX_LOSS_BLOCKS = 2048;
+constexpr int FINAL_THREADS = 512;  // loss_finalize_kernel: 4 block partials per thread
 
 enum { METRIC_RATIO = 0, METRIC_K1 = 1, METRIC_K2 = 2, METRIC_K3 = 3, METRIC_BINARY_KL = 4 };
 enum { AGG_SUM = 0, AGG_MEAN = 1, AGG_MAX = 2 };
@@ -130,10 +131,11 @@ DEVI bool in_bounds(float metric, const LossCfg& c) {
   return ok;
 }
 
-// Per-token divergence metric between proximal and behaviour policy.
-DEVI float rs_metric(float prox, float old, float lr_sane, int metric) {
+// Per-token divergence metric between proximal and behaviour policy. exp_lr = expf(lr_sane), which
+// the caller has already (the behaviour weight).
+DEVI float rs_metric(float prox, float old, float exp_lr, int metric) {
   switch (metric) {
-    case METRIC_RATIO: return expf(lr_sane);
+    case METRIC_RATIO: return exp_lr;
     case METRIC_K1: return prox - old;
     case METRIC_K2: { const float d = prox - old; return (d * d) / 2.0f; }
     case METRIC_K3: { const float d = -(prox - old); return (expf(d) - 1.0f) - d; }
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_rs_kernel(LossIO io, LossCfg
     if (!io.mask[t]) continue;
     const float prox = io.prox[t], old = io.old[t];
     const float lr = sane_log_ratio(prox, old);
-    const float v = log_agg ? lr : rs_metric(prox, old, lr, c.rs_metric);
+    const float v = log_agg ? lr : rs_metric(prox, old, 0.0f, c.rs_metric);  // (the ratio metric aggregates lr)
     cnt += 1;
     sum_lr += (double)lr;
     sum_m += (double)v;
@@ -239,7 +241,7 @@ DEVI bool rs_token(const LossIO& io, const LossCfg& c, int64_t t, bool m, float 
     w = torch_clamp(w, c.rs_has_lower ? c.rs_lower : 0.0f, c.rs_upper);
     counted = m && (orig != w);
   } else {
-    keep = in_bounds(rs_metric(prox, old, lr, c.rs_metric), c);
+    keep = in_bounds(rs_metric(prox, old, w, c.rs_metric), c);
     counted = m && !keep;
   }
   return c.rs_clamp ? m : (m && keep);
@@ -284,15 +286,17 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_is_kernel(LossIO io, LossCfg
 // Per-token arrays are moved VEC elements per thread and access: VEC = 4 takes 16-byte loads and
 // stores for the fp32 arrays and 4-byte ones for the byte masks (every array 16-byte, resp.
 // 4-byte, aligned; the host checks), VEC = 1 is the element-wise form for anything else and for
-// the last n % 4 tokens. Each array is read and written once: the accesses carry the non-temporal
-// hint.
+// the last n % 4 tokens. Plain loads and stores: a micro-batch's per-token arrays (a few hundred MB
+// at most) come from and go to kernels next to this one through the 256 MB memory-side cache,
+// which accesses with the non-temporal hint bypass (measured on 4 Mi tokens: 5.0 TB/s with the
+// hint, 6.5 to 7.5 without).
 template <int VEC>
 DEVI void load_f32(const float* p, int64_t t, float (&v)[VEC]) {
   if (p == nullptr) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[i] = 0.f;
   } else if (VEC == 4) {
-    const f32x4 x = __builtin_nontemporal_load((const f32x4*)(p + t));
+    const f32x4 x = *(const f32x4*)(p + t);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[i] = x[i];
   } else {
@@ -303,7 +307,7 @@ DEVI void load_f32(const float* p, int64_t t, float (&v)[VEC]) {
 template <int VEC>
 DEVI void load_mask(const uint8_t* p, int64_t t, bool (&v)[VEC]) {
   if (VEC == 4) {
-    const uint32_t x = __builtin_nontemporal_load((const uint32_t*)(p + t));
+    const uint32_t x = *(const uint32_t*)(p + t);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[i] = ((x >> (8 * i)) & 0xffu) != 0;
   } else {
@@ -316,7 +320,7 @@ DEVI void store_f32(float* p, int64_t t, const float (&v)[VEC]) {
   if (p == nullptr) return;
   if (VEC == 4) {
     const f32x4 x = {v[0], v[1], v[2], v[3]};
-    __builtin_nontemporal_store(x, (f32x4*)(p + t));
+    *(f32x4*)(p + t) = x;
   } else {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
@@ -329,7 +333,7 @@ DEVI void store_mask(uint8_t* p, int64_t t, const bool (&v)[VEC]) {
     uint32_t x = 0;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) x |= (v[i] ? 1u : 0u) << (8 * i);
-    __builtin_nontemporal_store(x, (uint32_t*)(p + t));
+    *(uint32_t*)(p + t) = x;
   } else {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
@@ -344,29 +348,23 @@ struct TokenAcc {
 
 // The logged statistics a thread reduces itself. The three 0/1-valued ones (clip_ratio,
 // dual_clip_ratio, behave_filtered_ratio) are not among them: their sums are the integer counters
-// and their extremes follow from those (loss_stats_finalize_kernel). it_sum collects the tokens of
-// one iteration in fp32 and is added to the fp64 sum once per iteration.
+// and their extremes follow from those (loss_finalize_kernel). A thread sees at most a few
+// thousand tokens (n / (MAX_LOSS_BLOCKS * LOSS_THREADS), 8 of 4 Mi), which it sums in fp32, as
+// the reference's tracker sums whole tensors; from the wave level on the sums are fp64.
 template <bool STATS>
 struct StatAcc {
-  double sum[STATS ? N_LOSS_STATS : 1];
-  float it_sum[STATS ? N_LOSS_STATS : 1], mn[STATS ? N_LOSS_STATS : 1], mx[STATS ? N_LOSS_STATS : 1];
+  float sum[STATS ? N_LOSS_STATS : 1], mn[STATS ? N_LOSS_STATS : 1], mx[STATS ? N_LOSS_STATS : 1];
   DEVI void init() {
     if (STATS) {
 #pragma unroll
-      for (int k = 0; k < N_LOSS_STATS; ++k) { sum[k] = 0.0; it_sum[k] = 0.f; mn[k] = pos_inf(); mx[k] = neg_inf(); }
+      for (int k = 0; k < N_LOSS_STATS; ++k) { sum[k] = 0.f; mn[k] = pos_inf(); mx[k] = neg_inf(); }
     }
   }
   DEVI void add(int k, float v) {
     if (STATS) {
-      it_sum[k] += v;
+      sum[k] += v;
       mn[k] = stat_min(mn[k], v);
       mx[k] = stat_max(mx[k], v);
-    }
-  }
-  DEVI void flush() {
-    if (STATS) {
-#pragma unroll
-      for (int k = 0; k < N_LOSS_STATS; ++k) { sum[k] += (double)it_sum[k]; it_sum[k] = 0.f; }
     }
   }
 };
@@ -498,29 +496,36 @@ DEVI void token_body(const LossIO& io, const LossCfg& c, int64_t t, const TokenI
   out.dual = dual;
 }
 
-template <bool STATS, int VEC>
-DEVI void token_group(const LossIO& io, const LossCfg& c, int64_t t, TokenAcc& acc, StatAcc<STATS>& st) {
+// The per-token inputs of VEC consecutive tokens, in registers.
+template <int VEC>
+struct TokenLoad {
   float lp[VEC], prox[VEC], old[VEC], adv[VEC], ent[VEC], x0[VEC], x1[VEC];
   bool m[VEC];
-  load_mask<VEC>(io.mask, t, m);
-  load_f32<VEC>(io.prox, t, prox);
-  load_f32<VEC>(io.old, t, old);
-  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.lp, t, lp);
-  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.adv, t, adv);
-  load_f32<VEC>(STATS ? io.entropy : nullptr, t, ent);
-  load_f32<VEC>(STATS ? io.extra0 : nullptr, t, x0);
-  load_f32<VEC>(STATS ? io.extra1 : nullptr, t, x1);
+};
+template <bool STATS, int VEC>
+DEVI void token_group_load(const LossIO& io, const LossCfg& c, int64_t t, TokenLoad<VEC>& in) {
+  load_mask<VEC>(io.mask, t, in.m);
+  load_f32<VEC>(io.prox, t, in.prox);
+  load_f32<VEC>(io.old, t, in.old);
+  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.lp, t, in.lp);
+  load_f32<VEC>(c.loss_kind == LOSS_NONE ? nullptr : io.adv, t, in.adv);
+  load_f32<VEC>(STATS ? io.entropy : nullptr, t, in.ent);
+  load_f32<VEC>(STATS ? io.extra0 : nullptr, t, in.x0);
+  load_f32<VEC>(STATS ? io.extra1 : nullptr, t, in.x1);
+}
+template <bool STATS, int VEC>
+DEVI void token_group_compute(const LossIO& io, const LossCfg& c, int64_t t, const TokenLoad<VEC>& ld,
+                              TokenAcc& acc, StatAcc<STATS>& st) {
   float dlp[VEC], loss[VEC], ratio[VEC], kl[VEC], bw[VEC], bkl[VEC];
   bool clip[VEC], dual[VEC], m2[VEC], bm[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
-    const TokenIn in{lp[i], prox[i], old[i], adv[i], ent[i], x0[i], x1[i], m[i]};
+    const TokenIn in{ld.lp[i], ld.prox[i], ld.old[i], ld.adv[i], ld.ent[i], ld.x0[i], ld.x1[i], ld.m[i]};
     TokenOut o;
     token_body<STATS>(io, c, t + i, in, o, acc, st);
     dlp[i] = o.dlp; loss[i] = o.loss; ratio[i] = o.ratio; kl[i] = o.kl; bw[i] = o.behave_w; bkl[i] = o.behave_kl;
     clip[i] = o.clip; dual[i] = o.dual; m2[i] = o.m2; bm[i] = o.bm;
   }
-  st.flush();
   if (c.rs_enabled) {
     store_mask<VEC>(io.new_mask, t, m2);
     store_f32<VEC>(io.behave_w, t, bw);
@@ -552,8 +557,16 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
   const int64_t n_vec = io.n - io.n % VEC;
-  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) token_group<STATS, VEC>(io, c, t, acc, st);
-  if (VEC > 1 && n_vec + gid < io.n) token_group<STATS, 1>(io, c, n_vec + gid, acc, st);
+  TokenLoad<VEC> in;
+  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) {
+    token_group_load<STATS, VEC>(io, c, t, in);
+    token_group_compute<STATS, VEC>(io, c, t, in, acc, st);
+  }
+  if (VEC > 1 && n_vec + gid < io.n) {
+    TokenLoad<1> tail;
+    token_group_load<STATS, 1>(io, c, n_vec + gid, tail);
+    token_group_compute<STATS, 1>(io, c, n_vec + gid, tail, acc, st);
+  }
 
   const double loss_sum = block_sum(acc.loss_sum, sm_d);
   const long long n_valid = block_sum((long long)acc.n_valid, sm_l);
@@ -573,7 +586,7 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
     for (int k = 0; k < N_LOSS_STATS; ++k) {
-      const double sv = wave_sum(st.sum[k]);
+      const double sv = wave_sum((double)st.sum[k]);
       float mn = st.mn[k], mx = st.mx[k];
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) {
@@ -604,20 +617,29 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
 // The three 0/1-valued statistics are not reduced per token: their sums are token counts and
 // their extremes follow from whether every / any counted token has the value 1. Each block sums
 // the counts it needs itself, so one launch does everything.
-__global__ __launch_bounds__(LOSS_THREADS) void loss_finalize_kernel(
+__global__ __launch_bounds__(FINAL_THREADS) void loss_finalize_kernel(
     const Partial* __restrict__ partials, const StatPartial* __restrict__ stat_partials, int nparts,
     float* loss_out, double* __restrict__ counters, double n_tokens, double* __restrict__ stats,
     int loss_active, int rs_enabled) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
-  __shared__ float sm_f[8];
+  __shared__ float sm_f[2 * (FINAL_THREADS / 64)];
   double ls = 0.0;
   long long a[6] = {0, 0, 0, 0, 0, 0};
-  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
-    const Partial p = partials[i];
-    ls += p.loss_sum;
-    a[0] += p.n_valid; a[1] += p.n_kept; a[2] += p.n_filtered;
-    a[3] += p.n_clip; a[4] += p.n_dual; a[5] += p.n_behave;
+  // the thread's partials are fetched together (one memory latency, not one per partial) and
+  // added in index order
+  constexpr int PER_THREAD = MAX_LOSS_BLOCKS / FINAL_THREADS;
+  Partial pp[PER_THREAD];
+#pragma unroll
+  for (int j = 0; j < PER_THREAD; ++j) {
+    const int i = threadIdx.x + j * FINAL_THREADS;
+    pp[j] = i < nparts ? partials[i] : Partial{0.0, 0, 0, 0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int j = 0; j < PER_THREAD; ++j) {
+    ls += pp[j].loss_sum;
+    a[0] += pp[j].n_valid; a[1] += pp[j].n_kept; a[2] += pp[j].n_filtered;
+    a[3] += pp[j].n_clip; a[4] += pp[j].n_dual; a[5] += pp[j].n_behave;
   }
   ls = block_sum(ls, sm_d);
   for (int k = 0; k < 6; ++k) a[k] = block_sum(a[k], sm_l);
@@ -662,10 +684,12 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_finalize_kernel(
     }
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     __syncthreads();
-    if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
+    constexpr int NW = FINAL_THREADS / 64;
+    if (lane == 0) { sm_f[w] = mn; sm_f[NW + w] = mx; }
     __syncthreads();
-    mn = stat_min(stat_min(sm_f[0], sm_f[1]), stat_min(sm_f[2], sm_f[3]));
-    mx = stat_max(stat_max(sm_f[4], sm_f[5]), stat_max(sm_f[6], sm_f[7]));
+    mn = sm_f[0]; mx = sm_f[NW];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) { mn = stat_min(mn, sm_f[i]); mx = stat_max(mx, sm_f[NW + i]); }
   }
   if (threadIdx.x == 0) {
     stats[4 * k + 0] = sum;
@@ -925,7 +949,9 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
   io.extra0 = with_stats ? sa->extra0 : nullptr;
   io.extra1 = with_stats ? sa->extra1 : nullptr;
 
-  const bool vec4 = aligned_to(logprobs, 16) && aligned_to(proximal, 16) && aligned_to(old_logprobs, 16) &&
+  // four tokens per thread once that still gives every CU a block; a smaller batch is bound by
+  // latency, not by bandwidth, and runs faster spread over four times as many threads
+  const bool vec4 = n_tokens >= (int64_t)4 * LOSS_THREADS * 256 && aligned_to(logprobs, 16) && aligned_to(proximal, 16) && aligned_to(old_logprobs, 16) &&
                     aligned_to(advantages, 16) && aligned_to(dlogprobs, 16) && aligned_to(stat_loss, 16) &&
                     aligned_to(stat_ratio, 16) && aligned_to(stat_approx_kl, 16) &&
                     aligned_to(behave_imp_weight, 16) && aligned_to(behave_approx_kl, 16) &&
@@ -962,7 +988,7 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
   }
   token_pass(io, c, with_stats);
   AREAL_CHECK_LAUNCH();
-  hipLaunchKernelGGL(loss_finalize_kernel, dim3(with_stats ? 1 + N_LOSS_STATS : 1), dim3(LOSS_THREADS), 0, stream,
+  hipLaunchKernelGGL(loss_finalize_kernel, dim3(with_stats ? 1 + N_LOSS_STATS : 1), dim3(FINAL_THREADS), 0, stream,
                      partials, stat_partials, grid, loss, counters, (double)n_tokens,
                      with_stats ? sa->stats : nullptr, c.loss_kind != LOSS_NONE ? 1 : 0, c.rs_enabled);
   AREAL_CHECK_LAUNCH();
@@ -979,7 +1005,7 @@ int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const d
   if (n_tokens < 0) return AREAL_ERR_BAD_ARG;
   if (n_tokens == 0) return AREAL_OK;
   if (!dlogprobs || !upstream || !counters || !grad_logprobs) return AREAL_ERR_BAD_ARG;
-  if (aligned_to(dlogprobs, 16) && aligned_to(grad_logprobs, 16))
+  if (n_tokens >= (int64_t)4 * LOSS_THREADS * 256 && aligned_to(dlogprobs, 16) && aligned_to(grad_logprobs, 16))
     hipLaunchKernelGGL(loss_grad_scale_kernel<4>, dim3(loss_grid(n_tokens, 4)), dim3(LOSS_THREADS), 0,
                        stream, dlogprobs, upstream, counters, grad_logprobs, n_tokens);
   else

@@ -147,6 +147,8 @@ class FusedLMHeadAdapter:
         self.compute_dtype = compute_dtype
         self.fuse_wgrad_accumulation = fuse_wgrad_accumulation
         self.save_probs = save_probs
+        self._compute_copy_key = None
+        self._compute_copy_value = None
 
     # -- pieces --------------------------------------------------------------------------
     def hidden_states(self, model_inputs: dict[str, Any]) -> torch.Tensor:
@@ -157,11 +159,24 @@ class FusedLMHeadAdapter:
             hidden = hidden.squeeze(0)
         return hidden.to(self.compute_dtype)
 
+    def _compute_copy(self, param: torch.Tensor) -> torch.Tensor:
+        """Detached compute-dtype copy of the master weight, made once per version of the
+        parameter: the micro-batches of a step (and forward-only calls between optimizer steps)
+        share it, and an in-place update of the parameter (the optimizer's) bumps its version
+        counter and invalidates it.  At Qwen3-8B size the cast reads 2.5 GB and writes 1.2 GB."""
+        key = (param.data_ptr(), param._version, tuple(param.shape), param.device)
+        if self._compute_copy_key != key:
+            self._compute_copy_value = param.detach().to(self.compute_dtype)
+            self._compute_copy_key = key
+        return self._compute_copy_value
+
     def _weight(self, hidden: torch.Tensor):
         """(compute copy of lm_head.weight, fp32 accumulator or None)."""
         param = self.module.lm_head.weight
         if param.dtype == self.compute_dtype:
             return param, None
+        if not torch.is_grad_enabled():
+            return self._compute_copy(param), None
         fused = (
             self.fuse_wgrad_accumulation
             and param.dtype == torch.float32
@@ -173,7 +188,7 @@ class FusedLMHeadAdapter:
             return param.to(self.compute_dtype), None  # autograd casts the gradient back
         if param.grad is None:
             param.grad = torch.zeros_like(param, memory_format=torch.contiguous_format)
-        return param.detach().to(self.compute_dtype), param.grad
+        return self._compute_copy(param), param.grad
 
     def _bias(self):
         return getattr(self.module.lm_head, "bias", None)

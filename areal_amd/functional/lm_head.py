@@ -110,6 +110,7 @@ class _FusedLMHead(torch.autograd.Function):
             save_probs = need <= SAVE_PROBS_BYTES_LIMIT and need <= 0.6 * _available_bytes(dev)
         probs = probs_ref = probs_status = None
         if save_probs and needs_grad and T > 0:
+            # rows padded to 128, columns to 64: areal_lmhead_probs_bytes(T, V)
             probs = torch.empty(
                 (_round_up(T, 128), _round_up(V, 64)), dtype=torch.bfloat16, device=dev
             )
@@ -123,7 +124,8 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(bias_f), _lib.ptr(labels_1d),
                 T, H, V, 1.0 / temperature, logit_scale,
                 *[_lib.ptr(o) for o in outs],
-                _lib.ptr(probs), _lib.ptr(probs_ref), _lib.ptr(probs_status),
+                _lib.ptr(probs), probs.numel() * 2 if probs is not None else 0,
+                _lib.ptr(probs_ref), _lib.ptr(probs_status),
                 _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
             )
             _lib.check(rc, "areal_lmhead_fwd")
@@ -207,7 +209,7 @@ class _FusedLMHead(torch.autograd.Function):
                 _lib.ptr(hidden_2d), _lib.ptr(weight_c), _lib.ptr(labels_1d),
                 _lib.ptr(row_max), _lib.ptr(sum_exp), _lib.ptr(ctx.label_logprobs), _lib.ptr(g),
                 T, H, V, 1.0 / ctx.temperature, ctx.logit_scale,
-                _lib.ptr(probs), _lib.ptr(probs_ref), _lib.ptr(probs_status),
+                _lib.ptr(probs), probs.numel() * 2, _lib.ptr(probs_ref), _lib.ptr(probs_status),
                 _lib.ptr(dh), _lib.ptr(dw_direct if direct else dw32),
                 2 if direct else (1 if accum is not None else 0),
                 _lib.ptr(db32), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),

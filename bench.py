@@ -13,6 +13,7 @@ import argparse
 import functools
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -79,6 +80,40 @@ def make_batch(name: str, device):
         cu_seqlens=cu.to(device), loss_mask=loss_mask.to(device), advantages=advantages.to(device),
         T=T, H=H, V=V_QWEN, seed=w["seed"],
     )
+
+
+def make_batch_on_device(name: str, device):
+    """The same shapes and distributions drawn with the device's generator (seeded): used for the
+    secondary workloads, whose host-side generation would take longer than their timed steps."""
+    import torch
+
+    w = WORKLOADS[name]
+    T, H = w["T"], w["H"]
+    g = torch.Generator().manual_seed(w["seed"])
+    lens = torch.randint(w["lo"], w["hi"] + 1, (w["n_seqs"],), generator=g)
+    if int(lens.sum()) > T:
+        lens = torch.clamp((lens.double() * T / lens.sum()).floor().long(), min=w["lo"])
+        while int(lens.sum()) > T:
+            lens[lens.argmax()] -= 1
+    pad = T - int(lens.sum())
+    seg = lens.tolist() + ([pad] if pad > 0 else [])
+    cu = torch.tensor([0] + torch.tensor(seg).cumsum(0).tolist(), dtype=torch.int32)
+    loss_mask = torch.ones(T, dtype=torch.bool)
+    loss_mask[cu[1 : w["n_seqs"] + 1].long() - 1] = False
+    if pad > 0:
+        loss_mask[T - pad :] = False
+    gd = torch.Generator(device=device).manual_seed(w["seed"])
+    hidden = torch.randn(T, H, generator=gd, device=device, dtype=torch.float32).bfloat16()
+    weight = torch.empty(V_QWEN, H, dtype=torch.bfloat16, device=device)
+    for i in range(0, V_QWEN, 32768):  # chunked to bound the fp32 temporaries
+        n = min(32768, V_QWEN - i)
+        weight[i : i + n] = (torch.randn(n, H, generator=gd, device=device) * 0.02).bfloat16()
+    labels = torch.randint(0, V_QWEN, (T,), generator=gd, device=device)
+    adv_seq = torch.randn(len(seg), generator=g)
+    advantages = adv_seq.repeat_interleave(torch.tensor(seg))
+    return dict(hidden=hidden, weight=weight, labels=labels, cu_seqlens=cu.to(device),
+                loss_mask=loss_mask.to(device), advantages=advantages.to(device), T=T, H=H, V=V_QWEN,
+                seed=w["seed"])
 
 
 def cpu_baseline(sample_tokens: int, H: int, seed: int, threads: int, repeats: int = 3):
@@ -429,6 +464,10 @@ def main() -> None:
                     help="skip timing torch.mm (the vendor library's bf16 GEMM) at the forward's shape")
     ap.add_argument("--no-other-mode", action="store_true",
                     help="skip the short second leg that times the other backward mode")
+    ap.add_argument("--only-hbm-kernels", action="store_true",
+                    help="time only the HBM-bound kernels (prints {\"hbm_rooflines\": [...]})")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short legs on the other BASELINE shapes (configs 1, 2 and 5)")
     ap.add_argument("--recompute", action="store_true",
                     help="backward recomputes the logits (save_probs=False) instead of using the "
                          "bf16 exponentials kept by the forward")
@@ -447,74 +486,85 @@ def main() -> None:
         sys.exit("bench.py needs an MI355X: the hot path has no CPU implementation")
     _lib.load()
     dev = torch.device("cuda:0")
-    b = make_batch(args.workload, dev)
-    T, H, V = b["T"], b["H"], b["V"]
-    hidden = b["hidden"].requires_grad_(True)
-    weight = b["weight"].requires_grad_(True)
+    if args.only_hbm_kernels:
+        print(json.dumps({"hbm_rooflines": hbm_rooflines(dev)}))
+        return
 
-    # rollout log-probs = train log-probs + Laplace(0, 0.1); proximal = train log-probs
-    with torch.no_grad():
-        logp0 = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0).logprobs
-    torch.manual_seed(b["seed"])
-    old = logp0 + torch.distributions.Laplace(0.0, 0.1).sample((T,)).to(dev)
-    input_data = dict(logprobs=old, advantages=b["advantages"], loss_mask=b["loss_mask"],
-                      prox_logp=logp0, cu_seqlens=b["cu_seqlens"])
-    loss_fn = functools.partial(
-        grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None,
-        rejection_sampling=RejectionSamplingConfig(level="token", action="mask", metric="ratio",
-                                                   lower=0.5, upper=2.0),
-        # the step is queued without waiting for the GPU: the loss's host scalars are read after
-        # the backward is queued (nothing is skipped on the device)
-        defer_host_reads=True,
-    )
+    class Workload:
+        """One packed micro-batch resident in HBM and the step that is timed on it: fused
+        forward, GRPO loss with IcePop masking, backward to dHidden and dWeight."""
 
-    # None: keep the exponentials if the bf16 [T, V] buffer fits the library's default limit
-    saved = False
+        def __init__(self, b):
+            self.b = b
+            self.T, self.H, self.V = b["T"], b["H"], b["V"]
+            self.hidden = b["hidden"].requires_grad_(True)
+            self.weight = b["weight"].requires_grad_(True)
+            # rollout log-probs = train log-probs + Laplace(0, 0.1); proximal = train log-probs
+            with torch.no_grad():
+                logp0 = fused_lm_head_logprobs_entropy(self.hidden, self.weight, b["labels"], temperature=1.0).logprobs
+            torch.manual_seed(b["seed"])
+            old = logp0 + torch.distributions.Laplace(0.0, 0.1).sample((self.T,)).to(dev)
+            self.input_data = dict(logprobs=old, advantages=b["advantages"], loss_mask=b["loss_mask"],
+                                   prox_logp=logp0, cu_seqlens=b["cu_seqlens"])
+            self.loss_fn = functools.partial(
+                grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None,
+                rejection_sampling=RejectionSamplingConfig(level="token", action="mask", metric="ratio",
+                                                           lower=0.5, upper=2.0),
+                # the step is queued without waiting for the GPU: the loss's host scalars are read
+                # after the backward is queued (nothing is skipped on the device)
+                defer_host_reads=True,
+            )
+            self.saved = False
 
-    def run_steps(n_steps: int, n_warm: int, save_probs):
-        """n_warm untimed steps, then n_steps timed ones between two synchronisations. The
-        phase times come from HIP events recorded on the launch stream (read after the last
-        step, so nothing waits on the host inside the timed region)."""
-        nonlocal saved
-        evs = []
-
-        def step(record: bool):
-            nonlocal saved
-            hidden.grad = None
-            weight.grad = None
+        def step(self, record: bool, save_probs, accum=None):
+            self.hidden.grad = None
+            self.weight.grad = None
             ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if record else None
             if record:
                 ev[0].record()
-            out = fused_lm_head_logprobs_entropy(hidden, weight, b["labels"], temperature=1.0,
-                                                 save_probs=save_probs)
-            saved = out.logprobs.grad_fn.probs is not None
+            out = fused_lm_head_logprobs_entropy(self.hidden, self.weight, self.b["labels"], temperature=1.0,
+                                                 save_probs=save_probs, weight_grad_accum=accum)
+            self.saved = out.logprobs.grad_fn.probs is not None
             if record:
                 ev[1].record()
-            loss = loss_fn(out.logprobs, out.entropy, input_data,
-                           vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
+            loss = self.loss_fn(out.logprobs, out.entropy, self.input_data,
+                                vocab_min_logits=out.vocab_min_logits, vocab_max_logits=out.vocab_max_logits)
             if record:
                 ev[2].record()
             loss.backward()
             if record:
                 ev[3].record()
+            return loss, ev
+
+        def run(self, n_steps: int, n_warm: int, save_probs, accum=None):
+            """n_warm untimed steps, then n_steps timed ones between two synchronisations. The
+            phase times come from HIP events recorded on the launch stream (read after the last
+            step, so nothing waits on the host inside the timed region)."""
+            evs = []
+            for _ in range(n_warm):
+                self.step(False, save_probs, accum)
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            t0 = time.perf_counter()
+            for _ in range(n_steps):
+                loss, ev = self.step(True, save_probs, accum)
                 evs.append(ev)
-            return loss
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+            phases = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) for i in range(3)]
+            return wall, phases, loss, torch.cuda.max_memory_allocated() / 1e9
 
-        for _ in range(n_warm):
-            step(False)
-        torch.cuda.synchronize()
-        torch.cuda.reset_peak_memory_stats()
-        t0 = time.perf_counter()
-        for _ in range(n_steps):
-            loss = step(True)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        phases = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) for i in range(3)]
-        return wall, phases, loss, torch.cuda.max_memory_allocated() / 1e9
+        def frac(self, ms_per_step: float) -> float:
+            return 6.0 * self.T * self.H * self.V / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
 
-    wall, (t_fwd, t_loss, t_bwd), loss, peak_hbm_gb = run_steps(
+    wl = Workload(make_batch(args.workload, dev))
+    b, T, H, V = wl.b, wl.T, wl.H, wl.V
+    hidden, weight, input_data, loss_fn = wl.hidden, wl.weight, wl.input_data, wl.loss_fn
+
+    # save_probs None: keep the exponentials if the bf16 [T, V] buffer fits the library's default limit
+    wall, (t_fwd, t_loss, t_bwd), loss, peak_hbm_gb = wl.run(
         args.steps, args.warmup, False if args.recompute else None)
-    main_saved = saved
+    saved = main_saved = wl.saved
     ms_per_step = wall * 1e3 / args.steps
     tokens_per_s = T * args.steps / wall
 
@@ -525,16 +575,30 @@ def main() -> None:
     other = None
     if not args.no_other_mode:
         n_other = max(1, min(args.steps, 5))
-        o_wall, o_ph, _, o_peak = run_steps(n_other, 1, None if args.recompute else False)
+        o_wall, o_ph, _, o_peak = wl.run(n_other, 1, None if args.recompute else False)
         other = {
-            "backward": "saved bf16 exponentials" if saved else "recompute logits",
+            "backward": "saved bf16 exponentials" if wl.saved else "recompute logits",
             "steps": n_other, "ms_per_step": o_wall * 1e3 / n_other,
-            "frac": 6.0 * T * H * V / (o_wall / n_other) / 1e12 / PEAK_BF16_TFLOPS,
+            "frac": wl.frac(o_wall * 1e3 / n_other),
             "peak_hbm_gb": o_peak,
             "ms": {"lmhead_fwd": o_ph[0] / n_other, "loss_fwd": o_ph[1] / n_other,
                    "loss_bwd+lmhead_bwd": o_ph[2] / n_other},
         }
     saved = main_saved
+
+    # The route an engine with fp32 master weights takes (FusedLMHeadAdapter's default, Megatron's
+    # main_grad, vocab_parallel_head.py:870-876): dWeight is ADDED to an fp32 [V, H] buffer by the
+    # contraction's epilogue instead of being stored as bf16.
+    fp32_accum = None
+    if not args.no_other_mode and not args.recompute:
+        n_acc = max(1, min(args.steps, 5))
+        acc = torch.zeros(V, H, dtype=torch.float32, device=dev)
+        a_wall, a_ph, _, a_peak = wl.run(n_acc, 1, None, accum=acc)
+        fp32_accum = {"steps": n_acc, "ms_per_step": a_wall * 1e3 / n_acc, "frac": wl.frac(a_wall * 1e3 / n_acc),
+                      "peak_hbm_gb": a_peak,
+                      "ms": {"lmhead_fwd": a_ph[0] / n_acc, "loss_fwd": a_ph[1] / n_acc,
+                             "loss_bwd+lmhead_bwd": a_ph[2] / n_acc}}
+        del acc
 
     # The two backward contractions on their own (median of three): a backward that asks for one
     # gradient launches one contraction, next to the loss backward and the operand preparation
@@ -625,10 +689,40 @@ def main() -> None:
         traffic_source = ("offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command "
                           "(profiles/lmhead_contraction_qwen3-8b.md), mean of the three contraction "
                           "launches; not re-measured by this run")
-    missing = [k for k in (KERNEL_FWD_SAVE, KERNEL_FWD, KERNEL_DHIDDEN, KERNEL_DWEIGHT, KERNEL_RECOMPUTE)
-               if not _lib.has_kernel(k)]
+    final_loss = float(loss.detach().item())
+    # The kernel names this line reports, checked against the loaded library (tests/test_bench_contract.py
+    # makes the same check a hard failure); a box without a symbol demangler still gets its line.
+    try:
+        missing = [k for k in (KERNEL_FWD_SAVE, KERNEL_FWD, KERNEL_DHIDDEN, KERNEL_DWEIGHT, KERNEL_RECOMPUTE)
+                   if not _lib.has_kernel(k)]
+        kernel_names_checked = True
+    except (OSError, subprocess.SubprocessError):
+        missing, kernel_names_checked = [], False
     if missing:
         sys.exit(f"bench.py names kernels that the loaded library does not contain: {missing}")
+
+    # The other BASELINE shapes, a short timed leg each (same step, saved-exponentials mode), after
+    # the default workload's tensors are released. Drawn on the device; small shapes get more
+    # warm-up steps (the caching allocator takes a few steps to stop re-splitting its blocks).
+    other_workloads = []
+    if not args.no_other_workloads and args.workload == "qwen3-8b":
+        del wl, b, hidden, weight, input_data, loss_fn, loss
+        torch.cuda.empty_cache()
+        for name, n_steps, n_warm in (("qwen2.5-0.5b", 40, 20), ("qwen2.5-1.5b", 20, 10), ("qwen3-14b-128k", 3, 1)):
+            w2 = Workload(make_batch_on_device(name, dev))
+            w_wall, w_ph, _, w_peak = w2.run(n_steps, n_warm, None)
+            ms = w_wall * 1e3 / n_steps
+            other_workloads.append({
+                "workload": f"{name}: {WORKLOADS[name]['desc']}", "tokens": w2.T, "hidden": w2.H, "vocab": w2.V,
+                "steps": n_steps, "warmup": n_warm, "ms_per_step": ms, "value": w2.T / (ms * 1e-3),
+                "unit": "tokens/s", "frac": w2.frac(ms),
+                "backward": "saved bf16 exponentials" if w2.saved else "recompute logits", "peak_hbm_gb": w_peak,
+                "ms": {"lmhead_fwd": w_ph[0] / n_steps, "loss_fwd": w_ph[1] / n_steps,
+                       "loss_bwd+lmhead_bwd": w_ph[2] / n_steps},
+            })
+            del w2
+            torch.cuda.empty_cache()
+        wl = None
 
     result = {
         "metric": "packed tokens/sec, logprob+entropy+PPO loss fwd+bwd; % bf16 MFMA peak",
@@ -647,7 +741,7 @@ def main() -> None:
             "workload": f"{args.workload}: {WORKLOADS[args.workload]['desc']}",
             "tokens": T, "hidden": H, "vocab": V,
             "loss": "PPO clip eps=0.2, rejection sampling ratio in [0.5, 2.0] (token, mask)",
-            "final_loss": float(loss.detach().item()),
+            "final_loss": final_loss,
             "host_reads": "deferred (grpo_loss_fn(defer_host_reads=True): no host wait between the launches of a step)",
             "backward": "saved bf16 exponentials" if saved else "recompute logits",
             "peak_hbm_gb": peak_hbm_gb,
@@ -673,10 +767,14 @@ def main() -> None:
             "backward_split_ms": backward_split,
             "other_backward_mode": other,
             "recompute_mode_ms": (ms_per_step if not saved else (other["ms_per_step"] if other else None)),
+            "fp32_wgrad_accum": fp32_accum,
+            "fp32_wgrad_accum_ms": fp32_accum["ms_per_step"] if fp32_accum else None,
+            "kernel_names_checked": kernel_names_checked,
         },
+        "other_workloads": other_workloads,
     }
     if not args.no_hbm_kernels:
-        del hidden, weight, b, input_data, old, logp0
+        wl = b = hidden = weight = input_data = loss_fn = loss = None
         torch.cuda.empty_cache()
         result["hbm_rooflines"] = hbm_rooflines(dev)
     if not args.no_cpu_baseline:

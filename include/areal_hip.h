@@ -24,6 +24,15 @@ extern "C" {
 
 typedef struct ihipStream_t* areal_stream_t; /* a hipStream_t */
 
+/* Version of this interface. It moves whenever an entry point's argument list or the size of a
+ * caller-allocated buffer changes; a caller built against another number must not call in.
+ * areal_abi_version() returns the number the loaded library was built with.
+ *   3: areal_lmhead_fwd / areal_lmhead_bwd_saved take probs_bytes and check it against
+ *      areal_lmhead_probs_bytes() (the buffer's rows are padded to 128, and
+ *      areal_lmhead_bwd_saved takes probs_status). */
+#define AREAL_HIP_ABI_VERSION 3
+int areal_abi_version(void);
+
 enum areal_status {
   AREAL_OK = 0,
   AREAL_ERR_BAD_ARG = -1,
@@ -42,6 +51,10 @@ enum areal_status {
 
 size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 
+/* Bytes of the bf16 buffer of saved softmax exponentials (`probs` below):
+ * round_up(T, 128) rows of round_up(V, 64) columns. */
+size_t areal_lmhead_probs_bytes(int64_t T, int64_t V);
+
 /* hidden [T,H] bf16, weight [V,H] bf16 (H % 8 == 0, 16-byte aligned), bias [V] fp32 or NULL,
  * labels [T] int64. Outputs fp32 [T]; row_max and sum_exp are the state saved for backward
  * (vocab_parallel_head.py:704-713). logits = (hidden . weight^T + bias) * logit_scale.
@@ -50,7 +63,9 @@ size_t areal_lmhead_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * exponentials for areal_lmhead_bwd_saved, the counterpart of autograd saving the logits in the
  * reference's logits-in path (_gather_logprobs_entropy,
  * areal/utils/functional/vocab_parallel.py:24-30): probs is bf16
- * [round_up(T,128)][round_up(V,64)] holding 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
+ * [round_up(T,128)][round_up(V,64)] (probs_bytes = its size in bytes, at least
+ * areal_lmhead_probs_bytes(T, V), else AREAL_ERR_WORKSPACE) holding
+ * 2^(x / T * log2(e) - probs_ref[t]); probs_ref is
  * fp32 [T], a per-row reference estimated from a few logits of the row (its label's among
  * them) before the sweep; *probs_status (one int32 on the device) is written 0 when every
  * row's exponentials are in range, 1 when some row's maximum lies more than 100 binades (69 nats
@@ -62,8 +77,8 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
                      float inv_temperature, float logit_scale, float* logprobs, float* entropy,
                      float* vocab_min, float* vocab_max, float* vocab_mean, float* vocab_norm,
-                     float* row_max, float* sum_exp, void* probs, float* probs_ref,
-                     int* probs_status, void* workspace, size_t workspace_bytes,
+                     float* row_max, float* sum_exp, void* probs, size_t probs_bytes,
+                     float* probs_ref, int* probs_status, void* workspace, size_t workspace_bytes,
                      areal_stream_t stream);
 
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk);
@@ -89,7 +104,8 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
  * chunk to save memory; an MI355X has the HBM to keep them) and no pass rewrites the [T, V]
  * buffer: dlogits[t][:] = f[t] * probs[t][:] with a per-row factor that dHidden applies to its
  * output rows and dWeight to the hidden states. Only the label's entry of each row of probs is
- * rewritten, so probs can be used once. logprobs (NULL allowed) are the forward's label
+ * rewritten (and rows [T, round_up(T, 128)) are cleared), so probs can be used once; probs_bytes
+ * as in areal_lmhead_fwd. logprobs (NULL allowed) are the forward's label
  * log-probabilities: with them the label's dlogit is -expm1(logprob) in fp32. dweight [V,H]:
  * dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store; dbias [V] fp32 or NULL
  * (added to in mode 1). Other arguments as areal_lmhead_bwd; the bias itself does not enter (it
@@ -100,7 +116,7 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V);
 int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t* labels,
                            const float* row_max, const float* sum_exp, const float* logprobs,
                            const float* grad_logprobs, int64_t T, int64_t H, int64_t V,
-                           float inv_temperature, float logit_scale, void* probs,
+                           float inv_temperature, float logit_scale, void* probs, size_t probs_bytes,
                            const float* probs_ref, const int* probs_status, void* dhidden, void* dweight,
                            int dweight_mode, float* dbias, void* workspace,
                            size_t workspace_bytes, areal_stream_t stream);

@@ -160,6 +160,32 @@ def test_adapter_bf16_parameters_get_bf16_gradients_and_bad_modules_are_refused(
         FusedLMHeadAdapter(nn.Linear(4, 4))
 
 
+def test_adapter_reuses_the_bf16_compute_copy_until_the_master_weight_changes(dev):
+    """The bf16 copy of an fp32 master lm_head.weight is made once per version of the parameter:
+    micro-batches and forward-only calls share it; an in-place update (an optimizer step) makes
+    the next call cast again, and the log-probabilities follow the new weights."""
+    torch.manual_seed(3)
+    lm = ToyLM().to(dev)
+    adapter = FusedLMHeadAdapter(lm)
+    sp = _micro_batch(192, 0, 4)
+    inputs = dict(input_ids=sp["ids"].to(dev))
+    lp0 = adapter.compute_logprobs(inputs)
+    copy0 = adapter._compute_copy_value
+    assert copy0.dtype == torch.bfloat16 and torch.equal(copy0, lm.lm_head.weight.detach().bfloat16())
+    mb = dict(logprobs=lp0 + sp["noise"].to(dev), advantages=sp["adv"].to(dev), loss_mask=sp["mask"].to(dev),
+              prox_logp=lp0)
+    loss_fn = functools.partial(grpo_loss_fn, eps_clip=0.2, eps_clip_higher=None, c_clip=None)
+    adapter.forward_backward_batch([dict(model_inputs=inputs, mb_input=mb)] * 2, loss_fn, _weight_fn)
+    assert adapter._compute_copy_value is copy0  # forward-only call and both micro-batches: one cast
+    assert torch.equal(adapter.compute_logprobs(inputs), lp0)
+    with torch.no_grad():
+        lm.lm_head.weight.mul_(1.5)  # what an optimizer step does: in place, the version counter moves
+    lp1 = adapter.compute_logprobs(inputs)
+    assert adapter._compute_copy_value is not copy0
+    assert torch.equal(adapter._compute_copy_value, lm.lm_head.weight.detach().bfloat16())
+    assert not torch.allclose(lp1, lp0)
+
+
 def test_step_is_queued_without_waiting_for_the_gpu(dev):
     """Forward, loss and backward of one micro-batch with deferred host reads: no call of the
     step may synchronise with the device before its last launch is queued (the saved-mode

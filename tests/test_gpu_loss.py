@@ -347,6 +347,6 @@ def test_reduced_stats_agree_with_the_tensor_mode_on_the_gpu(dev):
                              {"behave_imp_weight": t["unclipped_behave_tokens"]}))
     for k, w in want.items():
         assert r[k]["count"] == w["count"]
-        # the token pass adds the four tokens of one access in fp32 before its fp64 running sum
+        # a thread of the token pass adds its few tokens in fp32; from the wave level on sums are fp64
         assert r[k]["sum"] == pytest.approx(w["sum"], rel=1e-6, abs=1e-6), k
         assert r[k]["min"] == w["min"] and r[k]["max"] == w["max"], k
