@@ -80,7 +80,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_aux_loss_workspace_bytes": (SZ, [I64, I64]),
     "areal_sapo_loss": (
         I,
-        [P, P, P, P, P, I64, I64, I64, F, F, I, P, P, P, P, P, P, P, P, P, P, SZ, P],
+        [P, P, P, P, P, I64, I64, I64, F, F, I, P, P, P, P, P, P, P, P, P, P, P, P, P, P, SZ, P],
     ),
     "areal_critic_loss": (I, [P, P, P, P, I64, F, I, P, P, P, P, P, P, SZ, P]),
     "areal_m2po_mask_workspace_bytes": (SZ, [I64]),

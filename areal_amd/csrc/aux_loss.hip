@@ -28,8 +28,8 @@ DEVI T block_sum(T v, T* smem) {
   return r;
 }
 
-int aux_grid(int64_t n) {
-  int64_t b = ceil_div_i64(n, AUX_THREADS);
+int aux_grid(int64_t n, int vec = 1) {
+  int64_t b = ceil_div_i64(n, (int64_t)AUX_THREADS * vec);
   if (b > AUX_MAX_BLOCKS) b = AUX_MAX_BLOCKS;
   if (b < 1) b = 1;
   return (int)b;
@@ -60,13 +60,24 @@ struct SumCount {
   long long n_valid, n_clip;
 };
 
+// Block partial of one logged statistic.
+struct StatPart {
+  double sum;
+  float mn, mx;
+};
+
 // counters: [0] loss sum [1] masked-token count [4] clipped count [7] loss; the layout of the
 // actor loss, so that its gradient-scaling entry point serves these losses too.
 // denom_mode 0: sum / max(count, 1); 1: sum / count (0/0 = NaN, as torch); 2: sum / n_total.
-__global__ void aux_finalize_kernel(const SumCount* parts, int nparts, int denom_mode,
-                                    double n_total, float* loss_out, double* counters) {
+// With statistics (stat_parts [nparts][n_stats]), block 1 + k folds statistic k into
+// stats[k] = {sum, count, min, max}; count = the masked-token count for k < n_masked_stats, every
+// token for the rest. Each block sums the counts itself, so one launch does everything.
+__global__ __launch_bounds__(AUX_THREADS) void aux_finalize_kernel(
+    const SumCount* parts, int nparts, int denom_mode, double n_total, float* loss_out, double* counters,
+    const StatPart* __restrict__ stat_parts, int n_stats, int n_masked_stats, double* __restrict__ stats) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
+  __shared__ float sm_f[8];
   double s = 0.0;
   long long nv = 0, nc = 0;
   for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
@@ -75,6 +86,36 @@ __global__ void aux_finalize_kernel(const SumCount* parts, int nparts, int denom
   s = block_sum(s, sm_d);
   nv = block_sum(nv, sm_l);
   nc = block_sum(nc, sm_l);
+  if (blockIdx.x > 0) {
+    const int k = blockIdx.x - 1;
+    double sum = 0.0;
+    float mn = pos_inf(), mx = neg_inf();
+    for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+      const StatPart sp = stat_parts[(size_t)i * n_stats + k];
+      sum += sp.sum;
+      mn = stat_min(mn, sp.mn);
+      mx = stat_max(mx, sp.mx);
+    }
+    sum = block_sum(sum, sm_d);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      mn = stat_min(mn, __shfl_xor(mn, o, 64));
+      mx = stat_max(mx, __shfl_xor(mx, o, 64));
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      mn = stat_min(stat_min(sm_f[0], sm_f[1]), stat_min(sm_f[2], sm_f[3]));
+      mx = stat_max(stat_max(sm_f[4], sm_f[5]), stat_max(sm_f[6], sm_f[7]));
+      stats[4 * k + 0] = sum;
+      stats[4 * k + 1] = k < n_masked_stats ? (double)nv : n_total;
+      stats[4 * k + 2] = (double)mn;
+      stats[4 * k + 3] = (double)mx;
+    }
+    return;
+  }
   if (threadIdx.x == 0) {
     for (int k = 0; k < 8; ++k) counters[k] = 0.0;
     counters[0] = s;
@@ -117,7 +158,12 @@ struct SapoIO {
   float* soft_gate;
   float* gate_pos;
   float* gate_neg;
+  // optional per-token inputs of the reduced statistics
+  const float* entropy;
+  const float* extra0;
+  const float* extra1;
 };
+template <int N> struct IntTag { static constexpr int value = N; };
 
 // Per-sequence geometric-mean ratio and mean advantage over the mask (one block per sequence).
 __global__ __launch_bounds__(AUX_THREADS) void sapo_seq_kernel(SapoIO io, float* seq_stat) {
@@ -145,51 +191,132 @@ __global__ __launch_bounds__(AUX_THREADS) void sapo_seq_kernel(SapoIO io, float*
 
 DEVI float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-__global__ __launch_bounds__(AUX_THREADS) void sapo_token_kernel(SapoIO io, SumCount* parts) {
+// Statistics the token pass can reduce itself (sum, min, max per block) instead of writing the
+// per-token tensors: what grpo_loss_fn logs for a SAPO step (areal/trainer/ppo/actor.py:662-733,
+// :735-741), the first SAPO_MASKED_STATS under the loss mask, the extras over every token.
+enum {
+  SS_IMPORTANCE_WEIGHT = 0, SS_APPROX_KL, SS_NEW_LOGP, SS_OLD_LOGP, SS_ENTROPY, SS_ACTOR_LOSS, SS_LOGP_DIFF,
+  SS_LOGP_ABS_DIFF, SS_SOFT_GATE, SS_GATE_POS, SS_GATE_NEG, SS_EXTRA0, SS_EXTRA1, N_SAPO_STATS
+};
+constexpr int SAPO_MASKED_STATS = SS_EXTRA0;
+
+// VEC tokens per thread and access (see load_f32); STATS: per-thread fp32 sums and extremes of the
+// statistics above (a thread sees a few tokens; from the wave level on the sums are fp64).
+template <bool STATS, int VEC>
+__global__ __launch_bounds__(AUX_THREADS) void sapo_token_kernel(SapoIO io, SumCount* parts,
+                                                                 StatPart* stat_parts) {
   __shared__ double sm_d[8];
   __shared__ long long sm_l[8];
   double loss_sum = 0.0;
   long long n_valid = 0;
-  const float scale_pos = 4.0f / io.tau_pos, scale_neg = 4.0f / io.tau_neg;
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < io.n;
-       t += (int64_t)gridDim.x * blockDim.x) {
-    const bool m = io.mask[t] != 0;
-    const float kl = io.lp[t] - io.old[t];
-    float ratio, a, dscale;  // d ratio / d lp[t] = ratio * dscale (summed over the sequence)
-    if (io.seq_level) {
-      const int s = seq_of(io.seq, t);
-      ratio = m ? io.seq_stat[3 * s] : 0.0f;
-      a = m ? io.seq_stat[3 * s + 1] : 0.0f;
-      // every masked token of the sequence carries the same term; the sum over them of
-      // d ratio_s / d lp[t] = ratio_s / count is ratio_s
-      dscale = 1.0f;
-    } else {
-      ratio = expf(kl);
-      a = io.adv[t];
-      dscale = 1.0f;
-    }
-    const float gp = sigmoidf(io.tau_pos * (ratio - 1.0f));
-    const float gn = sigmoidf(io.tau_neg * (ratio - 1.0f));
-    const float sp = gp * scale_pos, sn = gn * scale_neg;
-    const bool pos = a > 0.0f;
-    const float gate = pos ? sp : sn;
-    const float pg = (-gate) * a;
-    // d gate / d ratio = scale * tau * g (1 - g) = 4 g (1 - g)
-    const float g = pos ? gp : gn;
-    const float dgate = 4.0f * g * (1.0f - g);
-    const float d = m ? ((-dgate) * a) * (ratio * dscale) : 0.0f;
-    if (m) { loss_sum += (double)pg; n_valid += 1; }
-    if (io.dlp) io.dlp[t] = d;
-    if (io.stat_loss) io.stat_loss[t] = pg;
-    if (io.stat_ratio) io.stat_ratio[t] = ratio;
-    if (io.stat_kl) io.stat_kl[t] = kl;
-    if (io.soft_gate) io.soft_gate[t] = gate;
-    if (io.gate_pos) io.gate_pos[t] = sp;
-    if (io.gate_neg) io.gate_neg[t] = sn;
+  float st_sum[STATS ? N_SAPO_STATS : 1], st_mn[STATS ? N_SAPO_STATS : 1], st_mx[STATS ? N_SAPO_STATS : 1];
+  if (STATS) {
+#pragma unroll
+    for (int k = 0; k < N_SAPO_STATS; ++k) { st_sum[k] = 0.f; st_mn[k] = pos_inf(); st_mx[k] = neg_inf(); }
   }
+  auto stat = [&](int k, float v) {
+    if (STATS) { st_sum[k] += v; st_mn[k] = stat_min(st_mn[k], v); st_mx[k] = stat_max(st_mx[k], v); }
+  };
+  const float scale_pos = 4.0f / io.tau_pos, scale_neg = 4.0f / io.tau_neg;
+  auto group = [&](auto vec_tag, int64_t t) {
+    constexpr int W = decltype(vec_tag)::value;
+    bool m[W];
+    float lp[W], old[W], adv[W], ent[W], x0[W], x1[W];
+    load_mask<W>(io.mask, t, m);
+    load_f32<W>(io.lp, t, lp);
+    load_f32<W>(io.old, t, old);
+    load_f32<W>(io.adv, t, adv);
+    load_f32<W>(STATS ? io.entropy : nullptr, t, ent);
+    load_f32<W>(STATS ? io.extra0 : nullptr, t, x0);
+    load_f32<W>(STATS ? io.extra1 : nullptr, t, x1);
+    float d[W], pg[W], ratio[W], kl[W], gate[W], sp[W], sn[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      kl[i] = lp[i] - old[i];
+      float a;
+      if (io.seq_level) {
+        // every masked token of the sequence carries the same term; the sum over them of
+        // d ratio_s / d lp[t] = ratio_s / count is ratio_s
+        const int s = seq_of(io.seq, t + i);
+        ratio[i] = m[i] ? io.seq_stat[3 * s] : 0.0f;
+        a = m[i] ? io.seq_stat[3 * s + 1] : 0.0f;
+      } else {
+        ratio[i] = expf(kl[i]);
+        a = adv[i];
+      }
+      const float gp = sigmoidf(io.tau_pos * (ratio[i] - 1.0f));
+      const float gn = sigmoidf(io.tau_neg * (ratio[i] - 1.0f));
+      sp[i] = gp * scale_pos;
+      sn[i] = gn * scale_neg;
+      const bool pos = a > 0.0f;
+      gate[i] = pos ? sp[i] : sn[i];
+      pg[i] = (-gate[i]) * a;
+      // d gate / d ratio = scale * tau * g (1 - g) = 4 g (1 - g)
+      const float g = pos ? gp : gn;
+      const float dgate = 4.0f * g * (1.0f - g);
+      d[i] = m[i] ? ((-dgate) * a) * ratio[i] : 0.0f;
+      if (m[i]) { loss_sum += (double)pg[i]; n_valid += 1; }
+      if (STATS) {
+        if (m[i]) {
+          stat(SS_IMPORTANCE_WEIGHT, ratio[i]);
+          stat(SS_APPROX_KL, kl[i]);
+          stat(SS_NEW_LOGP, lp[i]);
+          stat(SS_OLD_LOGP, old[i]);
+          if (io.entropy) stat(SS_ENTROPY, ent[i]);
+          stat(SS_ACTOR_LOSS, pg[i]);
+          stat(SS_LOGP_DIFF, old[i] - lp[i]);
+          stat(SS_LOGP_ABS_DIFF, fabsf(old[i] - lp[i]));
+          stat(SS_SOFT_GATE, gate[i]);
+          stat(SS_GATE_POS, sp[i]);
+          stat(SS_GATE_NEG, sn[i]);
+        }
+        if (io.extra0) stat(SS_EXTRA0, x0[i]);
+        if (io.extra1) stat(SS_EXTRA1, x1[i]);
+      }
+    }
+    store_f32<W>(io.dlp, t, d);
+    store_f32<W>(io.stat_loss, t, pg);
+    store_f32<W>(io.stat_ratio, t, ratio);
+    store_f32<W>(io.stat_kl, t, kl);
+    store_f32<W>(io.soft_gate, t, gate);
+    store_f32<W>(io.gate_pos, t, sp);
+    store_f32<W>(io.gate_neg, t, sn);
+  };
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n_vec = io.n - io.n % VEC;
+  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) group(IntTag<VEC>{}, t);
+  if (VEC > 1 && n_vec + gid < io.n) group(IntTag<1>{}, n_vec + gid);
   loss_sum = block_sum(loss_sum, sm_d);
   n_valid = block_sum(n_valid, sm_l);
   if (threadIdx.x == 0) parts[blockIdx.x] = SumCount{loss_sum, n_valid, 0};
+  if (STATS) {
+    __shared__ double sh_sum[AUX_THREADS / 64][N_SAPO_STATS];
+    __shared__ float sh_mn[AUX_THREADS / 64][N_SAPO_STATS], sh_mx[AUX_THREADS / 64][N_SAPO_STATS];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < N_SAPO_STATS; ++k) {
+      const double sv = wave_sum((double)st_sum[k]);
+      float mn = st_mn[k], mx = st_mx[k];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        mn = stat_min(mn, __shfl_xor(mn, o, 64));
+        mx = stat_max(mx, __shfl_xor(mx, o, 64));
+      }
+      if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
+    }
+    __syncthreads();
+    if (threadIdx.x < N_SAPO_STATS) {
+      const int k = threadIdx.x;
+      StatPart sp{sh_sum[0][k], sh_mn[0][k], sh_mx[0][k]};
+      for (int i = 1; i < AUX_THREADS / 64; ++i) {
+        sp.sum += sh_sum[i][k];
+        sp.mn = stat_min(sp.mn, sh_mn[i][k]);
+        sp.mx = stat_max(sp.mx, sh_mx[i][k]);
+      }
+      stat_parts[(size_t)blockIdx.x * N_SAPO_STATS + k] = sp;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -208,6 +335,7 @@ DEVI float value_loss(float x, float y, int huber, float& dx) {
   return (0.5f * e) * e;
 }
 
+template <int VEC>
 __global__ __launch_bounds__(AUX_THREADS) void critic_token_kernel(
     const float* value, const float* old_value, const float* target, const uint8_t* mask, int64_t n,
     float eps, int huber, float* dvalue, float* stat_loss, uint8_t* clip_mask, SumCount* parts) {
@@ -215,29 +343,46 @@ __global__ __launch_bounds__(AUX_THREADS) void critic_token_kernel(
   __shared__ long long sm_l[8];
   double loss_sum = 0.0;
   long long n_valid = 0, n_clip = 0;
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n;
-       t += (int64_t)gridDim.x * blockDim.x) {
-    const bool m = mask ? mask[t] != 0 : true;
-    const float v = value[t], ov = old_value[t], tg = target[t];
-    float d_orig, d_clip;
-    const float l_orig = value_loss(v, tg, huber, d_orig);
-    const float dv = v - ov;
-    const float dc = dv != dv ? dv : (dv < -eps ? -eps : (dv > eps ? eps : dv));
-    const float vc = ov + dc;
-    const float l_clip = value_loss(vc, tg, huber, d_clip);
-    // clamp passes the gradient inside the closed band; torch.max splits ties evenly
-    const float pass = (dv >= -eps && dv <= eps) ? 1.0f : 0.0f;
-    const float w_orig = l_orig > l_clip ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
-    const float w_clip = l_clip > l_orig ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
-    const float l = (l_orig != l_orig || l_clip != l_clip) ? __builtin_nanf("")
-                                                             : (l_orig > l_clip ? l_orig : l_clip);
-    const bool clip = (l_clip > l_orig) && m;
-    if (m) { loss_sum += (double)l; n_valid += 1; }
-    n_clip += clip;
-    if (dvalue) dvalue[t] = m ? (w_orig * d_orig + w_clip * (d_clip * pass)) : 0.0f;
-    if (stat_loss) stat_loss[t] = l;
-    if (clip_mask) clip_mask[t] = clip;
-  }
+  auto group = [&](auto vec_tag, int64_t t) {
+    constexpr int W = decltype(vec_tag)::value;
+    bool m[W], clip[W];
+    float v[W], ov[W], tg[W], dout[W], l[W];
+    if (mask != nullptr) {
+      load_mask<W>(mask, t, m);
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) m[i] = true;
+    }
+    load_f32<W>(value, t, v);
+    load_f32<W>(old_value, t, ov);
+    load_f32<W>(target, t, tg);
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      float d_orig, d_clip;
+      const float l_orig = value_loss(v[i], tg[i], huber, d_orig);
+      const float dv = v[i] - ov[i];
+      const float dc = dv != dv ? dv : (dv < -eps ? -eps : (dv > eps ? eps : dv));
+      const float vc = ov[i] + dc;
+      const float l_clip = value_loss(vc, tg[i], huber, d_clip);
+      // clamp passes the gradient inside the closed band; torch.max splits ties evenly
+      const float pass = (dv >= -eps && dv <= eps) ? 1.0f : 0.0f;
+      const float w_orig = l_orig > l_clip ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
+      const float w_clip = l_clip > l_orig ? 1.0f : (l_orig == l_clip ? 0.5f : 0.0f);
+      l[i] = (l_orig != l_orig || l_clip != l_clip) ? __builtin_nanf("") : (l_orig > l_clip ? l_orig : l_clip);
+      clip[i] = (l_clip > l_orig) && m[i];
+      if (m[i]) { loss_sum += (double)l[i]; n_valid += 1; }
+      n_clip += clip[i];
+      dout[i] = m[i] ? (w_orig * d_orig + w_clip * (d_clip * pass)) : 0.0f;
+    }
+    store_f32<W>(dvalue, t, dout);
+    store_f32<W>(stat_loss, t, l);
+    store_mask<W>(clip_mask, t, clip);
+  };
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const int64_t n_vec = n - n % VEC;
+  for (int64_t t = gid * VEC; t < n_vec; t += nthreads * VEC) group(IntTag<VEC>{}, t);
+  if (VEC > 1 && n_vec + gid < n) group(IntTag<1>{}, n_vec + gid);
   loss_sum = block_sum(loss_sum, sm_d);
   n_valid = block_sum(n_valid, sm_l);
   n_clip = block_sum(n_clip, sm_l);
@@ -541,18 +686,26 @@ extern "C" {
 size_t areal_aux_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs) {
   (void)n_tokens;
   if (n_seqs < 0) n_seqs = 0;
-  return (size_t)AUX_MAX_BLOCKS * sizeof(SumCount) + (size_t)n_seqs * 3 * sizeof(float) + 256;
+  return (size_t)AUX_MAX_BLOCKS * (sizeof(SumCount) + N_SAPO_STATS * sizeof(StatPart)) +
+         (size_t)n_seqs * 3 * sizeof(float) + 256;
 }
 
 // SAPO policy loss: forward, closed-form d(loss sum)/d logprobs (to be scaled with
 // areal_actor_loss_grad), per-token statistics. seq_level != 0 uses the geometric-mean ratio
 // and the mean advantage of each sequence (cu_seqlens or uniform_len).
+// stats (nullable) [13][4] double = {sum, count, min, max} of, in this order: importance_weight,
+// approx_kl, new_logp, old_logp, entropy, actor_loss, logp_diff, logp_abs_diff, sapo_soft_gate,
+// sapo_scaled_gate_pos, sapo_scaled_gate_neg (under the loss mask), extra0, extra1 (every token),
+// reduced in the token pass itself; entropy / extra0 / extra1 are optional per-token inputs of it
+// (a null one comes out as sum 0, min +inf, max -inf). With stats every per-token output may be
+// null: a caller that logs reduced values only moves 13 bytes per token in and 4 out.
 int areal_sapo_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                     const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
                     int64_t n_seqs, int64_t uniform_len, float tau_pos, float tau_neg,
                     int seq_level, float* loss, float* dlogprobs, float* stat_loss,
                     float* stat_ratio, float* stat_approx_kl, float* soft_gate, float* gate_pos,
-                    float* gate_neg, double* counters, void* workspace, size_t workspace_bytes,
+                    float* gate_neg, double* counters, const float* entropy, const float* extra0,
+                    const float* extra1, double* stats, void* workspace, size_t workspace_bytes,
                     hipStream_t stream) {
   if (n_tokens < 0 || counters == nullptr) return AREAL_ERR_BAD_ARG;
   if (!(tau_pos > 0.f) || !(tau_neg > 0.f)) return AREAL_ERR_BAD_ARG;
@@ -564,21 +717,37 @@ int areal_sapo_loss(const float* logprobs, const float* old_logprobs, const floa
     return AREAL_ERR_WORKSPACE;
   char* wp = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   SumCount* parts = (SumCount*)wp;
-  float* seq_stat = (float*)(wp + (size_t)AUX_MAX_BLOCKS * sizeof(SumCount));
+  StatPart* stat_parts = (StatPart*)(wp + (size_t)AUX_MAX_BLOCKS * sizeof(SumCount));
+  float* seq_stat = (float*)(stat_parts + (size_t)AUX_MAX_BLOCKS * N_SAPO_STATS);
+  const bool with_stats = stats != nullptr;
   SapoIO io{logprobs, old_logprobs, advantages, loss_mask,
             SeqLayout{cu_seqlens, (int)n_seqs, uniform_len}, n_tokens, tau_pos, tau_neg,
             seq_level, seq_stat, dlogprobs, stat_loss, stat_ratio, stat_approx_kl, soft_gate,
-            gate_pos, gate_neg};
-  const int grid = aux_grid(n_tokens);
+            gate_pos, gate_neg, with_stats ? entropy : nullptr, with_stats ? extra0 : nullptr,
+            with_stats ? extra1 : nullptr};
+  const bool vec4 = n_tokens >= VEC4_MIN_TOKENS && aligned_to(logprobs, 16) && aligned_to(old_logprobs, 16) &&
+                    aligned_to(advantages, 16) && aligned_to(loss_mask, 4) && aligned_to(dlogprobs, 16) &&
+                    aligned_to(stat_loss, 16) && aligned_to(stat_ratio, 16) && aligned_to(stat_approx_kl, 16) &&
+                    aligned_to(soft_gate, 16) && aligned_to(gate_pos, 16) && aligned_to(gate_neg, 16) &&
+                    aligned_to(io.entropy, 16) && aligned_to(io.extra0, 16) && aligned_to(io.extra1, 16);
+  const int grid = aux_grid(n_tokens, vec4 ? 4 : 1);
   if (seq_level && n_tokens > 0) {
     hipLaunchKernelGGL(sapo_seq_kernel, dim3((unsigned)n_seqs), dim3(AUX_THREADS), 0, stream, io,
                        seq_stat);
     AREAL_CHECK_LAUNCH();
   }
-  hipLaunchKernelGGL(sapo_token_kernel, dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts);
+  if (with_stats && vec4)
+    hipLaunchKernelGGL((sapo_token_kernel<true, 4>), dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts, stat_parts);
+  else if (with_stats)
+    hipLaunchKernelGGL((sapo_token_kernel<true, 1>), dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts, stat_parts);
+  else if (vec4)
+    hipLaunchKernelGGL((sapo_token_kernel<false, 4>), dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts, stat_parts);
+  else
+    hipLaunchKernelGGL((sapo_token_kernel<false, 1>), dim3(grid), dim3(AUX_THREADS), 0, stream, io, parts, stat_parts);
   AREAL_CHECK_LAUNCH();
-  hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid, 0,
-                     0.0, loss, counters);
+  hipLaunchKernelGGL(aux_finalize_kernel, dim3(with_stats ? 1 + N_SAPO_STATS : 1), dim3(AUX_THREADS), 0, stream,
+                     parts, grid, 0, (double)n_tokens, loss, counters, (const StatPart*)stat_parts, N_SAPO_STATS,
+                     SAPO_MASKED_STATS, stats);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -594,13 +763,22 @@ int areal_critic_loss(const float* value, const float* old_value, const float* t
   if (workspace == nullptr || workspace_bytes < areal_aux_loss_workspace_bytes(n, 0))
     return AREAL_ERR_WORKSPACE;
   SumCount* parts = (SumCount*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-  const int grid = aux_grid(n);
-  hipLaunchKernelGGL(critic_token_kernel, dim3(grid), dim3(AUX_THREADS), 0, stream, value,
-                     old_value, target_value, loss_mask, n, value_eps_clip, huber, dvalue,
-                     stat_loss, clip_mask, parts);
+  const bool vec4 = n >= VEC4_MIN_TOKENS && aligned_to(value, 16) && aligned_to(old_value, 16) &&
+                    aligned_to(target_value, 16) && aligned_to(loss_mask, 4) && aligned_to(dvalue, 16) &&
+                    aligned_to(stat_loss, 16) && aligned_to(clip_mask, 4);
+  const int grid = aux_grid(n, vec4 ? 4 : 1);
+  if (vec4)
+    hipLaunchKernelGGL(critic_token_kernel<4>, dim3(grid), dim3(AUX_THREADS), 0, stream, value,
+                       old_value, target_value, loss_mask, n, value_eps_clip, huber, dvalue,
+                       stat_loss, clip_mask, parts);
+  else
+    hipLaunchKernelGGL(critic_token_kernel<1>, dim3(grid), dim3(AUX_THREADS), 0, stream, value,
+                       old_value, target_value, loss_mask, n, value_eps_clip, huber, dvalue,
+                       stat_loss, clip_mask, parts);
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid,
-                     loss_mask ? 1 : 2, (double)n, loss, counters);
+                     loss_mask ? 1 : 2, (double)n, loss, counters, (const StatPart*)nullptr, 0, 0,
+                     (double*)nullptr);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -724,7 +902,7 @@ int areal_distill_terms(const float* logprobs, const float* old_logprobs, const 
                      old_logprobs, teacher_logprobs, loss_mask, n_tokens, mode, dlogprobs, term, parts);
   AREAL_CHECK_LAUNCH();
   hipLaunchKernelGGL(aux_finalize_kernel, dim3(1), dim3(AUX_THREADS), 0, stream, parts, grid, 0, 0.0,
-                     value, counters);
+                     value, counters, (const StatPart*)nullptr, 0, 0, (double*)nullptr);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

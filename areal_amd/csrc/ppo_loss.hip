@@ -109,11 +109,6 @@ DEVI float torch_clamp(float x, float lo, float hi) {
 }
 DEVI float torch_max(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a > b ? a : b); }
 DEVI float torch_min(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : (a < b ? a : b); }
-// The same for the running extremes of the logged statistics, where the sign of a zero does not
-// matter: IEEE 754-2019 minimum / maximum, one instruction each (v_minimum3_f32 / v_maximum3_f32).
-DEVI float stat_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
-DEVI float stat_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
-
 // Bernoulli KL(P||Q) with p = clamp(exp(log_p), 1e-8, 1 - 1e-8): in fp32 the upper bound
 // rounds to 1.0f, which is what the reference's fp32 tensors see.
 DEVI float binary_kl(float log_p, float log_q) {
@@ -283,63 +278,6 @@ __global__ __launch_bounds__(LOSS_THREADS) void seq_is_kernel(LossIO io, LossCfg
 // ---------------------------------------------------------------------------------------
 // Token kernel
 // ---------------------------------------------------------------------------------------
-// Per-token arrays are moved VEC elements per thread and access: VEC = 4 takes 16-byte loads and
-// stores for the fp32 arrays and 4-byte ones for the byte masks (every array 16-byte, resp.
-// 4-byte, aligned; the host checks), VEC = 1 is the element-wise form for anything else and for
-// the last n % 4 tokens. Plain loads and stores: a micro-batch's per-token arrays (a few hundred MB
-// at most) come from and go to kernels next to this one through the 256 MB memory-side cache,
-// which accesses with the non-temporal hint bypass (measured on 4 Mi tokens: 5.0 TB/s with the
-// hint, 6.5 to 7.5 without).
-template <int VEC>
-DEVI void load_f32(const float* p, int64_t t, float (&v)[VEC]) {
-  if (p == nullptr) {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = 0.f;
-  } else if (VEC == 4) {
-    const f32x4 x = *(const f32x4*)(p + t);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = x[i];
-  } else {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = p[t + i];
-  }
-}
-template <int VEC>
-DEVI void load_mask(const uint8_t* p, int64_t t, bool (&v)[VEC]) {
-  if (VEC == 4) {
-    const uint32_t x = *(const uint32_t*)(p + t);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = ((x >> (8 * i)) & 0xffu) != 0;
-  } else {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) v[i] = p[t + i] != 0;
-  }
-}
-template <int VEC>
-DEVI void store_f32(float* p, int64_t t, const float (&v)[VEC]) {
-  if (p == nullptr) return;
-  if (VEC == 4) {
-    const f32x4 x = {v[0], v[1], v[2], v[3]};
-    *(f32x4*)(p + t) = x;
-  } else {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
-  }
-}
-template <int VEC>
-DEVI void store_mask(uint8_t* p, int64_t t, const bool (&v)[VEC]) {
-  if (p == nullptr) return;
-  if (VEC == 4) {
-    uint32_t x = 0;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) x |= (v[i] ? 1u : 0u) << (8 * i);
-    *(uint32_t*)(p + t) = x;
-  } else {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) p[t + i] = v[i];
-  }
-}
-
 // Running sums of one thread. Counts fit 32 bits per thread (a thread sees n / gridsize tokens).
 struct TokenAcc {
   double loss_sum;
@@ -719,9 +657,6 @@ __global__ void loss_grad_scale_kernel(const float* __restrict__ dlp,
   }
   if (VEC > 1 && n_vec + gid < n) out[n_vec + gid] = (dlp[n_vec + gid] * g) / nv;
 }
-
-// VEC = 4 needs every per-token fp32 array 16-byte aligned and every byte array 4-byte aligned.
-bool aligned_to(const void* p, uintptr_t a) { return p == nullptr || ((uintptr_t)p & (a - 1)) == 0; }
 
 int loss_grid(int64_t n, int vec = 1) {
   int64_t b = ceil_div_i64(n, (int64_t)LOSS_THREADS * vec);

@@ -67,8 +67,12 @@ def sapo_loss_fn(
     loss_mask: torch.Tensor,
     importance_sampling_level: str = "token",
     cu_seqlens: torch.Tensor | None = None,
+    stat_reduction=None,
 ) -> tuple[torch.Tensor, dict]:
-    """SAPO loss with asymmetric sigmoid gates; ``stat`` keys as in ``functional.py:661-673``."""
+    """SAPO loss with asymmetric sigmoid gates; ``stat`` keys as in ``functional.py:661-673``.
+    ``stat_reduction`` (a ``StatReduction``; not in the reference): the token kernel reduces the
+    logged statistics itself and no per-token statistic tensor is written; ``stat`` then holds
+    the host scalars ``n_total_tokens`` and ``n_valid_tokens`` only."""
     if tau_pos <= 0 or tau_neg <= 0:
         raise ValueError("SAPO temperatures (tau_pos, tau_neg) must be positive.")
     if importance_sampling_level == "sequence":
@@ -94,13 +98,27 @@ def sapo_loss_fn(
     if seq_level:
         cu, n_seqs, uniform_len = _sequence_layout(shape, cu_seqlens, dev)
 
+    names = ("stat_loss", "ratio", "approx_kl", "soft_gate", "gate_pos", "gate_neg")
+    red = stat_reduction
+    ent = extras = None
+    if red is not None:
+        from areal_amd.functional.functional import SAPO_REDUCED_STAT_KEYS
+
+        extras = [_f32(t) for t in red.extras.values()]
+        ent = _f32(red.entropy) if red.entropy is not None else None
+        for t in extras + ([ent] if ent is not None else []):
+            if t.numel() != n:
+                raise ValueError(f"a statistic rides along with {t.numel()} elements, expected {n}")
+
     def launch(want_grad: bool):
         f32 = dict(dtype=torch.float32, device=dev)
-        out = {k: torch.empty(n, **f32) for k in
-               ("stat_loss", "ratio", "approx_kl", "soft_gate", "gate_pos", "gate_neg")}
+        out = {k: (torch.empty(n, **f32) if red is None else None) for k in names}
         out["loss"] = torch.empty((), **f32)
         out["dsum"] = torch.empty(n, **f32) if want_grad else None
-        out["counters"] = torch.empty(8, dtype=torch.float64, device=dev)
+        # counters [8] and, with a reduction, stats [13][4] in one buffer: one copy to the host
+        n_stats = len(SAPO_REDUCED_STAT_KEYS) if red is not None else 0
+        both = torch.empty(8 + 4 * n_stats, dtype=torch.float64, device=dev)
+        out["counters"], out["both"] = both[:8], both
         nbytes = lib.areal_aux_loss_workspace_bytes(n, n_seqs)
         ws = _lib.workspace(nbytes, dev)
         rc = lib.areal_sapo_loss(
@@ -109,6 +127,9 @@ def sapo_loss_fn(
             _lib.ptr(out["loss"]), _lib.ptr(out["dsum"]), _lib.ptr(out["stat_loss"]),
             _lib.ptr(out["ratio"]), _lib.ptr(out["approx_kl"]), _lib.ptr(out["soft_gate"]),
             _lib.ptr(out["gate_pos"]), _lib.ptr(out["gate_neg"]), _lib.ptr(out["counters"]),
+            _lib.ptr(ent), _lib.ptr(extras[0] if extras else None),
+            _lib.ptr(extras[1] if extras and len(extras) > 1 else None),
+            _lib.ptr(both[8:]) if red is not None else None,
             _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
         )
         _lib.check(rc, "areal_sapo_loss")
@@ -117,6 +138,12 @@ def sapo_loss_fn(
     runner = _Launch(launch)
     loss = _ScaledLoss.apply(logprobs, runner)
     out = runner.out
+    if red is not None:
+        host = out["both"].cpu()  # the one host synchronisation of the call
+        red._fill_sapo(host[8:].view(-1, 4), host[:8], n)
+        return loss, dict(n_total_tokens=float(n), n_valid_tokens=float(host[1]),
+                          n_masked_tokens=float(n) - float(host[1]),
+                          masked_token_ratio=1.0 - float(host[1]) / max(float(n), 1.0))
     stat = dict(
         loss=out["stat_loss"].view(shape),
         importance_weight=out["ratio"].view(shape),

@@ -49,6 +49,15 @@ REDUCED_STAT_KEYS = (
     ("clipped_new_logp", "clipped_tokens"), ("clipped_old_logp", "clipped_tokens"),
     ("extra0", "n_tokens"), ("extra1", "n_tokens"),
 )
+# The same for areal_sapo_loss's stats output.
+SAPO_REDUCED_STAT_KEYS = (
+    ("importance_weight", "n_valid_tokens"), ("approx_kl", "n_valid_tokens"),
+    ("new_logp", "n_valid_tokens"), ("old_logp", "n_valid_tokens"), ("entropy", "n_valid_tokens"),
+    ("actor_loss", "n_valid_tokens"), ("logp_diff", "n_valid_tokens"),
+    ("logp_abs_diff", "n_valid_tokens"), ("sapo_soft_gate", "n_valid_tokens"),
+    ("sapo_scaled_gate_pos", "n_valid_tokens"), ("sapo_scaled_gate_neg", "n_valid_tokens"),
+    ("extra0", "n_tokens"), ("extra1", "n_tokens"),
+)
 
 
 class _HostCopy:
@@ -150,12 +159,18 @@ class StatReduction:
     vocabulary min / max logits) are optional per-token inputs that ride along in the same pass.
     """
 
-    def __init__(self, entropy: torch.Tensor | None = None, extras: dict[str, torch.Tensor] | None = None):
+    def __init__(self, entropy: torch.Tensor | None = None, extras: dict[str, torch.Tensor] | None = None,
+                 keep_behave_mask: bool = False):
         extras = dict(extras or {})
         if len(extras) > 2:
             raise ValueError(f"at most two extra statistics ride along, got {len(extras)}")
         self.entropy = entropy
         self.extras = extras
+        # the one per-token output a caller may still need (1 byte per token): the tokens that pass
+        # rejection sampling with a positive weight, the denominator of the diagnostics that
+        # grpo_loss_fn reduces in a launch of their own
+        self.keep_behave_mask = keep_behave_mask
+        self.behave_mask: torch.Tensor | None = None
         self._results: dict[str, dict[str, float | None]] = {}
         self._denominators: dict[str, float] = {}
         self._pending = None  # (host copy, arguments of _fill) of a call with deferred host reads
@@ -167,6 +182,16 @@ class StatReduction:
             host = copy.host()
             self._fill(host[8:].view(-1, 4), host[:8], n_tokens, has_rs, has_old)
 
+    def _fill_sapo(self, host: torch.Tensor, counters, n_tokens: int) -> None:
+        """Results of ``areal_sapo_loss``'s reduction. SAPO clips nothing: the clip ratios are
+        zero on every token of the mask and the clipped-token statistics are empty."""
+        self._fill(host, counters, n_tokens, False, True, keys=SAPO_REDUCED_STAT_KEYS)
+        nv = float(counters[1])
+        zero = dict(sum=0.0, count=nv, avg=None if nv == 0 else 0.0, min=None if nv == 0 else 0.0,
+                    max=None if nv == 0 else 0.0, denominator="n_valid_tokens")
+        self._results["clip_ratio"] = dict(zero)
+        self._results["dual_clip_ratio"] = dict(zero)
+
     @property
     def results(self) -> dict[str, dict[str, float | None]]:
         self._resolve()
@@ -177,9 +202,10 @@ class StatReduction:
         self._resolve()
         return self._denominators
 
-    def _fill(self, host: torch.Tensor, counters, n_tokens: int, has_rs: bool, has_old: bool) -> None:
+    def _fill(self, host: torch.Tensor, counters, n_tokens: int, has_rs: bool, has_old: bool,
+              keys=REDUCED_STAT_KEYS) -> None:
         names = list(self.extras)
-        for i, (key, denom) in enumerate(REDUCED_STAT_KEYS):
+        for i, (key, denom) in enumerate(keys):
             if key == "entropy" and self.entropy is None:
                 continue
             if key.startswith("behave_") and not has_rs:
@@ -300,6 +326,8 @@ def _run_loss_kernel_reduced(lib, dev, cfg, n, n_seqs, uniform_len, cu, logprobs
     if need_seq_io:
         out["new_mask"] = torch.empty(n, dtype=torch.bool, device=dev)
         out["behave_imp_weight"] = torch.empty(n, **f32)
+    if reduction.keep_behave_mask and cfg.rs_enabled:
+        out["behave_mask"] = reduction.behave_mask = torch.empty(n, dtype=torch.bool, device=dev)
     # counters [8] and stats [17][4] share one buffer: one device-to-host copy serves both
     n_stats = len(REDUCED_STAT_KEYS)
     both = torch.empty(8 + 4 * n_stats, dtype=torch.float64, device=dev)
@@ -319,7 +347,7 @@ def _run_loss_kernel_reduced(lib, dev, cfg, n, n_seqs, uniform_len, cu, logprobs
         _lib.ptr(ent), _lib.ptr(extras[0] if len(extras) > 0 else None),
         _lib.ptr(extras[1] if len(extras) > 1 else None),
         _lib.ptr(out["loss"]), _lib.ptr(out["dlp"]), None, None, None, None, None,
-        _lib.ptr(out["new_mask"]), _lib.ptr(out["behave_imp_weight"]), None, None,
+        _lib.ptr(out["new_mask"]), _lib.ptr(out["behave_imp_weight"]), None, _lib.ptr(out["behave_mask"]),
         _lib.ptr(counters), _lib.ptr(stats), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev),
     )
     _lib.check(rc, "areal_actor_loss_stats")

@@ -84,24 +84,27 @@ def grpo_loss_fn(
 
     ``stats`` (optional dict) receives what the reference hands to its ``stats_tracker``.  With
     ``stats_mode="tensors"`` these are the bool denominators and fp32 statistics of the
-    micro-batch's token shape, as in the reference.  With ``stats_mode="reduced"`` (PPO and CISPO
-    losses) no per-token statistic tensor is written at all: the loss kernel reduces every
-    logged statistic under its denominator in its own pass and ``stats[key]`` is
+    micro-batch's token shape, as in the reference.  With ``stats_mode="reduced"`` (every loss
+    kind) no per-token statistic tensor comes back: the loss kernel reduces every logged
+    statistic under its denominator in its own pass and ``stats[key]`` is
     ``{"sum", "count", "avg", "min", "max", "denominator"}``, ``stats["denominator/<name>"]``
     the token counts (what the tracker's export computes from the clones, ``actor.py:662-733``,
-    ``stats_tracker.py:455-560``); the proximal-approximation and staleness diagnostics, which
-    need per-token tensors, are not collected in that mode.
+    ``stats_tracker.py:455-560``).  The ``compute_logp/...`` diagnostics of the proximal
+    approximations (``actor.py:1138-1226``) are functions of tensors the loss kernel does not
+    see; they are evaluated as in the other mode and reduced at once by one launch of the masked
+    statistics kernel, under the same denominator (``stats["denominator/compute_logp/
+    n_valid_tokens"]``); the staleness statistics are host scalars in both modes.
     """
     if stats_mode not in ("tensors", "reduced"):
         raise ValueError(f"stats_mode must be 'tensors' or 'reduced', got {stats_mode!r}")
     reduction = None
-    if stats is not None and stats_mode == "reduced" and not use_sapo_loss:
+    if stats is not None and stats_mode == "reduced":
         from areal_amd.functional.functional import StatReduction
 
         extras = {}
         if vocab_min_logits is not None and vocab_max_logits is not None:
             extras = dict(vocab_min_logits=vocab_min_logits, vocab_max_logits=vocab_max_logits)
-        reduction = StatReduction(entropy=entropy, extras=extras)
+        reduction = StatReduction(entropy=entropy, extras=extras, keep_behave_mask=True)
     if prox_logp_method not in PROX_LOGP_METHODS_ALL:
         raise ValueError(f"'{prox_logp_method}' is not a valid ProxLogpMethod")
     old_logp = input_data["logprobs"]
@@ -171,6 +174,7 @@ def grpo_loss_fn(
             loss_mask=loss_mask,
             importance_sampling_level=importance_sampling_level,
             cu_seqlens=input_data.get("cu_seqlens"),
+            stat_reduction=reduction,
         )
     else:
         loss, stat = ppo_actor_loss_fn(
@@ -210,12 +214,43 @@ def grpo_loss_fn(
             rkl_stat = term
 
     if reduction is not None:
-        if defer_host_reads:
+        defer = defer_host_reads and not use_sapo_loss
+        if defer:
             stats["reduction"] = reduction
         else:
             stats.update(reduction.results)
             for name, count in reduction.denominators.items():
                 stats["denominator/" + name] = count
+        # the compute_logp diagnostics: per-token tensors as in the other mode, reduced right away
+        from areal_amd.stats import masked_stats
+
+        lp = logprobs.detach()
+        diag_mask = reduction.behave_mask if reduction.behave_mask is not None else loss_mask
+        diag: dict = {}
+        _collect_proximal_approximation_stats(
+            diag, prox_logp_method, prox_logp_gt, old_logp, lp, input_data.get("versions"),
+            current_version, diag_mask.view(loss_mask.shape),
+        )
+        den = diag.pop("compute_logp/n_valid_tokens")
+        if diag:
+            reduced = masked_stats(diag, {k: den for k in diag}, defer=defer)
+            if defer:
+                stats["compute_logp_reduction"] = reduced
+            else:
+                for k, v in reduced.items():
+                    stats[k] = dict(v, denominator="compute_logp/n_valid_tokens")
+                stats["denominator/compute_logp/n_valid_tokens"] = next(iter(reduced.values()))["count"]
+        if "versions" in input_data and current_version is not None and not defer:
+            _collect_version_staleness_stats(stats, input_data["versions"], current_version, diag_mask.view(loss_mask.shape))
+        if vocab_mean_logits is not None or vocab_norm_logits is not None:
+            more = {k: v for k, v in (("vocab_mean_logits", vocab_mean_logits), ("vocab_norm_logits", vocab_norm_logits))
+                    if v is not None}
+            extra = masked_stats(more, {k: None for k in more}, defer=defer)
+            if defer:
+                stats["vocab_moments_reduction"] = extra
+            else:
+                for k, v in extra.items():
+                    stats[k] = dict(v, denominator="n_tokens")
         for key in ("n_total_tokens", "n_valid_tokens", "n_masked_tokens", "masked_token_ratio"):
             if key in stat:
                 stats["scalar/" + key] = stat[key]

@@ -18,16 +18,46 @@ from areal_amd import _lib
 MAX_TENSORS = 32
 
 
+class DeferredStats:
+    """Result of ``masked_stats(..., defer=True)``: the reductions are queued and their results
+    on their way to pinned host memory; ``results`` waits for them when first read."""
+
+    def __init__(self, pending):
+        self._pending = pending  # [(keys, pinned host tensor, event)]
+        self._results = None
+
+    @property
+    def results(self) -> dict[str, dict[str, float | None]]:
+        if self._results is None:
+            out = {}
+            for keys, host, event in self._pending:
+                event.synchronize()
+                _unpack(out, keys, host)
+            self._results, self._pending = out, None
+        return self._results
+
+
+def _unpack(out, keys, host) -> None:
+    for j, k in enumerate(keys):
+        s, c, mn, mx = host[j].tolist()
+        empty = c == 0
+        out[k] = dict(sum=s, count=c, avg=None if empty else s / c,
+                      min=None if empty else mn, max=None if empty else mx)
+
+
 def masked_stats(
     values: dict[str, torch.Tensor],
     denominators: dict[str, torch.Tensor | None],
-) -> dict[str, dict[str, float | None]]:
+    defer: bool = False,
+):
     """``{key: {"sum", "count", "avg", "min", "max"}}`` of ``values[key]`` where
     ``denominators[key]`` is true (``None``: everywhere).  ``avg`` / ``min`` / ``max`` are ``None``
-    for an empty mask, as ``_avg_of`` / ``_min_of`` / ``_max_of`` return."""
+    for an empty mask, as ``_avg_of`` / ``_min_of`` / ``_max_of`` return.  ``defer=True`` returns
+    a ``DeferredStats`` without waiting for the GPU."""
     lib = _lib.load()
     keys = list(values)
     out: dict[str, dict[str, float | None]] = {}
+    pending = []
     for i in range(0, len(keys), MAX_TENSORS):
         chunk = keys[i : i + MAX_TENSORS]
         vals, masks = [], []
@@ -51,10 +81,12 @@ def masked_stats(
         ws = _lib.workspace(nbytes, dev)
         rc = lib.areal_masked_stats(vptr, mptr, K, n, _lib.ptr(res), _lib.ptr(ws), nbytes, _lib.stream_ptr(dev))
         _lib.check(rc, "areal_masked_stats")
-        host = res.cpu()
-        for j, k in enumerate(chunk):
-            s, c, mn, mx = host[j].tolist()
-            empty = c == 0
-            out[k] = dict(sum=s, count=c, avg=None if empty else s / c,
-                          min=None if empty else mn, max=None if empty else mx)
-    return out
+        if defer:
+            host = torch.empty(res.shape, dtype=res.dtype, pin_memory=True)
+            host.copy_(res, non_blocking=True)
+            event = torch.cuda.Event()
+            event.record(torch.cuda.current_stream(dev))
+            pending.append((chunk, host, event))
+        else:
+            _unpack(out, chunk, res.cpu())
+    return DeferredStats(pending) if defer else out

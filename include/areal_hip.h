@@ -29,7 +29,8 @@ typedef struct ihipStream_t* areal_stream_t; /* a hipStream_t */
  * areal_abi_version() returns the number the loaded library was built with.
  *   3: areal_lmhead_fwd / areal_lmhead_bwd_saved take probs_bytes and check it against
  *      areal_lmhead_probs_bytes() (the buffer's rows are padded to 128, and
- *      areal_lmhead_bwd_saved takes probs_status). */
+ *      areal_lmhead_bwd_saved takes probs_status); areal_sapo_loss takes entropy, extra0,
+ *      extra1 and stats. */
 #define AREAL_HIP_ABI_VERSION 3
 int areal_abi_version(void);
 
@@ -253,13 +254,21 @@ int areal_actor_loss_grad(const float* dlogprobs, const float* upstream, const d
 size_t areal_aux_loss_workspace_bytes(int64_t n_tokens, int64_t n_seqs);
 
 /* seq_level != 0: geometric-mean ratio and mean advantage per sequence (functional.py:56-149;
- * cu_seqlens [n_seqs+1] or uniform_len > 0). Per-token outputs may be NULL. */
+ * cu_seqlens [n_seqs+1] or uniform_len > 0). Per-token outputs may be NULL.
+ * stats (NULL allowed) [13][4] double = {sum, count, min, max} of what grpo_loss_fn logs for a
+ * SAPO step (areal/trainer/ppo/actor.py:662-741), reduced inside the token pass instead of
+ * written as [n_tokens] tensors: importance_weight, approx_kl, new_logp, old_logp, entropy,
+ * actor_loss, logp_diff, logp_abs_diff, sapo_soft_gate, sapo_scaled_gate_pos,
+ * sapo_scaled_gate_neg (under the loss mask), extra0, extra1 (every token). entropy, extra0,
+ * extra1 [n_tokens] are optional inputs of that reduction (NULL: sum 0, min +inf, max -inf) and
+ * are ignored without stats. */
 int areal_sapo_loss(const float* logprobs, const float* old_logprobs, const float* advantages,
                     const uint8_t* loss_mask, const int32_t* cu_seqlens, int64_t n_tokens,
                     int64_t n_seqs, int64_t uniform_len, float tau_pos, float tau_neg,
                     int seq_level, float* loss, float* dlogprobs, float* stat_loss,
                     float* stat_ratio, float* stat_approx_kl, float* soft_gate, float* gate_pos,
-                    float* gate_neg, double* counters, void* workspace, size_t workspace_bytes,
+                    float* gate_neg, double* counters, const float* entropy, const float* extra0,
+                    const float* extra1, double* stats, void* workspace, size_t workspace_bytes,
                     areal_stream_t stream);
 
 /* loss = mean over the mask (or over all n when loss_mask is NULL) of

@@ -73,6 +73,102 @@ def test_sapo_matches_oracle(dev, level, layout):
     torch.testing.assert_close(x.grad.cpu(), lp_c.grad, rtol=1e-4, atol=1e-8)
 
 
+@pytest.mark.parametrize("n,level", [(70_001, "token"), (300_003, "token"), (70_001, "sequence")])
+def test_sapo_reduced_stats_match_oracle_masked_stats(dev, n, level):
+    """grpo_loss_fn(use_sapo_loss=True, stats_mode="reduced") writes no per-token statistic
+    tensor; what it reports equals the oracle's per-token SAPO tensors (assembled as
+    actor.py:662-741 hands them to the tracker) reduced by oracle.packing.masked_stats. The larger
+    batch takes the four-tokens-per-thread form of the kernel."""
+    from areal_amd.ppo.actor import grpo_loss_fn
+    from oracle.packing import masked_stats as oracle_masked_stats
+
+    g = torch.Generator().manual_seed(n)
+    lens = torch.randint(1, n // 40, (40,), generator=g)
+    lens[-1] = n - int(lens[:-1].sum())  # 40 sequences that cover the n tokens
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    assert int(cu[-1]) == n
+    lp = torch.randn(n, generator=g) * 0.3 - 1.0
+    old = lp + torch.randn(n, generator=g) * 0.2
+    adv = torch.randn(n, generator=g)
+    mask = torch.rand(n, generator=g) > 0.25
+    ent = torch.rand(n, generator=g) * 3
+    vmin, vmax = -torch.rand(n, generator=g) * 9 - 3, torch.rand(n, generator=g) * 20
+    lp_c = lp.clone().requires_grad_(True)
+    want_loss, so = A.sapo_loss(lp_c, old, adv, 1.0, 1.05, mask, level, cu)
+    want_loss.backward()
+    lpd = lp_c.detach()
+    diff = (old - lpd) * mask
+    zeros = torch.zeros(n)
+    vals = dict(importance_weight=so["importance_weight"], approx_kl=so["approx_kl"], new_logp=lpd, old_logp=old,
+                entropy=ent, actor_loss=so["loss"], clip_ratio=zeros, dual_clip_ratio=zeros, logp_diff=diff,
+                logp_abs_diff=diff.abs(), sapo_soft_gate=so["sapo_soft_gate"],
+                sapo_scaled_gate_pos=so["sapo_scaled_gate_pos"], sapo_scaled_gate_neg=so["sapo_scaled_gate_neg"],
+                vocab_min_logits=vmin, vocab_max_logits=vmax)
+    den = {k: mask for k in vals}
+    den["vocab_min_logits"] = den["vocab_max_logits"] = None
+    want = oracle_masked_stats(vals, den)
+
+    stats = {}
+    x = lp.to(dev).requires_grad_(True)
+    data = dict(logprobs=old.to(dev), advantages=adv.to(dev), loss_mask=mask.to(dev), cu_seqlens=cu.to(dev),
+                prox_logp=old.to(dev))
+    loss = grpo_loss_fn(x, ent.to(dev), data, 0.2, None, None, use_sapo_loss=True, sapo_tau_pos=1.0,
+                        sapo_tau_neg=1.05, importance_sampling_level=level, vocab_min_logits=vmin.to(dev),
+                        vocab_max_logits=vmax.to(dev), stats=stats, stats_mode="reduced")
+    loss.backward()
+    torch.testing.assert_close(loss.detach().cpu(), want_loss.detach(), rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(x.grad.cpu(), lp_c.grad, rtol=1e-4, atol=1e-8)
+    assert not any(torch.is_tensor(v) for v in stats.values())  # nothing of token shape comes back
+    assert set(want) <= set(stats), sorted(set(want) - set(stats))
+    for k, w in want.items():
+        got = stats[k]
+        assert got["count"] == w["count"], k
+        assert got["sum"] == pytest.approx(w["sum"], rel=2e-5, abs=1e-7 * max(1.0, w["count"])), k
+        assert got["min"] == pytest.approx(w["min"], rel=2e-6, abs=1e-6), k
+        assert got["max"] == pytest.approx(w["max"], rel=2e-6, abs=1e-6), k
+    assert stats["denominator/n_valid_tokens"] == float(mask.sum()) and stats["denominator/n_tokens"] == float(n)
+    # the compute_logp diagnostics of the tensor mode, reduced under the same mask
+    assert stats["compute_logp/prox_logp_gt"]["count"] == float(mask.sum())
+    assert stats["compute_logp/prox_logp_gt"]["sum"] == pytest.approx(float(old[mask].double().sum()), rel=1e-6)
+
+
+def test_reduced_mode_reduces_the_proximal_approximation_diagnostics(dev):
+    """stats_mode="reduced" with versions: the compute_logp/... entries of the tensor mode come
+    back as reduced values (sum, count, min, max under the behave mask), the staleness scalars
+    as they are."""
+    from areal_amd.config import RejectionSamplingConfig
+    from areal_amd.ppo.actor import grpo_loss_fn
+    from areal_amd.stats import masked_stats
+
+    g = torch.Generator().manual_seed(17)
+    n = 40_000
+    lp = torch.randn(n, generator=g) * 0.3 - 1.0
+    prox = lp + torch.randn(n, generator=g) * 0.05
+    old = prox + torch.randn(n, generator=g) * 0.3
+    ver = torch.randint(-1, 5, (n,), generator=g)
+    data = dict(logprobs=old.to(dev), advantages=torch.randn(n, generator=g).to(dev),
+                loss_mask=(torch.rand(n, generator=g) > 0.2).to(dev), prox_logp=prox.to(dev), versions=ver.to(dev))
+    rs = RejectionSamplingConfig(level="token", action="mask", metric="ratio", lower=0.5, upper=2.0)
+    out = {}
+    for mode in ("tensors", "reduced"):
+        st = {}
+        grpo_loss_fn(lp.to(dev).requires_grad_(True), torch.zeros(n, device=dev), data, 0.2, None, None,
+                     rejection_sampling=rs, current_version=5, prox_logp_method="metrics", stats=st, stats_mode=mode)
+        out[mode] = st
+    t, r = out["tensors"], out["reduced"]
+    keys = [k for k in t if k.startswith("compute_logp/") and k != "compute_logp/n_valid_tokens"]
+    assert "compute_logp/loglinear/abs_error" in keys and "compute_logp/kl_div_taylor" in keys
+    want = masked_stats({k: t[k] for k in keys}, {k: t["compute_logp/n_valid_tokens"] for k in keys})
+    assert not any(torch.is_tensor(v) for v in r.values())
+    for k in keys:
+        assert r[k]["count"] == want[k]["count"] == float(t["compute_logp/n_valid_tokens"].sum()), k
+        assert r[k]["sum"] == pytest.approx(want[k]["sum"], rel=1e-12) and r[k]["max"] == want[k]["max"], k
+    assert r["denominator/compute_logp/n_valid_tokens"] == float(t["unclipped_behave_tokens"].sum())
+    for k in t:
+        if k.startswith("scalar/version_stats/"):
+            assert r[k] == t[k], k
+
+
 @pytest.mark.parametrize("kind", ["mse", "huber"])
 @pytest.mark.parametrize("masked", [True, False])
 def test_critic_loss_matches_oracle(dev, kind, masked):
