@@ -27,6 +27,12 @@ Operand layouts: ``kc`` = k contiguous (row = i or j, 128 B of k per stage row, 
 XOR-swizzled), ``km`` = k major (row = k, 512 B of i or j per stage row, fetched with
 ``ds_read_b64_tr_b16``).  Variants: nt = (kc, kc), tn = (km, km), mix = (km, kc).
 
+An odd number of k-tiles runs as one more pair whose second k-tile is "dead": it keeps the
+pipeline's loads, fragment reads and barriers (the next output tile's first two k-tiles arrive in
+the same stages as always) and issues no MFMA.  The loads that would fetch the k-tile behind the
+last one are issued with the pointers held back by one k-tile (``S_PEN_*`` replaces the stride
+for one advance), so they fetch the last k-tile again and nothing outside the operands is read.
+
 Run ``python gen_mainloop16.py`` to rewrite ``mainloop16.inc`` next to this file.
 """
 
@@ -38,12 +44,13 @@ from pathlib import Path
 # ---- physical registers of the asm block (the C++ side binds its operands to the same names)
 S_PA, S_PB, S_PA_NEXT, S_PB_NEXT = 40, 42, 44, 46  # 64-bit pointers: s[n:n+1]
 S_CNT, S_LDSW, S_STRIDE_A, S_STRIDE_B = 48, 49, 50, 51
+# odd k-tile counts: S_ODD = 1 when the tile's last pair has a dead second k-tile (else 0);
+# S_PEN_* = what the pointers advance by after the loads of the tile's last real k-tile
+# (0 for an odd count, the stride otherwise); S_EFF_* are scratch
+S_ODD, S_PEN_A, S_PEN_B, S_EFF_A, S_EFF_B = 52, 53, 54, 55, 56
 
 HALF_BYTES = 32768            # one operand of one stage
 OPER_BYTES = 2 * HALF_BYTES   # both stages of one operand
-
-# Timing experiments (results are wrong with any of these set): drop one ingredient of the loop.
-FLAGS = set()
 
 
 class Variant:
@@ -92,9 +99,18 @@ class Variant:
                 f"global_load_lds_dwordx4 v{self.off[oper] + i}, s[{ptr}:{ptr + 1}]")
 
     @staticmethod
-    def advance(oper):
-        p, st = (S_PA, S_STRIDE_A) if oper == 0 else (S_PB, S_STRIDE_B)
+    def advance(oper, eff=False):
+        """Move the operand's pointer to the next k-tile; eff: by the amount select_advance() chose."""
+        p, st = (S_PA, S_EFF_A if eff else S_STRIDE_A) if oper == 0 else (S_PB, S_EFF_B if eff else S_STRIDE_B)
         return [f"s_add_u32 s{p}, s{p}, s{st}", f"s_addc_u32 s{p + 1}, s{p + 1}, 0"]
+
+    @staticmethod
+    def select_advance():
+        """In front of a pair: its first k-tile fetches the tile's last real k-tile exactly when
+        this is the last pair but one; the pointers then advance by S_PEN_* instead of the stride."""
+        return [f"s_cmp_eq_u32 s{S_CNT}, 2",
+                f"s_cselect_b32 s{S_EFF_A}, s{S_PEN_A}, s{S_STRIDE_A}",
+                f"s_cselect_b32 s{S_EFF_B}, s{S_PEN_B}, s{S_STRIDE_B}"]
 
     # ---------------------------------------------------------------- schedule
     def a_reads(self, buf, stage, ks):
@@ -110,18 +126,14 @@ class Variant:
                 out += self.reads(self.fb[parity][ks] + 4 * x, stage, ks, 1, x)
         return out
 
-    def kstep(self, abuf, bbuf, init, pre, post):
-        """64 MFMAs; pre[m] / post[m] are emitted in front of / behind MFMA m."""
+    def kstep(self, abuf, bbuf, init, pre, post, dead=False):
+        """64 MFMAs; pre[m] / post[m] are emitted in front of / behind MFMA m. dead: no MFMA."""
         out = []
         for m in range(64):
             out += pre.get(m, [])
-            if not ("no_mfma" in FLAGS and not init):
+            if not dead:
                 out.append(self.mfma(abuf, bbuf, m >> 3, m & 7, init))
             out += post.get(m, [])
-        if "no_reads" in FLAGS:
-            out = [ln for ln in out if not ln.startswith("ds_read")]
-        if "no_loads" in FLAGS:
-            out = [ln for ln in out if not ln.startswith("global_load") and "m0" not in ln]
         return out
 
     @staticmethod
@@ -146,18 +158,19 @@ class Variant:
             setm0, ld = self.load(stage, oper, i)
             pre.setdefault(i * step, []).append(setm0)
             post.setdefault(i * step, []).append(ld)
-        post.setdefault(7 * step + 1, []).extend(self.advance(oper))
+        # the first k-tile of a pair (stage 0) advances by the selected amount
+        post.setdefault(7 * step + 1, []).extend(self.advance(oper, eff=(stage == 0)))
 
-    def ktile(self, parity, init):
+    def ktile(self, parity, init, dead=False):
         stage = parity
-        barrier = [] if "no_barrier" in FLAGS else ["s_barrier"]
-        out = [f"; ---- k-tile on stage {stage}: k-step 0"]
+        barrier = ["s_barrier"]
+        out = [f"; ---- k-tile on stage {stage}{' (dead: no MFMA)' if dead else ''}: k-step 0"]
         # k-step 0: the B half of this stage is free (its fragments are in registers): refill
         # it with the k-tile after next; A fragments of k-step 1 -> A buffer 1
         pre, post = {}, {}
         self.put_loads(stage, 1, pre, post)
         self.spread(self.a_reads(1, stage, 1), 9, 40, post)
-        out += self.kstep(self.fa[0], self.fb[parity][0], init, pre, post)
+        out += self.kstep(self.fa[0], self.fb[parity][0], init, pre, post, dead)
         # own A reads done and own loads of one k-tile ago landed (the 8 newest may be in flight)
         out += ["s_waitcnt vmcnt(8) lgkmcnt(0)"] + barrier
         out += [f"; ---- k-tile on stage {stage}: k-step 1"]
@@ -167,28 +180,34 @@ class Variant:
         pre, post = {}, {}
         self.put_loads(stage, 0, pre, post)
         self.spread(self.a_reads(0, stage ^ 1, 0) + self.b_reads(parity ^ 1, stage ^ 1), 9, 52, post)
-        out += self.kstep(self.fa[1], self.fb[parity][1], False, pre, post)
+        out += self.kstep(self.fa[1], self.fb[parity][1], False, pre, post, dead)
         # every wave has the next k-tile's B fragments: the other stage's B half may be refilled
         out += ["s_waitcnt lgkmcnt(0)"] + barrier
         return out
 
-    def pair(self, init):
-        return self.ktile(0, init) + self.ktile(1, False)
+    def pair(self, init, dead_second=False):
+        return self.select_advance() + self.ktile(0, init) + self.ktile(1, False, dead_second)
 
     def tile_loop(self):
-        """One 256 x 256 tile: s48 pairs of k-tiles. On entry both stages hold (or are receiving)
-        k-tiles 0 and 1 and the pointers are on the next k-tile to fetch."""
+        """One 256 x 256 tile: s48 pairs of k-tiles, the second k-tile of the last pair dead when
+        s52 is 1 (an odd number of k-tiles; then at least two pairs). On entry both stages hold (or
+        are receiving) k-tiles 0 and 1 and the pointers are on the next k-tile to fetch."""
         out = ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_barrier"]
         out += self.a_reads(0, 0, 0) + self.b_reads(0, 0)
         out += ["s_waitcnt lgkmcnt(0)", "s_barrier"]
         out += self.pair(True)
         out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_eq_u32 s{S_CNT}, 0", "s_cbranch_scc1 2f", "1:",
+                # the last pair fetches the next tile's first k-tiles
                 f"s_cmp_eq_u32 s{S_CNT}, 1",
                 f"s_cselect_b64 s[{S_PA}:{S_PA + 1}], s[{S_PA_NEXT}:{S_PA_NEXT + 1}], s[{S_PA}:{S_PA + 1}]",
-                f"s_cselect_b64 s[{S_PB}:{S_PB + 1}], s[{S_PB_NEXT}:{S_PB_NEXT + 1}], s[{S_PB}:{S_PB + 1}]"]
+                f"s_cselect_b64 s[{S_PB}:{S_PB + 1}], s[{S_PB_NEXT}:{S_PB_NEXT + 1}], s[{S_PB}:{S_PB + 1}]",
+                # ... and is the one with the dead k-tile if the count is odd (s52 = 1; 0 never matches)
+                f"s_cmp_eq_u32 s{S_CNT}, s{S_ODD}", "s_cbranch_scc1 3f"]
         out += self.pair(False)
-        out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_lg_u32 s{S_CNT}, 0", "s_cbranch_scc1 1b", "2:",
-                "s_nop 15", "s_nop 15"]  # the last MFMAs retire before the accumulators are read
+        out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_lg_u32 s{S_CNT}, 0", "s_cbranch_scc1 1b",
+                "s_branch 2f", "3:"]
+        out += self.pair(False, dead_second=True)
+        out += ["2:", "s_nop 15", "s_nop 15"]  # the last MFMAs retire before the accumulators are read
         return out
 
     def prologue(self):
@@ -219,6 +238,9 @@ def emit():
             f"#define ML16_S_PB_NEXT \"{{s[{S_PB_NEXT}:{S_PB_NEXT + 1}]}}\"",
             f"#define ML16_S_CNT \"{{s{S_CNT}}}\"", f"#define ML16_S_LDSW \"{{s{S_LDSW}}}\"",
             f"#define ML16_S_STRIDE_A \"{{s{S_STRIDE_A}}}\"", f"#define ML16_S_STRIDE_B \"{{s{S_STRIDE_B}}}\"",
+            f"#define ML16_S_ODD \"{{s{S_ODD}}}\"", f"#define ML16_S_PEN_A \"{{s{S_PEN_A}}}\"",
+            f"#define ML16_S_PEN_B \"{{s{S_PEN_B}}}\"",
+            f"#define ML16_S_SCRATCH_CLOBBERS \"s{S_EFF_A}\", \"s{S_EFF_B}\"",
             f"#define ML16_HALF_BYTES {HALF_BYTES}", f"#define ML16_OPER_BYTES {OPER_BYTES}", ""]
     # The accumulators are not operands: the compiler must not know values live in a[0:255]
     # (it would move them around); the main loop lists them as clobbered.
@@ -250,9 +272,5 @@ def emit():
 
 if __name__ == "__main__":
     path = Path(__file__).resolve().parent / "mainloop16.inc"
-    args = sys.argv[1:]
-    if args and args[0] == "--out":
-        path = Path(args[1])
-        FLAGS.update(args[2:])
     path.write_text(emit())
     print(f"wrote {path}", file=sys.stderr)

@@ -1,24 +1,26 @@
 // Fused lm_head -> log-softmax -> label log-prob + entropy, forward and backward, for gfx950.
 //
 // Every matrix product of the path is one bf16 MFMA contraction D[i][j] = sum_k A[.]*B[.] over
-// 256 x 256 x 64 tiles; three kernels differ in how the operands are stored, the epilogues in
-// what happens to the accumulators:
-//   gemm_nt_sweep  (A[i][k], B[j][k], both k-contiguous)
-//     forward   : A = W [V,H],       B = hidden [T,H]     -> online softmax statistics, and in
-//                                                            the saving variant the bf16
-//                                                            exponentials e [T,V]
-//     recompute : A = W [V,H],       B = hidden [Tc,H]    -> dlogits (bf16, one or two layouts)
-//   gemm_mix_sweep (A[k][i] k-major, B[j][k] k-contiguous)
+// 256 x 256 x 64 tiles, by one kernel template in three operand layouts, with the epilogue (what
+// happens to the accumulators) as a template parameter:
+//   gemm16_sweep<VAR_NT>  (A[i][k], B[j][k], both k-contiguous)
+//     forward   : A = W [V,H],       B = hidden [T,H]     -> softmax statistics; the saving variant
+//                                                            also writes the bf16 exponentials e [T,V]
+//     recompute : A = W [V,H],       B = hidden [Tc,H]    -> dlogits (bf16)
+//   gemm16_sweep<VAR_MIX> (A[k][i] k-major, B[j][k] k-contiguous)
 //     dHidden   : A = W [V,H] as stored, B = e or dlogits [T,V'] -> bf16 store, rows scaled
-//                 (gemm_nt_sweep on a zero-padded W^T when V is not a multiple of 64)
-//   gemm_tn_sweep  (A[k][i], B[k][j], both k-major)
+//                 (VAR_NT on a zero-padded W^T when V is not a multiple of 64)
+//   gemm16_sweep<VAR_TN>  (A[k][i], B[k][j], both k-major)
 //     dWeight   : A = hidden [T,H] (scaled per row in the saved mode), B = e or dlogits [T,V']
-//                 -> bf16 store, or fp32 store / accumulate over token chunks
-//   gemm_nt_generic: any K (not a multiple of 64), register-staged loads.
-// The vocabulary is put on the MFMA "A" side of the forward so that, in the accumulator layout
-// of v_mfma_f32_32x32x16_bf16 (lane -> column j, registers -> rows i), each lane owns one token
-// and 16 vocabulary entries per 32x32 block: the softmax reductions over the vocabulary run
-// inside a lane and the fp32 logits never leave registers.
+//                 -> bf16 store, or fp32 store / accumulate
+// Its k-loop is the hand-scheduled v_mfma_f32_16x16x32_bf16 loop that gen_mainloop16.py writes into
+// mainloop16.inc (any K that is a multiple of 64, at least 128). gemm_nt_generic (both operands
+// k-contiguous, any K % 8 == 0, 32x32x16 MFMA, register-staged loads) takes every other shape,
+// with epilogues of the same arithmetic written for its accumulator layout.
+// The vocabulary is put on the MFMA "A" side of the forward: in a block column of the
+// accumulators 16 lanes own 16 tokens and four lane groups own 4 of every 16 vocabulary entries,
+// so the softmax reductions over the vocabulary run inside a lane and across four lanes, and the
+// fp32 logits never leave registers.
 //
 // Follows the algorithm of the reference's chunked LM head
 // (areal/models/mcore/vocab_parallel_head.py:564-735 forward, :737-938 backward) and the
@@ -42,7 +44,7 @@ struct GemmArgs {
   int K;                              // multiple of 8
   int acols, bcols;                   // k-major operands only: readable columns of A and B
                                       // (a k-major operand must have K readable rows)
-  // split-K (gemm_nt_sweep / gemm_mix_sweep with a store epilogue only): the grid is ksplit
+  // split-K (gemm16_sweep with a store epilogue only): the grid is ksplit
   // copies of the tile schedule; copy z contracts k-tiles [z*kt_per_split, (z+1)*kt_per_split)
   // and writes its partial result zstride bytes after the previous copy's. ksplit <= 1: off.
   int ksplit, kt_per_split;
@@ -233,538 +235,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_nt_generic(GemmArgs g, Sched sc
   Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
 }
 
-// ---------------------------------------------------------------------------------------
-// gemm_nt_sweep: the production main loop, for K % 64 == 0.
-//
-//  * Operand tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR staging). A wave
-//    instruction fills 8 rows x 128 B; which 16-byte chunk of its row a lane fetches is XOR
-//    swizzled so that the MFMA fragment reads (ds_read_b128, 32 rows x one chunk) hit every
-//    LDS bank exactly once (measured: 0 bank conflicts).
-//  * Two 64 KB stages form a ring over the flattened (A tile, k tile) sequence of the whole
-//    sweep: the loads of the next A tile are in flight while the epilogue of the current one
-//    runs. A stage is refilled right after the barrier that retires it (A half during the last
-//    k-step of the current k-tile, B half during the first k-step of the next).
-//  * The loop body is written as 8 slots per k-step, each {2 MFMA, 1 fragment read, 1 direct
-//    load}, fenced with sched_barrier so the compiler keeps the interleave.
-// ---------------------------------------------------------------------------------------
-constexpr int RING_OPER = TILE * BK;       // elements of one operand stage (32 KB)
-constexpr int RING_STAGE = 2 * RING_OPER;  // A then B
-DEVI int swz64(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 #define LDS_AS(p) ((void __attribute__((address_space(3)))*)(p))
-#define GLB_AS(p) ((const void __attribute__((address_space(1)))*)(p))
-
-template <class Epi>
-__global__ __launch_bounds__(NTHREADS) void gemm_nt_sweep(GemmArgs g, Sched sc,
-                                                          typename Epi::Params ep) {
-  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
-  int bj, split, ai_begin, ai_end;
-  int wg = blockIdx.x, nk = g.K / BK;
-  if (g.ksplit > 1) {
-    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
-    const int z = wg / per_copy;
-    wg -= z * per_copy;
-    // The schedule puts super-block sb on XCD sb % 8 (workgroup id % 8). Copies start on
-    // different XCDs, so that a schedule of fewer than 8 super-blocks still uses all of them.
-    wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);
-    const int kt0 = z * g.kt_per_split;
-    nk -= kt0;
-    nk = nk < g.kt_per_split ? nk : g.kt_per_split;
-    g.A += (int64_t)kt0 * BK;
-    g.B += (int64_t)kt0 * BK;
-    Epi::split_output(ep, (int64_t)z * g.zstride);
-    if (nk <= 0) return;
-  }
-  if (gemm_skipped(g)) return;
-  if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wa = wave >> 1, wb = wave & 1;
-
-  // ---- loader: lane -> (row of the wave's 64-row slice, swizzled chunk). A load address is a
-  // wave-uniform base (tile origin + k offset, scalar registers) plus a 32-bit byte offset per
-  // lane that is fixed for the tile, so the k loop spends no vector instructions on addresses.
-  // The host keeps 256 * ld * 2 below 2^32.
-  uint32_t oa[8], ob[8];
-  const u16* a_tile;  // origin of the A tile the loader is on
-  int l_ai = ai_begin, l_kt = 0;
-  auto set_a_rows = [&](int ai) {
-    a_tile = g.A + (int64_t)ai * TILE * g.lda;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = wave * 64 + i * 8 + (lane >> 3);
-      int rr = ai * TILE + r < g.M ? r : g.M - 1 - ai * TILE;  // clamped rows are discarded by the epilogue
-      oa[i] = 2u * ((uint32_t)rr * (uint32_t)g.lda + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
-    }
-  };
-  set_a_rows(ai_begin);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int r = wave * 64 + i * 8 + (lane >> 3);
-    int rr = bj * TILE + r < g.N ? r : g.N - 1 - bj * TILE;
-    ob[i] = 2u * ((uint32_t)rr * (uint32_t)g.ldb + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
-  }
-  const u16* b_tile = g.B + (int64_t)bj * TILE * g.ldb;
-  int l_stage = 0;  // stage the loader fills next
-  auto load_a = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + wave * 64 * BK + i * 8 * BK;
-    const char* base = (const char*)(a_tile + l_kt * BK);
-    __builtin_amdgcn_global_load_lds(GLB_AS(base + oa[i]), LDS_AS(dst), 16, 0, 0);
-  };
-  auto load_b = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + wave * 64 * BK + i * 8 * BK;
-    const char* base = (const char*)(b_tile + l_kt * BK);
-    // keeps the offset a 32-bit value up to the load, the form that selects the scalar-base
-    // addressing mode (hoisted out of the sweep it would be widened to 64 bits)
-    uint32_t o = ob[i];
-    asm volatile("" : "+v"(o));
-    __builtin_amdgcn_global_load_lds(GLB_AS(base + o), LDS_AS(dst), 16, 0, 0);
-  };
-  auto loader_advance = [&]() {  // after both halves of a stage were issued
-    l_stage ^= 1;
-    if (l_kt + 1 < nk) {
-      ++l_kt;
-    } else if (l_ai + 1 < ai_end) {
-      ++l_ai;
-      l_kt = 0;
-      set_a_rows(l_ai);
-    }  // else: keep re-loading the last k-tile into the idle stage (never consumed)
-  };
-
-  // ---- fragments
-  const int rl = lane & 31, ch = lane >> 5;
-  const int sw = swz64(rl);
-  bf16x8 af[2][4], bf[2][4];
-  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
-  auto dsr = [&](int st, int s, int buf, int f) {
-    const int slot = ((s * 2 + ch) ^ sw) * 8;
-    const u16* sA = lds + st * RING_STAGE + wa * 128 * BK + rl * BK + slot;
-    const u16* sB = lds + st * RING_STAGE + RING_OPER + wb * 128 * BK + rl * BK + slot;
-    if (f == 0) af[buf][0] = *(const bf16x8*)(sA);
-    else if (f <= 4) bf[buf][f - 1] = *(const bf16x8*)(sB + (f - 1) * 32 * BK);
-    else af[buf][f - 4] = *(const bf16x8*)(sA + (f - 4) * 32 * BK);
-  };
-  f32x16 acc[4][4];
-  auto mfma2 = [&](int buf, int p) {
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int idx = 2 * p + q, a = idx >> 2, b = idx & 3;
-      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
-    }
-  };
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  };
-
-  typename Epi::State st;
-  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
-
-  // ---- prologue: stage 0 completely, A half of stage 1
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_b(i);
-  loader_advance();
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-  zero_acc();
-  __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): everything but the last 8 loads has landed
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
-
-  // Outer loop over A tiles, inner (hot) loop over k-tiles; the loader state and the stage
-  // parity run on across tile boundaries.
-  int cs = 0;
-  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
-    for (int c_kt = 0; c_kt < nk; ++c_kt) {
-      // k-steps 0..2: fragments of the next k-step are fetched while this one multiplies;
-      // step 0 also issues the B half of the stage the loader is filling.
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-#pragma unroll
-        for (int p = 0; p < 8; ++p) {
-          mfma2(s & 1, p);
-          dsr(cs, s + 1, (s + 1) & 1, p);
-          if (s == 0) load_b(p);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (s == 0) loader_advance();
-      }
-      // every wave: own fragment reads done, own direct loads landed; then all waves agree
-      __builtin_amdgcn_s_waitcnt(0x0070);
-      __builtin_amdgcn_s_barrier();
-      // k-step 3, with the first fragments of the next k-tile and the A half of the stage
-      // that the barrier has just retired
-#pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        mfma2(1, p);
-        dsr(cs ^ 1, 0, 0, p);
-        load_a(p);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      cs ^= 1;
-    }
-    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
-    zero_acc();
-  }
-  __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
-  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
-}
-
-// ---------------------------------------------------------------------------------------
-// gemm_tn_sweep: D[i][j] = sum_k A[k][i] * B[k][j], both operands stored k-major (row = k,
-// the i / j index contiguous), K % 64 == 0. Used for dWeight[v][h] = sum_t dl[t][v] hidden[t][h]
-// straight from the row-major dlogits and hidden states, so no transposed copies are needed.
-//
-// A stage holds 64 k-rows x 256 columns per operand (512 B per row). Fragments are fetched with
-// ds_read_b64_tr_b16: inside a group of 16 lanes, lanes 4r..4r+3 point at 16 consecutive columns
-// of row k0+r (r = 0..3) and lane q receives column q for those four k. Two such reads give
-// the 8 k values one MFMA operand needs. The 64-byte chunks of a row are XOR swizzled with
-// (k & 3) so that the four rows a group reads fall into different LDS bank groups.
-// ---------------------------------------------------------------------------------------
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-// 16 bytes per lane from global memory straight into LDS (lane L lands at lds_addr + 16 L).
-// Issued as inline assembly in the k-major kernel: when the compiler sees the load-to-LDS
-// builtin next to ds_read_b64_tr_b16 it cannot prove they do not alias and puts a full
-// vmcnt(0) wait in front of every transposed read, which serialises the prefetch with the
-// math. The kernel orders the two itself with its explicit vmcnt waits and barriers.
-// The address is a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset per
-// lane, so advancing along k costs scalar adds only.
-DEVI void lds_dma16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-}
-DEVI uint32_t lds_addr_of(const u16* p) { return (uint32_t)(uintptr_t)LDS_AS(p); }
-
-template <class Epi>
-__global__ __launch_bounds__(NTHREADS) void gemm_tn_sweep(GemmArgs g, Sched sc,
-                                                          typename Epi::Params ep) {
-  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
-  int bj, split, ai_begin, ai_end;
-  if (gemm_skipped(g)) return;
-  if (!sched_decode(sc, blockIdx.x, bj, split, ai_begin, ai_end)) return;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wa = wave >> 1, wb = wave & 1;
-  const int nk = g.K / BK;
-
-  // ---- loader. Instruction i of a wave fills rows k = wave*16 + 2*i + (lane >> 5) of the
-  // stage; lane -> 16-byte piece (lane & 31) of the LDS row, i.e. chunk position cp = piece/4.
-  // It fetches the chunk ci = cp ^ (k & 3); k & 3 = ((i & 1) * 2 + (lane >> 5)) & 3.
-  const int hl = lane >> 5, piece = lane & 31;
-  uint32_t oa[2], ob[2];  // i even / odd: byte offset of the lane's piece of its row at k-tile 0
-  int l_ai = ai_begin, l_kt = 0;
-  // global 16-byte piece of instruction parity par for column tile `tile`
-  auto piece_col = [&](int tile, int ncols, int par) -> int {
-    const int k3 = (par * 2 + hl) & 3;
-    int gp = tile * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + (piece & 3);
-    const int last = ncols / 8 - 1;
-    gp = gp < last ? gp : last;  // columns past the end are discarded by the epilogue
-    return gp * 8;
-  };
-  // offsets stay below 2^32: the host checks 64 * ld * 2 + 2 * cols < 2^32
-  auto set_a_cols = [&](int ai) {
-#pragma unroll
-    for (int par = 0; par < 2; ++par)
-      oa[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.lda +
-                      (uint32_t)piece_col(ai, g.acols, par));
-  };
-  set_a_cols(ai_begin);
-#pragma unroll
-  for (int par = 0; par < 2; ++par)
-    ob[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.ldb +
-                    (uint32_t)piece_col(bj, g.bcols, par));
-  int l_stage = 0;
-  auto load_a = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
-    const u16* base = g.A + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
-    lds_dma16(base, oa[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
-  };
-  auto load_b = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + (wave * 16 + i * 2) * TILE;
-    const u16* base = g.B + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.ldb;
-    lds_dma16(base, ob[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
-  };
-  auto loader_advance = [&]() {
-    l_stage ^= 1;
-    if (l_kt + 1 < nk) {
-      ++l_kt;
-    } else if (l_ai + 1 < ai_end) {
-      ++l_ai;
-      l_kt = 0;
-      set_a_cols(l_ai);
-    }
-  };
-
-  // ---- fragments: group G = lane/16 -> column half (G & 1) and k half (G >> 1);
-  // q = lane%16 -> row r = q/4 of the four, column quad q%4.
-  const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
-  // byte offset inside a stage operand, without the block (x) and step (s, half) terms
-  const int frag_row = (G >> 1) * 8 + r4;                         // k within the k-step
-  const int frag_byte = (G & 1) * 32 + (q & 3) * 8;              // inside the 64-byte chunk
-  bf16x8 af[2][4], bf[2][4];
-  auto tr_read = [&](const u16* oper, int wsel, int x, int s) -> bf16x8 {
-    const int ci = wsel * 4 + x;
-    const char* base = (const char*)oper + ((ci ^ r4) << 6) + frag_byte;
-    const int k0 = s * 16 + frag_row;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)(base + (k0 << 9)));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)(base + ((k0 + 4) << 9)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, v);
-  };
-  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
-  auto dsr = [&](int st, int s, int buf, int f) {
-    const u16* sA = lds + st * RING_STAGE;
-    const u16* sB = sA + RING_OPER;
-    if (f == 0) af[buf][0] = tr_read(sA, wa, 0, s);
-    else if (f <= 4) bf[buf][f - 1] = tr_read(sB, wb, f - 1, s);
-    else af[buf][f - 4] = tr_read(sA, wa, f - 4, s);
-  };
-  f32x16 acc[4][4];
-  auto mfma2 = [&](int buf, int p) {
-#pragma unroll
-    for (int qq = 0; qq < 2; ++qq) {
-      const int idx = 2 * p + qq, a = idx >> 2, b = idx & 3;
-      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
-    }
-  };
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  };
-
-  typename Epi::State st;
-  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
-
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_b(i);
-  loader_advance();
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-  zero_acc();
-  __builtin_amdgcn_s_waitcnt(0x0F78);
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
-
-  int cs = 0;
-  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
-    for (int c_kt = 0; c_kt < nk; ++c_kt) {
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-#pragma unroll
-        for (int p = 0; p < 8; ++p) {
-          mfma2(s & 1, p);
-          dsr(cs, s + 1, (s + 1) & 1, p);
-          if (s == 0) load_b(p);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (s == 0) loader_advance();
-      }
-      __builtin_amdgcn_s_waitcnt(0x0070);
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        mfma2(1, p);
-        dsr(cs ^ 1, 0, 0, p);
-        load_a(p);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      cs ^= 1;
-    }
-    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
-    zero_acc();
-  }
-  __builtin_amdgcn_s_waitcnt(0x0070);
-  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
-}
-
-// ---------------------------------------------------------------------------------------
-// gemm_mix_sweep: D[i][j] = sum_k A[k][i] * B[j][k]: A stored k-major (row = k, i contiguous,
-// as gemm_tn_sweep reads it), B stored with k contiguous (as gemm_nt_sweep reads it),
-// K % 64 == 0 and A has K readable rows. Used for dHidden[t][h] = sum_v dl[t][v] W[v][h] straight
-// from the [V, H] weight: no transposed copy of the weight is made. The A half of a stage has
-// gemm_tn_sweep's layout and transposed fragment reads, the B half gemm_nt_sweep's; all direct
-// loads are inline assembly for the reason given at lds_dma16. Split-K as in gemm_nt_sweep.
-// ---------------------------------------------------------------------------------------
-template <class Epi>
-__global__ __launch_bounds__(NTHREADS) void gemm_mix_sweep(GemmArgs g, Sched sc,
-                                                           typename Epi::Params ep) {
-  __shared__ __attribute__((aligned(1024))) u16 lds[2 * RING_STAGE];
-  int bj, split, ai_begin, ai_end;
-  int wg = blockIdx.x, nk = g.K / BK;
-  if (g.ksplit > 1) {
-    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
-    const int z = wg / per_copy;
-    wg -= z * per_copy;
-    wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);  // copies start on different XCDs
-    const int kt0 = z * g.kt_per_split;
-    nk -= kt0;
-    nk = nk < g.kt_per_split ? nk : g.kt_per_split;
-    g.A += (int64_t)kt0 * BK * g.lda;
-    g.B += (int64_t)kt0 * BK;
-    Epi::split_output(ep, (int64_t)z * g.zstride);
-    if (nk <= 0) return;
-  }
-  if (gemm_skipped(g)) return;
-  if (!sched_decode(sc, wg, bj, split, ai_begin, ai_end)) return;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wa = wave >> 1, wb = wave & 1;
-
-  // ---- loader, A half (k-major): see gemm_tn_sweep
-  const int hl = lane >> 5, piece = lane & 31;
-  uint32_t oa[2], ob[8];
-  int l_ai = ai_begin, l_kt = 0;
-  auto set_a_cols = [&](int ai) {
-#pragma unroll
-    for (int par = 0; par < 2; ++par) {
-      const int k3 = (par * 2 + hl) & 3;
-      int gp = ai * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + (piece & 3);
-      const int last = g.acols / 8 - 1;
-      gp = gp < last ? gp : last;  // columns past the end are discarded by the epilogue
-      oa[par] = 2u * ((uint32_t)(wave * 16 + 2 * par + hl) * (uint32_t)g.lda + (uint32_t)(gp * 8));
-    }
-  };
-  set_a_cols(ai_begin);
-  // ---- loader, B half (k contiguous): see gemm_nt_sweep
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int r = wave * 64 + i * 8 + (lane >> 3);
-    const int rr = bj * TILE + r < g.N ? r : g.N - 1 - bj * TILE;
-    ob[i] = 2u * ((uint32_t)rr * (uint32_t)g.ldb + (uint32_t)(((lane & 7) ^ swz64(r)) * 8));
-  }
-  const u16* b_tile = g.B + (int64_t)bj * TILE * g.ldb;
-  int l_stage = 0;
-  auto load_a = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + (wave * 16 + i * 2) * TILE;
-    const u16* base = g.A + ((int64_t)l_kt * BK + (i >> 1) * 4) * g.lda;
-    lds_dma16(base, oa[i & 1], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
-  };
-  auto load_b = [&](int i) {
-    u16* dst = lds + l_stage * RING_STAGE + RING_OPER + wave * 64 * BK + i * 8 * BK;
-    lds_dma16(b_tile + l_kt * BK, ob[i], __builtin_amdgcn_readfirstlane(lds_addr_of(dst)));
-  };
-  auto loader_advance = [&]() {
-    l_stage ^= 1;
-    if (l_kt + 1 < nk) {
-      ++l_kt;
-    } else if (l_ai + 1 < ai_end) {
-      ++l_ai;
-      l_kt = 0;
-      set_a_cols(l_ai);
-    }
-  };
-
-  // ---- fragments: A by transposed reads (gemm_tn_sweep), B by 16-byte reads (gemm_nt_sweep)
-  const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
-  const int frag_row = (G >> 1) * 8 + r4;
-  const int frag_byte = (G & 1) * 32 + (q & 3) * 8;
-  const int rl = lane & 31, ch = lane >> 5;
-  const int sw = swz64(rl);
-  bf16x8 af[2][4], bf[2][4];
-  auto tr_read = [&](const u16* oper, int x, int s) -> bf16x8 {
-    const int ci = wa * 4 + x;
-    const char* base = (const char*)oper + ((ci ^ r4) << 6) + frag_byte;
-    const int k0 = s * 16 + frag_row;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)(base + (k0 << 9)));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)(base + ((k0 + 4) << 9)));
-    typedef short s16x8 __attribute__((ext_vector_type(8)));
-    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, v);
-  };
-  // fragment f (order a0,b0,b1,b2,b3,a1,a2,a3) of k-step s from stage st into buffer buf
-  auto dsr = [&](int st, int s, int buf, int f) {
-    const u16* sA = lds + st * RING_STAGE;
-    const u16* sB = sA + RING_OPER + wb * 128 * BK + rl * BK + ((s * 2 + ch) ^ sw) * 8;
-    if (f == 0) af[buf][0] = tr_read(sA, 0, s);
-    else if (f <= 4) bf[buf][f - 1] = *(const bf16x8*)(sB + (f - 1) * 32 * BK);
-    else af[buf][f - 4] = tr_read(sA, f - 4, s);
-  };
-  f32x16 acc[4][4];
-  auto mfma2 = [&](int buf, int p) {
-#pragma unroll
-    for (int qq = 0; qq < 2; ++qq) {
-      const int idx = 2 * p + qq, a = idx >> 2, b = idx & 3;
-      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[buf][a], bf[buf][b], acc[a][b], 0, 0, 0);
-    }
-  };
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
-  };
-
-  typename Epi::State st;
-  Epi::begin(st, ep, bj * TILE + wb * 128, split, wa, lane);
-
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_b(i);
-  loader_advance();
-#pragma unroll
-  for (int i = 0; i < 8; ++i) load_a(i);
-  zero_acc();
-  __builtin_amdgcn_s_waitcnt(0x0F78);
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int f = 0; f < 8; ++f) dsr(0, 0, 0, f);
-
-  int cs = 0;
-  for (int c_ai = ai_begin; c_ai < ai_end; ++c_ai) {
-    for (int c_kt = 0; c_kt < nk; ++c_kt) {
-#pragma unroll
-      for (int s = 0; s < 3; ++s) {
-#pragma unroll
-        for (int p = 0; p < 8; ++p) {
-          mfma2(s & 1, p);
-          dsr(cs, s + 1, (s + 1) & 1, p);
-          if (s == 0) load_b(p);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (s == 0) loader_advance();
-      }
-      __builtin_amdgcn_s_waitcnt(0x0070);
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int p = 0; p < 8; ++p) {
-        mfma2(1, p);
-        dsr(cs ^ 1, 0, 0, p);
-        load_a(p);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      cs ^= 1;
-    }
-    Epi::tile(st, ep, acc, c_ai * TILE + wa * 128, bj * TILE + wb * 128, lane);
-    zero_acc();
-  }
-  __builtin_amdgcn_s_waitcnt(0x0070);
-  Epi::end(st, ep, bj * TILE + wb * 128, split, wa, lane);
-}
 
 // ---------------------------------------------------------------------------------------
 // Epilogues. Each is a template on EDGE: the interior of the tile grid (every tile fully inside
@@ -1564,7 +1035,10 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
   const char* pb = (const char*)(B_KM ? g.B : g.B + (int64_t)bj * TILE * g.ldb);
   const char* pb_next = pb;
   const uint32_t ldsw = lds_base + (uint32_t)wave * 8192u;
-  const int npairs = nk >> 1;
+  // an odd number of k-tiles: one more pair whose second k-tile is dead (see gen_mainloop16.py)
+  const int npairs = (nk + 1) >> 1;
+  const int odd = nk & 1;
+  const uint32_t pen_a = odd ? 0u : stride_a, pen_b = odd ? 0u : stride_b;
   u16* stage = (u16*)(lds + RING16_BYTES + wave * STAGE16_BYTES);
 
   if (VAR == VAR_NT)
@@ -1599,23 +1073,23 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
       asm volatile(ML16_NT_TILE
                    : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
                    : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
-                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
-                     ML16_NT_VGPR_INPUTS(oa, ob, ra, rb)
-                   : "memory", "scc", ML16_NT_CLOBBERS, ML16_ACC_CLOBBERS);
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
+                     ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_NT_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_NT_CLOBBERS, ML16_ACC_CLOBBERS);
     else if (VAR == VAR_TN)
       asm volatile(ML16_TN_TILE
                    : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
                    : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
-                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
-                     ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
-                   : "memory", "scc", ML16_TN_CLOBBERS, ML16_ACC_CLOBBERS);
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
+                     ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_TN_CLOBBERS, ML16_ACC_CLOBBERS);
     else
       asm volatile(ML16_MIX_TILE
                    : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
                    : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
-                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b),
-                     ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
-                   : "memory", "scc", ML16_MIX_CLOBBERS, ML16_ACC_CLOBBERS);
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
+                     ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_MIX_CLOBBERS, ML16_ACC_CLOBBERS);
     // The lane number goes through an empty block so that nothing of the epilogue's per-lane
     // address arithmetic is computed ahead of the main loop, which leaves the compiler only
     // v[0:ML16_*_FIRST_VGPR) for values that live across it.
@@ -2038,11 +1512,10 @@ int pick_splits(int nbj, int nai, int target_wgs) {
   return S;
 }
 
-enum { KERNEL_GENERIC = 0, KERNEL_NT = 1, KERNEL_TN = 2, KERNEL_MIX = 3,
-       KERNEL16_NT = 4, KERNEL16_TN = 5, KERNEL16_MIX = 6 };
+enum { KERNEL_GENERIC = 0, KERNEL16_NT = 4, KERNEL16_TN = 5, KERNEL16_MIX = 6 };
 
-// K ranges the hand-scheduled main loop takes: whole pairs of k-tiles.
-bool k16_ok(int64_t K) { return K >= 2 * BK && K % (2 * BK) == 0; }
+// K ranges the hand-scheduled main loop takes: at least two whole k-tiles.
+bool k16_ok(int64_t K) { return K >= 2 * BK && K % BK == 0; }
 
 template <class Epi, int KERNEL>
 int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
@@ -2051,48 +1524,36 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
   if (S > nai) S = nai;
   if (S < 1) S = 1;
   const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
-  if constexpr (KERNEL == KERNEL_NT) {
-    // the loader addresses a tile as a 64-bit base plus 32-bit byte offsets per lane
-    if (g.lda > (1 << 22) || g.ldb > (1 << 22)) return AREAL_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((gemm_nt_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
-                       dim3(NTHREADS), 0, stream, g, sc, ep);
-  }
-  else if constexpr (KERNEL == KERNEL_MIX) {
-    if (g.lda > (1 << 24) || g.ldb > (1 << 22)) return AREAL_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((gemm_mix_sweep<Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
-                       dim3(NTHREADS), 0, stream, g, sc, ep);
-  } else if constexpr (KERNEL == KERNEL_TN) {
-    // the loader addresses a k-tile as a 64-bit base plus 32-bit byte offsets per lane
-    if (g.lda > (1 << 24) || g.ldb > (1 << 24)) return AREAL_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((gemm_tn_sweep<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
-                       sc, ep);
-  }
-  else if constexpr (KERNEL >= KERNEL16_NT) {
+  if constexpr (KERNEL >= KERNEL16_NT) {
     constexpr int VAR = KERNEL == KERNEL16_NT ? VAR_NT : KERNEL == KERNEL16_TN ? VAR_TN : VAR_MIX;
+    // the loader addresses a tile as a 64-bit base plus 32-bit byte offsets per lane
     if (g.lda > (VAR == VAR_NT ? (1 << 22) : (1 << 24)) || g.ldb > (VAR == VAR_TN ? (1 << 24) : (1 << 22)))
       return AREAL_ERR_UNSUPPORTED;
-    if (!k16_ok(g.K) || (g.ksplit > 1 && (g.kt_per_split & 1))) return AREAL_ERR_UNSUPPORTED;
+    // every copy of a split-K launch needs two k-tiles too (split_ktiles() sees to the last one)
+    if (!k16_ok(g.K) || (g.ksplit > 1 && (g.kt_per_split < 2 || g.K / BK - (g.ksplit - 1) * g.kt_per_split < 2)))
+      return AREAL_ERR_UNSUPPORTED;
     // a k-major A operand carries its tile column in the lane offsets: one A tile per workgroup
     if (VAR != VAR_NT && S != nai) return AREAL_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm16_sweep<VAR, Epi>), dim3(sched_grid(sc) * (g.ksplit > 1 ? g.ksplit : 1)),
                        dim3(NTHREADS), 0, stream, g, sc, ep);
-  }
-  else
+  } else {
+    if (g.ksplit > 1) return AREAL_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm_nt_generic<Epi>), dim3(sched_grid(sc)), dim3(NTHREADS), 0, stream, g,
                        sc, ep);
+  }
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
 
-// How a GEMM is cut into launches. K % 64 == 0 takes the fast kernel: interior tiles with the
-// predicate-free epilogue, then the ragged last B tile and the ragged last A tile with the
-// EDGE epilogue. Any other K takes the generic kernel over all tiles in one launch.
+// How a GEMM is cut into launches. The hand-scheduled kernel (k16: K a multiple of 64, at least
+// 128, and the caller's epilogue and operand layout allow it) runs the interior tiles with the
+// predicate-free epilogue, then the ragged last B tile and the ragged last A tile with the EDGE
+// epilogue. Everything else is one launch of the generic kernel over all tiles.
 struct Regions {
-  bool fast;
-  int nai_full, nbj_full;  // tiles entirely inside M and N
+  bool k16;
+  int nai_full, nbj_full;  // tiles entirely inside M and N (k16), else all tiles
   bool ragged_a, ragged_b;
   int S;                   // splits used for the interior and the ragged-B launch
-  bool k16;                // K suits the hand-scheduled main loop (callers may still clear it)
   bool fold_a;             // the ragged last A tile runs as rows [M - 256, M) at the end of the last
                            // split's sweep (GemmArgs::overlap_last_a) instead of a launch of its own;
                            // set by fold_ragged_a() for the epilogues that support it
@@ -2101,14 +1562,13 @@ struct Regions {
 // main launch when there is a full tile for it to overlap and whole 64-column groups (the stores
 // of the saved buffers are 16-byte pieces, and columns [V, round_up(V, 64)) would stay unwritten).
 void fold_ragged_a(Regions& r, int64_t M) {
-  r.fold_a = r.fast && r.k16 && r.ragged_a && r.nai_full >= 1 && M % BK == 0;
+  r.fold_a = r.k16 && r.ragged_a && r.nai_full >= 1 && M % BK == 0;
 }
-Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixed) {
+Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixed, bool allow16 = true) {
   Regions r;
-  r.fast = (K > 0 && K % BK == 0);
-  r.k16 = k16_ok(K);
+  r.k16 = allow16 && k16_ok(K);
   r.fold_a = false;
-  if (r.fast) {
+  if (r.k16) {
     r.nai_full = (int)(M / TILE); r.nbj_full = (int)(N / TILE);
     r.ragged_a = (M % TILE) != 0; r.ragged_b = (N % TILE) != 0;
   } else {
@@ -2121,38 +1581,38 @@ Regions plan_regions(int64_t M, int64_t N, int64_t K, int target_wgs, int S_fixe
   return r;
 }
 
-// EpiT<EDGE>; ep_edge_a is the parameter block of the ragged-A launch (it may differ from ep in
-// where it writes its partial results).
+// Epi16<EDGE> is the epilogue written for the hand-scheduled kernel's accumulator layout, Epi32<EDGE>
+// the same arithmetic for the generic kernel's; ep_edge_a is the parameter block of the ragged-A
+// launch (it may differ from ep in where it writes its partial results).
 // MERGE_EDGES: epilogues whose bounds predicates are cheap (plain stores) run ONE launch of the
 // EDGE = true instance over all tiles when any tile is ragged: a separate launch for the last
 // row of tiles has too few workgroups to fill the chip and each walks the whole K range.
-template <template <bool> class EpiT, class P, int FAST_KERNEL = KERNEL_NT, bool MERGE_EDGES = false>
+template <template <bool> class Epi16, template <bool> class Epi32, class P, int KERNEL16, bool MERGE_EDGES = false>
 int launch_gemm(const GemmArgs& g, const Regions& r, const P& ep, const P& ep_edge_a,
                 hipStream_t stream) {
   int rc;
-  if constexpr (FAST_KERNEL >= KERNEL16_NT) {
-    if (!r.fast || !r.k16) return AREAL_ERR_UNSUPPORTED;  // these epilogues have no generic kernel
-  } else if (!r.fast) {
-    return launch_region<EpiT<true>, KERNEL_GENERIC>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
+  if (!r.k16) {
+    if constexpr (KERNEL16 != KERNEL16_NT) return AREAL_ERR_UNSUPPORTED;  // the generic kernel reads k-contiguous operands
+    return launch_region<Epi32<true>, KERNEL_GENERIC>(g, 0, r.nbj_full, 0, r.nai_full, r.S, ep, stream);
   }
   if (MERGE_EDGES && (r.ragged_a || r.ragged_b)) {
     const int nai = r.nai_full + (r.ragged_a ? 1 : 0);
-    return launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), 0, nai,
-                                                  r.S == r.nai_full ? nai : r.S, ep, stream);
+    return launch_region<Epi16<true>, KERNEL16>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), 0, nai,
+                                                r.S == r.nai_full ? nai : r.S, ep, stream);
   }
   GemmArgs gm = g;
   int nai_main = r.nai_full;
-  if constexpr (FAST_KERNEL == KERNEL16_NT) {
+  if constexpr (KERNEL16 == KERNEL16_NT) {
     if (r.fold_a) { gm.overlap_last_a = 1; ++nai_main; }
   }
-  if ((rc = launch_region<EpiT<false>, FAST_KERNEL>(gm, 0, r.nbj_full, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
+  if ((rc = launch_region<Epi16<false>, KERNEL16>(gm, 0, r.nbj_full, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_b &&
-      (rc = launch_region<EpiT<true>, FAST_KERNEL>(gm, r.nbj_full, 1, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
+      (rc = launch_region<Epi16<true>, KERNEL16>(gm, r.nbj_full, 1, 0, nai_main, r.S, ep, stream)) != AREAL_OK)
     return rc;
   if (r.ragged_a && nai_main == r.nai_full &&
-      (rc = launch_region<EpiT<true>, FAST_KERNEL>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
-                                                   ep_edge_a, stream)) != AREAL_OK)
+      (rc = launch_region<Epi16<true>, KERNEL16>(g, 0, r.nbj_full + (r.ragged_b ? 1 : 0), r.nai_full, 1, 1,
+                                                 ep_edge_a, stream)) != AREAL_OK)
     return rc;
   return AREAL_OK;
 }
@@ -2169,26 +1629,20 @@ int check_operand(const void* p, int64_t ld) {
 int fwd_slots_per_split(const Regions& r) { return r.k16 ? 2 : 4; }
 int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + ((r.ragged_a && !r.fold_a) ? 1 : 0)); }
 
-// The four plain-store epilogues over either family of kernels. mode: 0 bf16, 1 fp32,
-// 2 fp32 accumulate, 3 bf16 with a factor per output row. The hand-scheduled kernels write bf16
-// as 16-byte pieces of whole rows.
-template <int KERNEL, int KERNEL16>
-int launch_store(const GemmArgs& g, const Regions& r, const StoreParams& ep, int mode, hipStream_t stream) {
-  bool use16 = r.k16;
-  if (mode == 0 || mode == 3) use16 = use16 && ep.ldo % 8 == 0 && aligned16(ep.out) && ep.M % 8 == 0;
-  if (use16) {
-    switch (mode) {
-      case 0: return launch_gemm<Store16Bf16, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
-      case 1: return launch_gemm<Store16F32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
-      case 2: return launch_gemm<Accum16F32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
-      default: return launch_gemm<Store16Bf16Scaled, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
-    }
-  }
+// The four plain-store epilogues over either kernel. mode: 0 bf16, 1 fp32, 2 fp32 accumulate,
+// 3 bf16 with a factor per output row. The hand-scheduled kernel writes bf16 as 16-byte pieces of
+// whole rows, which needs aligned output rows; the generic kernel (k-contiguous operands only)
+// takes what it cannot. S_fixed as plan_regions (stores want one A tile per workgroup).
+template <int KERNEL16>
+int launch_store(const GemmArgs& g, const StoreParams& ep, int mode, hipStream_t stream) {
+  bool allow16 = true;
+  if (mode == 0 || mode == 3) allow16 = ep.ldo % 8 == 0 && aligned16(ep.out) && ep.M % 8 == 0;
+  const Regions r = plan_regions(ep.M, ep.N, g.K, 0, 1 << 20, allow16);
   switch (mode) {
-    case 0: return launch_gemm<StoreBf16, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
-    case 1: return launch_gemm<StoreF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
-    case 2: return launch_gemm<AccumF32, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
-    default: return launch_gemm<StoreBf16Scaled, StoreParams, KERNEL, true>(g, r, ep, ep, stream);
+    case 0: return launch_gemm<Store16Bf16, StoreBf16, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+    case 1: return launch_gemm<Store16F32, StoreF32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+    case 2: return launch_gemm<Accum16F32, AccumF32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
+    default: return launch_gemm<Store16Bf16Scaled, StoreBf16Scaled, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
   }
 }
 
@@ -2215,6 +1669,18 @@ double sched_cost(const Sched& sc, int z) {
   return (double)ceil_div_i64(worst, 32) / z + 0.03 * (z - 1);
 }
 
+// k-tiles per copy of a launch whose nk k-tiles are split over (up to) z copies: whole pairs (an
+// even count runs without a dead k-tile), no empty copy, and at least two k-tiles in the last one.
+void split_ktiles(int nk, int& z, int& kps) {
+  kps = (int)ceil_div_i64(nk, z);
+  kps += kps & 1;
+  z = (int)ceil_div_i64(nk, kps);
+  if (z > 1 && nk - (z - 1) * kps < 2) {  // a single k-tile left over: the last copy but one takes it
+    kps += 2;
+    z = (int)ceil_div_i64(nk, kps);
+  }
+}
+
 int dh_ksplit(int64_t H, int64_t T, int64_t K) {
   const int64_t tiles = ceil_div_i64(H, TILE) * ceil_div_i64(T, TILE);
   if (tiles >= 2048 || K % BK != 0) return 1;
@@ -2235,30 +1701,29 @@ size_t dh_partial_bytes(int64_t H, int64_t T, int64_t K) {
 }
 
 // The weight can be contracted as stored ([V, H], k-major for dHidden) when its V rows cover the
-// K = round_up(V, 64) rows the kernel reads; otherwise a zero-padded transposed copy is used.
-bool dh_weight_in_place(int64_t V) { return V % BK == 0; }
+// K = round_up(V, 64) rows the kernel reads (and make two k-tiles, which the kernel that reads
+// k-major operands needs); otherwise a zero-padded transposed copy is used.
+bool dh_weight_in_place(int64_t V) { return V % BK == 0 && V >= 2 * BK; }
 
 // dHidden[t, h] = tscale[t] * sum_v dl[t, v] * W[v, h] (tscale = 1 when null), bf16 out;
 // split-K through `partial` when it pays. w is the weight itself [V, H] when
 // dh_weight_in_place(V), else its transposed copy W^T [H, ldv].
-template <int KERNEL, int KERNEL16>
+template <int KERNEL16>
 int launch_dhidden_k(const GemmArgs& g0, int64_t H, int64_t T, int64_t ldv, void* dhidden,
                      float* partial, const float* tscale, hipStream_t stream) {
   GemmArgs g = g0;
-  const Regions r = plan_regions(H, T, ldv, 0, 1 << 20);
   int z = dh_ksplit(H, T, ldv);
-  int kps = z > 1 ? (int)ceil_div_i64(ldv / BK, z) : 0;
-  if (r.k16) kps += kps & 1;  // the hand-scheduled loop walks pairs of k-tiles
-  if (z > 1) z = (int)ceil_div_i64(ldv / BK, kps);  // no empty split
+  int kps = 0;
+  if (z > 1) split_ktiles((int)(ldv / BK), z, kps);
   if (z <= 1 || partial == nullptr) {
     const StoreParams ep{dhidden, H, (int)H, (int)T, tscale};
-    return launch_store<KERNEL, KERNEL16>(g, r, ep, tscale != nullptr ? 3 : 0, stream);
+    return launch_store<KERNEL16>(g, ep, tscale != nullptr ? 3 : 0, stream);
   }
   g.ksplit = z;
   g.kt_per_split = kps;
   g.zstride = T * H * (int64_t)sizeof(float);
   const StoreParams ep{partial, H, (int)H, (int)T, nullptr};
-  int rc = launch_store<KERNEL, KERNEL16>(g, r, ep, 1, stream);
+  int rc = launch_store<KERNEL16>(g, ep, 1, stream);
   if (rc != AREAL_OK) return rc;
   int64_t blocks = ceil_div_i64(T * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
@@ -2273,11 +1738,11 @@ int launch_dhidden(const u16* w, int64_t V, const u16* dl, int64_t ldv, int64_t 
   if (dh_weight_in_place(V)) {
     GemmArgs g{w, H, (int)H, dl, ldv, (int)T, (int)ldv, (int)H, 0};
     g.skip_if_set = skip_if_set;
-    return launch_dhidden_k<KERNEL_MIX, KERNEL16_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
+    return launch_dhidden_k<KERNEL16_MIX>(g, H, T, ldv, dhidden, partial, tscale, stream);
   }
   GemmArgs g{w, ldv, (int)H, dl, ldv, (int)T, (int)ldv, 0, 0};
   g.skip_if_set = skip_if_set;
-  return launch_dhidden_k<KERNEL_NT, KERNEL16_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
+  return launch_dhidden_k<KERNEL16_NT>(g, H, T, ldv, dhidden, partial, tscale, stream);
 }
 
 // dWeight [V, H] in bf16 has ceil(V / 256) x ceil(H / 256) output tiles, one per workgroup, in
@@ -2314,9 +1779,8 @@ DwTail plan_dw_tail(int64_t H, int64_t V, int64_t Tpad) {
   const double before = (double)ceil_div_i64(sc.n_sb, 8), after = (double)(nj * n_sb_s / 8) + best_cost;
   if (best <= 1 || (before - after) * (double)nk < 16.0) return t;
   t.nbj_main = nj * sc.RB;
-  t.kps = (int)ceil_div_i64(nk, best);
-  t.kps += t.kps & 1;  // the hand-scheduled loop walks pairs of k-tiles
-  t.z = (int)ceil_div_i64(nk, t.kps);
+  t.z = best;
+  split_ktiles((int)nk, t.z, t.kps);
   t.rows = V - (int64_t)t.nbj_main * TILE;
   if (t.z <= 1) t = DwTail{nbj, 1, 0, 0};
   return t;
@@ -2336,13 +1800,13 @@ int launch_dweight_bf16(GemmArgs g, int64_t H, int64_t V, int64_t ldv, void* dwe
   int rc;
   if (tail.z <= 1) {
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
-    return launch_store<KERNEL_TN, KERNEL16_TN>(g, plan_regions(H, V, K, 0, 1 << 20), ep, 0, stream);
+    return launch_store<KERNEL16_TN>(g, ep, 0, stream);
   }
   const int64_t v0 = (int64_t)tail.nbj_main * TILE;
   GemmArgs gm = g;
   gm.N = (int)v0;
   const StoreParams ep{dweight, H, (int)H, (int)v0, nullptr};
-  rc = launch_store<KERNEL_TN, KERNEL16_TN>(gm, plan_regions(H, v0, K, 0, 1 << 20), ep, 0, stream);
+  rc = launch_store<KERNEL16_TN>(gm, ep, 0, stream);
   if (rc != AREAL_OK) return rc;
   GemmArgs gt = g;
   gt.B = g.B + v0;
@@ -2352,7 +1816,7 @@ int launch_dweight_bf16(GemmArgs g, int64_t H, int64_t V, int64_t ldv, void* dwe
   gt.kt_per_split = tail.kps;
   gt.zstride = tail.rows * H * (int64_t)sizeof(float);
   const StoreParams ept{dw_part, H, (int)H, (int)tail.rows, nullptr};
-  rc = launch_store<KERNEL_TN, KERNEL16_TN>(gt, plan_regions(H, tail.rows, K, 0, 1 << 20), ept, 1, stream);
+  rc = launch_store<KERNEL16_TN>(gt, ept, 1, stream);
   if (rc != AREAL_OK) return rc;
   int64_t blocks = ceil_div_i64(tail.rows * H, 256 * 4);
   if (blocks > 65535) blocks = 65535;
@@ -2385,9 +1849,8 @@ int areal_gemm_nt_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, v
   if (out_mode == 0 ? (ldo % 4 != 0 || ((uintptr_t)out & 7)) : (ldo % 4 != 0 || !aligned16(out)))
     return AREAL_ERR_ALIGNMENT;
   GemmArgs g{(const u16*)A, lda, (int)M, (const u16*)B, ldb, (int)N, (int)K, 0, 0};
-  const Regions r = plan_regions(M, N, K, 0, 1 << 20);  // one A tile per workgroup
   const StoreParams ep{out, ldo, (int)M, (int)N};
-  return launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, out_mode, stream);
+  return launch_store<KERNEL16_NT>(g, ep, out_mode, stream);
 }
 
 int areal_abi_version(void) { return 3; }  // AREAL_HIP_ABI_VERSION of include/areal_hip.h
@@ -2456,11 +1919,18 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                        logit_scale, c2, probs_ref, probs_status);
     AREAL_CHECK_LAUNCH();
   }
-  auto fwd16_plain = [&](const GemmArgs& gg) {
-    if (!affine && !moments) return launch_gemm<Fwd16Plain, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
-    if (!affine) return launch_gemm<Fwd16PlainMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
-    if (!moments) return launch_gemm<Fwd16Affine, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
-    return launch_gemm<Fwd16AffineMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+  // (each launch_gemm names the epilogue for the hand-scheduled kernel and the one for the generic kernel)
+  auto fwd_plain = [&](const GemmArgs& gg) {
+    if (!affine && !moments) return launch_gemm<Fwd16Plain, FwdPlain, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!affine) return launch_gemm<Fwd16PlainMom, FwdPlainMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!moments) return launch_gemm<Fwd16Affine, FwdAffine, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    return launch_gemm<Fwd16AffineMom, FwdAffineMom, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+  };
+  auto fwd_save = [&](const GemmArgs& gg) {
+    if (!affine && !moments) return launch_gemm<Fwd16PlainSave, FwdPlainSave, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!affine) return launch_gemm<Fwd16PlainMomSave, FwdPlainMomSave, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    if (!moments) return launch_gemm<Fwd16AffineSave, FwdAffineSave, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
+    return launch_gemm<Fwd16AffineMomSave, FwdAffineMomSave, FwdParams, KERNEL16_NT>(gg, r, ep, ep_a, stream);
   };
   auto merge = [&](int ref_sums, const float* ref, const int* gate, int gate_run_if_set) {
     hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)ceil_div_i64(T, 64)), dim3(64 * MERGE_WAVES),
@@ -2468,8 +1938,8 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
                        entropy, vocab_min, vocab_max, vocab_mean, vocab_norm, row_max, sum_exp, ref,
                        probs_status, gate, gate_run_if_set);
   };
-  if (r.k16 && probs == nullptr) {
-    if ((rc = fwd16_plain(g)) != AREAL_OK) return rc;
+  if (probs == nullptr) {
+    if ((rc = fwd_plain(g)) != AREAL_OK) return rc;
     merge(0, nullptr, nullptr, 0);
   } else if (r.k16) {
     // The saving sweep takes its sums relative to the row references, which is only right for rows
@@ -2477,31 +1947,18 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
     // some row is outside; the plain sweep and its merge are queued behind it and do their work
     // only in that case (otherwise every workgroup of them returns at once), so the outputs are
     // right either way without the host looking at the status in between.
-    if (!affine && !moments) rc = launch_gemm<Fwd16PlainSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else if (!affine) rc = launch_gemm<Fwd16PlainMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else if (!moments) rc = launch_gemm<Fwd16AffineSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    else rc = launch_gemm<Fwd16AffineMomSave, FwdParams, KERNEL16_NT>(g, r, ep, ep_a, stream);
-    if (rc != AREAL_OK) return rc;
+    if ((rc = fwd_save(g)) != AREAL_OK) return rc;
     merge(1, probs_ref, nullptr, 0);
     AREAL_CHECK_LAUNCH();
     GemmArgs gf = g;
     gf.skip_if_set = probs_status;
     gf.run_if_set = 1;
-    if ((rc = fwd16_plain(gf)) != AREAL_OK) return rc;
+    if ((rc = fwd_plain(gf)) != AREAL_OK) return rc;
     merge(0, nullptr, probs_status, 1);
   } else {
-    if (probs == nullptr) {
-      if (!affine && !moments) rc = launch_gemm<FwdPlain>(g, r, ep, ep_a, stream);
-      else if (!affine) rc = launch_gemm<FwdPlainMom>(g, r, ep, ep_a, stream);
-      else if (!moments) rc = launch_gemm<FwdAffine>(g, r, ep, ep_a, stream);
-      else rc = launch_gemm<FwdAffineMom>(g, r, ep, ep_a, stream);
-    } else {
-      if (!affine && !moments) rc = launch_gemm<FwdPlainSave>(g, r, ep, ep_a, stream);
-      else if (!affine) rc = launch_gemm<FwdPlainMomSave>(g, r, ep, ep_a, stream);
-      else if (!moments) rc = launch_gemm<FwdAffineSave>(g, r, ep, ep_a, stream);
-      else rc = launch_gemm<FwdAffineMomSave>(g, r, ep, ep_a, stream);
-    }
-    if (rc != AREAL_OK) return rc;
+    // the generic kernel's saving epilogue keeps its sums relative to each tile's maximum: the
+    // outputs do not depend on the row reference, only the saved buffer does
+    if ((rc = fwd_save(g)) != AREAL_OK) return rc;
     merge(0, probs_ref, nullptr, 0);
   }
   AREAL_CHECK_LAUNCH();
@@ -2509,14 +1966,14 @@ int areal_lmhead_fwd(const void* hidden, const void* weight, const float* bias,
 }
 
 // Backward workspace (bf16): W^T [H, ldv] + dl [Tc, ldv] per token chunk; chunks that are not a
-// multiple of 64 tokens also need hidden^T [H, ldt] and dlT [V, ldt] (token_chunk a multiple of
-// 64 and T a multiple of 64 avoid them).
+// multiple of 64 tokens (or shorter than 128) also need hidden^T [H, ldt] and dlT [V, ldt]
+// (token_chunk a multiple of 64 and T a multiple of 64, both at least 128, avoid them).
 size_t areal_lmhead_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int64_t token_chunk) {
   if (T <= 0 || H <= 0 || V <= 0 || token_chunk <= 0) return 0;
   const int64_t Tc = token_chunk < T ? token_chunk : T;
   const int64_t ldv = round_up_i64(V, BK), ldt = round_up_i64(Tc, BK);
   int64_t elems = (dh_weight_in_place(V) ? 0 : H * ldv) + Tc * ldv;
-  const bool ragged = (Tc % BK != 0) || (T % Tc) % BK != 0;  // some chunk is not a multiple of 64
+  const bool ragged = !k16_ok(Tc) || ((T % Tc) != 0 && !k16_ok(T % Tc));  // some chunk cannot be read k-major
   if (ragged) elems += H * ldt + V * ldt;
   // slack for 256-byte sub-buffer alignment
   // (the last term: partial results of the bf16 dWeight store, one chunk covering the batch)
@@ -2561,7 +2018,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     return (u16*)r;
   };
   char* wp = (char*)workspace;
-  const bool ragged = (Tc_max % BK != 0) || (T % Tc_max) % BK != 0;
+  const bool ragged = !k16_ok(Tc_max) || ((T % Tc_max) != 0 && !k16_ok(T % Tc_max));
   const bool w_in_place = dh_weight_in_place(V);
   u16* wT = w_in_place ? nullptr : carve(wp, H * ldv * 2);
   u16* dl = carve(wp, Tc_max * ldv * 2);
@@ -2584,25 +2041,23 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     const int64_t ldt_c = round_up_i64(Tc, BK);
     const u16* hid_c = (const u16*)hidden + t0 * H;
     // dWeight reads dl and hidden k-major (no transposed copies) when the chunk is a multiple
-    // of 64 tokens; otherwise it goes through dlT and hidden^T.
-    const bool tn = (Tc % BK == 0) && dweight_f32 != nullptr;
+    // of 64 tokens (at least 128); otherwise it goes through dlT and hidden^T.
+    const bool tn = k16_ok(Tc) && dweight_f32 != nullptr;
     const bool need_dlT = dweight_f32 != nullptr && !tn;
     // 1. recompute logits of the chunk, emit dlogits
     {
       GemmArgs g{(const u16*)weight, H, (int)V, hid_c, H, (int)Tc, (int)H, 0, 0};
       BwdParams ep{labels + t0, row_max + t0, sum_exp + t0, grad_logprobs + t0, (int)Tc,
                    (int)V, logit_scale, c2, inv_temperature, bias, dl, ldv, dlT, ldt_c};
-      Regions r = plan_regions(V, Tc, H, 512, 0);
-      if (!need_dlT) fold_ragged_a(r, V);
+      // the token-contiguous copy dlT is written by the generic kernel's epilogue only
+      Regions r = plan_regions(V, Tc, H, 512, 0, !need_dlT);
+      fold_ragged_a(r, V);
       if (need_dlT)
-        rc = affine ? launch_gemm<BwdAffineT>(g, r, ep, ep, stream)
-                    : launch_gemm<BwdPlainT>(g, r, ep, ep, stream);
-      else if (r.k16)
-        rc = affine ? launch_gemm<Bwd16Affine, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream)
-                    : launch_gemm<Bwd16Plain, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream);
+        rc = affine ? launch_gemm<Bwd16Affine, BwdAffineT, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream)
+                    : launch_gemm<Bwd16Plain, BwdPlainT, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream);
       else
-        rc = affine ? launch_gemm<BwdAffine>(g, r, ep, ep, stream)
-                    : launch_gemm<BwdPlain>(g, r, ep, ep, stream);
+        rc = affine ? launch_gemm<Bwd16Affine, BwdAffine, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream)
+                    : launch_gemm<Bwd16Plain, BwdPlain, BwdParams, KERNEL16_NT>(g, r, ep, ep, stream);
       if (rc != AREAL_OK) return rc;
     }
     // 2. dHidden[t, h] = sum_v dl[t, v] * W^T[h, v]
@@ -2621,9 +2076,8 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
     if (tn) {
       GemmArgs g{hid_c, H, (int)H, dl, ldv, (int)V, (int)Tc, (int)H, (int)ldv};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
-      const Regions r = plan_regions(H, V, Tc, 0, 1 << 20);
       rc = dw_bf16 ? launch_dweight_bf16(g, H, V, ldv, dweight, dw_part, stream)
-                   : launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
+                   : launch_store<KERNEL16_TN>(g, ep, (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     } else if (dweight_f32 != nullptr) {
       hipLaunchKernelGGL(transpose_pad_bf16_kernel,
@@ -2632,8 +2086,7 @@ int areal_lmhead_bwd(const void* hidden, const void* weight, const float* bias,
       AREAL_CHECK_LAUNCH();
       GemmArgs g{hT, ldt_c, (int)H, dlT, ldt_c, (int)V, (int)ldt_c, 0, 0};
       const StoreParams ep{dweight_f32, H, (int)H, (int)V};
-      const Regions r = plan_regions(H, V, ldt_c, 0, 1 << 20);
-      rc = launch_store<KERNEL_NT, KERNEL16_NT>(g, r, ep, dw_bf16 ? 0 : (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
+      rc = launch_store<KERNEL16_NT>(g, ep, dw_bf16 ? 0 : (accumulate == 1 || t0 > 0) ? 2 : 1, stream);
       if (rc != AREAL_OK) return rc;
     }
   }
@@ -2723,8 +2176,7 @@ int areal_lmhead_bwd_saved(const void* hidden, const void* weight, const int64_t
     g.skip_if_set = probs_status;
     if (dweight_mode == 2) return launch_dweight_bf16(g, H, V, ldv, dweight, dw_part, stream);
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
-    const Regions r = plan_regions(H, V, Tpad, 0, 1 << 20);
-    rc = launch_store<KERNEL_TN, KERNEL16_TN>(g, r, ep, dweight_mode == 1 ? 2 : 1, stream);
+    rc = launch_store<KERNEL16_TN>(g, ep, dweight_mode == 1 ? 2 : 1, stream);
     if (rc != AREAL_OK) return rc;
   }
   return AREAL_OK;

@@ -349,7 +349,7 @@ def hbm_rooflines(dev):
         rc = lib.areal_actor_loss_grad(p(dlp), p(gout), p(both[:8]), p(grad), Tl, _lib.stream_ptr(dev))
         _lib.check(rc, "areal_actor_loss_grad")
 
-    add("loss_token<stats>+loss_finalize+loss_stats_finalize+loss_grad_scale",
+    add("loss_token<stats>+loss_finalize+loss_grad_scale",
         "PPO + IcePop, 4 Mi tokens, fwd+bwd kernels through the C ABI with the 13 logged statistics reduced in "
         "the token pass instead of written as [T] tensors: 25 B/token + 8 B/token grad scale",
         33 * Tl, timed(loss_kernels_reduced, iters=50))
@@ -394,6 +394,28 @@ def hbm_rooflines(dev):
 
     add("sapo_token_kernel + backward (API level)", "SAPO, 4 Mi tokens, 7 output tensors, 41 B/token + 8 B/token grad scale",
         49 * Tl, timed(sapo_step))
+    # the same kernels through the C ABI, back to back on the stream (no host work between them)
+    p = _lib.ptr
+    strm2 = _lib.stream_ptr(dev)
+    aux_nb = lib.areal_aux_loss_workspace_bytes(Tl, 0)
+    aux_ws = torch.empty(aux_nb, dtype=torch.uint8, device=dev)
+    s_out = [torch.empty(Tl, device=dev) for _ in range(7)]  # dsum + 6 statistic tensors
+    s_cnt = torch.empty(8 + 4 * 13, dtype=torch.float64, device=dev)
+
+    def sapo_kernels(reduced):
+        outs = [None] * 6 if reduced else [p(t) for t in s_out[1:]]
+        rc = lib.areal_sapo_loss(p(lp32), p(old), p(adv), p(mask_b), None, Tl, 0, 0, 1.0, 1.05, 0, p(loss_out),
+                                 p(s_out[0]), *outs, p(s_cnt[:8]), p(ent) if reduced else None, None, None,
+                                 p(s_cnt[8:]) if reduced else None, p(aux_ws), aux_nb, strm2)
+        _lib.check(rc, "areal_sapo_loss")
+        rc = lib.areal_actor_loss_grad(p(s_out[0]), p(gout), p(s_cnt[:8]), p(grad), Tl, strm2)
+        _lib.check(rc, "areal_actor_loss_grad")
+
+    add("sapo_token+aux_finalize+loss_grad_scale (C ABI)", "SAPO, 4 Mi tokens, fwd+bwd kernels through the C ABI, "
+        "41 B/token + 8 B/token grad scale", 49 * Tl, timed(lambda: sapo_kernels(False), iters=50))
+    add("sapo_token<stats>+aux_finalize+loss_grad_scale (C ABI)", "SAPO, 4 Mi tokens, the 11 logged statistics reduced "
+        "in the token pass instead of written as [T] tensors: 13 B/token in + 4 B entropy + 4 B gradient out + "
+        "8 B/token grad scale", 29 * Tl, timed(lambda: sapo_kernels(True), iters=50))
     val = torch.randn(Tl, device=dev).requires_grad_(True)
     oldv, tgt = val.detach() + 0.1 * torch.randn(Tl, device=dev), torch.randn(Tl, device=dev)
 
@@ -404,6 +426,18 @@ def hbm_rooflines(dev):
 
     add("critic_token_kernel + backward (API level)", "clipped value loss, 4 Mi tokens, 22 B/token + 8 B/token grad scale",
         30 * Tl, timed(critic_step))
+    c_dv, c_sl, c_cm = torch.empty(Tl, device=dev), torch.empty(Tl, device=dev), torch.empty(Tl, dtype=torch.bool, device=dev)
+    val32 = val.detach()
+
+    def critic_kernels():
+        rc = lib.areal_critic_loss(p(val32), p(oldv), p(tgt), p(mask_b), Tl, 0.2, 0, p(loss_out), p(c_dv), p(c_sl),
+                                   p(c_cm), p(s_cnt[:8]), p(aux_ws), aux_nb, strm2)
+        _lib.check(rc, "areal_critic_loss")
+        rc = lib.areal_actor_loss_grad(p(c_dv), p(gout), p(s_cnt[:8]), p(grad), Tl, strm2)
+        _lib.check(rc, "areal_actor_loss_grad")
+
+    add("critic_token+aux_finalize+loss_grad_scale (C ABI)", "clipped value loss, 4 Mi tokens, fwd+bwd kernels through "
+        "the C ABI, 22 B/token + 8 B/token grad scale", 30 * Tl, timed(critic_kernels, iters=50))
     add("m2_hist x4 + m2_select x4 + m2_tie_count + m2_apply (API level)",
         "M2PO mask by radix select, 4 Mi tokens, 6 passes x 9 B/token",
         54 * Tl, timed(lambda: _apply_m2po_masking(old, prox, mask, 0.04)))
@@ -423,6 +457,24 @@ def hbm_rooflines(dev):
     add("rowlens + cu_scan + pack_kernel (API level)",
         f"pack_tensor_dict: [1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write",
         2 * 25 * n_packed + bsz * Lp, timed(lambda: pack_tensor_dict(dict(pdata))))
+    # the same launches through the C ABI into preallocated outputs
+    pk_mask = pattn.contiguous().view(torch.uint8)
+    pk_lens = torch.empty(bsz, dtype=torch.int32, device=dev)
+    pk_cu = torch.empty(bsz + 1, dtype=torch.int32, device=dev)
+    pk_max = torch.empty(1, dtype=torch.int32, device=dev)
+    pk_src = [pdata[k].contiguous() for k in ("input_ids", "loss_mask", "logprobs", "advantages")]
+    pk_src.append(torch.zeros(bsz, Lp, dtype=torch.long, device=dev))  # a second 8-byte tensor (position ids)
+    pk_dst = [torch.empty(n_packed, dtype=t.dtype, device=dev) for t in pk_src]
+
+    def pack_kernels():
+        rc = lib.areal_seqlens_from_mask(p(pk_mask), bsz, Lp, p(pk_lens), p(pk_cu), p(pk_max), strm2)
+        for s_, d_ in zip(pk_src, pk_dst):
+            rc |= lib.areal_pack_padded(p(s_), p(d_), p(pk_cu), bsz, Lp, s_.element_size(), n_packed, strm2)
+        assert rc == 0
+
+    add("rowlens + cu_scan + pack_kernel x5 (C ABI)",
+        f"[1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write, and the "
+        "attention mask read once", 2 * 25 * n_packed + bsz * Lp, timed(pack_kernels, iters=50))
     turn_ids = (torch.cumsum((torch.rand(bsz, Lp, device=dev) < 0.002).int(), dim=1)).to(torch.int32)
     tr = torch.zeros(bsz, Lp, device=dev)
     tr[torch.arange(bsz, device=dev), (plens - 2).clamp(min=0)] = 1.0

@@ -23,7 +23,9 @@ def _rel(a, b):
                                    # K a multiple of 128: the hand-scheduled main loop (one pair of
                                    # k-tiles, several, ragged M and N, M not a multiple of 8)
                                    (256, 256, 128), (512, 256, 1024), (300, 200, 256), (520, 1000, 384),
-                                   (96, 13, 128), (264, 513, 1280)])
+                                   (96, 13, 128), (264, 513, 1280),
+                                   # an odd number of k-tiles (3, 5, 7, 21): the last pair's second k-tile is dead
+                                   (256, 256, 192), (520, 300, 320), (512, 1000, 448), (264, 513, 1344)])
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_gemm_nt(dev, M, N, K, mode):
     lib = _lib.load()

@@ -46,6 +46,12 @@ def _case_list():
     cases.append((2048, 640, 20403))
     # token count 64 short of a multiple of 128 with a contraction long enough to split
     cases.append((1984, 256, 9000))
+    # contraction lengths that are an odd number of 64-deep steps (the main loop's last pair of
+    # k-tiles then has a dead second k-tile): hidden size (forward, recompute), vocabulary
+    # (dHidden: 31, 65, 575 steps, the last one split over copies of the schedule), token count
+    # (dWeight in recompute mode: 3 and 7 steps)
+    cases += [(192, 192, 1984), (448, 320, 4160), (1000, 960, 5000), (320, 448, 1536), (2048, 192, 36764),
+              (256, 128 + 64, 640)]
     return sorted(set(cases))
 
 
