@@ -96,6 +96,9 @@ SIGNATURES: dict[str, tuple] = {
     ),
     "areal_gae_padded_row_stats": (I, [P, P, P, P, P, I64, I64, F, F, P, P, P, P]),
     "areal_group_norm_from_row_stats": (I, [P, P, I64, I64, P, P, I64, I64, I, I, I, I, D, P, P, P]),
+    "areal_gae_segment_stats_bytes": (SZ, [I64, I64]),
+    "areal_gae_packed_group_stats": (I, [P, P, P, P, P, P, I64, I64, F, F, P, I64, P, P, P, SZ, P]),
+    "areal_group_norm_from_segment_stats": (I, [P, P, I64, P, P, I64, I64, I, I, I, I, D, P, P, P]),
     "areal_seqlens_from_mask": (I, [P, I64, I64, P, P, P, P]),
     "areal_pack_padded": (I, [P, P, P, I64, I64, I64, I64, P]),
     "areal_unpack_to_padded": (I, [P, P, P, P, I64, I64, I64, P, I, P]),

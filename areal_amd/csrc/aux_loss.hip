@@ -97,11 +97,8 @@ __global__ __launch_bounds__(AUX_THREADS) void aux_finalize_kernel(
       mx = stat_max(mx, sp.mx);
     }
     sum = block_sum(sum, sm_d);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      mn = stat_min(mn, __shfl_xor(mn, o, 64));
-      mx = stat_max(mx, __shfl_xor(mx, o, 64));
-    }
+    mn = wave_stat_min(mn);
+    mx = wave_stat_max(mx);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     __syncthreads();
     if (lane == 0) { sm_f[w] = mn; sm_f[4 + w] = mx; }
@@ -298,11 +295,8 @@ __global__ __launch_bounds__(AUX_THREADS) void sapo_token_kernel(SapoIO io, SumC
     for (int k = 0; k < N_SAPO_STATS; ++k) {
       const double sv = wave_sum((double)st_sum[k]);
       float mn = st_mn[k], mx = st_mx[k];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        mn = stat_min(mn, __shfl_xor(mn, o, 64));
-        mx = stat_max(mx, __shfl_xor(mx, o, 64));
-      }
+      mn = wave_stat_min(mn);
+      mx = wave_stat_max(mx);
       if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
     }
     __syncthreads();

@@ -57,23 +57,82 @@ DEVI float bf16_bits_to_f32(u16 b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
 }
 
-// Wave-wide (64 lanes) reductions through cross-lane shuffles.
+// ---------------------------------------------------------------------------------------
+// Cross-lane movement inside a 64-lane wave without the LDS crossbar. A ds_bpermute shuffle goes
+// through the CU's one LDS unit, which every wave of the CU shares: a block-end reduction of a few
+// values by sixteen resident waves queues there for microseconds. DPP operands (data-parallel
+// primitives: a VALU instruction reads its source from another lane of the same row of 16) and
+// v_readlane stay inside the SIMD.
+// ---------------------------------------------------------------------------------------
+constexpr int DPP_ROW_SHL = 0x100;  // + n (1..15): lane i reads lane i + n of its row
+constexpr int DPP_ROW_SHR = 0x110;  // + n: lane i reads lane i - n of its row
+constexpr int DPP_ROW_ROR = 0x120;  // + n: lane i reads lane (i - n) mod 16 of its row
+
+// x of the lane CTRL names; a lane whose source falls outside its row keeps `old`.
+template <int CTRL>
+DEVI int dpp_move(int old, int x) { return __builtin_amdgcn_update_dpp(old, x, CTRL, 0xf, 0xf, false); }
+template <int CTRL>
+DEVI unsigned dpp_move(unsigned old, unsigned x) { return (unsigned)dpp_move<CTRL>((int)old, (int)x); }
+template <int CTRL>
+DEVI float dpp_move(float old, float x) {
+  return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x)));
+}
+template <int CTRL>
+DEVI double dpp_move(double old, double x) {
+  const int2 o = __builtin_bit_cast(int2, old), v = __builtin_bit_cast(int2, x);
+  int2 r;
+  r.x = dpp_move<CTRL>(o.x, v.x);
+  r.y = dpp_move<CTRL>(o.y, v.y);
+  return __builtin_bit_cast(double, r);
+}
+template <int CTRL>
+DEVI long long dpp_move(long long old, long long x) {
+  return __builtin_bit_cast(long long, dpp_move<CTRL>(__builtin_bit_cast(double, old), __builtin_bit_cast(double, x)));
+}
+
+template <int CTRL>
+DEVI unsigned long long dpp_move(unsigned long long old, unsigned long long x) {
+  return (unsigned long long)dpp_move<CTRL>((long long)old, (long long)x);
+}
+template <int CTRL>
+DEVI long dpp_move(long old, long x) { return (long)dpp_move<CTRL>((long long)old, (long long)x); }
+
+// x of lane `lane` (a constant) in every lane.
+DEVI int lane_value(int x, int lane) { return __builtin_amdgcn_readlane(x, lane); }
+DEVI unsigned lane_value(unsigned x, int lane) { return (unsigned)__builtin_amdgcn_readlane((int)x, lane); }
+DEVI float lane_value(float x, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+DEVI double lane_value(double x, int lane) {
+  const int2 v = __builtin_bit_cast(int2, x);
+  int2 r;
+  r.x = __builtin_amdgcn_readlane(v.x, lane);
+  r.y = __builtin_amdgcn_readlane(v.y, lane);
+  return __builtin_bit_cast(double, r);
+}
+DEVI long long lane_value(long long x, int lane) {
+  return __builtin_bit_cast(long long, lane_value(__builtin_bit_cast(double, x), lane));
+}
+DEVI unsigned long long lane_value(unsigned long long x, int lane) {
+  return (unsigned long long)lane_value((long long)x, lane);
+}
+DEVI long lane_value(long x, int lane) { return (long)lane_value((long long)x, lane); }
+
+// Wave-wide (64 lanes) reduction with a commutative, associative op; the result in every lane.
+// Four rotations leave each row's result in all of its lanes; the four rows are then combined
+// from lanes 0, 16, 32 and 48 in that order, so the result does not depend on the calling lane.
+template <typename T, typename Op>
+DEVI T wave_reduce(T v, Op op) {
+  v = op(v, dpp_move<DPP_ROW_ROR + 8>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 4>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 2>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 1>(v, v));
+  return op(op(lane_value(v, 0), lane_value(v, 16)), op(lane_value(v, 32), lane_value(v, 48)));
+}
 template <typename T>
-DEVI T wave_sum(T v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-DEVI float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-DEVI float wave_min(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
-  return v;
-}
+DEVI T wave_sum(T v) { return wave_reduce(v, [](T a, T b) { return a + b; }); }
+DEVI float wave_max(float v) { return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); }); }
+DEVI float wave_min(float v) { return wave_reduce(v, [](float a, float b) { return fminf(a, b); }); }
 
 // ---------------------------------------------------------------------------------------
 // Streaming per-token kernels (losses, statistics)
@@ -140,6 +199,8 @@ DEVI void store_mask(uint8_t* p, int64_t t, const bool (&v)[VEC]) {
 // zero does not matter there): IEEE 754-2019 minimum / maximum, one instruction each.
 DEVI float stat_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 DEVI float stat_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+DEVI float wave_stat_min(float v) { return wave_reduce(v, [](float a, float b) { return stat_min(a, b); }); }
+DEVI float wave_stat_max(float v) { return wave_reduce(v, [](float a, float b) { return stat_max(a, b); }); }
 
 // VEC = 4 needs every per-token fp32 array 16-byte aligned and every byte array 4-byte aligned
 // (null pointers pass); it pays once the batch gives every CU a block of four-token threads.

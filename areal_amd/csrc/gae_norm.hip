@@ -20,6 +20,7 @@ namespace {
 constexpr int GAE_THREADS = 256;
 constexpr int GAE_ITEMS = 8;
 constexpr int GAE_TILE = GAE_THREADS * GAE_ITEMS;
+constexpr int GAE_SEG_WAVES = GAE_THREADS / 64;  // entries per (tile, group) segment of GaeArgs::seg_stats
 
 // R = double in the three-launch scan (maps composed over the whole array); R = float in the
 // single-pass kernel, where a map spans at most one tile and the state carried from tile to
@@ -47,13 +48,55 @@ DEVI MapT<R> compose(const MapT<R>& f, const MapT<R>& g) {
   r.b2 = fma(f.a22, g.b2, f.b2);
   return r;
 }
-template <class R>
-DEVI MapT<R> shfl_down_map(const MapT<R>& m, int d) {
+// The map of the lane that CTRL names (common.hpp); the identity where that lane lies outside
+// the row of 16.
+template <int CTRL, class R>
+DEVI MapT<R> dpp_map(const MapT<R>& m) {
   MapT<R> r;
-  r.a11 = __shfl_down(m.a11, d, 64); r.a12 = __shfl_down(m.a12, d, 64);
-  r.a22 = __shfl_down(m.a22, d, 64); r.b1 = __shfl_down(m.b1, d, 64);
-  r.b2 = __shfl_down(m.b2, d, 64);
+  r.a11 = dpp_move<CTRL>(R(1), m.a11); r.a12 = dpp_move<CTRL>(R(0), m.a12);
+  r.a22 = dpp_move<CTRL>(R(1), m.a22); r.b1 = dpp_move<CTRL>(R(0), m.b1);
+  r.b2 = dpp_move<CTRL>(R(0), m.b2);
   return r;
+}
+template <class R>
+DEVI MapT<R> lane_map(const MapT<R>& m, int lane) {
+  return MapT<R>{lane_value(m.a11, lane), lane_value(m.a12, lane), lane_value(m.a22, lane),
+                 lane_value(m.b1, lane), lane_value(m.b2, lane)};
+}
+// Inclusive suffix scan inside each row of 16 lanes: lane i gets the composition of the maps of
+// lanes i..15 of its row (lane i applied last). No LDS traffic: the sixteen waves of a CU would
+// queue at its one LDS unit with ds_bpermute shuffles.
+template <class R>
+DEVI MapT<R> row_suffix_scan(MapT<R> acc) {
+  acc = compose(acc, dpp_map<DPP_ROW_SHL + 1>(acc));
+  acc = compose(acc, dpp_map<DPP_ROW_SHL + 2>(acc));
+  acc = compose(acc, dpp_map<DPP_ROW_SHL + 4>(acc));
+  acc = compose(acc, dpp_map<DPP_ROW_SHL + 8>(acc));
+  return acc;
+}
+// Composition of the maps of all 64 lanes (lane 0 applied last), in every lane.
+template <class R>
+DEVI MapT<R> wave_total_map(const MapT<R>& mine) {
+  const MapT<R> acc = row_suffix_scan(mine);
+  return compose(lane_map(acc, 0), compose(lane_map(acc, 16), compose(lane_map(acc, 32), lane_map(acc, 48))));
+}
+// Inclusive suffix scan over the wave: lane i gets the composition of lanes i..63.
+template <class R>
+DEVI MapT<R> wave_suffix_scan(const MapT<R>& mine, MapT<R>& total) {
+  const MapT<R> acc = row_suffix_scan(mine);
+  const MapT<R> t0 = lane_map(acc, 0), t1 = lane_map(acc, 16), t2 = lane_map(acc, 32), t3 = lane_map(acc, 48);
+  const MapT<R> r1 = compose(t2, t3);  // all that lies right of row 1
+  const MapT<R> r0 = compose(t1, r1);  // right of row 0
+  total = compose(t0, r0);
+  const int row = (threadIdx.x & 63) >> 4;
+  const MapT<R> id = map_identity_t<R>();
+  MapT<R> right;
+  right.a11 = row == 0 ? r0.a11 : row == 1 ? r1.a11 : row == 2 ? t3.a11 : id.a11;
+  right.a12 = row == 0 ? r0.a12 : row == 1 ? r1.a12 : row == 2 ? t3.a12 : id.a12;
+  right.a22 = row == 0 ? r0.a22 : row == 1 ? r1.a22 : row == 2 ? t3.a22 : id.a22;
+  right.b1 = row == 0 ? r0.b1 : row == 1 ? r1.b1 : row == 2 ? t3.b1 : id.b1;
+  right.b2 = row == 0 ? r0.b2 : row == 1 ? r1.b2 : row == 2 ? t3.b2 : id.b2;
+  return compose(acc, right);
 }
 
 // N sums at once: one pair of barriers instead of N.
@@ -94,6 +137,14 @@ struct GaeArgs {
   double* row_stats;         // nullable, with block_per_seq only: [5][n_seqs] sums over each row of
                              // m, x m, m^2, m^2 x, m^2 x^2 (x = the advantage written, m = mask):
                              // the statistics pass of the normalisation that follows, for free
+  // packed tile kernel with statistics: the same five sums per (tile, group) segment. goff [G+1]
+  // are the groups' token offsets (a partition of [0, n)); segment (tile k, group j) lands in slot
+  // k + j of seg_stats [5][seg_slots][4] (one entry per wave of the tile's block), seg_slots =
+  // tiles + G. Slots no segment maps to are zeroed.
+  const int64_t* goff;
+  int n_groups;
+  double* seg_stats;
+  int64_t seg_slots;
 };
 
 DEVI int gae_seq_of(const GaeArgs& g, int64_t t) {
@@ -174,14 +225,10 @@ DEVI Map thread_total(const Map (&mp)[GAE_ITEMS]) {
 template <class R>
 DEVI MapT<R> block_suffix_scan(MapT<R> mine, MapT<R>* smem, MapT<R>& block_total) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  MapT<R> acc = mine;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const MapT<R> other = shfl_down_map(acc, d);
-    if (lane + d < 64) acc = compose(acc, other);
-  }
+  MapT<R> wave_total;
+  const MapT<R> acc = wave_suffix_scan(mine, wave_total);
   __syncthreads();
-  if (lane == 0) smem[w] = acc;  // wave total (lanes 0..63)
+  if (lane == 0) smem[w] = wave_total;
   __syncthreads();
   const int nw = blockDim.x >> 6;
   MapT<R> right = map_identity_t<R>();
@@ -285,7 +332,8 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_apply_kernel(GaeArgs g, const
 
 // #{i in [0, n) : ends[i] <= x} for a non-decreasing array, by one wave: every round probes 64
 // positions and keeps the gap after the last probe that is <= x.
-DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
+template <class I>
+DEVI int wave_count_le(const I* ends, int n, int64_t x, int lane) {
   int base = 0, len = n;
   while (len > 0) {
     const int step = (len + 63) >> 6;
@@ -308,6 +356,7 @@ DEVI int wave_count_le(const int32_t* ends, int n, int64_t x, int lane) {
 // holds one of those tokens (cu_own[0] <= t_begin, cu_own[n_own] >= t_end); with uniform rows
 // cu_own is unused. (A0, nv0) is the fp64 state entering the tile from its right and is replaced
 // by the state leaving it on the left. rs: the row sums of GaeArgs::row_stats (STATS only).
+// oa receives the advantages of the thread's owned tokens (zero elsewhere).
 // The thread's 8 consecutive tokens from t0 (a multiple of 8) as raw inputs; zeros where `want`
 // is false and beyond the array.
 DEVI void gae_load_items(const GaeArgs& g, int64_t t0, bool want, float (&rw)[GAE_ITEMS],
@@ -353,7 +402,7 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
                        int n_own, const int32_t* cu_own, double& A0, double& nv0,
                        double (&rs)[STATS ? 5 : 1], MapF* smem, MapF* all,
                        const float (&rw)[GAE_ITEMS], const float (&v)[GAE_ITEMS],
-                       const float (&ms)[GAE_ITEMS]) {
+                       const float (&ms)[GAE_ITEMS], float (&oa)[GAE_ITEMS]) {
   constexpr bool uniform = LAYOUT != GAE_LAYOUT_CU;
   const int tid = threadIdx.x;
   const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
@@ -449,8 +498,10 @@ DEVI void gae_one_tile(const GaeArgs& g, int64_t tile, int64_t t_begin, int64_t 
   // tile applied to the fp64 state entering the tile
   float A = (float)fma((double)excl.a11, A0, fma((double)excl.a12, nv0, (double)excl.b1));
   float nv = (float)fma((double)excl.a22, nv0, (double)excl.b2);
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) oa[i] = 0.f;
   if (any) {
-    float oa[GAE_ITEMS], orr[GAE_ITEMS];
+    float orr[GAE_ITEMS];
 #pragma unroll
     for (int i = GAE_ITEMS - 1; i >= 0; --i) {
       const MapF f = token_map(i);
@@ -526,10 +577,10 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_owned_kernel(GaeArgs g) {
     const int64_t t0 = tile * GAE_TILE + (int64_t)tid * GAE_ITEMS;
     int i_lo, i_hi;
     gae_owned_items(t0, t_begin, t_end, i_lo, i_hi);
-    float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS];
+    float rw[GAE_ITEMS], v[GAE_ITEMS], ms[GAE_ITEMS], oa[GAE_ITEMS];
     gae_load_items(g, t0, i_lo < i_hi, rw, v, ms);
     gae_one_tile<STATS, ONE_ROW ? GAE_LAYOUT_ONE_ROW : GAE_LAYOUT_ROWS, LAMBDAS>(
-        g, tile, t_begin, t_end, s_first, n_own, nullptr, A0, nv0, rs, smem, all, rw, v, ms);
+        g, tile, t_begin, t_end, s_first, n_own, nullptr, A0, nv0, rs, smem, all, rw, v, ms, oa);
   }
   if constexpr (STATS) {  // block = row: uniform for the block
     __shared__ double s_rs[4 * 5];
@@ -544,23 +595,124 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_owned_kernel(GaeArgs g) {
 // Single-pass GAE for packed sequences of ordinary length, one block per tile. What enters the
 // tile from its right is the state of the sequence that crosses the tile's right edge, and it
 // depends only on that sequence's tokens beyond the edge: the block reads them too (rewards,
-// values, mask; nothing written), two tiles' worth at a time with all loads in flight together,
-// and composes their maps onto the zero state. No block waits for another, and the remainder is
-// read once per tile of the sequence, from L2 mostly: the blocks of an XCD are neighbours in the
-// array. Against blocks that walk the sequences they own tile by tile, carrying the state (the
-// padded-row kernel above, which also took cu_seqlens once): equal on 1024 sequences of mean
-// length 1760 (18.7 / 18.3 us; of the tile kernel's time 6.5 us are the tile's loads and stores,
-// 1.3 us the sequence layout, 5.7 us the remainder and 5.2 us the scan), 19 against 24 us on
-// 64 x 16384 tokens and 24 against 38 us on 4 x 32768, where a walking block has 16 tiles in a
-// row. The kernel is bound by vector instruction issue (about 1400 per wave and tile), so it is
-// held to 128 registers: all blocks of a 1.8 M-token batch are then resident at once (186
-// registers with three tiles per round: two rounds of blocks, 25.6 us).
-constexpr int GAE_CARRY_BATCH = 2;
+// values, mask; nothing written), one tile's worth at a time, and composes their maps onto the
+// zero state; a wave whose 512 tokens lie beyond the sequence's end skips its share. No block
+// waits for another, and the remainder is read once per tile of the sequence, from L2 mostly:
+// the blocks of an XCD are neighbours in the array. Against blocks that walk the sequences they
+// own tile by tile, carrying the state (the padded-row kernel above, which also took cu_seqlens
+// once): faster on 64 x 16384 tokens and on 4 x 32768, where a walking block has 16 tiles in a row.
+// The kernel is bound by vector instruction issue (about 1150 vector and 250 scalar instructions
+// per wave and tile on 1024 sequences of mean length 1760) with four blocks resident per CU, so
+// that all blocks of a 1.8 M-token batch run at once; that leaves 128 registers. Two remainder
+// tiles per round need 148 and spill 20 of them into scratch memory: 19.9 against 15.4 us.
+constexpr int GAE_CARRY_BATCH = 1;
 constexpr int GAE_CU_LDS = 16 * GAE_THREADS;  // entries of cu_seqlens the block can hold (>= TILE + 2)
 
-template <bool LAMBDAS>
+// Groups of a tile for GaeArgs::seg_stats: those of the tile's first and last token and of the next
+// tile's first token, each the number of group ends at or before the token. Waves 0..2 search
+// (their loads go out with the tile's own); s_grp is valid after the block's next barrier.
+DEVI void gae_tile_group_search(const GaeArgs& g, int64_t lo, int64_t hi, int* s_grp /* [3] */) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave < 3) {
+    const int64_t x = wave == 0 ? lo : (wave == 1 ? hi - 1 : hi);
+    const int r = wave_count_le(g.goff + 1, g.n_groups, x, lane);
+    if (lane == 0) s_grp[wave] = r;
+  }
+}
+
+// Group bounds of a tile relative to its first token, kept in registers from the start of the
+// kernel to its end: b[i] = goff[g_first + i] - lo for the first three bounds.
+struct GaeTileGroups {
+  int g_first, g_last, g_next;
+  int64_t b[3];
+};
+DEVI GaeTileGroups gae_tile_groups(const GaeArgs& g, int64_t lo, const int* s_grp) {
+  GaeTileGroups r;
+  r.g_first = s_grp[0];
+  r.g_last = s_grp[1] < g.n_groups ? s_grp[1] : g.n_groups - 1;
+  r.g_next = s_grp[2];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int j = r.g_first + i <= g.n_groups ? r.g_first + i : g.n_groups;
+    r.b[i] = g.goff[j] - lo;
+  }
+  return r;
+}
+
+// The five masked sums of the tile's advantages per group and wave (GaeArgs::seg_stats): x = oa
+// (zero for tokens outside every sequence), m = the thread's 8 mask values (zero beyond the
+// array). Every wave writes its own entry, so no wave waits for another. Every thread of the
+// block calls it.
+DEVI void gae_tile_group_stats(const GaeArgs& g, int64_t tile, int64_t lo, int64_t hi,
+                               const GaeTileGroups& tg, const float (&oa)[GAE_ITEMS],
+                               const float (&ms)[GAE_ITEMS]) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t rel = (int64_t)tid * GAE_ITEMS;  // the thread's first token relative to lo
+  const int64_t st = GAE_SEG_WAVES * g.seg_slots;
+  // the usual 0/1 mask (decided per wave): sum m^2 = sum m, sum m^2 x = sum m x, and sum m is a count
+  bool other = false;
+#pragma unroll
+  for (int i = 0; i < GAE_ITEMS; ++i) other |= ms[i] != 0.f && ms[i] != 1.f;
+  const bool binary = __builtin_amdgcn_ballot_w64(other) == 0;
+  for (int gi = tg.g_first; gi <= tg.g_last; ++gi) {
+    const int k = gi - tg.g_first;
+    // the group's bounds relative to the thread's tokens, clamped to them
+    // (selects, not an index: an indexed register array would live in scratch memory)
+    const int64_t d0 = (k == 0 ? tg.b[0] : k == 1 ? tg.b[1] : k == 2 ? tg.b[2] : g.goff[gi] - lo) - rel;
+    const int64_t d1 = (k == 0 ? tg.b[1] : k == 1 ? tg.b[2] : g.goff[gi + 1] - lo) - rel;
+    const int i0 = d0 <= 0 ? 0 : (d0 >= GAE_ITEMS ? GAE_ITEMS : (int)d0);
+    const int i1 = d1 <= 0 ? 0 : (d1 >= GAE_ITEMS ? GAE_ITEMS : (int)d1);
+    double rs[5];
+    if (binary) {
+      int cnt = 0;
+      double s1 = 0.0, s4 = 0.0;
+#pragma unroll
+      for (int i = 0; i < GAE_ITEMS; ++i) {
+        const bool on = i >= i0 && i < i1 && ms[i] != 0.f;
+        const double x = on ? (double)oa[i] : 0.0;
+        cnt += on ? 1 : 0;
+        s1 += x;
+        s4 += x * x;
+      }
+      rs[0] = (double)wave_sum(cnt);
+      rs[1] = wave_sum(s1);
+      rs[4] = wave_sum(s4);
+      rs[2] = rs[0];
+      rs[3] = rs[1];
+    } else {
+#pragma unroll
+      for (int q = 0; q < 5; ++q) rs[q] = 0.0;
+#pragma unroll
+      for (int i = 0; i < GAE_ITEMS; ++i) {
+        const double m = (i >= i0 && i < i1) ? (double)ms[i] : 0.0;
+        const double xm = (double)oa[i] * m, mm = m * m;
+        rs[0] += m; rs[1] += xm; rs[2] += mm; rs[3] += xm * m; rs[4] += xm * xm;
+      }
+#pragma unroll
+      for (int q = 0; q < 5; ++q) rs[q] = wave_sum(rs[q]);
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int q = 0; q < 5; ++q) g.seg_stats[(int64_t)q * st + GAE_SEG_WAVES * (tile + gi) + wave] = rs[q];
+    }
+  }
+  // slots that no segment maps to: before the first tile's first group, between this tile's last
+  // group and the next tile's first, and after the last tile's last group
+  const int64_t z_lo = tile == 0 ? 0 : tile + tg.g_first;
+  const int64_t r_lo = tile + tg.g_first, r_hi = tile + tg.g_last + 1;  // the slots written above
+  const int64_t z_hi = hi < g.n ? tile + 1 + tg.g_next : g.seg_slots;
+  for (int64_t j = GAE_SEG_WAVES * z_lo + tid; j < GAE_SEG_WAVES * z_hi; j += GAE_THREADS) {
+    if (j >= GAE_SEG_WAVES * r_lo && j < GAE_SEG_WAVES * r_hi) continue;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) g.seg_stats[(int64_t)q * st + j] = 0.0;
+  }
+}
+
+// STATS: also leaves the per-(tile, group) sums of GaeArgs::seg_stats.
+template <bool LAMBDAS, bool STATS>
 __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
   __shared__ MapF smem[GAE_THREADS / 64];
+  __shared__ int s_grp[3];
   __shared__ MapF all[GAE_THREADS];
   __shared__ MapF s_part[GAE_THREADS / 64][GAE_CARRY_BATCH];
   __shared__ int32_t s_cu[GAE_CU_LDS];
@@ -586,6 +738,8 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
       const int i = tid + k * GAE_THREADS;
       c[k] = i <= g.n_seqs ? g.cu[i] : 0;
     }
+    // (after the loads above are on their way: the search waits for its own)
+    if constexpr (STATS) gae_tile_group_search(g, lo, hi, s_grp);
 #pragma unroll
     for (int k = 0; k < GAE_CU_LDS / GAE_THREADS; ++k) s_cu[tid + k * GAE_THREADS] = c[k];
     if (tid < 2) s_own[tid] = 0;
@@ -593,6 +747,7 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
     cov_lo = (int64_t)s_cu[0];
     cov_hi = (int64_t)s_cu[g.n_seqs];
   } else {
+    if constexpr (STATS) gae_tile_group_search(g, lo, hi, s_grp);
     cov_lo = (int64_t)g.cu[0];
     cov_hi = (int64_t)g.cu[g.n_seqs];
   }
@@ -603,7 +758,14 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
   }
   const int64_t t_begin = lo > cov_lo ? lo : cov_lo;
   const int64_t t_end = hi < cov_hi ? hi : cov_hi;
-  if (t_end <= t_begin) return;  // uniform for the block
+  if (t_end <= t_begin) {  // uniform for the block
+    if constexpr (STATS) {
+      const float zero[GAE_ITEMS] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      __syncthreads();
+      gae_tile_group_stats(g, tile, lo, hi, gae_tile_groups(g, lo, s_grp), zero, ms);
+    }
+    return;
+  }
 
   // sequences holding the first and the last token of [t_begin, t_end): the number of sequence
   // ends at or before each
@@ -640,6 +802,8 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
     }
   }
   const int n_own = s_last - s_first + 1;
+  GaeTileGroups tg;
+  if constexpr (STATS) tg = gae_tile_groups(g, lo, s_grp);  // a barrier has passed since the search
 
   // the crossing sequence's tokens [t_end, e): in whole tiles from t_end (a multiple of the tile
   // when e > t_end), the rightmost batch first
@@ -681,6 +845,9 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
       for (int k = 0; k < GAE_CARRY_BATCH; ++k) {
         const int64_t t0 = t_end + (j0 + k) * GAE_TILE + (int64_t)tid * GAE_ITEMS;
         MapF acc = map_identity_t<float>();
+        part[k] = acc;
+        // a wave whose 512 tokens all lie beyond the sequence contributes the identity
+        if (!(j0 + k < j && t0 - (int64_t)lane * GAE_ITEMS < e)) continue;
 #pragma unroll
         for (int i = GAE_ITEMS - 1; i >= 0; --i) {
           const int64_t t = t0 + i;
@@ -695,10 +862,7 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
           if (j0 + k < j && t == e - 1) f = MapF{0.f, 0.f, 0.f, 0.f, boot ? v[k][i] : 0.f};
           acc = compose(f, acc);
         }
-        // wave total in lane 0 (the upper lanes' values are not used)
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) acc = compose(acc, shfl_down_map(acc, d));
-        part[k] = acc;
+        part[k] = wave_total_map(acc);
       }
       __syncthreads();  // the previous batch's readers are done
       if (lane == 0) {
@@ -719,14 +883,17 @@ __global__ __launch_bounds__(GAE_THREADS, 4) void gae_tile_kernel(GaeArgs g) {
     }
   }
   double rs[1];
+  float oa[GAE_ITEMS];
   gae_one_tile<false, GAE_LAYOUT_CU, LAMBDAS>(g, tile, t_begin, t_end, s_first, n_own, cu_own, A0, nv0, rs, smem,
-                                              all, rw, v, ms);
+                                              all, rw, v, ms, oa);
+  if constexpr (STATS) gae_tile_group_stats(g, tile, lo, hi, tg, oa, ms);
 }
 
 // ---------------------------------------------------------------------------------------
 // Normalisation
 // ---------------------------------------------------------------------------------------
 constexpr int NORM_THREADS = 256;
+constexpr int SEG_APPLY_ELEMS = 16 * NORM_THREADS;  // elements per block of the apply pass after the packed GAE
 enum { LEVEL_NONE = 0, LEVEL_BATCH = 1, LEVEL_GROUP = 2 };
 
 struct NormArgs {
@@ -748,7 +915,10 @@ struct NormArgs {
   // closed form only: where the five sums of a group are. part_rows == 0: [5][G][nsplit], written
   // by norm_stats5_kernel. part_rows > 0: [5][part_rows], one entry per row of row_len elements
   // (written by the GAE kernel); group g owns the rows from goff[g] / row_len on, grows[g] of them.
+  // part_tile > 0: [5][part_slots][4], four entries per (tile of part_tile tokens, group) segment
+  // in slot tile + group (written by the packed GAE kernel, GaeArgs::seg_stats); unused slots are zero.
   int64_t part_rows, row_len;
+  int64_t part_tile, part_slots;
 };
 
 DEVI double block_sum_d(double v, double* smem) {
@@ -922,25 +1092,78 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_apply_cf_kernel(NormArgs a)
   int64_t lo, hi;
   split_range(a, g, sp, lo, hi);
   const bool any_batch = a.mean_level == LEVEL_BATCH || a.std_level == LEVEL_BATCH;
-  const int64_t st = a.part_rows > 0 ? a.part_rows : (int64_t)a.G * a.nsplit;
-  const int64_t p0 = a.part_rows > 0 ? a.goff[g] / a.row_len : (int64_t)g * a.nsplit;
-  const int64_t pn = a.part_rows > 0 ? (g == a.tail_group ? a.part_rows - p0 : a.grows[g]) : a.nsplit;
+  // The block's first 16 elements per thread are requested before the partial sums, which then
+  // arrive while those loads are in flight.
+  int64_t mid_lo = (lo + 3) & ~(int64_t)3, mid_hi = hi & ~(int64_t)3;
+  if (mid_lo > mid_hi) { mid_lo = hi; mid_hi = hi; }
+  const int64_t step = 4 * (int64_t)blockDim.x;
+  f32x4 xv[4], mv[4];
+  auto fetch = [&](int64_t i) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t j = i + u * step;
+      xv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      mv[u] = f32x4{1.f, 1.f, 1.f, 1.f};
+      if (j < mid_hi) {
+        xv[u] = *(const f32x4*)(a.x + j);
+        if (has_mask) mv[u] = *(const f32x4*)(a.mask + j);
+      }
+    }
+  };
+  const int64_t i0 = mid_lo + 4 * (int64_t)threadIdx.x;
+  fetch(i0);
+  int64_t st, p0, pn;  // the group's partial sums: entries [p0, p0 + pn) of arrays of st entries
+  if (a.part_tile > 0) {
+    const int64_t g0 = a.goff[g], g1 = a.goff[g + 1];
+    st = GAE_SEG_WAVES * a.part_slots;
+    p0 = GAE_SEG_WAVES * (g0 / a.part_tile + g);
+    pn = g1 > g0 ? GAE_SEG_WAVES * ((g1 - 1) / a.part_tile - g0 / a.part_tile + 1) : 0;
+  } else if (a.part_rows > 0) {
+    st = a.part_rows;
+    p0 = a.goff[g] / a.row_len;
+    pn = g == a.tail_group ? a.part_rows - p0 : a.grows[g];
+  } else {
+    st = (int64_t)a.G * a.nsplit;
+    p0 = (int64_t)g * a.nsplit;
+    pn = a.nsplit;
+  }
   double v[10];  // group sums 0..4, batch sums 5..9
 #pragma unroll
   for (int k = 0; k < 10; ++k) v[k] = 0.0;
-  for (int64_t i = threadIdx.x; i < pn; i += blockDim.x) {
-#pragma unroll
-    for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + p0 + i];
-  }
   if (any_batch) {
+    for (int64_t i = threadIdx.x; i < pn; i += blockDim.x) {
+#pragma unroll
+      for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + p0 + i];
+    }
     for (int64_t i = threadIdx.x; i < st; i += blockDim.x) {
 #pragma unroll
       for (int k = 0; k < 5; ++k) v[5 + k] += a.part[k * st + i];
     }
-  } else if (has_mask) {
-    for (int64_t i = threadIdx.x; i < st; i += blockDim.x) v[5] += a.part[i];
+    block_sum_n<10>(v, smem);
+  } else {
+    // group level only: the first wave sums the group's entries, the others wait for it
+    if (threadIdx.x < 64) {
+      for (int64_t i = threadIdx.x; i < pn; i += 64) {
+#pragma unroll
+        for (int k = 0; k < 5; ++k) v[k] += a.part[k * st + p0 + i];
+      }
+#pragma unroll
+      for (int k = 0; k < 5; ++k) v[k] = wave_sum(v[k]);
+      if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 5; ++k) smem[k] = v[k];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 5; ++k) v[k] = smem[k];
+    v[5] = v[0];
+    if (has_mask && v[0] == 0.0) {  // nothing active in the group: is anything active at all?
+      double c = 0.0;
+      for (int64_t i = threadIdx.x; i < st; i += blockDim.x) c += a.part[i];
+      v[5] = block_sum_d(c, smem + 8);
+    }
   }
-  block_sum_n<10>(v, smem);
   if (has_mask && v[5] == 0.0) {  // nothing active: the input is returned unchanged
     for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) a.out[i] = a.x[i];
     return;
@@ -988,22 +1211,9 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_apply_cf_kernel(NormArgs a)
     if (has_mask) c = c * m;
     return c / ((float)std_d + (float)eps);
   };
-  int64_t mid_lo = (lo + 3) & ~(int64_t)3, mid_hi = hi & ~(int64_t)3;
-  if (mid_lo > mid_hi) { mid_lo = hi; mid_hi = hi; }
   for (int64_t i = lo + threadIdx.x; i < mid_lo; i += blockDim.x) a.out[i] = one(a.x[i], has_mask ? a.mask[i] : 1.0f);
-  const int64_t step = 4 * (int64_t)blockDim.x;
-  for (int64_t i = mid_lo + 4 * (int64_t)threadIdx.x; i < mid_hi; i += 4 * step) {
-    f32x4 xv[4], mv[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int64_t j = i + u * step;
-      xv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-      mv[u] = f32x4{1.f, 1.f, 1.f, 1.f};
-      if (j < mid_hi) {
-        xv[u] = *(const f32x4*)(a.x + j);
-        if (has_mask) mv[u] = *(const f32x4*)(a.mask + j);
-      }
-    }
+  for (int64_t i = i0; i < mid_hi; i += 4 * step) {
+    if (i != i0) fetch(i);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int64_t j = i + u * step;
@@ -1610,9 +1820,9 @@ int areal_gae_packed(const float* rewards, const float* values, const float* los
     // packed sequences: block = tile, the state entering from the right recomputed per tile
     const dim3 grid((unsigned)(ceil_div_i64(nb, 8) * 8));
     if (lambda_seq != nullptr)
-      hipLaunchKernelGGL(gae_tile_kernel<true>, grid, dim3(GAE_THREADS), 0, stream, g);
+      hipLaunchKernelGGL((gae_tile_kernel<true, false>), grid, dim3(GAE_THREADS), 0, stream, g);
     else
-      hipLaunchKernelGGL(gae_tile_kernel<false>, grid, dim3(GAE_THREADS), 0, stream, g);
+      hipLaunchKernelGGL((gae_tile_kernel<false, false>), grid, dim3(GAE_THREADS), 0, stream, g);
     AREAL_CHECK_LAUNCH();
     return AREAL_OK;
   }
@@ -1655,6 +1865,48 @@ int areal_gae_padded_row_stats(const float* rewards, const float* values, const 
   GaeArgs g{rewards, values, loss_mask, nullptr, no_eos, lambda_seq, n_seqs * uniform_len, (int)n_seqs,
             uniform_len, discount, gae_lambda, advantages, returns, 1, row_stats};
   launch_gae_owned<true>(g, n_seqs, stream);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// Packed GAE that also leaves the statistics pass of a group normalisation of its advantages:
+// groups are runs of whole sequences, group_offsets [n_groups + 1] (int64, device) their token
+// offsets (group_offsets[0] = 0, group_offsets[n_groups] = n_tokens). segment_stats receives
+// [5][slots][4] fp64 sums (slots = 2048-token tiles + groups) for
+// areal_group_norm_from_segment_stats. One launch. AREAL_ERR_UNSUPPORTED when the batch is not one
+// for the single-pass kernel (sequences longer than 16384 tokens on average) or the groups are
+// shorter than 256 tokens on average: the caller then runs areal_gae_packed and areal_group_norm.
+size_t areal_gae_segment_stats_bytes(int64_t n_tokens, int64_t n_groups) {
+  if (n_tokens <= 0 || n_groups <= 0) return 0;
+  return (size_t)5 * GAE_SEG_WAVES * (size_t)(ceil_div_i64(n_tokens, GAE_TILE) + n_groups) * sizeof(double);
+}
+
+int areal_gae_packed_group_stats(const float* rewards, const float* values, const float* loss_mask,
+                                 const int32_t* cu_seqlens, const uint8_t* no_eos,
+                                 const float* lambda_seq, int64_t n_tokens, int64_t n_seqs,
+                                 float discount, float gae_lambda, const int64_t* group_offsets,
+                                 int64_t n_groups, float* advantages, float* returns,
+                                 double* segment_stats, size_t segment_stats_bytes,
+                                 hipStream_t stream) {
+  if (n_tokens < 0 || n_seqs < 0 || n_groups < 0) return AREAL_ERR_BAD_ARG;
+  if (n_tokens == 0) return AREAL_OK;
+  if (!rewards || !values || !loss_mask || !advantages || !returns || !cu_seqlens || !group_offsets ||
+      !segment_stats || n_seqs == 0 || n_groups == 0)
+    return AREAL_ERR_BAD_ARG;
+  if (n_seqs > (1 << 30) || n_groups > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  const int64_t nb = ceil_div_i64(n_tokens, GAE_TILE);
+  if (nb > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  if (n_tokens / n_seqs > 8 * GAE_TILE || n_tokens / n_groups < 256) return AREAL_ERR_UNSUPPORTED;
+  if (segment_stats_bytes < areal_gae_segment_stats_bytes(n_tokens, n_groups)) return AREAL_ERR_WORKSPACE;
+  GaeArgs g{rewards, values, loss_mask, cu_seqlens, no_eos, lambda_seq, n_tokens, (int)n_seqs,
+            0, discount, gae_lambda, advantages, returns, 0, nullptr};
+  g.goff = group_offsets; g.n_groups = (int)n_groups; g.seg_stats = segment_stats;
+  g.seg_slots = nb + n_groups;
+  const dim3 grid((unsigned)(ceil_div_i64(nb, 8) * 8));
+  if (lambda_seq != nullptr)
+    hipLaunchKernelGGL((gae_tile_kernel<true, true>), grid, dim3(GAE_THREADS), 0, stream, g);
+  else
+    hipLaunchKernelGGL((gae_tile_kernel<false, true>), grid, dim3(GAE_THREADS), 0, stream, g);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -1756,7 +2008,7 @@ int areal_group_norm(const float* x, const float* mask, int64_t n, const int64_t
   // batch-level deviation does not sit on top of per-group means; otherwise the deviations need
   // a pass of their own.
   a.closed_form = (!leave_one_out && !(mean_level == LEVEL_GROUP && std_level == LEVEL_BATCH)) ? 1 : 0;
-  a.part_rows = 0; a.row_len = 0;
+  a.part_rows = 0; a.row_len = 0; a.part_tile = 0; a.part_slots = 0;
   const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
   if (a.closed_form) {
     hipLaunchKernelGGL(norm_stats5_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
@@ -1799,7 +2051,42 @@ int areal_group_norm_from_row_stats(const float* x, const float* mask, int64_t n
   a.part = const_cast<double*>(row_stats);
   a.out = out;
   a.closed_form = 1;
-  a.part_rows = n_rows; a.row_len = row_len;
+  a.part_rows = n_rows; a.row_len = row_len; a.part_tile = 0; a.part_slots = 0;
+  const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
+  hipLaunchKernelGGL(norm_apply_cf_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
+  AREAL_CHECK_LAUNCH();
+  return AREAL_OK;
+}
+
+// The apply pass of areal_group_norm alone on a packed array whose per-segment sums
+// (segment_stats, as areal_gae_packed_group_stats leaves them for the same n and group_offsets)
+// are already known: one launch. Same level restrictions as areal_group_norm_from_row_stats.
+int areal_group_norm_from_segment_stats(const float* x, const float* mask, int64_t n,
+                                        const int64_t* group_offsets, const int64_t* group_rows,
+                                        int64_t n_groups, int64_t max_group_len, int tail_group,
+                                        int mean_level, int std_level, int unbiased, double eps,
+                                        const double* segment_stats, float* out, hipStream_t stream) {
+  if (n < 0 || n_groups < 0) return AREAL_ERR_BAD_ARG;
+  if (n == 0) return AREAL_OK;
+  if (!x || !out || !group_offsets || !group_rows || !segment_stats || n_groups == 0) return AREAL_ERR_BAD_ARG;
+  if (mean_level < 0 || mean_level > 2 || std_level < 0 || std_level > 2) return AREAL_ERR_BAD_ARG;
+  if (mean_level == LEVEL_GROUP && std_level == LEVEL_BATCH) return AREAL_ERR_UNSUPPORTED;
+  if (n_groups > 65535 * 16) return AREAL_ERR_UNSUPPORTED;
+  NormArgs a;
+  a.x = x; a.mask = mask; a.n = n; a.goff = group_offsets; a.grows = group_rows;
+  a.G = (int)n_groups; a.tail_group = tail_group;
+  // the partial sums do not depend on the split: one round of 16 elements per thread
+  int64_t ns = ceil_div_i64(max_group_len, (int64_t)SEG_APPLY_ELEMS);
+  if (ns > 65535) ns = 65535;
+  if (ns < 1) ns = 1;
+  a.nsplit = (int)ns;
+  a.mean_level = mean_level; a.std_level = std_level; a.leave1out = 0;
+  a.unbiased = unbiased; a.eps = eps;
+  a.part = const_cast<double*>(segment_stats);
+  a.out = out;
+  a.closed_form = 1;
+  a.part_rows = 0; a.row_len = 0;
+  a.part_tile = GAE_TILE; a.part_slots = ceil_div_i64(n, GAE_TILE) + n_groups;
   const dim3 grid((unsigned)n_groups, (unsigned)a.nsplit);
   hipLaunchKernelGGL(norm_apply_cf_kernel, grid, dim3(NORM_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();

@@ -526,11 +526,8 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
     for (int k = 0; k < N_LOSS_STATS; ++k) {
       const double sv = wave_sum((double)st.sum[k]);
       float mn = st.mn[k], mx = st.mx[k];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        mn = stat_min(mn, __shfl_xor(mn, o, 64));
-        mx = stat_max(mx, __shfl_xor(mx, o, 64));
-      }
+      mn = wave_stat_min(mn);
+      mx = wave_stat_max(mx);
       if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
     }
     __syncthreads();
@@ -615,11 +612,8 @@ __global__ __launch_bounds__(FINAL_THREADS) void loss_finalize_kernel(
       mx = stat_max(mx, sp.mx);
     }
     sum = block_sum(sum, sm_d);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      mn = stat_min(mn, __shfl_xor(mn, o, 64));
-      mx = stat_max(mx, __shfl_xor(mx, o, 64));
-    }
+    mn = wave_stat_min(mn);
+    mx = wave_stat_max(mx);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     __syncthreads();
     constexpr int NW = FINAL_THREADS / 64;

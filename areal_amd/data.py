@@ -148,6 +148,59 @@ class Normalization:
         return out
 
 
+    @torch.no_grad()
+    def packed(self, x: torch.Tensor, mask_f32: torch.Tensor | None, cu_seqlens: torch.Tensor,
+               group_sizes: list[int] | None = None, max_group_tokens: int | None = None,
+               segment_stats: torch.Tensor | None = None) -> torch.Tensor:
+        """``self`` over a packed 1-D fp32 ``x``: sequence ``i`` is ``[cu_seqlens[i],
+        cu_seqlens[i+1])`` and plays the part of row ``i`` of the padded form, so groups are runs
+        of ``group_size`` (or ``group_sizes``) whole sequences.  ``segment_stats``: the sums the
+        packed GAE kernel left for these groups (``_packed_gae_with_segment_stats``), which make
+        this one launch; the configuration must satisfy ``needs_one_statistics_pass``.
+        ``max_group_tokens``: an upper bound of a group's token count (read back from
+        ``cu_seqlens`` when not given, which waits for the GPU)."""
+        lib = _lib.load()
+        dev = _lib.require_gpu(x, mask_f32, cu_seqlens)
+        if x.ndim != 1:
+            raise ValueError(f"packed normalisation expects a 1D tensor, got ndim={x.ndim}")
+        n, n_seqs = x.numel(), cu_seqlens.numel() - 1
+        if n == 0:
+            return x.clone()
+        index, rows, tail_group = self._packed_groups(n_seqs, group_sizes, dev)
+        offsets = cu_seqlens.to(torch.int64)[index]
+        if max_group_tokens is None:
+            max_group_tokens = int((offsets[1:] - offsets[:-1]).max())
+        out = torch.empty_like(x)
+        levels = (_LEVEL_ID[self.mean_level], _LEVEL_ID[self.std_level])
+        if segment_stats is not None:
+            rc = lib.areal_group_norm_from_segment_stats(
+                _lib.ptr(x), _lib.ptr(mask_f32), n, _lib.ptr(offsets), _lib.ptr(rows), rows.numel(),
+                max_group_tokens, tail_group, *levels, int(bool(self.std_unbiased)), float(self.eps),
+                _lib.ptr(segment_stats), _lib.ptr(out), _lib.stream_ptr(dev),
+            )
+            _lib.check(rc, "areal_group_norm_from_segment_stats")
+            return out
+        nbytes = lib.areal_group_norm_workspace_bytes(rows.numel(), max_group_tokens)
+        ws = _lib.workspace(nbytes, dev)
+        rc = lib.areal_group_norm(
+            _lib.ptr(x), _lib.ptr(mask_f32), n, _lib.ptr(offsets), _lib.ptr(rows), rows.numel(),
+            max_group_tokens, tail_group, *levels, int(bool(self.mean_leave1out)),
+            int(bool(self.std_unbiased)), float(self.eps), _lib.ptr(out), _lib.ptr(ws), nbytes,
+            _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_group_norm")
+        return out
+
+    def _packed_groups(self, n_seqs: int, group_sizes, dev):
+        """(index of each group's first sequence plus ``n_seqs`` [G+1], sequences per group [G],
+        tail group) as device tensors, for groups of whole sequences."""
+        if self.mean_level == "group" or self.std_level == "group":
+            groups, tail = self._group_rows(n_seqs, group_sizes)
+        else:
+            groups, tail = (n_seqs,), 0
+        return _group_tables(groups, tail, 1, str(dev))[:3]
+
+
 class KLEstimator:
     """k1 / k2 / k3 estimators of KL(new || base) from log-probabilities
     (``data.py:1640-1698``).  Elementwise tensor arithmetic on whatever device holds the

@@ -122,6 +122,53 @@ def compute_gae_packed(
     )
 
 
+def compute_gae_packed_normalized(
+    rewards: torch.Tensor,
+    values: torch.Tensor,
+    loss_mask: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    seq_no_eos_mask: torch.Tensor | None,
+    discount: float,
+    gae_lambda: float | torch.Tensor,
+    adv_norm,
+    group_sizes: list[int] | None = None,
+    max_group_tokens: int | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``compute_gae_packed`` followed by ``adv_norm`` (a ``Normalization``) of the advantages
+    under ``loss_mask``, with groups of whole sequences: what ``compute_advantages`` does after
+    GAE (``areal/trainer/ppo/actor.py:344-350``), on the packed layout.  Returns ``(normalised
+    advantages, returns, raw advantages)``.  Two launches when the normalisation needs one
+    statistics pass (the GAE kernel leaves the sums), else GAE and the three normalisation passes."""
+    if rewards.ndim != 1:
+        raise ValueError(f"packed GAE expects 1D tensors, got ndim={rewards.ndim}")
+    lib = _lib.load()
+    dev = _lib.require_gpu(rewards, values, loss_mask, cu_seqlens)
+    cu = cu_seqlens.to(device=dev, dtype=torch.int32).contiguous()
+    n, n_seqs = rewards.numel(), cu.numel() - 1
+    r = rewards.to(torch.float32).contiguous()
+    v = values.to(torch.float32).contiguous()
+    m = loss_mask.to(torch.float32).contiguous()
+    if n > 0 and n_seqs > 0 and adv_norm.needs_one_statistics_pass():
+        lam_seq, lam = _split_lambda(gae_lambda, n_seqs, dev)
+        no_eos = seq_no_eos_mask.to(device=dev, dtype=torch.bool).contiguous() if seq_no_eos_mask is not None else None
+        index, rows, _ = adv_norm._packed_groups(n_seqs, group_sizes, dev)
+        offsets = cu.to(torch.int64)[index]
+        nbytes = lib.areal_gae_segment_stats_bytes(n, rows.numel())
+        seg = torch.empty(nbytes // 8, dtype=torch.float64, device=dev)
+        adv, ret = torch.empty_like(r), torch.empty_like(r)
+        rc = lib.areal_gae_packed_group_stats(
+            _lib.ptr(r), _lib.ptr(v), _lib.ptr(m), _lib.ptr(cu), _lib.ptr(no_eos), _lib.ptr(lam_seq), n, n_seqs,
+            float(discount), float(lam), _lib.ptr(offsets), rows.numel(), _lib.ptr(adv), _lib.ptr(ret),
+            _lib.ptr(seg), nbytes, _lib.stream_ptr(dev),
+        )
+        if rc != _lib.ERR_UNSUPPORTED:
+            _lib.check(rc, "areal_gae_packed_group_stats")
+            normed = adv_norm.packed(adv, m, cu, group_sizes, max_group_tokens, segment_stats=seg)
+            return normed, ret, adv
+    adv, ret = compute_gae_packed(r, v, m, cu, seq_no_eos_mask, discount, gae_lambda)
+    return adv_norm.packed(adv, m, cu, group_sizes, max_group_tokens), ret, adv
+
+
 _TURN_ID_ERRORS = (
     (1, "turn_ids must be non-negative at every active loss token"),
     (2, "turn_ids at active loss tokens must be smaller than the sequence length"),

@@ -247,7 +247,23 @@ def hbm_rooflines(dev):
     add("gae_tile_kernel + norm_stats5_kernel + norm_apply_cf_kernel (C ABI)",
         f"config 3: 1024 packed sequences, {T} tokens, GAE then group normalisation of the advantages, "
         "launches back to back, 20 + 20 B/token", 40 * T, timed(gae_then_norm))
-    del adv_o, ret_o, nrm_o
+    # the same in two launches: the GAE kernel leaves the per-(tile, group) sums of its advantages,
+    # the apply pass of the normalisation starts from them
+    seg_n = lib_.areal_gae_segment_stats_bytes(T, 64)
+    seg = torch.empty(seg_n // 8, dtype=torch.float64, device=dev)
+
+    def gae_stats_then_apply():
+        rc = lib_.areal_gae_packed_group_stats(L_.ptr(r), L_.ptr(v), L_.ptr(m), L_.ptr(cu), None, None, T, 1024, 1.0,
+                                               0.95, L_.ptr(goff), 64, L_.ptr(adv_o), L_.ptr(ret_o), L_.ptr(seg), seg_n,
+                                               strm)
+        rc |= lib_.areal_group_norm_from_segment_stats(L_.ptr(adv_o), L_.ptr(m), T, L_.ptr(goff), L_.ptr(grow), 64,
+                                                       max_glen, -1, 2, 2, 1, 1e-5, L_.ptr(seg), L_.ptr(nrm_o), strm)
+        assert rc == 0
+
+    add("gae_tile_kernel<stats> + norm_apply_cf_kernel (C ABI)",
+        f"config 3: 1024 packed sequences, {T} tokens, GAE that leaves the normalisation's sums, then the apply "
+        "pass: two launches, 20 + 20 B/token", 40 * T, timed(gae_stats_then_apply))
+    del adv_o, ret_o, nrm_o, seg
     # the padded drop-in signature on the same batch: [1024, 8192] (8.39 M slots)
     from areal_amd.ppo.gae import _compute_token_level_gae
 

@@ -342,6 +342,23 @@ int areal_gae_padded_row_stats(const float* rewards, const float* values, const 
                                float* advantages, float* returns, double* row_stats,
                                areal_stream_t stream);
 
+/* areal_gae_packed on packed sequences (cu_seqlens) that also leaves the statistics pass of a
+ * group normalisation of the advantages under loss_mask (areal/trainer/ppo/actor.py:344-350 on
+ * the packed layout): groups are runs of whole sequences, group_offsets [n_groups + 1] (int64,
+ * device) their token offsets from 0 to n_tokens. segment_stats (fp64,
+ * areal_gae_segment_stats_bytes(n_tokens, n_groups) bytes) receives the five sums of
+ * areal_gae_padded_row_stats per (2048-token tile, group) segment, for
+ * areal_group_norm_from_segment_stats. One launch. AREAL_ERR_UNSUPPORTED when sequences average
+ * more than 16384 tokens or groups fewer than 256: run areal_gae_packed and areal_group_norm. */
+size_t areal_gae_segment_stats_bytes(int64_t n_tokens, int64_t n_groups);
+int areal_gae_packed_group_stats(const float* rewards, const float* values, const float* loss_mask,
+                                 const int32_t* cu_seqlens, const uint8_t* no_eos,
+                                 const float* lambda_seq, int64_t n_tokens, int64_t n_seqs,
+                                 float discount, float gae_lambda, const int64_t* group_offsets,
+                                 int64_t n_groups, float* advantages, float* returns,
+                                 double* segment_stats, size_t segment_stats_bytes,
+                                 areal_stream_t stream);
+
 /* Turn-level GAE (areal/trainer/ppo/gae.py:82-163) on padded [bs, max_seqlen] tensors: every
  * generated turn is one timestep. turn_ids int32 (-1 in prompt / tool gaps; non-decreasing over
  * the active tokens of a row), loss_mask fp32 (nonzero = active). *status (device int, zeroed
@@ -387,6 +404,15 @@ int areal_group_norm_from_row_stats(const float* x, const float* mask, int64_t n
                                     int64_t n_groups, int64_t max_group_len, int tail_group,
                                     int mean_level, int std_level, int unbiased, double eps,
                                     const double* row_stats, float* out, areal_stream_t stream);
+
+/* The same apply pass on a packed array of n elements whose segment sums
+ * areal_gae_packed_group_stats left (same n and group_offsets): one launch, same restrictions. */
+int areal_group_norm_from_segment_stats(const float* x, const float* mask, int64_t n,
+                                        const int64_t* group_offsets, const int64_t* group_rows,
+                                        int64_t n_groups, int64_t max_group_len, int tail_group,
+                                        int mean_level, int std_level, int unbiased, double eps,
+                                        const double* segment_stats, float* out,
+                                        areal_stream_t stream);
 
 size_t areal_masked_norm_workspace_bytes(int64_t n);
 

@@ -431,3 +431,120 @@ def test_compute_advantages_fused_gae_and_normalisation_equal_the_two_stage_rout
     want = N.normalization(want_a, fused["loss_mask"].cpu().float(), mean_level=mean_level, std_level=std_level,
                            group_size=8)
     torch.testing.assert_close(fused["advantages"].cpu(), want, rtol=1e-4, atol=1e-5 * want.abs().max().item())
+
+
+def _pad_packed(x, cu, fill=0.0):
+    lens = (cu[1:] - cu[:-1]).long()
+    L = max(int(lens.max()), 1)
+    out = torch.full((lens.numel(), L), fill, dtype=x.dtype)
+    pos = torch.arange(x.numel()) - cu[:-1].long().repeat_interleave(lens)
+    rows = torch.arange(lens.numel()).repeat_interleave(lens)
+    out[rows, pos] = x
+    return out, (rows, pos)
+
+
+PACKED_NORM_LAYOUTS = {
+    # sequences per tile of 2048 tokens: several groups inside one tile
+    "short": dict(lens=[300, 17, 450, 1, 612, 95, 800, 333, 64, 2, 700, 410, 129, 256, 31, 999], group_size=2),
+    # groups that cross tile boundaries, one sequence of several tiles, an empty sequence
+    "long": dict(lens=[5000, 1200, 0, 2048, 4096, 37, 7000, 2047, 2049, 1], group_size=2),
+    # explicit uneven groups
+    "uneven": dict(lens=[1500, 700, 2600, 90, 3100, 512, 800, 1300, 1900], group_sizes=[1, 3, 2, 3]),
+    # rows after the last whole group form the tail (mean 0, deviation 0 at group level)
+    "tail": dict(lens=[900, 1100, 2100, 700, 1600, 450, 3000], group_size=3),
+}
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(mean_level="group", std_level="group"),
+    dict(mean_level="group", std_level="group", std_unbiased=False, eps=0.0),
+    dict(mean_level="batch", std_level="batch"),
+    dict(mean_level="batch", std_level="group"),
+    dict(mean_level="group", std_level=None),
+    dict(mean_level="group", std_level="batch"),           # needs the second statistics pass
+    dict(mean_level="group", std_level="group", mean_leave1out=True),  # so does leave-one-out
+], ids=["gg", "gg_biased", "bb", "bg", "g_none", "gb", "gg_loo"])
+@pytest.mark.parametrize("layout", list(PACKED_NORM_LAYOUTS))
+@pytest.mark.parametrize("float_mask", [False, True], ids=["mask01", "maskf"])
+def test_packed_gae_then_normalisation_matches_oracle(dev, cfg, layout, float_mask):
+    """GAE over packed sequences whose kernel also leaves the normalisation's sums, then the one
+    apply launch: against the oracle's GAE and its normalisation of the padded form."""
+    from areal_amd.ppo.gae import compute_gae_packed_normalized
+
+    spec = PACKED_NORM_LAYOUTS[layout]
+    lens = torch.tensor(spec["lens"])
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    T = int(cu[-1])
+    g = torch.Generator().manual_seed(T)
+    r = torch.randn(T, generator=g) * 0.3
+    v = torch.randn(T, generator=g)
+    m = (torch.rand(T, generator=g) > 0.3).float()
+    if float_mask:
+        m = m * (0.5 + torch.rand(T, generator=g))
+    ne = torch.rand(lens.numel(), generator=g) > 0.5
+    group_sizes = spec.get("group_sizes")
+    full = dict(cfg, group_size=spec.get("group_size", 1))
+    norm = Normalization(NormConfig(**full))
+    got, ret, raw = compute_gae_packed_normalized(r.to(dev), v.to(dev), m.to(dev), cu.to(dev), ne.to(dev), 0.99, 0.9,
+                                                  norm, group_sizes=group_sizes)
+    want_a, want_r = G.gae_packed(r, v, m, cu, ne, 0.99, 0.9)
+    scale = want_a.abs().max().item()
+    torch.testing.assert_close(raw.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
+    torch.testing.assert_close(ret.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
+    # the oracle normalises the padded form of the advantages the kernel wrote
+    pa, idx = _pad_packed(raw.cpu(), cu)
+    pm, _ = _pad_packed(m, cu)
+    want = N.normalization(pa, pm, group_sizes=group_sizes, **full)[idx]
+    big = max(1.0, want[torch.isfinite(want)].abs().max().item())
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-5 * big, equal_nan=True)  # 0 / 0 in a tail group with eps 0
+    # and the separate statistics pass gives the same
+    two_stage = norm.packed(raw, m.to(dev), cu.to(dev), group_sizes)
+    torch.testing.assert_close(got, two_stage, rtol=1e-5, atol=1e-6 * big, equal_nan=True)
+
+
+def test_packed_gae_segment_sums_equal_fp64_group_sums(dev):
+    """The (tile, group) segment sums the packed GAE kernel leaves (four entries per segment, one
+    per wave of the tile's block) add up, per segment, per group and over the whole array, to the
+    fp64 sums of the advantages it wrote; slots of no segment are zero."""
+    from areal_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(11)
+    lens = torch.clamp((torch.randn(96, generator=g) + 6.5).exp().long(), 1, 6000)
+    lens[7] = 0
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    T, S = int(cu[-1]), lens.numel()
+    seq_off = torch.tensor([0, 8, 9, 9, 24, 40, 60, 96])  # uneven groups of whole sequences, one empty
+    goff = cu.long()[seq_off]
+    G_ = goff.numel() - 1
+    r = torch.randn(T, generator=g)
+    v = torch.randn(T, generator=g)
+    m = (torch.rand(T, generator=g) > 0.4).float() * (0.25 + torch.rand(T, generator=g))
+    nbytes = lib.areal_gae_segment_stats_bytes(T, G_)
+    slots = nbytes // 160
+    assert slots == (T + 2047) // 2048 + G_
+    seg = torch.full((5, slots, 4), float("nan"), dtype=torch.float64, device=dev)
+    adv, ret = torch.empty(T, device=dev), torch.empty(T, device=dev)
+    rd, vd, md, cud, gd = r.to(dev), v.to(dev), m.to(dev), cu.to(dev), goff.to(dev)
+    rc = lib.areal_gae_packed_group_stats(_lib.ptr(rd), _lib.ptr(vd), _lib.ptr(md), _lib.ptr(cud), None, None, T, S,
+                                          1.0, 0.95, _lib.ptr(gd), G_, _lib.ptr(adv), _lib.ptr(ret), _lib.ptr(seg),
+                                          nbytes, _lib.stream_ptr(dev))
+    assert rc == 0
+    seg = seg.cpu()
+    assert torch.isfinite(seg).all()
+    seg = seg.sum(2)
+    x, md64 = adv.cpu().double(), m.double()
+    terms = torch.stack([md64, x * md64, md64 * md64, md64 * md64 * x, (md64 * x) ** 2])
+    used = torch.zeros(slots, dtype=torch.bool)
+    for j in range(G_):
+        a, b = int(goff[j]), int(goff[j + 1])
+        if b == a:
+            continue
+        k0, k1 = a // 2048, (b - 1) // 2048
+        used[k0 + j:k1 + j + 1] = True
+        torch.testing.assert_close(seg[:, k0 + j:k1 + j + 1].sum(1), terms[:, a:b].sum(1), rtol=1e-12, atol=1e-12)
+        for k in range(k0, k1 + 1):  # every segment on its own
+            lo, hi = max(a, k * 2048), min(b, (k + 1) * 2048)
+            torch.testing.assert_close(seg[:, k + j], terms[:, lo:hi].sum(1), rtol=1e-12, atol=1e-12)
+    assert (seg[:, ~used] == 0).all()
+    torch.testing.assert_close(seg.sum(1), terms.sum(1), rtol=1e-12, atol=1e-12)

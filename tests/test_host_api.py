@@ -42,12 +42,13 @@ def test_library_exports_every_declared_symbol():
 
 def test_workspace_size_queries_run_without_gpu():
     lib = _lib.load()
-    # H a multiple of 128 (hand-scheduled kernels, 2 slots per split): 4 vocabulary splits; the ragged
+    # H a multiple of 64 (hand-scheduled kernels, 2 slots per split): 4 vocabulary splits; the ragged
     # last vocabulary tile rides in the last split's sweep (a vocabulary that is not a multiple of 64
-    # keeps a launch and a slot pair of its own). Other H: 4 slots per split, + 1 split for the ragged tile
+    # keeps a launch and a slot pair of its own). Other H (generic kernel): 4 slots per split
     assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096, 151936) == 7 * 8 * 32768 * 4
     assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096, 151936 - 8) == 7 * 10 * 32768 * 4
-    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096 + 64, 151936) == 7 * 20 * 32768 * 4
+    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096 + 64, 151936) == 7 * 8 * 32768 * 4
+    assert lib.areal_lmhead_fwd_workspace_bytes(32768, 4096 + 8, 151936) == 7 * 16 * 32768 * 4
     # W^T [64, 1024] + dlogits [256, 1024]; a ragged chunk adds the two transposed copies
     assert lib.areal_lmhead_bwd_workspace_bytes(1024, 64, 1000, 256) >= 2 * (64 * 1024 + 256 * 1024)
     assert (lib.areal_lmhead_bwd_workspace_bytes(1000, 64, 1000, 256)
