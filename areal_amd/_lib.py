@@ -101,6 +101,7 @@ SIGNATURES: dict[str, tuple] = {
     "areal_group_norm_from_segment_stats": (I, [P, P, I64, P, P, I64, I64, I, I, I, I, D, P, P, P]),
     "areal_seqlens_from_mask": (I, [P, I64, I64, P, P, P, P]),
     "areal_pack_padded": (I, [P, P, P, I64, I64, I64, I64, P]),
+    "areal_pack_padded_multi": (I, [P, P, P, I, P, I64, I64, I64, P]),
     "areal_unpack_to_padded": (I, [P, P, P, P, I64, I64, I64, P, I, P]),
     "areal_realign_packed": (I, [P, P, P, I64, P, I64, I64, P, I, I, I64, P]),
     "areal_masked_stats_workspace_bytes": (SZ, [I]),

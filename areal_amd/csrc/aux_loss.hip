@@ -288,22 +288,24 @@ __global__ __launch_bounds__(AUX_THREADS) void sapo_token_kernel(SapoIO io, SumC
   n_valid = block_sum(n_valid, sm_l);
   if (threadIdx.x == 0) parts[blockIdx.x] = SumCount{loss_sum, n_valid, 0};
   if (STATS) {
-    __shared__ double sh_sum[AUX_THREADS / 64][N_SAPO_STATS];
-    __shared__ float sh_mn[AUX_THREADS / 64][N_SAPO_STATS], sh_mx[AUX_THREADS / 64][N_SAPO_STATS];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    // reduced inside each row of 16 lanes; the block's 16 row results meet in LDS and are combined
+    // in a fixed order
+    constexpr int NROW = AUX_THREADS / 16;
+    __shared__ double sh_sum[NROW][N_SAPO_STATS];
+    __shared__ float sh_mn[NROW][N_SAPO_STATS], sh_mx[NROW][N_SAPO_STATS];
+    const int row = threadIdx.x >> 4;
 #pragma unroll
     for (int k = 0; k < N_SAPO_STATS; ++k) {
-      const double sv = wave_sum((double)st_sum[k]);
-      float mn = st_mn[k], mx = st_mx[k];
-      mn = wave_stat_min(mn);
-      mx = wave_stat_max(mx);
-      if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
+      const double sv = row_reduce((double)st_sum[k], [](double a, double b) { return a + b; });
+      const float mn = row_reduce(st_mn[k], [](float a, float b) { return stat_min(a, b); });
+      const float mx = row_reduce(st_mx[k], [](float a, float b) { return stat_max(a, b); });
+      if ((threadIdx.x & 15) == 0) { sh_sum[row][k] = sv; sh_mn[row][k] = mn; sh_mx[row][k] = mx; }
     }
     __syncthreads();
     if (threadIdx.x < N_SAPO_STATS) {
       const int k = threadIdx.x;
       StatPart sp{sh_sum[0][k], sh_mn[0][k], sh_mx[0][k]};
-      for (int i = 1; i < AUX_THREADS / 64; ++i) {
+      for (int i = 1; i < NROW; ++i) {
         sp.sum += sh_sum[i][k];
         sp.mn = stat_min(sp.mn, sh_mn[i][k]);
         sp.mx = stat_max(sp.mx, sh_mx[i][k]);

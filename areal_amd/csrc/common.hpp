@@ -129,10 +129,40 @@ DEVI T wave_reduce(T v, Op op) {
   v = op(v, dpp_move<DPP_ROW_ROR + 1>(v, v));
   return op(op(lane_value(v, 0), lane_value(v, 16)), op(lane_value(v, 32), lane_value(v, 48)));
 }
+// The first half of wave_reduce alone: each row's result in all 16 lanes of the row (lanes 0, 16,
+// 32 and 48 then hold the wave's four partial results).
+template <typename T, typename Op>
+DEVI T row_reduce(T v, Op op) {
+  v = op(v, dpp_move<DPP_ROW_ROR + 8>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 4>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 2>(v, v));
+  v = op(v, dpp_move<DPP_ROW_ROR + 1>(v, v));
+  return v;
+}
 template <typename T>
 DEVI T wave_sum(T v) { return wave_reduce(v, [](T a, T b) { return a + b; }); }
 DEVI float wave_max(float v) { return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); }); }
 DEVI float wave_min(float v) { return wave_reduce(v, [](float a, float b) { return fminf(a, b); }); }
+
+// #{i in [0, n) : ends[i] <= x} for a non-decreasing array, by one wave: every round probes 64
+// positions and keeps the gap after the last probe that is <= x.
+template <class I>
+DEVI int wave_count_le(const I* ends, int n, int64_t x, int lane) {
+  int base = 0, len = n;
+  while (len > 0) {
+    const int step = (len + 63) >> 6;
+    const int idx = base + lane * step;
+    const bool le = (idx < base + len) && ((int64_t)ends[idx] <= x);
+    const int cnt = __popcll(__builtin_amdgcn_ballot_w64(le));
+    if (cnt == 0) break;  // ends[base] > x
+    const int hit = base + (cnt - 1) * step;  // last probe <= x
+    const int lim = base + len;
+    base = hit + 1;
+    len = step - 1;
+    if (base + len > lim) len = lim - base;
+  }
+  return base;
+}
 
 // ---------------------------------------------------------------------------------------
 // Streaming per-token kernels (losses, statistics)

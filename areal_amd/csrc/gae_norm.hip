@@ -330,26 +330,6 @@ __global__ __launch_bounds__(GAE_THREADS) void gae_apply_kernel(GaeArgs g, const
 // three-launch scan above when sequences are long on average.
 // ---------------------------------------------------------------------------------------
 
-// #{i in [0, n) : ends[i] <= x} for a non-decreasing array, by one wave: every round probes 64
-// positions and keeps the gap after the last probe that is <= x.
-template <class I>
-DEVI int wave_count_le(const I* ends, int n, int64_t x, int lane) {
-  int base = 0, len = n;
-  while (len > 0) {
-    const int step = (len + 63) >> 6;
-    const int idx = base + lane * step;
-    const bool le = (idx < base + len) && ((int64_t)ends[idx] <= x);
-    const int cnt = __popcll(__builtin_amdgcn_ballot_w64(le));
-    if (cnt == 0) break;  // ends[base] > x
-    const int hit = base + (cnt - 1) * step;  // last probe <= x
-    const int lim = base + len;
-    base = hit + 1;
-    len = step - 1;
-    if (base + len > lim) len = lim - base;
-  }
-  return base;
-}
-
 // One tile of the single-pass kernels: the block's 256 threads take 8 consecutive tokens each
 // of tile `tile` (tokens [tile * TILE, (tile + 1) * TILE)), of which [t_begin, t_end) are this
 // block's to write. cu_own[i] = cu[s_first + i] for i in [0, n_own] covers every sequence that

@@ -287,8 +287,9 @@ struct TokenAcc {
 // The logged statistics a thread reduces itself. The three 0/1-valued ones (clip_ratio,
 // dual_clip_ratio, behave_filtered_ratio) are not among them: their sums are the integer counters
 // and their extremes follow from those (loss_finalize_kernel). A thread sees at most a few
-// thousand tokens (n / (MAX_LOSS_BLOCKS * LOSS_THREADS), 8 of 4 Mi), which it sums in fp32, as
-// the reference's tracker sums whole tensors; from the wave level on the sums are fp64.
+// thousand tokens (n / (grid * LOSS_THREADS), 16 of 4 Mi), which it sums in fp32, as the
+// reference's tracker sums whole tensors; so are the 16 threads of a row, and from there on the
+// sums are fp64.
 template <bool STATS>
 struct StatAcc {
   float sum[STATS ? N_LOSS_STATS : 1], mn[STATS ? N_LOSS_STATS : 1], mx[STATS ? N_LOSS_STATS : 1];
@@ -487,8 +488,6 @@ template <bool STATS, int VEC>
 __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, LossCfg c,
                                                                    Partial* partials,
                                                                    StatPartial* stat_partials) {
-  __shared__ double sm_d[8];
-  __shared__ long long sm_l[8];
   TokenAcc acc{0.0, 0, 0, 0, 0, 0, 0};
   StatAcc<STATS> st;
   st.init();
@@ -506,35 +505,51 @@ __global__ __launch_bounds__(LOSS_THREADS) void loss_token_kernel(LossIO io, Los
     token_group_compute<STATS, 1>(io, c, n_vec + gid, tail, acc, st);
   }
 
-  const double loss_sum = block_sum(acc.loss_sum, sm_d);
-  const long long n_valid = block_sum((long long)acc.n_valid, sm_l);
-  const long long n_kept = block_sum((long long)acc.n_kept, sm_l);
-  const long long n_filtered = block_sum((long long)acc.n_filtered, sm_l);
-  const long long n_clip = block_sum((long long)acc.n_clip, sm_l);
-  const long long n_dual = block_sum((long long)acc.n_dual, sm_l);
-  const long long n_behave = block_sum((long long)acc.n_behave, sm_l);
+  // One barrier pair for everything the block hands on. A wave sums its counters as 32-bit integers
+  // (a thread sees at most a few thousand tokens); statistics are reduced inside each row of 16
+  // lanes only, and the 16 row results of the block are combined from LDS in a fixed order.
+  constexpr int NW = LOSS_THREADS / 64, NROW = LOSS_THREADS / 16;
+  __shared__ double sh_loss[NW];
+  __shared__ int sh_cnt[NW][6];
+  __shared__ double sh_sum[STATS ? NROW : 1][STATS ? N_LOSS_STATS : 1];
+  __shared__ float sh_mn[STATS ? NROW : 1][STATS ? N_LOSS_STATS : 1], sh_mx[STATS ? NROW : 1][STATS ? N_LOSS_STATS : 1];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  {
+    const double ls = wave_sum(acc.loss_sum);
+    const int cnt[6] = {wave_sum(acc.n_valid), wave_sum(acc.n_kept), wave_sum(acc.n_filtered),
+                        wave_sum(acc.n_clip), wave_sum(acc.n_dual), wave_sum(acc.n_behave)};
+    if (lane == 0) {
+      sh_loss[w] = ls;
+#pragma unroll
+      for (int k = 0; k < 6; ++k) sh_cnt[w][k] = cnt[k];
+    }
+  }
+  if (STATS) {
+    const int row = threadIdx.x >> 4;
+#pragma unroll
+    for (int k = 0; k < N_LOSS_STATS; ++k) {
+      // (the 16 threads' fp32 sums are added in fp32 like the thread's own tokens; fp64 from here)
+      const double sv = (double)row_reduce(st.sum[k], [](float a, float b) { return a + b; });
+      const float mn = row_reduce(st.mn[k], [](float a, float b) { return stat_min(a, b); });
+      const float mx = row_reduce(st.mx[k], [](float a, float b) { return stat_max(a, b); });
+      if ((threadIdx.x & 15) == 0) { sh_sum[row][k] = sv; sh_mn[row][k] = mn; sh_mx[row][k] = mx; }
+    }
+  }
+  __syncthreads();
   if (threadIdx.x == 0) {
-    Partial p{loss_sum, n_valid, n_kept, n_filtered, n_clip, n_dual, n_behave};
+    Partial p{sh_loss[0], sh_cnt[0][0], sh_cnt[0][1], sh_cnt[0][2], sh_cnt[0][3], sh_cnt[0][4], sh_cnt[0][5]};
+    for (int i = 1; i < NW; ++i) {
+      p.loss_sum += sh_loss[i];
+      p.n_valid += sh_cnt[i][0]; p.n_kept += sh_cnt[i][1]; p.n_filtered += sh_cnt[i][2];
+      p.n_clip += sh_cnt[i][3]; p.n_dual += sh_cnt[i][4]; p.n_behave += sh_cnt[i][5];
+    }
     partials[blockIdx.x] = p;
   }
   if (STATS) {
-    // wave shuffles, then the four waves' values meet in LDS and are combined in wave order
-    __shared__ double sh_sum[LOSS_THREADS / 64][N_LOSS_STATS];
-    __shared__ float sh_mn[LOSS_THREADS / 64][N_LOSS_STATS], sh_mx[LOSS_THREADS / 64][N_LOSS_STATS];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-#pragma unroll
-    for (int k = 0; k < N_LOSS_STATS; ++k) {
-      const double sv = wave_sum((double)st.sum[k]);
-      float mn = st.mn[k], mx = st.mx[k];
-      mn = wave_stat_min(mn);
-      mx = wave_stat_max(mx);
-      if (lane == 0) { sh_sum[w][k] = sv; sh_mn[w][k] = mn; sh_mx[w][k] = mx; }
-    }
-    __syncthreads();
-    if (threadIdx.x < N_LOSS_STATS) {
-      const int k = threadIdx.x;
+    if (threadIdx.x >= 64 && threadIdx.x < 64 + N_LOSS_STATS) {  // a wave other than thread 0's
+      const int k = threadIdx.x - 64;
       StatPartial sp{sh_sum[0][k], sh_mn[0][k], sh_mx[0][k]};
-      for (int i = 1; i < LOSS_THREADS / 64; ++i) {
+      for (int i = 1; i < NROW; ++i) {
         sp.sum += sh_sum[i][k];
         sp.mn = stat_min(sp.mn, sh_mn[i][k]);
         sp.mx = stat_max(sp.mx, sh_mx[i][k]);
@@ -556,47 +571,78 @@ __global__ __launch_bounds__(FINAL_THREADS) void loss_finalize_kernel(
     const Partial* __restrict__ partials, const StatPartial* __restrict__ stat_partials, int nparts,
     float* loss_out, double* __restrict__ counters, double n_tokens, double* __restrict__ stats,
     int loss_active, int rs_enabled) {
-  __shared__ double sm_d[8];
-  __shared__ long long sm_l[8];
-  __shared__ float sm_f[2 * (FINAL_THREADS / 64)];
-  double ls = 0.0;
-  long long a[6] = {0, 0, 0, 0, 0, 0};
+  constexpr int NW = FINAL_THREADS / 64;
+  __shared__ double sh_d[NW][2];     // loss sum, statistic sum
+  __shared__ long long sh_l[NW][6];
+  __shared__ float sh_f[NW][2];      // statistic minimum, maximum
+  const int k = (int)blockIdx.x - 1;  // the block's statistic; block 0: the counters and the loss
+  const bool reduced = k >= 0 && !(k == ST_CLIP_RATIO || k == ST_DUAL_CLIP_RATIO || k == ST_BEHAVE_FILTERED_RATIO);
   // the thread's partials are fetched together (one memory latency, not one per partial) and
   // added in index order
   constexpr int PER_THREAD = MAX_LOSS_BLOCKS / FINAL_THREADS;
   Partial pp[PER_THREAD];
+  StatPartial sp[PER_THREAD];
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     const int i = threadIdx.x + j * FINAL_THREADS;
     pp[j] = i < nparts ? partials[i] : Partial{0.0, 0, 0, 0, 0, 0, 0};
+    sp[j] = StatPartial{0.0, pos_inf(), neg_inf()};
+    if (reduced && i < nparts) sp[j] = stat_partials[(size_t)i * N_LOSS_STATS + k];
   }
+  double ls = 0.0, sum = 0.0;
+  long long a[6] = {0, 0, 0, 0, 0, 0};
+  float mn = pos_inf(), mx = neg_inf();
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     ls += pp[j].loss_sum;
     a[0] += pp[j].n_valid; a[1] += pp[j].n_kept; a[2] += pp[j].n_filtered;
     a[3] += pp[j].n_clip; a[4] += pp[j].n_dual; a[5] += pp[j].n_behave;
+    sum += sp[j].sum;
+    mn = stat_min(mn, sp[j].mn);
+    mx = stat_max(mx, sp[j].mx);
   }
-  ls = block_sum(ls, sm_d);
-  for (int k = 0; k < 6; ++k) a[k] = block_sum(a[k], sm_l);
-  if (blockIdx.x == 0) {
-    if (threadIdx.x == 0) {
-      counters[0] = ls;
-      for (int k = 0; k < 6; ++k) counters[1 + k] = (double)a[k];
-      const double denom = a[0] > 0 ? (double)a[0] : 1.0;
-      const float loss = (float)ls / (float)denom;
-      counters[7] = (double)loss;
-      if (loss_out) *loss_out = loss;
-    }
+  // wave results into LDS, one barrier, then thread 0 adds the waves in order
+  ls = wave_sum(ls);
+#pragma unroll
+  for (int q = 0; q < 6; ++q) a[q] = wave_sum(a[q]);
+  if (reduced) {
+    sum = wave_sum(sum);
+    mn = wave_stat_min(mn);
+    mx = wave_stat_max(mx);
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) {
+    sh_d[w][0] = ls; sh_d[w][1] = sum;
+#pragma unroll
+    for (int q = 0; q < 6; ++q) sh_l[w][q] = a[q];
+    sh_f[w][0] = mn; sh_f[w][1] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  ls = sh_d[0][0]; sum = sh_d[0][1]; mn = sh_f[0][0]; mx = sh_f[0][1];
+#pragma unroll
+  for (int q = 0; q < 6; ++q) a[q] = sh_l[0][q];
+  for (int i = 1; i < NW; ++i) {
+    ls += sh_d[i][0]; sum += sh_d[i][1];
+#pragma unroll
+    for (int q = 0; q < 6; ++q) a[q] += sh_l[i][q];
+    mn = stat_min(mn, sh_f[i][0]); mx = stat_max(mx, sh_f[i][1]);
+  }
+  if (k < 0) {
+    counters[0] = ls;
+    for (int q = 0; q < 6; ++q) counters[1 + q] = (double)a[q];
+    const double denom = a[0] > 0 ? (double)a[0] : 1.0;
+    const float loss = (float)ls / (float)denom;
+    counters[7] = (double)loss;
+    if (loss_out) *loss_out = loss;
     return;
   }
-  const int k = blockIdx.x - 1;
   const long long n_valid = a[0], n_clip = a[3], n_dual = a[4], n_behave = a[5];
   const int d = STAT_DENOM[k];
   const double count = d == 0 ? (double)n_valid : (d == 1 ? (double)n_clip : (d == 2 ? (double)n_behave : n_tokens));
-  double sum = 0.0;
-  float mn = pos_inf(), mx = neg_inf();
-  if (k == ST_CLIP_RATIO || k == ST_DUAL_CLIP_RATIO || k == ST_BEHAVE_FILTERED_RATIO) {
+  if (!reduced) {
     // ones among the n_valid tokens under the loss mask
+    sum = 0.0; mn = pos_inf(); mx = neg_inf();
     const bool on = loss_active && (k != ST_BEHAVE_FILTERED_RATIO || rs_enabled);
     const long long ones = k == ST_CLIP_RATIO ? n_clip : (k == ST_DUAL_CLIP_RATIO ? n_dual : n_valid - n_behave);
     if (on && n_valid > 0) {
@@ -604,31 +650,11 @@ __global__ __launch_bounds__(FINAL_THREADS) void loss_finalize_kernel(
       mn = ones == n_valid ? 1.0f : 0.0f;
       mx = ones > 0 ? 1.0f : 0.0f;
     }
-  } else {
-    for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
-      const StatPartial sp = stat_partials[(size_t)i * N_LOSS_STATS + k];
-      sum += sp.sum;
-      mn = stat_min(mn, sp.mn);
-      mx = stat_max(mx, sp.mx);
-    }
-    sum = block_sum(sum, sm_d);
-    mn = wave_stat_min(mn);
-    mx = wave_stat_max(mx);
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    __syncthreads();
-    constexpr int NW = FINAL_THREADS / 64;
-    if (lane == 0) { sm_f[w] = mn; sm_f[NW + w] = mx; }
-    __syncthreads();
-    mn = sm_f[0]; mx = sm_f[NW];
-#pragma unroll
-    for (int i = 1; i < NW; ++i) { mn = stat_min(mn, sm_f[i]); mx = stat_max(mx, sm_f[NW + i]); }
   }
-  if (threadIdx.x == 0) {
-    stats[4 * k + 0] = sum;
-    stats[4 * k + 1] = count;
-    stats[4 * k + 2] = (double)mn;
-    stats[4 * k + 3] = (double)mx;
-  }
+  stats[4 * k + 0] = sum;
+  stats[4 * k + 1] = count;
+  stats[4 * k + 2] = (double)mn;
+  stats[4 * k + 3] = (double)mx;
 }
 
 // out[t] = dlp[t] * upstream[0] / max(n_valid, 1); VEC as in the token kernel
@@ -887,7 +913,9 @@ int actor_loss_impl(const float* logprobs, const float* proximal, const float* o
                     aligned_to(io.entropy, 16) && aligned_to(io.extra0, 16) && aligned_to(io.extra1, 16) &&
                     aligned_to(loss_mask, 4) && aligned_to(clip_mask, 4) && aligned_to(dual_clip_mask, 4) &&
                     aligned_to(new_mask, 4) && aligned_to(behave_mask, 4);
-  const int grid = loss_grid(n_tokens, vec4 ? 4 : 1);
+  // with statistics a block's end costs a third of eight tokens' work per thread: half the blocks
+  int grid = loss_grid(n_tokens, vec4 ? 4 : 1);
+  if (with_stats && grid > MAX_LOSS_BLOCKS / 2) grid = MAX_LOSS_BLOCKS / 2;
   auto token_pass = [&](const LossIO& i, const LossCfg& cc, bool stats) {
     if (stats && vec4)
       hipLaunchKernelGGL((loss_token_kernel<true, 4>), dim3(grid), dim3(LOSS_THREADS), 0, stream, i, cc, partials, stat_partials);

@@ -35,59 +35,148 @@ DEVI void fill_elem(char* dst, const char* pattern, int pb, int64_t eb) {
   for (int64_t i = 0; i < eb; ++i) dst[i] = pattern[i % pb];
 }
 
-// lens[b] = number of nonzero entries of mask row b (one block per row).
+// 16 bytes at any address. The compiler picks the access the target allows for the alignment
+// (gfx950 runs with unaligned access enabled, where this is still one 16-byte instruction).
+struct __attribute__((packed, aligned(1))) Bytes16 { uint32_t w[4]; };
+
+// number of nonzero bytes among the four of x
+DEVI int nonzero_bytes(uint32_t x) {
+  x = (x | (x >> 4)) & 0x0f0f0f0fu;
+  x = (x | (x >> 2)) & 0x03030303u;
+  x = (x | (x >> 1)) & 0x01010101u;
+  return __popc(x);
+}
+
+// lens[b] = number of nonzero entries of mask row b (one block per row), 16 mask bytes per load.
 __global__ __launch_bounds__(PK_THREADS) void rowlens_kernel(const uint8_t* mask, int64_t S,
                                                              int32_t* lens) {
   __shared__ int sm[4];
   const uint8_t* row = mask + (int64_t)blockIdx.x * S;
   int len = 0;
-  for (int64_t s = threadIdx.x; s < S; s += blockDim.x) len += row[s] != 0;
+  const int64_t n16 = S >> 4;
+  for (int64_t i = threadIdx.x; i < n16; i += blockDim.x) {
+    const Bytes16 v = *(const Bytes16*)(row + 16 * i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) len += nonzero_bytes(v.w[k]);
+  }
+  for (int64_t s = 16 * n16 + threadIdx.x; s < S; s += blockDim.x) len += row[s] != 0;
   len = wave_sum(len);
   if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = len;
   __syncthreads();
   if (threadIdx.x == 0) lens[blockIdx.x] = sm[0] + sm[1] + sm[2] + sm[3];
 }
-// cu = exclusive prefix sums of lens, *max_len = max(lens) (one block).
-__global__ __launch_bounds__(PK_THREADS) void cu_scan_kernel(const int32_t* lens, int64_t B,
-                                                             int32_t* cu, int32_t* max_len) {
-  __shared__ int sm[PK_THREADS];
-  __shared__ int carry, mx;
-  if (threadIdx.x == 0) { carry = 0; mx = 0; cu[0] = 0; }
-  __syncthreads();
-  for (int64_t b0 = 0; b0 < B; b0 += PK_THREADS) {
-    const int64_t b = b0 + threadIdx.x;
-    const int len = b < B ? lens[b] : 0;
-    sm[threadIdx.x] = len;
-    __syncthreads();
-    for (int d = 1; d < PK_THREADS; d <<= 1) {
-      const int v = threadIdx.x >= d ? sm[threadIdx.x - d] : 0;
-      __syncthreads();
-      sm[threadIdx.x] += v;
-      __syncthreads();
-    }
-    if (b < B) {
-      cu[b + 1] = carry + sm[threadIdx.x];
-      atomicMax(&mx, len);
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) carry += sm[PK_THREADS - 1];
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) *max_len = mx;
+
+// Inclusive prefix sum over the wave's 64 lanes: inside each row of 16 through DPP, then the
+// totals of the rows to the left (lanes 15, 31, 47) are added.
+DEVI int wave_inclusive_sum(int v) {
+  v += dpp_move<DPP_ROW_SHR + 1>(0, v);
+  v += dpp_move<DPP_ROW_SHR + 2>(0, v);
+  v += dpp_move<DPP_ROW_SHR + 4>(0, v);
+  v += dpp_move<DPP_ROW_SHR + 8>(0, v);
+  const int t0 = lane_value(v, 15), t1 = lane_value(v, 31), t2 = lane_value(v, 47);
+  const int row = (threadIdx.x & 63) >> 4;
+  return v + (row == 0 ? 0 : row == 1 ? t0 : row == 2 ? t0 + t1 : t0 + t1 + t2);
 }
 
-// packed[cu[b] + j] = padded[b][j] for j < cu[b+1] - cu[b]   (pack = true)
-// padded[b][j] = j < len_b ? packed[cu[b] + j] : fill         (pack = false)
-__global__ __launch_bounds__(PK_THREADS) void pack_kernel(const char* padded, char* packed,
-                                                          const int32_t* cu, int n_seqs, int64_t S,
-                                                          int64_t eb, int64_t total) {
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total;
-       t += (int64_t)gridDim.x * blockDim.x) {
-    const int b = seq_of_cu(cu, n_seqs, t);
-    const int64_t j = t - cu[b];
-    copy_elem(packed + t * eb, padded + ((int64_t)b * S + j) * eb, eb);
+// cu = exclusive prefix sums of lens, *max_len = max(lens) (one block; 4 entries per thread and
+// round, two barriers per round).
+constexpr int SCAN_ITEMS = 4;
+__global__ __launch_bounds__(PK_THREADS) void cu_scan_kernel(const int32_t* lens, int64_t B,
+                                                             int32_t* cu, int32_t* max_len) {
+  __shared__ int sm_sum[PK_THREADS / 64], sm_max[PK_THREADS / 64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int carry = 0, mx = 0;
+  if (threadIdx.x == 0) cu[0] = 0;
+  for (int64_t b0 = 0; b0 < B; b0 += PK_THREADS * SCAN_ITEMS) {
+    const int64_t b = b0 + (int64_t)threadIdx.x * SCAN_ITEMS;
+    int len[SCAN_ITEMS];
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i) len[i] = b + i < B ? lens[b + i] : 0;
+    int tot = 0;
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i) { tot += len[i]; mx = len[i] > mx ? len[i] : mx; }
+    const int incl = wave_inclusive_sum(tot);
+    __syncthreads();  // the previous round's readers are done
+    if (lane == 63) sm_sum[w] = incl;
+    __syncthreads();
+    int base = carry + incl - tot;
+    for (int i = 0; i < w; ++i) base += sm_sum[i];
+#pragma unroll
+    for (int i = 0; i < SCAN_ITEMS; ++i) {
+      base += len[i];
+      if (b + i < B) cu[b + i + 1] = base;
+    }
+    for (int i = 0; i < PK_THREADS / 64; ++i) carry += sm_sum[i];
+  }
+  mx = wave_reduce(mx, [](int a, int b) { return a > b ? a : b; });
+  __syncthreads();
+  if (lane == 0) sm_max[w] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < PK_THREADS / 64; ++i) mx = sm_max[i] > mx ? sm_max[i] : mx;
+    *max_len = mx;
   }
 }
+
+// Copy of n contiguous bytes by the whole block: 16 bytes per thread and access, whatever the
+// two addresses' alignment, four loads in flight per thread before the first store; then the
+// last n % 16 bytes one by one.
+DEVI void block_copy_bytes(char* dst, const char* src, int64_t n) {
+  const int64_t n16 = n >> 4;
+  for (int64_t i0 = threadIdx.x; i0 < n16; i0 += 4 * (int64_t)blockDim.x) {
+    Bytes16 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * (int64_t)blockDim.x;
+      if (i < n16) v[u] = *(const Bytes16*)(src + 16 * i);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * (int64_t)blockDim.x;
+      if (i < n16) *(Bytes16*)(dst + 16 * i) = v[u];
+    }
+  }
+  for (int64_t i = 16 * n16 + threadIdx.x; i < n; i += blockDim.x) dst[i] = src[i];
+}
+
+// Several tensors packed in one launch. Block (c, k) writes packed tokens [c * chunk, (c + 1) *
+// chunk) of tensor k: it finds the sequence of its first token (every wave searches cu_seqlens
+// with 64 probes per round) and then walks the sequences its chunk touches, each one contiguous
+// run of a padded row to one contiguous run of the packed array. No block is empty. The chunk is
+// 16 KiB of the widest tensor (at most 2048 tokens), so a thread has four loads of 16 bytes in
+// flight at once.
+constexpr int PK_MAX_TENSORS = 8;
+constexpr int PK_CHUNK_BYTES = 16384, PK_CHUNK_MAX = 2048;
+struct PackArgs {
+  const char* src[PK_MAX_TENSORS];
+  char* dst[PK_MAX_TENSORS];
+  int64_t eb[PK_MAX_TENSORS];  // bytes of one token's trailing dimensions
+  const int32_t* cu;
+  int n_seqs;
+  int64_t S, total;
+  int chunk;  // tokens per block
+};
+__global__ __launch_bounds__(PK_THREADS) void pack_rows_kernel(PackArgs a) {
+  const int k = blockIdx.y;
+  int64_t t = (int64_t)blockIdx.x * a.chunk;
+  const int64_t t1 = t + a.chunk < a.total ? t + a.chunk : a.total;
+  // (selects, not an index into the argument arrays: those would be copied to scratch memory)
+  const char* src = a.src[0]; char* dst = a.dst[0]; int64_t eb = a.eb[0];
+#pragma unroll
+  for (int i = 1; i < PK_MAX_TENSORS; ++i)
+    if (k == i) { src = a.src[i]; dst = a.dst[i]; eb = a.eb[i]; }
+  // sequence of token t: the number of sequence ends at or before it (same value in every wave)
+  int b = wave_count_le(a.cu + 1, a.n_seqs, t, threadIdx.x & 63);
+  while (t < t1 && b < a.n_seqs) {
+    const int64_t start = a.cu[b], end = a.cu[b + 1];
+    const int64_t stop = end < t1 ? end : t1;
+    if (stop > t) block_copy_bytes(dst + t * eb, src + ((int64_t)b * a.S + (t - start)) * eb, (stop - t) * eb);
+    t = stop > t ? stop : t;
+    ++b;
+  }
+}
+
+// padded[b][j] = j < len_b ? packed[cu[b] + j] : fill
 struct Fill { char bytes[16]; int n; };
 __global__ __launch_bounds__(PK_THREADS) void unpack_kernel(const char* packed, char* padded,
                                                             const int32_t* cu, const int32_t* row_seq,
@@ -244,16 +333,38 @@ int areal_seqlens_from_mask(const uint8_t* attention_mask, int64_t B, int64_t S,
 }
 
 // packed [total, E] <- the first len_b tokens of every row of padded [B, S, E]; elem_bytes = bytes
-// of one token's trailing dimensions (data.py:535-541).
-int areal_pack_padded(const void* padded, void* packed, const int32_t* cu_seqlens, int64_t B,
-                      int64_t S, int64_t elem_bytes, int64_t total, hipStream_t stream) {
-  if (B < 0 || S < 0 || elem_bytes <= 0 || total < 0) return AREAL_ERR_BAD_ARG;
-  if (total == 0) return AREAL_OK;
-  if (!padded || !packed || !cu_seqlens || B == 0) return AREAL_ERR_BAD_ARG;
-  hipLaunchKernelGGL(pack_kernel, dim3(pk_grid(total)), dim3(PK_THREADS), 0, stream,
-                     (const char*)padded, (char*)packed, cu_seqlens, (int)B, S, elem_bytes, total);
+// of one token's trailing dimensions (data.py:535-541). Up to 8 tensors of one batch (host
+// arrays of device pointers and of element sizes) in one launch.
+int areal_pack_padded_multi(const void* const* padded, void* const* packed, const int64_t* elem_bytes,
+                            int n_tensors, const int32_t* cu_seqlens, int64_t B, int64_t S,
+                            int64_t total, hipStream_t stream) {
+  if (B < 0 || S < 0 || total < 0 || n_tensors < 0 || n_tensors > PK_MAX_TENSORS) return AREAL_ERR_BAD_ARG;
+  if (total == 0 || n_tensors == 0) return AREAL_OK;
+  if (!padded || !packed || !elem_bytes || !cu_seqlens || B == 0) return AREAL_ERR_BAD_ARG;
+  PackArgs a;
+  for (int k = 0; k < PK_MAX_TENSORS; ++k) { a.src[k] = nullptr; a.dst[k] = nullptr; a.eb[k] = 0; }
+  for (int k = 0; k < n_tensors; ++k) {
+    if (!padded[k] || !packed[k] || elem_bytes[k] <= 0) return AREAL_ERR_BAD_ARG;
+    a.src[k] = (const char*)padded[k]; a.dst[k] = (char*)packed[k]; a.eb[k] = elem_bytes[k];
+  }
+  int64_t max_eb = 1;
+  for (int k = 0; k < n_tensors; ++k) max_eb = elem_bytes[k] > max_eb ? elem_bytes[k] : max_eb;
+  int64_t chunk = PK_CHUNK_BYTES / max_eb;
+  chunk = chunk < 1 ? 1 : (chunk > PK_CHUNK_MAX ? PK_CHUNK_MAX : chunk);
+  const int64_t chunks = ceil_div_i64(total, chunk);
+  if (chunks >= ((int64_t)1 << 31) || B > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  a.cu = cu_seqlens; a.n_seqs = (int)B; a.S = S; a.total = total; a.chunk = (int)chunk;
+  const dim3 grid((unsigned)chunks, (unsigned)n_tensors);
+  hipLaunchKernelGGL(pack_rows_kernel, grid, dim3(PK_THREADS), 0, stream, a);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
+}
+
+int areal_pack_padded(const void* padded, void* packed, const int32_t* cu_seqlens, int64_t B,
+                      int64_t S, int64_t elem_bytes, int64_t total, hipStream_t stream) {
+  if (elem_bytes <= 0) return AREAL_ERR_BAD_ARG;
+  if (total > 0 && (!padded || !packed)) return AREAL_ERR_BAD_ARG;
+  return areal_pack_padded_multi(&padded, &packed, &elem_bytes, 1, cu_seqlens, B, S, total, stream);
 }
 
 // padded [B, S, E] <- packed sequences, the rest filled with the fill pattern (fill_bytes <= 16

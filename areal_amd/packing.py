@@ -20,6 +20,7 @@ import torch
 from areal_amd import _lib
 
 N_TOKENS_PER_PAGE = 256  # data.py:819
+_PACK_MAX_TENSORS = 8  # tensors per areal_pack_padded_multi launch
 
 
 def _elem_bytes(t: torch.Tensor, lead_dims: int) -> int:
@@ -52,6 +53,7 @@ def pack_tensor_dict(data: dict[str, Any]) -> dict[str, Any]:
     _lib.check(rc, "areal_seqlens_from_mask")
     total_length, max_seqlen = torch.stack([cu_seqlens[-1], max_len[0]]).tolist()  # the one host copy
     packed_data: dict[str, Any] = {}
+    moved = []  # (contiguous source, packed destination) of the tensors that are packed
     for key, value in data.items():
         if key == "attention_mask":
             packed_data["cu_seqlens"] = cu_seqlens
@@ -61,14 +63,21 @@ def pack_tensor_dict(data: dict[str, Any]) -> dict[str, Any]:
             _lib.require_gpu(value)
             src = value.contiguous()
             packed = torch.empty((total_length, *value.shape[2:]), dtype=value.dtype, device=value.device)
-            rc = lib.areal_pack_padded(
-                _lib.ptr(src), _lib.ptr(packed), _lib.ptr(cu_seqlens), bs, seq_len,
-                _elem_bytes(src, 2), total_length, _lib.stream_ptr(dev),
-            )
-            _lib.check(rc, "areal_pack_padded")
+            moved.append((src, packed))
             packed_data[key] = packed
         else:
             packed_data[key] = value
+    # eight tensors per launch
+    for i in range(0, len(moved), _PACK_MAX_TENSORS):
+        part = moved[i : i + _PACK_MAX_TENSORS]
+        n = len(part)
+        srcs = (ctypes.c_void_p * n)(*[s.data_ptr() for s, _ in part])
+        dsts = (ctypes.c_void_p * n)(*[d.data_ptr() for _, d in part])
+        sizes = (ctypes.c_int64 * n)(*[_elem_bytes(s, 2) for s, _ in part])
+        rc = lib.areal_pack_padded_multi(
+            srcs, dsts, sizes, n, _lib.ptr(cu_seqlens), bs, seq_len, total_length, _lib.stream_ptr(dev),
+        )
+        _lib.check(rc, "areal_pack_padded_multi")
     return packed_data
 
 

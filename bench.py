@@ -470,7 +470,7 @@ def hbm_rooflines(dev):
                  loss_mask=pattn & (ppos >= (plens // 4)[:, None]), logprobs=torch.randn(bsz, Lp, device=dev),
                  advantages=torch.randn(bsz, Lp, device=dev))
     n_packed = int(plens.sum())
-    add("rowlens + cu_scan + pack_kernel (API level)",
+    add("rowlens + cu_scan + pack_rows (API level)",
         f"pack_tensor_dict: [1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write",
         2 * 25 * n_packed + bsz * Lp, timed(lambda: pack_tensor_dict(dict(pdata))))
     # the same launches through the C ABI into preallocated outputs
@@ -482,13 +482,18 @@ def hbm_rooflines(dev):
     pk_src.append(torch.zeros(bsz, Lp, dtype=torch.long, device=dev))  # a second 8-byte tensor (position ids)
     pk_dst = [torch.empty(n_packed, dtype=t.dtype, device=dev) for t in pk_src]
 
+    import ctypes
+
+    pk_srcs = (ctypes.c_void_p * 5)(*[t.data_ptr() for t in pk_src])
+    pk_dsts = (ctypes.c_void_p * 5)(*[t.data_ptr() for t in pk_dst])
+    pk_sizes = (ctypes.c_int64 * 5)(*[t.element_size() for t in pk_src])
+
     def pack_kernels():
         rc = lib.areal_seqlens_from_mask(p(pk_mask), bsz, Lp, p(pk_lens), p(pk_cu), p(pk_max), strm2)
-        for s_, d_ in zip(pk_src, pk_dst):
-            rc |= lib.areal_pack_padded(p(s_), p(d_), p(pk_cu), bsz, Lp, s_.element_size(), n_packed, strm2)
+        rc |= lib.areal_pack_padded_multi(pk_srcs, pk_dsts, pk_sizes, 5, p(pk_cu), bsz, Lp, n_packed, strm2)
         assert rc == 0
 
-    add("rowlens + cu_scan + pack_kernel x5 (C ABI)",
+    add("rowlens + cu_scan + pack_rows (C ABI)",
         f"[1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write, and the "
         "attention mask read once", 2 * 25 * n_packed + bsz * Lp, timed(pack_kernels, iters=50))
     turn_ids = (torch.cumsum((torch.rand(bsz, Lp, device=dev) < 0.002).int(), dim=1)).to(torch.int32)

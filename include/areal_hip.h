@@ -455,6 +455,12 @@ int areal_seqlens_from_mask(const uint8_t* attention_mask, int64_t B, int64_t S,
                             int32_t* cu_seqlens, int32_t* max_len, areal_stream_t stream);
 int areal_pack_padded(const void* padded, void* packed, const int32_t* cu_seqlens, int64_t B,
                       int64_t S, int64_t elem_bytes, int64_t total, areal_stream_t stream);
+/* The tensors of one batch (pack_tensor_dict's loop over the dict, data.py:519-543) in one launch:
+ * padded / packed / elem_bytes are HOST arrays of n_tensors (at most 8) device pointers, resp.
+ * element sizes. */
+int areal_pack_padded_multi(const void* const* padded, void* const* packed,
+                            const int64_t* elem_bytes, int n_tensors, const int32_t* cu_seqlens,
+                            int64_t B, int64_t S, int64_t total, areal_stream_t stream);
 int areal_unpack_to_padded(const void* packed, void* padded, const int32_t* cu_seqlens,
                            const int32_t* row_seq, int64_t B, int64_t S, int64_t elem_bytes,
                            const void* fill, int fill_bytes, areal_stream_t stream);
