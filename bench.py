@@ -746,17 +746,17 @@ def main() -> None:
     # FETCH_SIZE / WRITE_SIZE runs of this command on this workload (KiB per dispatch, scaled by
     # the factors the same counters show for copy-like kernels of known size, the operand-prep
     # and the bf16 transpose: fetch x2.0, write x1.0); profiles/lmhead_contraction_qwen3-8b.md
-    # has the commands and the table. The forward's fetch count moves by +-20 % from run to run
-    # with L2 hit timing.
+    # has the commands and the table. The forward's fetch count moves by +-5 % from launch to
+    # launch with L2 hit timing.
     traffic = None
     traffic_detail = None
     traffic_source = None
     if args.workload == "qwen3-8b" and saved:
         kib = 1024.0
         traffic_detail = {
-            KERNEL_FWD_SAVE + " forward": 3.09126e7 * kib * 2.0 + 9.72083e6 * kib,
-            KERNEL_DHIDDEN + " dHidden": 2.92022e7 * kib * 2.0 + 2.64192e5 * kib,
-            KERNEL_DWEIGHT + " dWeight": 2.92275e7 * kib * 2.0 + 1.22189e6 * kib,
+            KERNEL_FWD_SAVE + " forward": 3.1562e7 * kib * 2.0 + 9.729e6 * kib,  # fetch: mean of 7 launches
+            KERNEL_DHIDDEN + " dHidden": 2.9199e7 * kib * 2.0 + 2.6419e5 * kib,
+            KERNEL_DWEIGHT + " dWeight": (2.9205e7 + 1.5956e5) * kib * 2.0 + 1.2219e6 * kib,  # with its 384-row tail
         }
         traffic = sum(traffic_detail.values()) / 3.0
         traffic_source = ("offline rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command "
