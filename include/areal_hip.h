@@ -222,8 +222,10 @@ int areal_actor_loss_stats(const float* logprobs, const float* proximal_logprobs
                            size_t workspace_bytes, areal_stream_t stream);
 
 /* areal_actor_loss without the workspace argument: the block partials and per-sequence
- * aggregates live in a static device array inside the library (about 1.6 MB per GPU, held until
- * the process ends), so nothing on the call path allocates. It has no counterpart in the
+ * aggregates live in a static device array inside the library (about 1.7 MB per GPU, held until
+ * the process ends), so nothing on the call path allocates. The first call on a device looks the
+ * array's address up (hipGetSymbolAddress, once per device): make one call per device outside any
+ * stream capture before a call is captured into a graph. It has no counterpart in the
  * reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc. Call it with the stream's device current. At most
  * 65536 sequences (n_seqs beyond that: AREAL_ERR_UNSUPPORTED). All calls on one GPU share that
