@@ -56,6 +56,20 @@ def test_pack_tensor_dict_matches_oracle(dev, bs, S):
         pack_tensor_dict(dict(x=data["input_ids"].to(dev)))
 
 
+def test_pack_more_tensors_than_one_launch_takes_and_a_wide_one(dev):
+    """Ten packed tensors (two launches of at most eight) and one with 8 KiB per token, whose
+    chunks are two tokens long."""
+    g = torch.Generator().manual_seed(7)
+    bs, S = 9, 300
+    lens = torch.randint(1, S + 1, (bs,), generator=g)
+    mask = torch.arange(S)[None] < lens[:, None]
+    data = dict(attention_mask=mask, wide=torch.randn(bs, S, 2048, generator=g))
+    for i in range(9):
+        data[f"t{i}"] = torch.randint(-1000, 1000, (bs, S), generator=g).to(
+            [torch.int64, torch.int32, torch.int16, torch.int8][i % 4])
+    _same(pack_tensor_dict(_to(data, dev)), P.pack_tensor_dict(data))
+
+
 @pytest.mark.parametrize("align", [None, 8, 256])
 @pytest.mark.parametrize("three", [False, True])
 def test_pad_packed_tensor_dict_matches_oracle(dev, align, three):
