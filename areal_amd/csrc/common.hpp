@@ -67,6 +67,7 @@ DEVI float bf16_bits_to_f32(u16 b) {
 constexpr int DPP_ROW_SHL = 0x100;  // + n (1..15): lane i reads lane i + n of its row
 constexpr int DPP_ROW_SHR = 0x110;  // + n: lane i reads lane i - n of its row
 constexpr int DPP_ROW_ROR = 0x120;  // + n: lane i reads lane (i - n) mod 16 of its row
+constexpr int DPP_WAVE_SHR1 = 0x138;  // lane i reads lane i - 1 of the wave (lane 0 has no source)
 
 // x of the lane CTRL names; a lane whose source falls outside its row keeps `old`.
 template <int CTRL>
@@ -139,6 +140,27 @@ DEVI T row_reduce(T v, Op op) {
   v = op(v, dpp_move<DPP_ROW_ROR + 1>(v, v));
   return v;
 }
+// Inclusive prefix scan over the wave's 64 lanes with an associative, commutative op: inside each
+// row of 16 through DPP shifts (a lane without a source takes the identity), then the results of
+// the rows to the left (lanes 15, 31, 47) are folded in.
+template <typename T, typename Op>
+DEVI T wave_inclusive_scan(T v, T identity, Op op) {
+  v = op(v, dpp_move<DPP_ROW_SHR + 1>(identity, v));
+  v = op(v, dpp_move<DPP_ROW_SHR + 2>(identity, v));
+  v = op(v, dpp_move<DPP_ROW_SHR + 4>(identity, v));
+  v = op(v, dpp_move<DPP_ROW_SHR + 8>(identity, v));
+  const T t0 = lane_value(v, 15), t1 = lane_value(v, 31), t2 = lane_value(v, 47);
+  const int row = (threadIdx.x & 63) >> 4;
+  T left = identity;
+  if (row >= 1) left = t0;
+  if (row >= 2) left = op(left, t1);
+  if (row >= 3) left = op(left, t2);
+  return op(left, v);
+}
+// The value of the lane before (lane 0: the identity).
+template <typename T>
+DEVI T wave_shift_up(T v, T identity) { return dpp_move<DPP_WAVE_SHR1>(identity, v); }
+
 template <typename T>
 DEVI T wave_sum(T v) { return wave_reduce(v, [](T a, T b) { return a + b; }); }
 DEVI float wave_max(float v) { return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); }); }

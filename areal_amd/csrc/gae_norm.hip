@@ -1518,31 +1518,33 @@ struct TurnCarry { int count; int maxid; double sum; };
 // included. smem: [TURN_THREADS] of each.
 DEVI TurnCarry turn_block_exclusive(int cnt, int mx, double sm, const TurnCarry& carry, int* s_cnt,
                                     int* s_max, double* s_sum, TurnCarry& chunk_total) {
-  const int tid = threadIdx.x;
+  // s_cnt / s_max / s_sum: one entry per wave. Scans inside a wave through DPP, the waves' totals
+  // through LDS: two barriers.
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int ic = wave_inclusive_scan(cnt, 0, [](int a, int b) { return a + b; });
+  const int im = wave_inclusive_scan(mx, -1, [](int a, int b) { return a > b ? a : b; });
+  const double is = wave_inclusive_scan(sm, 0.0, [](double a, double b) { return a + b; });
+  __syncthreads();  // the previous chunk's readers are done
+  if (lane == 63) { s_cnt[w] = ic; s_max[w] = im; s_sum[w] = is; }
   __syncthreads();
-  s_cnt[tid] = cnt; s_max[tid] = mx; s_sum[tid] = sm;
-  __syncthreads();
-  // Hillis-Steele inclusive scan (256 threads, 8 steps)
-  for (int d = 1; d < TURN_THREADS; d <<= 1) {
-    int c = 0, m = -1; double v = 0.0;
-    if (tid >= d) { c = s_cnt[tid - d]; m = s_max[tid - d]; v = s_sum[tid - d]; }
-    __syncthreads();
-    if (tid >= d) {
-      s_cnt[tid] += c;
-      s_max[tid] = s_max[tid] > m ? s_max[tid] : m;
-      s_sum[tid] += v;
-    }
-    __syncthreads();
-  }
   TurnCarry ex = carry;
-  if (tid > 0) {
-    ex.count += s_cnt[tid - 1];
-    ex.maxid = ex.maxid > s_max[tid - 1] ? ex.maxid : s_max[tid - 1];
-    ex.sum += s_sum[tid - 1];
+  for (int i = 0; i < w; ++i) {
+    ex.count += s_cnt[i];
+    ex.maxid = ex.maxid > s_max[i] ? ex.maxid : s_max[i];
+    ex.sum += s_sum[i];
   }
-  chunk_total.count = carry.count + s_cnt[TURN_THREADS - 1];
-  chunk_total.maxid = carry.maxid > s_max[TURN_THREADS - 1] ? carry.maxid : s_max[TURN_THREADS - 1];
-  chunk_total.sum = carry.sum + s_sum[TURN_THREADS - 1];
+  chunk_total = carry;
+  for (int i = 0; i < TURN_THREADS / 64; ++i) {
+    chunk_total.count += s_cnt[i];
+    chunk_total.maxid = chunk_total.maxid > s_max[i] ? chunk_total.maxid : s_max[i];
+    chunk_total.sum += s_sum[i];
+  }
+  // the lanes before this one in its wave
+  const int pc = wave_shift_up(ic, 0), pm = wave_shift_up(im, -1);
+  const double ps = wave_shift_up(is, 0.0);
+  ex.count += pc;
+  ex.maxid = ex.maxid > pm ? ex.maxid : pm;
+  ex.sum += ps;
   return ex;
 }
 
