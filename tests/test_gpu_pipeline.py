@@ -175,7 +175,8 @@ def _lognormal_lengths(n, mu, sigma, lo, hi, g):
 
 def test_config3_gae_and_group_norm_full_size(dev):
     """1024 sequences, lognormal(7, 1) lengths in [16, 8192] (~1.6 M tokens), gamma 1, lambda 0.95,
-    then group-of-16 normalisation: oracle on the first 48 sequences, properties on all."""
+    then group-of-16 normalisation: the packed oracle on the first 48 sequences, the padded oracle and
+    properties on all."""
     g = torch.Generator().manual_seed(2)
     lens = _lognormal_lengths(1024, 7.0, 1.0, 16, 8192, g)
     cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
@@ -209,6 +210,14 @@ def test_config3_gae_and_group_norm_full_size(dev):
     idx = (torch.arange(1024).repeat_interleave(lens), pos)
     padded_adv[idx] = a
     padded_mask[idx] = mask
+    # every sequence against the oracle's padded recurrence (vectorised over the rows; the mask is 0 on
+    # each sequence's last token and on the padding, where the packed and the padded form agree)
+    padded_r = torch.zeros(1024, L_pad)
+    padded_v = torch.zeros(1024, L_pad)
+    padded_r[idx] = rewards
+    padded_v[idx] = values
+    want_pa, _ = G.gae_padded(padded_r, padded_v, padded_mask, torch.zeros(1024), 1.0, 0.95)
+    torch.testing.assert_close(a, want_pa[idx], rtol=1e-4, atol=1e-5 * scale)
     out = norm(padded_adv.to(dev), padded_mask.to(dev)).cpu()
     want = N.normalization(padded_adv[:32], padded_mask[:32], mean_level="group", std_level="group", group_size=16)
     torch.testing.assert_close(out[:32], want, rtol=1e-4, atol=1e-5)
@@ -216,6 +225,17 @@ def test_config3_gae_and_group_norm_full_size(dev):
         vals = out[gi * 16:(gi + 1) * 16][padded_mask[gi * 16:(gi + 1) * 16].bool()].double()
         assert abs(vals.mean().item()) < 1e-4 and abs(vals.std().item() - 1.0) < 1e-3
     assert (out[padded_mask == 0] == 0).all()
+    # the two-launch packed route (the GAE kernel leaves the normalisation's sums) on the whole batch,
+    # against the oracle's normalisation of all 64 groups
+    from areal_amd.ppo.gae import compute_gae_packed_normalized
+
+    normed, ret2, raw2 = compute_gae_packed_normalized(rewards.to(dev), values.to(dev), mask.to(dev), cu.to(dev), None,
+                                                       1.0, 0.95, norm)
+    torch.testing.assert_close(raw2.cpu(), a, rtol=0, atol=0)
+    torch.testing.assert_close(ret2.cpu(), ret.cpu(), rtol=0, atol=0)
+    want_all = N.normalization(padded_adv, padded_mask, mean_level="group", std_level="group", group_size=16)
+    torch.testing.assert_close(normed.cpu(), want_all[idx], rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(normed.cpu(), out[idx], rtol=1e-5, atol=1e-6)
 
 
 def test_config4_full_size_masks_bit_exact(dev):
@@ -364,7 +384,8 @@ def test_config4_full_size_forward_backward(dev, save_probs):
 
 
 def test_config2_full_size_decoupled_ppo(dev):
-    """T=16384, H=1536, 64 sequences; proximal and behaviour log-probs drawn independently."""
+    """T=16384, H=1536, 64 packed sequences of lognormal lengths (their packed GAE gives the advantages);
+    proximal and behaviour log-probs drawn independently."""
     T, H, V = 16384, 1536, 151936
     g, hidden, weight, labels = _make_lm_inputs(T, H, V, 1, dev)
     h, w = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
@@ -372,8 +393,24 @@ def test_config2_full_size_decoupled_ppo(dev):
     lp = out.logprobs.detach()
     prox = lp + 0.1 * torch.randn(T, generator=g).to(dev)
     old = lp + 0.1 * torch.randn(T, generator=g).to(dev)
-    adv = torch.randn(T, generator=g).to(dev)
     mask = (torch.rand(T, generator=g) > 0.2).to(dev)
+    # the batch's packing: 64 sequences of lognormal lengths filling the 16384 tokens; the advantages
+    # come from packed GAE over them, checked against the oracle's padded recurrence
+    lens = _lognormal_lengths(64, 5.4, 0.6, 16, 2048, g)
+    lens = torch.clamp((lens.double() * (T / lens.sum().item())).floor().long(), min=2)
+    lens[-1] += T - int(lens.sum())
+    assert int(lens.sum()) == T and int(lens.min()) >= 2
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    pos = torch.arange(T) - cu[:-1].long().repeat_interleave(lens)
+    gae_mask = (mask.cpu() & (pos < lens.repeat_interleave(lens) - 1)).float()
+    values = torch.randn(T, generator=g)
+    rewards = torch.zeros(T)
+    rewards[cu[1:].long() - 2] = torch.randn(64, generator=g)
+    adv, _ = compute_gae_packed(rewards.to(dev), values.to(dev), gae_mask.to(dev), cu.to(dev), None, 1.0, 0.95)
+    idx = (torch.arange(64).repeat_interleave(lens), pos)
+    pad = lambda x: torch.zeros(64, int(lens.max())).index_put_(idx, x)
+    want_adv, _ = G.gae_padded(pad(rewards), pad(values), pad(gae_mask), torch.zeros(64), 1.0, 0.95)
+    torch.testing.assert_close(adv.cpu(), want_adv[idx], rtol=1e-4, atol=1e-5 * want_adv.abs().max().item())
     rs = dict(level="token", action="clamp", metric="ratio", upper=5.0, lower=0.0)
     cfg = RejectionSamplingConfig(level="token", action="clamp", metric="ratio", upper=5.0)  # lower -> 0.0
     loss, stat = ppo_actor_loss_fn(out.logprobs, prox, old, adv, 0.2, mask, eps_clip_higher=0.28, c_clip=3.0,
