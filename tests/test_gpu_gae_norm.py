@@ -485,9 +485,11 @@ def test_packed_gae_then_normalisation_matches_oracle(dev, cfg, layout, float_ma
     group_sizes = spec.get("group_sizes")
     full = dict(cfg, group_size=spec.get("group_size", 1))
     norm = Normalization(NormConfig(**full))
-    got, ret, raw = compute_gae_packed_normalized(r.to(dev), v.to(dev), m.to(dev), cu.to(dev), ne.to(dev), 0.99, 0.9,
-                                                  norm, group_sizes=group_sizes)
-    want_a, want_r = G.gae_packed(r, v, m, cu, ne, 0.99, 0.9)
+    # a lambda per sequence on the float-mask runs, one scalar otherwise
+    lam = (0.5 + 0.5 * torch.rand(lens.numel(), generator=g)) if float_mask else 0.9
+    got, ret, raw = compute_gae_packed_normalized(r.to(dev), v.to(dev), m.to(dev), cu.to(dev), ne.to(dev), 0.99,
+                                                  lam.to(dev) if float_mask else lam, norm, group_sizes=group_sizes)
+    want_a, want_r = G.gae_packed(r, v, m, cu, ne, 0.99, lam)
     scale = want_a.abs().max().item()
     torch.testing.assert_close(raw.cpu(), want_a, rtol=1e-4, atol=1e-5 * scale)
     torch.testing.assert_close(ret.cpu(), want_r, rtol=1e-4, atol=1e-5 * scale)
