@@ -893,8 +893,8 @@ __global__ void cast_f32_to_bf16_kernel(const float* __restrict__ src, u16* __re
 // =======================================================================================
 // The contraction with the hand-scheduled main loop (mainloop16.inc, written by
 // gen_mainloop16.py): v_mfma_f32_16x16x32_bf16, accumulators in a[0:255], k-loop as one assembly
-// block per output tile. Same tile (256 x 256 x 64, four waves of 128 x 128), same operand
-// layouts as the three kernels above (nt / tn / mix), for K % 128 == 0.
+// block per output tile: a 256 x 256 x 64 tile, four waves of 128 x 128, three operand layouts
+// (nt / tn / mix), any K that is a multiple of 64 and at least 128.
 //
 // Accumulator layout of a wave: block (ia, jb) of 16 x 16, register r of a lane:
 //   i = ia*16 + 4*(lane/16) + r     (A row inside the wave's 128)
@@ -982,9 +982,10 @@ DEVI void setup_operand16(int64_t ld, int first, int nvalid, int W, int oper, in
 }
 
 // A workgroup sweeps the A tiles [ai_begin, ai_end) against one B tile. Requirements checked by
-// the host: K % 128 == 0; a sweep of more than one A tile has only full A tiles (a ragged last one
-// as rows [M - 256, M), see GemmArgs::overlap_last_a) and a k-contiguous A (the loader's lane
-// offsets are those of the first tile); split-K ranges are an even number of k-tiles.
+// the host: K % 64 == 0 and K >= 128; a sweep of more than one A tile has only full A tiles (a
+// ragged last one as rows [M - 256, M), see GemmArgs::overlap_last_a) and a k-contiguous A (the
+// loader's lane offsets are those of the first tile); every copy of a split-K launch has at least
+// two k-tiles (an even number in all but the last, see split_ktiles).
 // Epi::tile gets the first row of the tile's sub-block of this wave and, last, the first row of the
 // tile that no earlier tile of the sweep covered.
 template <int VAR, class Epi>
@@ -2107,8 +2108,8 @@ size_t areal_lmhead_bwd_saved_workspace_bytes(int64_t T, int64_t H, int64_t V) {
 // read back as 0): no logits are recomputed and no pass rewrites the [T, V] buffer. Per row,
 // dlogits = f[t] * e' with a row factor f; dHidden scales its output rows by f and dWeight
 // contracts e' with f[t] * hidden[t]. Only the label's entry of each row of probs is rewritten
-// (and rows [T, round_up(T, 128)) are cleared: the token range of dWeight's contraction is whole
-// pairs of k-tiles, which the hand-scheduled main loop walks), so probs can be used once. logprobs (nullable)
+// (and rows [T, round_up(T, 128)) are cleared: dWeight contracts over that padded token range, so
+// that any T takes the hand-scheduled main loop), so probs can be used once. logprobs (nullable)
 // are the label log-probabilities of the forward; with them the label's entry is evaluated in
 // fp32. dweight [V,H]: dweight_mode 0 = fp32 store, 1 = fp32 accumulate, 2 = bf16 store (the
 // whole batch is one contraction, so no fp32 staging is needed). probs_status (nullable): the
