@@ -12,29 +12,6 @@ namespace {
 
 constexpr int PK_THREADS = 256;
 
-DEVI int seq_of_cu(const int32_t* cu, int n_seqs, int64_t t) {
-  int lo = 0, hi = n_seqs;  // last s with cu[s] <= t
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if ((int64_t)cu[mid] <= t) lo = mid; else hi = mid;
-  }
-  return lo;
-}
-
-// Copies `eb` bytes (one token's trailing dimensions) with the widest aligned access.
-DEVI void copy_elem(char* dst, const char* src, int64_t eb) {
-  if (((eb | (uintptr_t)dst | (uintptr_t)src) & 15) == 0) {
-    for (int64_t i = 0; i < eb; i += 16) *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
-  } else if (((eb | (uintptr_t)dst | (uintptr_t)src) & 3) == 0) {
-    for (int64_t i = 0; i < eb; i += 4) *(uint32_t*)(dst + i) = *(const uint32_t*)(src + i);
-  } else {
-    for (int64_t i = 0; i < eb; ++i) dst[i] = src[i];
-  }
-}
-DEVI void fill_elem(char* dst, const char* pattern, int pb, int64_t eb) {
-  for (int64_t i = 0; i < eb; ++i) dst[i] = pattern[i % pb];
-}
-
 // 16 bytes at any address. The compiler picks the access the target allows for the alignment
 // (gfx950 runs with unaligned access enabled, where this is still one 16-byte instruction).
 struct __attribute__((packed, aligned(1))) Bytes16 { uint32_t w[4]; };
@@ -176,45 +153,87 @@ __global__ __launch_bounds__(PK_THREADS) void pack_rows_kernel(PackArgs a) {
   }
 }
 
-// padded[b][j] = j < len_b ? packed[cu[b] + j] : fill
 struct Fill { char bytes[16]; int n; };
+
+// n bytes at dst (the start of an element) filled with the pattern by the whole block: 16-byte
+// stores of the repeated pattern when its length divides 16, byte by byte otherwise and at the end.
+DEVI void block_fill_bytes(char* dst, int64_t n, const Fill& f) {
+  int64_t done = 0;
+  if ((16 % f.n) == 0) {
+    Bytes16 pat;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t x = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x |= (uint32_t)(uint8_t)f.bytes[(4 * w + k) % f.n] << (8 * k);
+      pat.w[w] = x;
+    }
+    const int64_t n16 = n >> 4;
+    for (int64_t i = threadIdx.x; i < n16; i += blockDim.x) *(Bytes16*)(dst + 16 * i) = pat;
+    done = 16 * n16;
+  }
+  for (int64_t i = done + threadIdx.x; i < n; i += blockDim.x) dst[i] = f.bytes[i % f.n];
+}
+
+// Tokens per block of the row-wise kernels below: 16 KiB of an element, at most 2048 tokens.
+static int64_t pk_chunk_tokens(int64_t eb) {
+  const int64_t c = PK_CHUNK_BYTES / eb;
+  return c < 1 ? 1 : (c > PK_CHUNK_MAX ? PK_CHUNK_MAX : c);
+}
+
+// padded[row][j] = j < len_b ? packed[cu[b] + j] : fill, b = row_seq[row] (or row). Block
+// (row, c) writes tokens [c * chunk, (c + 1) * chunk) of its row: one contiguous copy, one fill.
 __global__ __launch_bounds__(PK_THREADS) void unpack_kernel(const char* packed, char* padded,
                                                             const int32_t* cu, const int32_t* row_seq,
-                                                            int64_t B, int64_t S, int64_t eb,
-                                                            Fill fill) {
-  const int64_t total = B * S;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t row = i / S, j = i - row * S;
-    const int64_t b = row_seq ? row_seq[row] : row;  // packed sequence shown in this row
-    const int64_t len = (int64_t)cu[b + 1] - cu[b];
-    if (j < len) copy_elem(padded + i * eb, packed + ((int64_t)cu[b] + j) * eb, eb);
-    else fill_elem(padded + i * eb, fill.bytes, fill.n, eb);
-  }
+                                                            int64_t S, int64_t eb, Fill fill, int chunks,
+                                                            int chunk) {
+  const int64_t row = blockIdx.x / chunks;
+  const int64_t j0 = (int64_t)(blockIdx.x % chunks) * chunk;
+  const int64_t nj = S - j0 < chunk ? S - j0 : chunk;
+  const int64_t b = row_seq ? row_seq[row] : row;  // packed sequence shown in this row
+  const int64_t start = cu[b], len = (int64_t)cu[b + 1] - start;
+  int64_t ncopy = len - j0;
+  ncopy = ncopy < 0 ? 0 : (ncopy > nj ? nj : ncopy);
+  char* d = padded + (row * S + j0) * eb;
+  if (ncopy > 0) block_copy_bytes(d, packed + (start + j0) * eb, ncopy * eb);
+  if (ncopy < nj) block_fill_bytes(d + ncopy * eb, (nj - ncopy) * eb, fill);
 }
 
 // dst[cu_new[s] + j] = j < old length of s ? src[cu_old[s] + j] : fill; sequences of cu_new
 // beyond n_old (a trailing pad segment) are all fill. arange != 0: dst is int64 position ids,
-// and the fill is j (position inside the new sequence) instead.
+// and the fill is j (position inside the new sequence, src == NULL) or j - old length instead.
+// Block c writes tokens [c * chunk, (c + 1) * chunk) of dst, sequence by sequence as pack_rows_kernel.
 __global__ __launch_bounds__(PK_THREADS) void realign_kernel(const char* src, char* dst,
                                                              const int32_t* cu_old, int n_old,
                                                              const int32_t* cu_new, int n_new,
                                                              int64_t eb, Fill fill, int arange,
-                                                             int64_t total_new) {
-  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total_new;
-       t += (int64_t)gridDim.x * blockDim.x) {
-    const int s = seq_of_cu(cu_new, n_new, t);
-    const int64_t j = t - cu_new[s];
-    const int64_t len = s < n_old ? (int64_t)cu_old[s + 1] - cu_old[s] : 0;
-    char* d = dst + t * eb;
-    if (j < len && src != nullptr) {
-      copy_elem(d, src + ((int64_t)cu_old[s] + j) * eb, eb);
-    } else if (arange) {
-      const int64_t v = (src == nullptr) ? j : j - len;  // whole-sequence arange, or pad arange
-      for (int64_t k = 0; k < eb; k += 8) *(int64_t*)(d + k) = v;
-    } else {
-      fill_elem(d, fill.bytes, fill.n, eb);
+                                                             int64_t total_new, int chunk) {
+  int64_t t = (int64_t)blockIdx.x * chunk;
+  const int64_t t1 = t + chunk < total_new ? t + chunk : total_new;
+  int s = wave_count_le(cu_new + 1, n_new, t, threadIdx.x & 63);
+  while (t < t1 && s < n_new) {
+    const int64_t start = cu_new[s], end = cu_new[s + 1];
+    const int64_t stop = end < t1 ? end : t1;
+    if (stop > t) {
+      const int64_t j0 = t - start, j1 = stop - start;  // positions inside the new sequence
+      const int64_t len = (s < n_old && src != nullptr) ? (int64_t)cu_old[s + 1] - cu_old[s] : 0;
+      const int64_t jc = j1 < len ? j1 : len;            // copied positions are [j0, jc)
+      if (jc > j0) block_copy_bytes(dst + t * eb, src + ((int64_t)cu_old[s] + j0) * eb, (jc - j0) * eb);
+      const int64_t jf = j0 > len ? j0 : len;            // filled positions are [jf, j1)
+      if (jf < j1) {
+        char* d = dst + (start + jf) * eb;
+        if (arange) {
+          const int64_t shift = src == nullptr ? 0 : (s < n_old ? (int64_t)cu_old[s + 1] - cu_old[s] : 0);
+          const int64_t per = eb >> 3;  // int64 channels per token
+          for (int64_t i = threadIdx.x; i < (j1 - jf) * per; i += blockDim.x)
+            ((int64_t*)d)[i] = jf + i / per - shift;
+        } else {
+          block_fill_bytes(d, (j1 - jf) * eb, fill);
+        }
+      }
+      t = stop;
     }
+    ++s;
   }
 }
 
@@ -295,12 +314,6 @@ __global__ __launch_bounds__(PK_THREADS) void stats_final_kernel(const StatPart*
   }
 }
 
-int pk_grid(int64_t n) {
-  int64_t b = ceil_div_i64(n, PK_THREADS);
-  if (b > 65535) b = 65535;
-  if (b < 1) b = 1;
-  return (int)b;
-}
 bool make_fill(const void* fill, int fill_bytes, Fill& f) {
   if (fill_bytes < 0 || fill_bytes > 16) return false;
   f.n = fill_bytes > 0 ? fill_bytes : 1;
@@ -349,8 +362,7 @@ int areal_pack_padded_multi(const void* const* padded, void* const* packed, cons
   }
   int64_t max_eb = 1;
   for (int k = 0; k < n_tensors; ++k) max_eb = elem_bytes[k] > max_eb ? elem_bytes[k] : max_eb;
-  int64_t chunk = PK_CHUNK_BYTES / max_eb;
-  chunk = chunk < 1 ? 1 : (chunk > PK_CHUNK_MAX ? PK_CHUNK_MAX : chunk);
+  const int64_t chunk = pk_chunk_tokens(max_eb);
   const int64_t chunks = ceil_div_i64(total, chunk);
   if (chunks >= ((int64_t)1 << 31) || B > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
   a.cu = cu_seqlens; a.n_seqs = (int)B; a.S = S; a.total = total; a.chunk = (int)chunk;
@@ -378,8 +390,11 @@ int areal_unpack_to_padded(const void* packed, void* padded, const int32_t* cu_s
   if (!padded || !cu_seqlens) return AREAL_ERR_BAD_ARG;
   Fill f;
   if (!make_fill(fill, fill_bytes, f)) return AREAL_ERR_BAD_ARG;
-  hipLaunchKernelGGL(unpack_kernel, dim3(pk_grid(B * S)), dim3(PK_THREADS), 0, stream,
-                     (const char*)packed, (char*)padded, cu_seqlens, row_seq, B, S, elem_bytes, f);
+  const int64_t chunk = pk_chunk_tokens(elem_bytes), chunks = ceil_div_i64(S, chunk);
+  if (chunks * B >= ((int64_t)1 << 31)) return AREAL_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)(chunks * B)), dim3(PK_THREADS), 0, stream,
+                     (const char*)packed, (char*)padded, cu_seqlens, row_seq, S, elem_bytes, f, (int)chunks,
+                     (int)chunk);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }
@@ -400,9 +415,11 @@ int areal_realign_packed(const void* src, void* dst, const int32_t* cu_old, int6
   if (!position_ids && src == nullptr && n_old > 0) return AREAL_ERR_BAD_ARG;
   Fill f;
   if (!make_fill(fill, fill_bytes, f)) return AREAL_ERR_BAD_ARG;
-  hipLaunchKernelGGL(realign_kernel, dim3(pk_grid(total_new)), dim3(PK_THREADS), 0, stream,
+  const int64_t chunk = pk_chunk_tokens(elem_bytes), chunks = ceil_div_i64(total_new, chunk);
+  if (chunks >= ((int64_t)1 << 31) || n_new > (1 << 30)) return AREAL_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(realign_kernel, dim3((unsigned)chunks), dim3(PK_THREADS), 0, stream,
                      (const char*)src, (char*)dst, cu_old, (int)n_old, cu_new, (int)n_new,
-                     elem_bytes, f, position_ids, total_new);
+                     elem_bytes, f, position_ids, total_new, (int)chunk);
   AREAL_CHECK_LAUNCH();
   return AREAL_OK;
 }

@@ -496,6 +496,20 @@ def hbm_rooflines(dev):
     add("rowlens + cu_scan + pack_rows (C ABI)",
         f"[1024, 8192] padded -> {n_packed} packed tokens, 5 tensors (8+8+1+4+4 B), read + write, and the "
         "attention mask read once", 2 * 25 * n_packed + bsz * Lp, timed(pack_kernels, iters=50))
+    # back to the padded layout: five launches of the row-wise unpack kernel (pad value 0)
+    pk_back = [torch.empty_like(t) for t in pk_src]
+
+    def unpack_kernels():
+        rc = 0
+        for s_, d_ in zip(pk_dst, pk_back):
+            rc |= lib.areal_unpack_to_padded(p(s_), p(d_), p(pk_cu), None, bsz, Lp, s_.element_size(), None, 0, strm2)
+        assert rc == 0
+
+    pack_kernels()
+    add("unpack_kernel x5 (C ABI)",
+        f"{n_packed} packed tokens -> [1024, 8192] padded, 5 tensors (8+8+1+4+4 B): packed read, every padded slot "
+        "written", 25 * n_packed + 25 * bsz * Lp, timed(unpack_kernels, iters=50))
+    del pk_back
     turn_ids = (torch.cumsum((torch.rand(bsz, Lp, device=dev) < 0.002).int(), dim=1)).to(torch.int32)
     tr = torch.zeros(bsz, Lp, device=dev)
     tr[torch.arange(bsz, device=dev), (plens - 2).clamp(min=0)] = 1.0
