@@ -443,7 +443,10 @@ def _pad_packed(x, cu, fill=0.0):
     return out, (rows, pos)
 
 
+_MANY = torch.Generator().manual_seed(99)
 PACKED_NORM_LAYOUTS = {
+    # more sequences than the kernel keeps of cu_seqlens in LDS, six or seven groups per 2048-token tile
+    "many": dict(lens=torch.randint(1, 40, (5000,), generator=_MANY).tolist(), group_size=16),
     # sequences per tile of 2048 tokens: several groups inside one tile
     "short": dict(lens=[300, 17, 450, 1, 612, 95, 800, 333, 64, 2, 700, 410, 129, 256, 31, 999], group_size=2),
     # groups that cross tile boundaries, one sequence of several tiles, an empty sequence
