@@ -113,9 +113,9 @@ class Variant:
                 f"s_cselect_b32 s{S_EFF_B}, s{S_PEN_B}, s{S_STRIDE_B}"]
 
     # ---------------------------------------------------------------- schedule
-    def a_reads(self, buf, stage, ks):
+    def a_reads(self, buf, stage, ks, na=8):
         out = []
-        for x in range(8):
+        for x in range(na):
             out += self.reads(self.fa[buf] + 4 * x, stage, ks, 0, x)
         return out
 
@@ -126,12 +126,13 @@ class Variant:
                 out += self.reads(self.fb[parity][ks] + 4 * x, stage, ks, 1, x)
         return out
 
-    def kstep(self, abuf, bbuf, init, pre, post, dead=False):
-        """64 MFMAs; pre[m] / post[m] are emitted in front of / behind MFMA m. dead: no MFMA."""
+    def kstep(self, abuf, bbuf, init, pre, post, dead=False, na=8):
+        """64 MFMA slots; pre[m] / post[m] are emitted in front of / behind slot m. dead: no MFMA;
+        na < 8: the slots of the A blocks ia >= na stay empty (a narrower A tile)."""
         out = []
         for m in range(64):
             out += pre.get(m, [])
-            if not dead:
+            if not dead and (m >> 3) < na:
                 out.append(self.mfma(abuf, bbuf, m >> 3, m & 7, init))
             out += post.get(m, [])
         return out
@@ -161,7 +162,7 @@ class Variant:
         # the first k-tile of a pair (stage 0) advances by the selected amount
         post.setdefault(7 * step + 1, []).extend(self.advance(oper, eff=(stage == 0)))
 
-    def ktile(self, parity, init, dead=False):
+    def ktile(self, parity, init, dead=False, na=8):
         stage = parity
         barrier = ["s_barrier"]
         out = [f"; ---- k-tile on stage {stage}{' (dead: no MFMA)' if dead else ''}: k-step 0"]
@@ -169,8 +170,8 @@ class Variant:
         # it with the k-tile after next; A fragments of k-step 1 -> A buffer 1
         pre, post = {}, {}
         self.put_loads(stage, 1, pre, post)
-        self.spread(self.a_reads(1, stage, 1), 9, 40, post)
-        out += self.kstep(self.fa[0], self.fb[parity][0], init, pre, post, dead)
+        self.spread(self.a_reads(1, stage, 1, na), 9, 40, post)
+        out += self.kstep(self.fa[0], self.fb[parity][0], init, pre, post, dead, na)
         # own A reads done and own loads of one k-tile ago landed (the 8 newest may be in flight)
         out += ["s_waitcnt vmcnt(8) lgkmcnt(0)"] + barrier
         out += [f"; ---- k-tile on stage {stage}: k-step 1"]
@@ -179,23 +180,27 @@ class Variant:
         # of the next k-tile -> the other pair of B buffers
         pre, post = {}, {}
         self.put_loads(stage, 0, pre, post)
-        self.spread(self.a_reads(0, stage ^ 1, 0) + self.b_reads(parity ^ 1, stage ^ 1), 9, 52, post)
-        out += self.kstep(self.fa[1], self.fb[parity][1], False, pre, post, dead)
+        # the last fragment read sits 11 MFMAs in front of the k-step's end, whatever its length
+        self.spread(self.a_reads(0, stage ^ 1, 0, na) + self.b_reads(parity ^ 1, stage ^ 1), 9, 8 * na - 12, post)
+        out += self.kstep(self.fa[1], self.fb[parity][1], False, pre, post, dead, na)
         # every wave has the next k-tile's B fragments: the other stage's B half may be refilled
         out += ["s_waitcnt lgkmcnt(0)"] + barrier
         return out
 
-    def pair(self, init, dead_second=False):
-        return self.select_advance() + self.ktile(0, init) + self.ktile(1, False, dead_second)
+    def pair(self, init, dead_second=False, na=8):
+        return self.select_advance() + self.ktile(0, init, False, na) + self.ktile(1, False, dead_second, na)
 
-    def tile_loop(self):
+    def tile_loop(self, na=8):
         """One 256 x 256 tile: s48 pairs of k-tiles, the second k-tile of the last pair dead when
         s52 is 1 (an odd number of k-tiles; then at least two pairs). On entry both stages hold (or
-        are receiving) k-tiles 0 and 1 and the pointers are on the next k-tile to fetch."""
+        are receiving) k-tiles 0 and 1 and the pointers are on the next k-tile to fetch.
+        na < 8: a tile of 32 na x 256, each wave's sub-tile 16 na x 128: the loads, barriers and B
+        fragment reads are those of the full tile; the fragment reads and MFMAs of the A blocks
+        ia >= na are left out."""
         out = ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_barrier"]
-        out += self.a_reads(0, 0, 0) + self.b_reads(0, 0)
+        out += self.a_reads(0, 0, 0, na) + self.b_reads(0, 0)
         out += ["s_waitcnt lgkmcnt(0)", "s_barrier"]
-        out += self.pair(True)
+        out += self.pair(True, False, na)
         out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_eq_u32 s{S_CNT}, 0", "s_cbranch_scc1 2f", "1:",
                 # the last pair fetches the next tile's first k-tiles
                 f"s_cmp_eq_u32 s{S_CNT}, 1",
@@ -203,10 +208,10 @@ class Variant:
                 f"s_cselect_b64 s[{S_PB}:{S_PB + 1}], s[{S_PB_NEXT}:{S_PB_NEXT + 1}], s[{S_PB}:{S_PB + 1}]",
                 # ... and is the one with the dead k-tile if the count is odd (s52 = 1; 0 never matches)
                 f"s_cmp_eq_u32 s{S_CNT}, s{S_ODD}", "s_cbranch_scc1 3f"]
-        out += self.pair(False)
+        out += self.pair(False, False, na)
         out += [f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1", f"s_cmp_lg_u32 s{S_CNT}, 0", "s_cbranch_scc1 1b",
                 "s_branch 2f", "3:"]
-        out += self.pair(False, dead_second=True)
+        out += self.pair(False, True, na)
         out += ["2:", "s_nop 15", "s_nop 15"]  # the last MFMAs retire before the accumulators are read
         return out
 
@@ -266,6 +271,8 @@ def emit():
         out.append(f"#define ML16_{n}_CLOBBERS " + ", ".join(f'"{c}"' for c in v.clobbers()))
         out.append(f"#define ML16_{n}_PROLOGUE \\\n" + cstring(v.prologue()))
         out.append(f"#define ML16_{n}_TILE \\\n" + cstring(v.tile_loop()))
+        if v.km[0]:  # narrower A tiles exist for a k-major A (its tile column is a lane offset)
+            out.append(f"#define ML16_{n}_TILE7 \\\n" + cstring(v.tile_loop(7)))
         out.append("")
     return "\n".join(out) + "\n"
 

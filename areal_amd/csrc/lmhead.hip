@@ -944,11 +944,13 @@ enum { VAR_NT = 0, VAR_TN = 1, VAR_MIX = 2 };
 DEVI int swz16(int r) { return r & 7; }
 
 // Per-lane byte offsets of the 8 direct loads of one operand half, and the LDS read addresses
-// (stage 0) of its fragments. KM: k-major operand (`first` = its 256-column tile, nvalid = readable
-// columns); otherwise k-contiguous (`first` = the tile's first row, nvalid = rows).
+// (stage 0) of its fragments. KM: k-major operand (`first` = its tile of 32 nblk columns, nvalid =
+// readable columns; the loads fetch 256 columns from the tile's first one whatever nblk is, and
+// wave row / column W reads the nblk blocks of 16 columns from block W * nblk on); otherwise
+// k-contiguous (`first` = the tile's first row, nvalid = rows; nblk = 8).
 template <bool KM>
 DEVI void setup_operand16(int64_t ld, int first, int nvalid, int W, int oper, int wave, int lane,
-                          uint32_t lds_base, uint32_t (&off)[8], uint32_t (&rd)[8]) {
+                          uint32_t lds_base, uint32_t (&off)[8], uint32_t (&rd)[8], int nblk = 8) {
   if (!KM) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -968,16 +970,18 @@ DEVI void setup_operand16(int64_t ld, int first, int nvalid, int W, int oper, in
     for (int i = 0; i < 8; ++i) {
       const int kr = wave * 16 + 2 * i + hl;
       const int k3 = kr & 3, cf = ((kr >> 3) & 1) * 2;
-      int gp = first * (TILE / 8) + (((piece >> 2) ^ k3) << 2) + ((piece & 3) ^ cf);
+      int gp = first * (nblk * 4) + (((piece >> 2) ^ k3) << 2) + ((piece & 3) ^ cf);
       const int last = nvalid / 8 - 1;
       gp = gp < last ? gp : last;  // columns past the end are discarded later
       off[i] = 2u * ((uint32_t)kr * (uint32_t)ld + (uint32_t)(gp * 8));
     }
     const int G = lane >> 4, q = lane & 15, r4 = q >> 2;
 #pragma unroll
-    for (int x = 0; x < 8; ++x)
-      rd[x] = lds_base + oper * ML16_OPER_BYTES + (G * 8 + r4) * 512 + (((W * 4 + (x >> 1)) ^ r4) << 6) +
-              ((((x & 1) ^ G) & 1) << 5) + (q & 3) * 8;
+    for (int x = 0; x < 8; ++x) {
+      const int y = W * nblk + x;  // block of 16 columns inside the 256 loaded ones
+      rd[x] = lds_base + oper * ML16_OPER_BYTES + (G * 8 + r4) * 512 + ((((y >> 1) & 7) ^ r4) << 6) +
+              ((((y & 1) ^ G) & 1) << 5) + (q & 3) * 8;
+    }
   }
 }
 
@@ -988,10 +992,16 @@ DEVI void setup_operand16(int64_t ld, int first, int nvalid, int W, int oper, in
 // two k-tiles (an even number in all but the last, see split_ktiles).
 // Epi::tile gets the first row of the tile's sub-block of this wave and, last, the first row of the
 // tile that no earlier tile of the sweep covered.
+// NA < 8 (k-major A only): A tiles of 32 NA columns, each wave row taking NA blocks of 16; the MFMAs
+// of the missing blocks are not issued (a tile costs NA / 8 of a full one), so an M that fills its
+// last 256-wide tile badly (896 = 3.5 x 256 = 4 x 224) wastes nothing. NA is the epilogue's (Epi::NA).
 template <int VAR, class Epi>
 __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, typename Epi::Params ep) {
   __shared__ __attribute__((aligned(1024))) unsigned char lds[RING16_BYTES + 4 * STAGE16_BYTES];
   constexpr bool A_KM = VAR != VAR_NT, B_KM = VAR == VAR_TN;
+  constexpr int NA = Epi::NA;
+  static_assert(NA == 8 || (NA == 7 && A_KM), "narrow A tiles need a k-major A");
+  constexpr int TM = NA * 32;  // A rows (output index i) per tile
   int bj, split, ai_begin, ai_end;
   int wg = blockIdx.x, nk = g.K / BK;
   if (g.ksplit > 1) {
@@ -1017,12 +1027,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
 
   // first row of A tile ai (k-contiguous A): the last tile of a ragged M may overlap its predecessor
   auto a_row0 = [&](int ai) -> int {
-    const int r = ai * TILE;
+    const int r = ai * TM;
     return (VAR == VAR_NT && g.overlap_last_a != 0 && r + TILE > g.M) ? g.M - TILE : r;
   };
   uint32_t oa[8], ob[8], ra[8], rb[8];
   setup_operand16<A_KM>(g.lda, A_KM ? ai_begin : a_row0(ai_begin), A_KM ? g.acols : g.M, wa, 0, wave, lane,
-                        lds_base, oa, ra);
+                        lds_base, oa, ra, NA);
   setup_operand16<B_KM>(g.ldb, B_KM ? bj : bj * TILE, B_KM ? g.bcols : g.N, wb, 1, wave, lane, lds_base, ob, rb);
 
   // pointers to the next k-tile to fetch and their advance per k-tile in bytes. A k-major
@@ -1077,6 +1087,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
                      ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
                      ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_NT_VGPR_INPUTS(oa, ob, ra, rb)
                    : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_NT_CLOBBERS, ML16_ACC_CLOBBERS);
+    else if (VAR == VAR_TN && NA == 7)
+      asm volatile(ML16_TN_TILE7
+                   : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
+                   : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
+                     ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_TN_CLOBBERS, ML16_ACC_CLOBBERS);
     else if (VAR == VAR_TN)
       asm volatile(ML16_TN_TILE
                    : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
@@ -1084,6 +1101,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
                      ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
                      ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_TN_VGPR_INPUTS(oa, ob, ra, rb)
                    : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_TN_CLOBBERS, ML16_ACC_CLOBBERS);
+    else if (NA == 7)
+      asm volatile(ML16_MIX_TILE7
+                   : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
+                   : ML16_S_PA_NEXT(pa_next), ML16_S_PB_NEXT(pb_next), ML16_S_LDSW(ldsw),
+                     ML16_S_STRIDE_A(stride_a), ML16_S_STRIDE_B(stride_b), ML16_S_ODD(odd),
+                     ML16_S_PEN_A(pen_a), ML16_S_PEN_B(pen_b), ML16_MIX_VGPR_INPUTS(oa, ob, ra, rb)
+                   : "memory", "scc", ML16_S_SCRATCH_CLOBBERS, ML16_MIX_CLOBBERS, ML16_ACC_CLOBBERS);
     else
       asm volatile(ML16_MIX_TILE
                    : "+" ML16_S_PA(pa), "+" ML16_S_PB(pb), "+" ML16_S_CNT(cnt)
@@ -1097,7 +1121,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
     Epi::open(st, ep, bj * TILE + wb * 128, split, wa, lane_e, ai == ai_begin);
-    Epi::tile(st, ep, a_row0(ai) + wa * 128, bj * TILE + wb * 128, lane_e, stage, ai * TILE);
+    Epi::tile(st, ep, a_row0(ai) + wa * (NA * 16), bj * TILE + wb * 128, lane_e, stage, ai * TM);
     Epi::close(st, ep, bj * TILE + wb * 128, split, wa, lane_e);
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // drain the trailing (unused) loads before LDS is released
@@ -1131,8 +1155,12 @@ DEVI void stage16_put(u16* stage, int lane, int ia, u32x2 v) {
 }
 
 // ---- plain store (dHidden, dWeight, stand-alone GEMM): out[j * ldo + i]
-template <bool EDGE, int MODE>
-struct Store16 {
+// NA < 8: the wave's sub-tile has only NA blocks of 16 values i (gemm16_sweep's narrow A tiles); the
+// bounds of the EDGE instance then also stop at the sub-tile's width.
+template <bool EDGE, int MODE, int NA_>
+struct Store16Impl {
+  static_assert(NA_ == 8 || EDGE, "narrow tiles use the bounds-checked instance");
+  static constexpr int NA = NA_;
   typedef StoreParams Params;
   struct State {};
   static DEVI void open(State&, const Params&, int, int, int, int, bool) {}
@@ -1151,7 +1179,7 @@ struct Store16 {
         float js = 1.f;
         if (MODE == 3) js = (!EDGE || j < p.N) ? p.jscale[j] : 0.f;
 #pragma unroll
-        for (int a = 0; a < 8; ++a) {
+        for (int a = 0; a < NA; ++a) {
           float x0 = x[a * 4], x1 = x[a * 4 + 1], x2 = x[a * 4 + 2], x3 = x[a * 4 + 3];
           if (MODE == 3) { x0 *= js; x1 *= js; x2 *= js; x3 *= js; }
           u32x2 v;
@@ -1159,11 +1187,13 @@ struct Store16 {
           v[1] = pack_bf16x2(x2, x3);
           stage16_put(stage, lane, a, v);
         }
+        int cols_valid = p.M - i0;
+        if (NA < 8) cols_valid = cols_valid < NA * 16 ? cols_valid : NA * 16;
         flush_stage16<EDGE>(stage, (u16*)p.out + (int64_t)(j0 + b * 16) * p.ldo + i0, p.ldo,
-                            p.N - (j0 + b * 16), p.M - i0, 0, lane);
+                            p.N - (j0 + b * 16), cols_valid, 0, lane);
       } else {
 #pragma unroll
-        for (int a = 0; a < 8; ++a) {
+        for (int a = 0; a < NA; ++a) {
           const int i = i0 + a * 16 + 4 * (lane >> 4);
           if (!EDGE || (j < p.N && i < p.M)) {
             f32x4* dst = (f32x4*)((float*)p.out + (int64_t)j * p.ldo + i);
@@ -1176,6 +1206,8 @@ struct Store16 {
     });
   }
 };
+template <bool EDGE, int MODE> struct Store16 : Store16Impl<EDGE, MODE, 8> {};
+template <int MODE> struct Store16Narrow : Store16Impl<true, MODE, 7> {};
 template <bool E> using Store16Bf16 = Store16<E, 0>;
 template <bool E> using Store16F32 = Store16<E, 1>;
 template <bool E> using Accum16F32 = Store16<E, 2>;
@@ -1231,6 +1263,7 @@ constexpr float MASKED_LOGIT = -1e30f;
 
 template <bool EDGE, bool AFFINE, bool MOMENTS, bool SAVE>
 struct Fwd16 {
+  static constexpr int NA = 8;
   typedef FwdParams Params;
   // SAVE: s and q are relative to the row reference of the saved exponentials (fixed for the whole
   // sweep: nothing is rescaled); otherwise relative to the running maximum m.
@@ -1436,6 +1469,7 @@ template <bool E> using Fwd16AffineMomSave = Fwd16<E, true, true, true>;
 // ---- recompute: dlogits = (onehot - p) * g * invT * scale in bf16, [Tc, ldv] (see BwdEpi)
 template <bool EDGE, bool AFFINE>
 struct Bwd16 {
+  static constexpr int NA = 8;
   typedef BwdParams Params;
   struct State {
     float nb[8], gs[8];
@@ -1634,11 +1668,28 @@ int fwd_slots(const Regions& r) { return fwd_slots_per_split(r) * (r.S + ((r.rag
 // 3 bf16 with a factor per output row. The hand-scheduled kernel writes bf16 as 16-byte pieces of
 // whole rows, which needs aligned output rows; the generic kernel (k-contiguous operands only)
 // takes what it cannot. S_fixed as plan_regions (stores want one A tile per workgroup).
+// A k-major A whose n = ceil(M / 256) tiles are filled to 7 / 8 at most (M <= 224 n, e.g. 896 =
+// 3.5 x 256): n tiles of 224 cover M too and each costs 7 / 8 of a full tile.
+bool narrow_a_tiles(int64_t M) {
+  const int64_t n = ceil_div_i64(M, TILE);
+  return M % TILE != 0 && M <= n * (TILE - 32);
+}
 template <int KERNEL16>
 int launch_store(const GemmArgs& g, const StoreParams& ep, int mode, hipStream_t stream) {
   bool allow16 = true;
   if (mode == 0 || mode == 3) allow16 = ep.ldo % 8 == 0 && aligned16(ep.out) && ep.M % 8 == 0;
   const Regions r = plan_regions(ep.M, ep.N, g.K, 0, 1 << 20, allow16);
+  if constexpr (KERNEL16 != KERNEL16_NT) {
+    // the modes the two backward contractions use: dWeight 0 - 2, dHidden 0, 1 and 3
+    constexpr int UNUSED_MODE = KERNEL16 == KERNEL16_TN ? 3 : 2;
+    if (r.k16 && mode != UNUSED_MODE && narrow_a_tiles(ep.M)) {
+      const int nai = (int)ceil_div_i64(ep.M, TILE), nbj = (int)ceil_div_i64(ep.N, TILE);
+      if (mode == 0) return launch_region<Store16Narrow<0>, KERNEL16>(g, 0, nbj, 0, nai, nai, ep, stream);
+      if (mode == 1) return launch_region<Store16Narrow<1>, KERNEL16>(g, 0, nbj, 0, nai, nai, ep, stream);
+      constexpr int LAST_MODE = KERNEL16 == KERNEL16_TN ? 2 : 3;
+      return launch_region<Store16Narrow<LAST_MODE>, KERNEL16>(g, 0, nbj, 0, nai, nai, ep, stream);
+    }
+  }
   switch (mode) {
     case 0: return launch_gemm<Store16Bf16, StoreBf16, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);
     case 1: return launch_gemm<Store16F32, StoreF32, StoreParams, KERNEL16, true>(g, r, ep, ep, stream);

@@ -83,3 +83,30 @@ def test_shapes_against_fp32_torch(dev, T, H, V, save_probs):
     assert _rel(h.grad.float(), dh) < 1e-2
     assert _rel(w.grad.float(), dw) < 1e-2
     assert (h.grad[::5] == 0).all()
+
+
+@pytest.mark.parametrize("accumulate", [False, True], ids=["bf16", "fp32_accumulate"])
+@pytest.mark.parametrize("save_probs", [True, False], ids=["saved", "recompute"])
+@pytest.mark.parametrize("H", [136, 640, 896, 1344])
+def test_hidden_sizes_tiled_224_wide_elementwise(dev, H, save_probs, accumulate):
+    """Hidden sizes that fill their 256-wide output tiles to 7/8 at most run dHidden and dWeight on
+    224-wide tiles (896 = 4 x 224; 640 = 224 + 224 + 192; 136 in one; 1344 = 6 x 224). Every
+    gradient element is compared, so a misplaced or missing block of 16 columns cannot hide in a
+    norm: |error| <= 2 % of the gradient's largest magnitude (bf16 outputs of bf16 operands)."""
+    T, V = 512, 2112
+    g = torch.Generator(device="cpu").manual_seed(H)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    weight = (torch.randn(V, H, generator=g) * (2.0 / H ** 0.5)).bfloat16().to(dev)
+    labels = torch.randint(0, V, (T,), generator=g).to(dev)
+    grad = torch.randn(T, generator=g).to(dev)
+    h = hidden.clone().requires_grad_(True)
+    w = weight.clone().requires_grad_(True)
+    main_grad = torch.full((V, H), 0.25, dtype=torch.float32, device=dev) if accumulate else None
+    out = fused_lm_head_logprobs_entropy(h, w, labels, save_probs=save_probs, weight_grad_accum=main_grad)
+    (out.logprobs * grad).sum().backward()
+    lp, _, _, _, dh, dw = _reference(hidden, weight, labels, grad, 1.0, 1.0)
+    assert (out.logprobs.detach() - lp).abs().max().item() < 2e-3
+    got_dw = main_grad - 0.25 if accumulate else w.grad.float()
+    for got, want in ((h.grad.float(), dh), (got_dw, dw)):
+        err = (got - want).abs()
+        assert err.max().item() <= 2e-2 * want.abs().max().item(), (int(err.argmax()) % H, err.max().item())
