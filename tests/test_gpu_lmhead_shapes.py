@@ -110,3 +110,37 @@ def test_hidden_sizes_tiled_224_wide_elementwise(dev, H, save_probs, accumulate)
     for got, want in ((h.grad.float(), dh), (got_dw, dw)):
         err = (got - want).abs()
         assert err.max().item() <= 2e-2 * want.abs().max().item(), (int(err.argmax()) % H, err.max().item())
+
+
+# (hidden size, vocabulary) of published model families, at a ragged 1.5 token tiles.
+MODEL_SHAPES = [
+    (1024, 151936),   # Qwen3-0.6B
+    (2048, 151936),   # Qwen3-1.7B
+    (2560, 151936),   # Qwen3-4B
+    (3584, 152064),   # Qwen2.5-7B
+    (5120, 152064),   # Qwen2.5-14B / 32B
+    (4096, 128256),   # Llama-3-8B
+    (8192, 128256),   # Llama-3-70B
+]
+
+
+@pytest.mark.parametrize("save_probs", [True, False], ids=["saved", "recompute"])
+@pytest.mark.parametrize("H,V", MODEL_SHAPES)
+def test_model_family_shapes(dev, H, V, save_probs):
+    """Hidden sizes and vocabularies of common model families run and agree with fp32 torch (the
+    launch plan depends on both: tile counts, splits of the contraction, the last partial round)."""
+    T = 384
+    g = torch.Generator(device=dev).manual_seed(H + V)  # on the device: the weight has up to 1 G entries
+    hidden = torch.randn(T, H, generator=g, device=dev).bfloat16()
+    weight = (torch.randn(V, H, generator=g, device=dev) * (2.0 / H ** 0.5)).bfloat16()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    grad = torch.randn(T, generator=g, device=dev)
+    h = hidden.clone().requires_grad_(True)
+    w = weight.clone().requires_grad_(True)
+    out = fused_lm_head_logprobs_entropy(h, w, labels, save_probs=save_probs)
+    (out.logprobs * grad).sum().backward()
+    lp, ent, _, _, dh, dw = _reference(hidden, weight, labels, grad, 1.0, 1.0)
+    assert (out.logprobs.detach() - lp).abs().max().item() < 2e-3
+    assert (out.entropy - ent).abs().max().item() < 2e-3
+    assert _rel(h.grad.float(), dh) < 1e-2
+    assert _rel(w.grad.float(), dw) < 1e-2
