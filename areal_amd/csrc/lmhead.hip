@@ -59,6 +59,8 @@ struct GemmArgs {
   // is rows [M - 256, M) (it overlaps its predecessor) instead of a ragged tile; the epilogue is
   // told which of its rows are new. Needs M >= 256.
   int overlap_last_a;
+  // Workgroups per super-block of the schedule (32 or 8; 0 = 32), see Sched.
+  int sb_wgs;
 };
 DEVI bool gate_closed(const int* flag, int run_if_set) {
   return flag != nullptr && ((*flag != 0) != (run_if_set != 0));
@@ -68,20 +70,22 @@ DEVI bool gemm_skipped(const GemmArgs& g) { return gate_closed(g.skip_if_set, g.
 // Mapping of workgroup ids onto (B tile, A-range split). Workgroup ids go round-robin over
 // the 8 XCDs, so the 32 workgroups resident on one XCD are id = xcd + 8*q for 32 consecutive
 // q. They are laid out as an RB x RS block of (B tiles) x (splits) so that they share operand
-// tiles through that XCD's L2.
+// tiles through that XCD's L2. A launch with fewer workgroups than the chip has CUs can use
+// super-blocks of 8 instead, which spread over the XCDs more evenly (several share an XCD's round).
 struct Sched {
   int bj0, nbj;  // B tiles [bj0, bj0 + nbj)
   int ai0, nai;  // A tiles [ai0, ai0 + nai)
   int S;         // splits of the A-tile range
-  int RB, RS;    // RB * RS == 32
+  int RB, RS;    // RB * RS == 1 << sb_log2
+  int sb_log2;   // log2 of the workgroups per super-block: 5 or 3
   int n_sb_j;    // super-blocks along j
   int n_sb;      // total super-blocks
 };
 
 DEVI bool sched_decode(const Sched& sc, int id, int& bj, int& split, int& ai_begin, int& ai_end) {
   const int xcd = id & 7, q = id >> 3;
-  const int sb = (q >> 5) * 8 + xcd;
-  const int r = q & 31;
+  const int sb = (q >> sc.sb_log2) * 8 + xcd;
+  const int r = q & ((1 << sc.sb_log2) - 1);
   if (sb >= sc.n_sb) return false;
   const int sbj = sb % sc.n_sb_j, sbs = sb / sc.n_sb_j;
   const int bl = sbj * sc.RB + (r % sc.RB);
@@ -93,17 +97,20 @@ DEVI bool sched_decode(const Sched& sc, int id, int& bj, int& split, int& ai_beg
   return ai_begin < ai_end;
 }
 
-static Sched make_sched(int bj0, int nbj, int ai0, int nai, int S) {
+static Sched make_sched(int bj0, int nbj, int ai0, int nai, int S, int sb_wgs = 32) {
   Sched sc;
   sc.bj0 = bj0; sc.nbj = nbj; sc.ai0 = ai0; sc.nai = nai; sc.S = S;
+  sc.sb_log2 = sb_wgs == 8 ? 3 : 5;
+  const int rs_max = sb_wgs == 8 ? 4 : 8;
   sc.RS = S >= 8 ? 8 : (S >= 4 ? 4 : (S >= 2 ? 2 : 1));
-  sc.RB = 32 / sc.RS;
+  if (sc.RS > rs_max) sc.RS = rs_max;
+  sc.RB = (1 << sc.sb_log2) / sc.RS;
   sc.n_sb_j = (nbj + sc.RB - 1) / sc.RB;
   const int n_sb_s = (S + sc.RS - 1) / sc.RS;
   sc.n_sb = sc.n_sb_j * n_sb_s;
   return sc;
 }
-static int sched_grid(const Sched& sc) { return ((sc.n_sb + 7) / 8) * 8 * 32; }
+static int sched_grid(const Sched& sc) { return ((sc.n_sb + 7) / 8) * 8 * (1 << sc.sb_log2); }
 
 // ---------------------------------------------------------------------------------------
 // Main loop pieces
@@ -1005,7 +1012,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm16_sweep(GemmArgs g, Sched sc, t
   int bj, split, ai_begin, ai_end;
   int wg = blockIdx.x, nk = g.K / BK;
   if (g.ksplit > 1) {
-    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 256
+    const int per_copy = gridDim.x / g.ksplit;  // a multiple of 8 super-blocks
     const int z = wg / per_copy;
     wg -= z * per_copy;
     wg = (wg & ~7) | ((wg - z * sc.n_sb) & 7);  // copies start on different XCDs
@@ -1558,7 +1565,7 @@ int launch_region(const GemmArgs& g, int bj0, int nbj, int ai0, int nai, int S,
   if (nbj <= 0 || nai <= 0) return AREAL_OK;
   if (S > nai) S = nai;
   if (S < 1) S = 1;
-  const Sched sc = make_sched(bj0, nbj, ai0, nai, S);
+  const Sched sc = make_sched(bj0, nbj, ai0, nai, S, g.sb_wgs == 8 ? 8 : 32);
   if constexpr (KERNEL >= KERNEL16_NT) {
     constexpr int VAR = KERNEL == KERNEL16_NT ? VAR_NT : KERNEL == KERNEL16_TN ? VAR_TN : VAR_MIX;
     // the loader addresses a tile as a 64-bit base plus 32-bit byte offsets per lane
@@ -1807,10 +1814,11 @@ struct DwTail {
   int nbj_main;  // B tiles of the first launch
   int z, kps;    // copies and k-tiles per copy of the second (z <= 1: there is none)
   int64_t rows;  // vocabulary rows of the second launch
+  int sb_wgs;    // workgroups per super-block of the second launch's schedule
 };
 DwTail plan_dw_tail(int64_t H, int64_t V, int64_t Tpad) {
   const int nai = (int)ceil_div_i64(H, TILE), nbj = (int)ceil_div_i64(V, TILE);
-  DwTail t{nbj, 1, 0, 0};
+  DwTail t{nbj, 1, 0, 0, 32};
   if (!k16_ok(Tpad) || H % 8 != 0) return t;
   const Sched sc = make_sched(0, nbj, 0, nai, nai);
   if (sc.n_sb % 8 == 0) return t;
@@ -1818,13 +1826,15 @@ DwTail plan_dw_tail(int64_t H, int64_t V, int64_t Tpad) {
   int nj = sc.n_sb_j;
   while (nj > 0 && (nj * n_sb_s) % 8 != 0) --nj;
   if (nj == 0) return t;
-  const Sched st = make_sched(nj * sc.RB, nbj - nj * sc.RB, 0, nai, nai);
   const int64_t nk = Tpad / BK;
-  int best = 1;
-  double best_cost = sched_cost(st, 1);
-  for (int z = 2; z <= 8 && z <= nk / 8; ++z) {
-    const double cost = sched_cost(st, z);
-    if (cost < best_cost - 1e-9) { best_cost = cost; best = z; }
+  int best = 1, best_sb = 32;
+  double best_cost = sched_cost(make_sched(nj * sc.RB, nbj - nj * sc.RB, 0, nai, nai), 1);
+  for (int sb_wgs = 32; sb_wgs >= 8; sb_wgs -= 24) {
+    const Sched st = make_sched(nj * sc.RB, nbj - nj * sc.RB, 0, nai, nai, sb_wgs);
+    for (int z = 2; z <= 8 && z <= nk / 8; ++z) {
+      const double cost = sched_cost(st, z);
+      if (cost < best_cost - 1e-9) { best_cost = cost; best = z; best_sb = sb_wgs; }
+    }
   }
   // rounds of a whole K range: before, and after with the first launch's even rounds. A k-tile
   // takes about a microsecond; the two extra launches have to be paid for.
@@ -1832,9 +1842,10 @@ DwTail plan_dw_tail(int64_t H, int64_t V, int64_t Tpad) {
   if (best <= 1 || (before - after) * (double)nk < 16.0) return t;
   t.nbj_main = nj * sc.RB;
   t.z = best;
+  t.sb_wgs = best_sb;
   split_ktiles((int)nk, t.z, t.kps);
   t.rows = V - (int64_t)t.nbj_main * TILE;
-  if (t.z <= 1) t = DwTail{nbj, 1, 0, 0};
+  if (t.z <= 1) t = DwTail{nbj, 1, 0, 0, 32};
   return t;
 }
 size_t dw_tail_bytes(int64_t H, int64_t V, int64_t Tpad) {
@@ -1848,7 +1859,7 @@ size_t dw_tail_bytes(int64_t H, int64_t V, int64_t Tpad) {
 int launch_dweight_bf16(GemmArgs g, int64_t H, int64_t V, int64_t ldv, void* dweight, float* dw_part,
                         hipStream_t stream) {
   const int64_t K = g.K;
-  const DwTail tail = dw_part != nullptr ? plan_dw_tail(H, V, K) : DwTail{0, 1, 0, 0};
+  const DwTail tail = dw_part != nullptr ? plan_dw_tail(H, V, K) : DwTail{0, 1, 0, 0, 32};
   int rc;
   if (tail.z <= 1) {
     const StoreParams ep{dweight, H, (int)H, (int)V, nullptr};
@@ -1866,6 +1877,7 @@ int launch_dweight_bf16(GemmArgs g, int64_t H, int64_t V, int64_t ldv, void* dwe
   gt.bcols = (int)(ldv - v0);
   gt.ksplit = tail.z;
   gt.kt_per_split = tail.kps;
+  gt.sb_wgs = tail.sb_wgs;
   gt.zstride = tail.rows * H * (int64_t)sizeof(float);
   const StoreParams ept{dw_part, H, (int)H, (int)tail.rows, nullptr};
   rc = launch_store<KERNEL16_TN>(gt, ept, 1, stream);
